@@ -1,0 +1,201 @@
+/*
+ * litekv.h -- C ABI of liblitekv.so: the paged-KV-cache attention path of
+ * lite_llama, written for one AMD Instinct MI355X (gfx950).
+ *
+ * Conventions shared by every entry point
+ *   - every pointer is a DEVICE pointer, 16-byte aligned, owned by the caller;
+ *     the library never allocates, frees or synchronises;
+ *   - calls only enqueue work on `stream` (a hipStream_t passed as void*;
+ *     NULL is the default stream) and return at once;
+ *   - the return value is a status: LITEKV_OK, or non-zero with a message
+ *     readable through litekv_last_error() (thread local);
+ *   - launch shapes depend only on the host scalars passed in, never on device
+ *     data, so a call sequence can be recorded once and replayed;
+ *   - data is fp16 ("half"), indices are int32, element strides are in
+ *     elements (not bytes) and passed as int64.
+ *
+ * KV pool layout (one per layer), identical to the reference's
+ * `gpu_kv_buffer[l]` (lite_llama/executor/paged_attention.py:54-62):
+ *     kv_pool[num_pages * page_size][2 * num_kv_heads][head_dim]  fp16
+ * heads [0, Hkv) of a slot are K, heads [Hkv, 2*Hkv) are V
+ * (lite_llama/models/qwen3.py:68-69). slot = page_id * page_size + offset
+ * (lite_llama/executor/paged_attention.py:141-146, 347-354), so a page is one
+ * contiguous run of page_size * 2 * Hkv * head_dim * 2 bytes.
+ *
+ * Supported shapes: head_dim == 128, page_size == 16, Hq % Hkv == 0,
+ * Hq / Hkv <= 16.
+ */
+#ifndef LITEKV_H
+#define LITEKV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LITEKV_OK 0
+#define LITEKV_ERR_INVALID_ARGUMENT 1
+#define LITEKV_ERR_LAUNCH 2
+
+#define LITEKV_ABI_VERSION 1
+
+/* ABI version of the loaded library (LITEKV_ABI_VERSION at build time). */
+int litekv_abi_version(void);
+
+/* Message of the last failing call made by this thread ("" if none). */
+const char *litekv_last_error(void);
+
+/*
+ * KV append. Replaces `update_kv_buffer(KV_Values, Select_Index, KV_Buffer)`
+ * (lite_llama/kernels/update_kv_buffer.py:46-81) together with the
+ * `torch.cat([xk, xv], dim=-2)` its callers run first
+ * (lite_llama/models/qwen3.py:29, 62):
+ *     kv_pool[slot_mapping[t]][0:Hkv]     = k[t]
+ *     kv_pool[slot_mapping[t]][Hkv:2*Hkv] = v[t]      for t in [0, num_tokens)
+ * k and v are [num_tokens][Hkv][head_dim] with the given token strides (the
+ * inner [Hkv][head_dim] block contiguous), so the two halves of an already
+ * concatenated [T][2*Hkv][D] tensor can be passed without a copy.
+ * A slot outside [0, num_slots) is skipped (padding rows of a replayed batch).
+ * The copy is bit exact.
+ */
+int litekv_kv_append(const void *k, const void *v,
+                     int64_t k_token_stride, int64_t v_token_stride,
+                     const int32_t *slot_mapping, void *kv_pool,
+                     int32_t num_tokens, int32_t num_kv_heads, int32_t head_dim,
+                     int64_t num_slots, void *stream);
+
+/*
+ * Page gather / page copy. The reference has no page-move operation (its
+ * allocator never moves KV: lite_llama/executor/paged_attention.py:1-11);
+ * these serve copy-on-write of a shared page and pool compaction:
+ *     dst_pool[page dst_ids[i]] = src_pool[page src_ids[i]]   for i in [0, n)
+ * dst_ids == NULL means dst page i. page_bytes must be a multiple of 16.
+ * src_pool may equal dst_pool (litekv_page_copy) provided no destination page
+ * is also a source page of a different move and destinations are distinct.
+ * Ids outside [0, num_src_pages) / [0, num_dst_pages) are skipped. Bit exact.
+ */
+int litekv_page_gather(const void *src_pool, void *dst_pool,
+                       const int32_t *src_ids, const int32_t *dst_ids,
+                       int32_t n, int64_t page_bytes,
+                       int64_t num_src_pages, int64_t num_dst_pages,
+                       void *stream);
+
+int litekv_page_copy(void *kv_pool, const int32_t *src_ids,
+                     const int32_t *dst_ids, int32_t n, int64_t page_bytes,
+                     int64_t num_pages, void *stream);
+
+/*
+ * Paged flash-decoding. Replaces `flash_decoding(q, k_cache, v_cache,
+ * qk_scale, b_req_tokens_table, b_seq_len, max_actual_seq_len)`
+ * (lite_llama/kernels/flashdecoding.py:294-342; stage 1 :6-138, stage 2
+ * :199-267):  out[b][h] = softmax(q[b][h] . K_b[h / (Hq/Hkv)]^T * scale) V_b,
+ * over the seq_lens[b] tokens of sequence b, whose token t lives in page
+ * block_table[b][t / page_size] at offset t % page_size.
+ *
+ *   q            [B][Hq][D] fp16, batch stride q_batch_stride, heads contiguous
+ *   block_table  [B][block_table_stride] int32 page ids (the per-page
+ *                equivalent of the reference's per-token
+ *                b_req_tokens_table, paged_attention.py:166-170)
+ *   seq_lens     [B] int32, tokens to attend over (already counting the token
+ *                appended this step, model_executor.py:893-911); 0 gives zeros
+ *   out          [B][Hq][D] fp16, contiguous
+ *   max_splits   S >= 1: upper bound of KV splits per sequence = grid extent
+ *   min_pages_per_split  sequence b uses
+ *                n_b = clamp(ceil(pages_b / min_pages_per_split), 1, S) splits
+ *                with page boundaries floor(s * pages_b / n_b): a pure function
+ *                of (seq_lens[b], S, min_pages_per_split), so results do not
+ *                depend on timing
+ *   workspace    litekv_paged_decode_workspace_bytes(B, Hq, D, S) bytes:
+ *                fp32 partial outputs [B][Hq][S][D] then natural-log
+ *                log-sum-exp [B][Hq][S] (the reference's mid_o /
+ *                mid_o_logexpsum, flashdecoding.py:310-321); may be NULL when
+ *                S == 1
+ *   softmax_scale natural scale (1/sqrt(D)); exp, not exp2, semantics
+ * Two launches: split kernel, then the merge in split-index order.
+ */
+size_t litekv_paged_decode_workspace_bytes(int32_t batch, int32_t num_q_heads,
+                                           int32_t head_dim, int32_t max_splits);
+
+int litekv_paged_decode(const void *q, int64_t q_batch_stride,
+                        const void *kv_pool, const int32_t *block_table,
+                        int32_t block_table_stride, const int32_t *seq_lens,
+                        void *out, void *workspace, size_t workspace_bytes,
+                        int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                        int32_t head_dim, int32_t page_size, int64_t num_pages,
+                        int32_t max_splits, int32_t min_pages_per_split,
+                        float softmax_scale, void *stream);
+
+/*
+ * The two stages of litekv_paged_decode on their own (same arguments), for
+ * callers that time or schedule them separately
+ * (flash_decode_stage1 / flash_decode_stage2, flashdecoding.py:141-196,
+ * 270-291).
+ */
+int litekv_paged_decode_split(const void *q, int64_t q_batch_stride,
+                              const void *kv_pool, const int32_t *block_table,
+                              int32_t block_table_stride, const int32_t *seq_lens,
+                              void *out, void *workspace, size_t workspace_bytes,
+                              int32_t batch, int32_t num_q_heads,
+                              int32_t num_kv_heads, int32_t head_dim,
+                              int32_t page_size, int64_t num_pages,
+                              int32_t max_splits, int32_t min_pages_per_split,
+                              float softmax_scale, void *stream);
+
+int litekv_paged_decode_merge(const int32_t *seq_lens, void *out,
+                              const void *workspace, size_t workspace_bytes,
+                              int32_t batch, int32_t num_q_heads,
+                              int32_t head_dim, int32_t page_size,
+                              int32_t max_splits, int32_t min_pages_per_split,
+                              void *stream);
+
+/*
+ * Varlen causal prefill over paged KV. Replaces
+ * `paged_chunk_flash_attention(q, k_cache, v_cache, sm_scale, req_token_table,
+ * req_ids, q_start_loc, context_lens, q_seq_lens, max_q_len)`
+ * (lite_llama/kernels/paged_chunk_flashattention.py:225-327, kernel :58-176):
+ * query row m of sequence b sits at logical position context_lens[b] + m and
+ * attends to keys 0 .. context_lens[b] + m read through block_table[b].
+ * With context_lens == NULL (all zero) it is the paged form of
+ * `flash_attention2_no_pad` (lite_llama/kernels/flashattention2_nopad.py:169-221).
+ *
+ *   q, out        [T][Hq][D] fp16 packed rows, token strides given
+ *   cu_q_lens     [B+1] int32, rows of sequence b are
+ *                 [cu_q_lens[b], cu_q_lens[b+1])
+ *   context_lens  [B] int32 or NULL
+ *   max_q_len     host upper bound of the per-sequence query length (grid)
+ *   softmax_scale natural scale; callers holding the reference's
+ *                 log2(e)-folded scale (lite_llama/models/qwen3.py:295-298)
+ *                 divide it out first
+ */
+int litekv_paged_prefill(const void *q, int64_t q_token_stride,
+                         const void *kv_pool, const int32_t *block_table,
+                         int32_t block_table_stride, const int32_t *cu_q_lens,
+                         const int32_t *context_lens, void *out,
+                         int64_t out_token_stride, int32_t batch,
+                         int32_t num_q_heads, int32_t num_kv_heads,
+                         int32_t head_dim, int32_t page_size, int64_t num_pages,
+                         int32_t max_q_len, float softmax_scale, void *stream);
+
+/*
+ * Varlen causal prefill over packed contiguous K/V. Replaces
+ * `flash_attention2_no_pad(q, k, v, sm_scale, b_start_loc, b_seq_len,
+ * max_seq_len)` (lite_llama/kernels/flashattention2_nopad.py:169-221) for
+ * callers that hold the fresh K/V rows rather than pages
+ * (lite_llama/models/qwen3.py:47-50).
+ *   q, out [T][Hq][D]; k, v [T][Hkv][D]; seq_starts, seq_lens [B] int32
+ */
+int litekv_varlen_prefill(const void *q, int64_t q_token_stride,
+                          const void *k, int64_t k_token_stride,
+                          const void *v, int64_t v_token_stride,
+                          const int32_t *seq_starts, const int32_t *seq_lens,
+                          void *out, int64_t out_token_stride, int32_t batch,
+                          int32_t num_q_heads, int32_t num_kv_heads,
+                          int32_t head_dim, int32_t max_seq_len,
+                          int64_t num_tokens, float softmax_scale, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LITEKV_H */

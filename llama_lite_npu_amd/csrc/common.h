@@ -1,0 +1,61 @@
+// Shared declarations of liblitekv: vector types, MFMA fragment helpers,
+// host-side argument checks and the thread-local error string.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/litekv.h"
+
+namespace litekv {
+
+typedef _Float16 half_t;
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kHeadDim = 128;   // elements per head row (256 bytes of fp16)
+constexpr int kPageSize = 16;   // tokens per page
+constexpr int kWave = 64;       // lanes per wavefront on CDNA
+
+// ---- host side -----------------------------------------------------------
+
+// Records `msg` as this thread's last error and returns `code`.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void clear_error();
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Turns the status of the launch just issued into an ABI status.
+int check_launch(const char *what);
+
+#define LITEKV_REQUIRE(cond, ...)                                         \
+  do {                                                                    \
+    if (!(cond)) return ::litekv::fail(LITEKV_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
+  } while (0)
+
+// ---- device side ---------------------------------------------------------
+
+// 2^x on the transcendental unit (v_exp_f32); exp2(-inf) == 0.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// Value held by lane (lane ^ mask) of the same wavefront.
+__device__ __forceinline__ float xor_lane(float v, int mask) { return __shfl_xor(v, mask, kWave); }
+
+// D(16x16) += A(16x32) * B(32x16), fp16 inputs, fp32 accumulate.
+// Lane l supplies A[l % 16][8*(l/16) .. +7] and B[8*(l/16) .. +7][l % 16];
+// it receives D[4*(l/16) + i][l % 16] in element i.
+__device__ __forceinline__ float4_t mfma_16x16x32(half8_t a, half8_t b, float4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+// D(16x16) += A(16x16) * B(16x16): lane l supplies A[l % 16][4*(l/16) .. +3] and
+// B[4*(l/16) .. +3][l % 16]; D as above.
+__device__ __forceinline__ float4_t mfma_16x16x16(half4_t a, half4_t b, float4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0);
+}
+
+}  // namespace litekv

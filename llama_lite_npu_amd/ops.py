@@ -1,0 +1,225 @@
+"""Block-table-native operators over liblitekv (PyTorch-ROCm tensors in, C ABI out).
+
+PyTorch supplies device memory and the current stream; every byte of the path
+is moved or computed by the HIP kernels behind include/litekv.h. All calls only
+enqueue work on ``torch.cuda.current_stream()``.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+PAGE_SIZE = 16
+HEAD_DIM = 128
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _dev_half(name: str, t: torch.Tensor) -> None:
+    _need(t.is_cuda, f"{name} must live on the GPU")
+    _need(t.dtype == torch.float16, f"{name} must be float16, got {t.dtype}")
+
+
+def _dev_i32(name: str, t: torch.Tensor) -> torch.Tensor:
+    _need(t.is_cuda, f"{name} must live on the GPU")
+    if t.dtype != torch.int32:
+        t = t.to(torch.int32)  # device-side cast, no host sync
+    return t.contiguous()
+
+
+def _rows(name: str, t: torch.Tensor) -> int:
+    """Token stride of a [T, H, D] tensor whose [H, D] block is contiguous."""
+    _need(t.dim() == 3, f"{name} must be [tokens, heads, head_dim]")
+    _need(t.stride(2) == 1 and t.stride(1) == t.shape[2], f"{name}: [heads, head_dim] block must be contiguous")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1] * t.shape[2])
+
+
+def pool_geometry(kv_pool: torch.Tensor, page_size: int = PAGE_SIZE):
+    """(num_slots, num_kv_heads, head_dim, num_pages, page_bytes) of a [slots, 2*Hkv, D] pool."""
+    _need(kv_pool.dim() == 3 and kv_pool.is_contiguous(), "kv_pool must be contiguous [slots, 2*Hkv, D]")
+    slots, two_h, d = kv_pool.shape
+    _need(two_h % 2 == 0, "kv_pool dim 1 must be 2 * num_kv_heads")
+    _need(slots % page_size == 0, "kv_pool slots must be a multiple of page_size")
+    return slots, two_h // 2, d, slots // page_size, page_size * two_h * d * kv_pool.element_size()
+
+
+def kv_append(k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor, kv_pool: torch.Tensor) -> None:
+    """kv_pool[slot_mapping[t]] = concat(k[t], v[t]) for every token t (bit exact, in place)."""
+    _dev_half("k", k), _dev_half("v", v), _dev_half("kv_pool", kv_pool)
+    slots, hkv, d, _, _ = pool_geometry(kv_pool, 1)
+    _need(k.shape == v.shape, "k and v must have the same shape")
+    _need(k.shape[1] == hkv and k.shape[2] == d, f"k/v heads {tuple(k.shape[1:])} do not match pool ({hkv}, {d})")
+    slot_mapping = _dev_i32("slot_mapping", slot_mapping)
+    t = k.shape[0]
+    _need(slot_mapping.numel() == t, "slot_mapping must hold one slot per token")
+    lib = _lib.load()
+    _lib.check(lib.litekv_kv_append(_ptr(k), _ptr(v), _rows("k", k), _rows("v", v), _ptr(slot_mapping),
+                                    _ptr(kv_pool), t, hkv, d, slots, _stream()))
+
+
+def page_gather(src_pool: torch.Tensor, dst_pool: torch.Tensor, src_ids: torch.Tensor,
+                dst_ids: Optional[torch.Tensor] = None, page_size: int = PAGE_SIZE) -> None:
+    """dst_pool[page dst_ids[i]] = src_pool[page src_ids[i]]; dst_ids None means page i."""
+    _dev_half("src_pool", src_pool), _dev_half("dst_pool", dst_pool)
+    _, hs, ds, n_src, page_bytes = pool_geometry(src_pool, page_size)
+    _, hd, dd, n_dst, page_bytes_d = pool_geometry(dst_pool, page_size)
+    _need((hs, ds) == (hd, dd) and page_bytes == page_bytes_d, "pools differ in page geometry")
+    src_ids = _dev_i32("src_ids", src_ids)
+    if dst_ids is not None:
+        dst_ids = _dev_i32("dst_ids", dst_ids)
+        _need(dst_ids.numel() == src_ids.numel(), "src_ids and dst_ids differ in length")
+    lib = _lib.load()
+    _lib.check(lib.litekv_page_gather(_ptr(src_pool), _ptr(dst_pool), _ptr(src_ids), _ptr(dst_ids),
+                                      src_ids.numel(), page_bytes, n_src, n_dst, _stream()))
+
+
+def page_copy(kv_pool: torch.Tensor, src_ids: torch.Tensor, dst_ids: torch.Tensor,
+              page_size: int = PAGE_SIZE) -> None:
+    """kv_pool[page dst_ids[i]] = kv_pool[page src_ids[i]] (copy-on-write move inside one pool)."""
+    _dev_half("kv_pool", kv_pool)
+    _, _, _, n_pages, page_bytes = pool_geometry(kv_pool, page_size)
+    src_ids = _dev_i32("src_ids", src_ids)
+    dst_ids = _dev_i32("dst_ids", dst_ids)
+    _need(dst_ids.numel() == src_ids.numel(), "src_ids and dst_ids differ in length")
+    lib = _lib.load()
+    _lib.check(lib.litekv_page_copy(_ptr(kv_pool), _ptr(src_ids), _ptr(dst_ids), src_ids.numel(),
+                                    page_bytes, n_pages, _stream()))
+
+
+def decode_split_plan(batch: int, num_kv_heads: int, max_blocks: int,
+                      num_splits: Optional[int] = None) -> tuple[int, int]:
+    """(max_splits, min_pages_per_split) for a decode launch.
+
+    ``num_splits`` fixes the split count per sequence (every sequence with at
+    least that many pages uses exactly that many). Otherwise pages per split
+    are chosen so the launch has a few thousand wavefronts of at least 8 pages.
+    """
+    if num_splits is not None:
+        return max(1, int(num_splits)), 1
+    items = max(1, batch * num_kv_heads)
+    target_waves = 4096
+    pps = max(8, min(64, (items * max_blocks + target_waves - 1) // target_waves))
+    return max(1, (max_blocks + pps - 1) // pps), pps
+
+
+def decode_workspace(batch: int, num_q_heads: int, max_splits: int, device) -> Optional[torch.Tensor]:
+    nbytes = _lib.load().litekv_paged_decode_workspace_bytes(batch, num_q_heads, HEAD_DIM, max_splits)
+    if nbytes == 0:
+        return None
+    return torch.empty(nbytes // 4, dtype=torch.float32, device=device)
+
+
+def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tensor,
+                 seq_lens: torch.Tensor, softmax_scale: Optional[float] = None,
+                 num_splits: Optional[int] = None, min_pages_per_split: Optional[int] = None,
+                 max_splits: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                 workspace: Optional[torch.Tensor] = None, page_size: int = PAGE_SIZE,
+                 stage: str = "both") -> torch.Tensor:
+    """Decode attention of q [B, Hq, D] over the pages named by block_table [B, max_blocks]."""
+    _dev_half("q", q), _dev_half("kv_pool", kv_pool)
+    _need(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2], "q must be [B, Hq, D] with contiguous heads")
+    b, hq, d = q.shape
+    _, hkv, dk, n_pages, _ = pool_geometry(kv_pool, page_size)
+    _need(d == dk, "q and kv_pool differ in head_dim")
+    _need(block_table.dim() == 2 and block_table.shape[0] == b, "block_table must be [B, max_blocks]")
+    block_table = _dev_i32("block_table", block_table)
+    seq_lens = _dev_i32("seq_lens", seq_lens)
+    _need(seq_lens.numel() == b, "seq_lens must be [B]")
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    if max_splits is None or min_pages_per_split is None:
+        s, pps = decode_split_plan(b, hkv, block_table.shape[1], num_splits)
+        max_splits = s if max_splits is None else max_splits
+        min_pages_per_split = pps if min_pages_per_split is None else min_pages_per_split
+    if out is None:
+        out = torch.empty((b, hq, d), dtype=torch.float16, device=q.device)
+    else:
+        _dev_half("out", out)
+        _need(out.shape == (b, hq, d) and out.is_contiguous(), "out must be contiguous [B, Hq, D]")
+    if workspace is None:
+        workspace = decode_workspace(b, hq, max_splits, q.device)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    lib = _lib.load()
+    q_stride = q.stride(0) if b > 1 else max(q.stride(0), hq * d)
+    if stage in ("both", "split"):
+        fn = lib.litekv_paged_decode if stage == "both" else lib.litekv_paged_decode_split
+        _lib.check(fn(_ptr(q), q_stride, _ptr(kv_pool), _ptr(block_table), block_table.stride(0),
+                      _ptr(seq_lens), _ptr(out), _ptr(workspace), ws_bytes, b, hq, hkv, d, page_size,
+                      n_pages, max_splits, min_pages_per_split, float(softmax_scale), _stream()))
+    elif stage == "merge":
+        _lib.check(lib.litekv_paged_decode_merge(_ptr(seq_lens), _ptr(out), _ptr(workspace), ws_bytes, b,
+                                                 hq, d, page_size, max_splits, min_pages_per_split,
+                                                 _stream()))
+    else:
+        raise ValueError(f"unknown stage {stage!r}")
+    return out
+
+
+def paged_prefill(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tensor,
+                  cu_q_lens: torch.Tensor, context_lens: Optional[torch.Tensor], max_q_len: int,
+                  softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
+                  page_size: int = PAGE_SIZE) -> torch.Tensor:
+    """Causal varlen attention of packed q [T, Hq, D] over paged KV (history + the chunk itself)."""
+    _dev_half("q", q), _dev_half("kv_pool", kv_pool)
+    q_stride = _rows("q", q)
+    t, hq, d = q.shape
+    _, hkv, dk, n_pages, _ = pool_geometry(kv_pool, page_size)
+    _need(d == dk, "q and kv_pool differ in head_dim")
+    cu_q_lens = _dev_i32("cu_q_lens", cu_q_lens)
+    b = cu_q_lens.numel() - 1
+    _need(block_table.dim() == 2 and block_table.shape[0] == b, "block_table must be [B, max_blocks]")
+    block_table = _dev_i32("block_table", block_table)
+    if context_lens is not None:
+        context_lens = _dev_i32("context_lens", context_lens)
+        _need(context_lens.numel() == b, "context_lens must be [B]")
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    if out is None:
+        out = torch.empty((t, hq, d), dtype=torch.float16, device=q.device)
+    lib = _lib.load()
+    _lib.check(lib.litekv_paged_prefill(_ptr(q), q_stride, _ptr(kv_pool), _ptr(block_table),
+                                        block_table.stride(0), _ptr(cu_q_lens), _ptr(context_lens),
+                                        _ptr(out), _rows("out", out), b, hq, hkv, d, page_size, n_pages,
+                                        int(max_q_len), float(softmax_scale), _stream()))
+    return out
+
+
+def varlen_prefill(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, seq_starts: torch.Tensor,
+                   seq_lens: torch.Tensor, max_seq_len: int, softmax_scale: Optional[float] = None,
+                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal varlen attention of packed q over packed contiguous k, v ([T, Hkv, D])."""
+    _dev_half("q", q), _dev_half("k", k), _dev_half("v", v)
+    q_stride, k_stride, v_stride = _rows("q", q), _rows("k", k), _rows("v", v)
+    t, hq, d = q.shape
+    _need(k.shape == v.shape and k.shape[0] == t and k.shape[2] == d, "k/v shape mismatch")
+    hkv = k.shape[1]
+    seq_starts = _dev_i32("seq_starts", seq_starts)
+    seq_lens = _dev_i32("seq_lens", seq_lens)
+    b = seq_lens.numel()
+    _need(seq_starts.numel() == b, "seq_starts and seq_lens differ in length")
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    if out is None:
+        out = torch.empty((t, hq, d), dtype=torch.float16, device=q.device)
+    lib = _lib.load()
+    _lib.check(lib.litekv_varlen_prefill(_ptr(q), q_stride, _ptr(k), k_stride, _ptr(v), v_stride,
+                                         _ptr(seq_starts), _ptr(seq_lens), _ptr(out), _rows("out", out),
+                                         b, hq, hkv, d, int(max_seq_len), t, float(softmax_scale),
+                                         _stream()))
+    return out

@@ -1,0 +1,142 @@
+"""GPU parity of paged flash-decoding against the CPU oracle, through the C ABI."""
+
+import numpy as np
+import pytest
+import torch
+
+from llama_lite_npu_amd import ops, workloads
+from oracle import c_oracle
+from tests.parity import assert_attention_close, to_np16
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _oracle(case, seq_lens=None):
+    sl = case.seq_lens if seq_lens is None else seq_lens
+    return c_oracle.paged_decode(to_np16(case.q), to_np16(case.kv_pool), case.block_table.cpu().numpy(),
+                                 sl.cpu().numpy(), case.softmax_scale)
+
+
+def _run(case, **kw):
+    out = ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, case.softmax_scale, **kw)
+    torch.cuda.synchronize()
+    return out
+
+
+def test_c1_append_then_decode():
+    print("decode C1", flush=True)
+    case = workloads.config_c1(DEV)
+    ops.kv_append(case.k_new, case.v_new, case.slot_mapping, case.kv_pool)
+    ref = _oracle(case)
+    for kw in ({}, {"num_splits": 1}, {"num_splits": 4}, {"max_splits": 8, "min_pages_per_split": 8}):
+        print("  ", kw, flush=True)
+        assert_attention_close(_run(case, **kw), ref, f"C1 {kw}")
+
+
+@pytest.mark.parametrize("hq,hkv", [(16, 8), (64, 8), (32, 4), (8, 8), (16, 1), (4, 2)])
+def test_head_layouts_and_ragged_lengths(hq, hkv):
+    print(f"decode heads {hq}/{hkv}", flush=True)
+    lens = [0, 1, 15, 16, 17, 255, 256, 700]  # context; +1 appended => 1, 2, 16, 17, 18, ...
+    case = workloads.make_decode_case("ragged", 50 + hq + hkv, lens, hq, hkv, device=DEV)
+    ref = _oracle(case)
+    for kw in ({"num_splits": 1}, {"num_splits": 3}, {"max_splits": 16, "min_pages_per_split": 2}):
+        assert_attention_close(_run(case, **kw), ref, f"ragged {hq}/{hkv} {kw}")
+
+
+def test_zero_length_sequence_gives_zeros():
+    print("decode zero length", flush=True)
+    case = workloads.make_decode_case("zero", 77, [40, 3, 90], 16, 8, device=DEV)
+    case.seq_lens[1] = 0
+    ref = _oracle(case)
+    for kw in ({"num_splits": 1}, {"num_splits": 4}):
+        out = _run(case, **kw)
+        assert_attention_close(out, ref, f"zero {kw}")
+        assert float(out[1].abs().max()) == 0.0
+
+
+def test_split_count_and_page_permutation_invariance():
+    """Same logical KV under another physical page assignment and any split count."""
+    print("decode invariance", flush=True)
+    case = workloads.make_decode_case("inv", 91, [1500, 333, 2047, 64], 64, 8, device=DEV)
+    ref = _oracle(case)
+    base = _run(case, num_splits=1)
+    assert_attention_close(base, ref, "inv base")
+    for s in (2, 5, 16, 200):
+        out = _run(case, num_splits=s)
+        assert_attention_close(out, ref, f"inv splits={s}")
+        assert float((out.float() - base.float()).abs().max()) <= 1e-3
+    # move every page to a new physical location; logical content unchanged
+    n = case.num_pages
+    perm = torch.randperm(n, generator=torch.Generator().manual_seed(5)).to(DEV)
+    pool2 = torch.empty_like(case.kv_pool)
+    pool2.view(n, -1)[perm] = case.kv_pool.view(n, -1)
+    table2 = perm[case.block_table.long()].to(torch.int32)
+    out2 = ops.paged_decode(case.q, pool2, table2, case.seq_lens, case.softmax_scale, num_splits=1)
+    torch.cuda.synchronize()
+    assert torch.equal(out2, base), "page permutation changed the result"
+
+
+def test_deterministic_bitwise():
+    print("decode determinism", flush=True)
+    case = workloads.make_decode_case("det", 93, [3000, 4096, 257, 1024] * 4, 64, 8, device=DEV)
+    a = _run(case)
+    b = _run(case)
+    assert torch.equal(a, b)
+
+
+def test_closed_forms():
+    """One token: out == v. Equal keys: out == mean(V) over the sequence."""
+    print("decode closed forms", flush=True)
+    case = workloads.make_decode_case("one", 95, [0, 0], 16, 8, device=DEV)
+    out = _run(case, num_splits=1)
+    for b in range(2):
+        slot = int(case.block_table[b, 0]) * 16
+        v = case.kv_pool[slot, 8:].float()                     # [Hkv, D]
+        want = v.repeat_interleave(2, dim=0)
+        assert float((out[b].float() - want).abs().max()) <= 1e-3
+    case = workloads.make_decode_case("mean", 96, [199], 16, 8, device=DEV)
+    n = int(case.seq_lens[0])
+    slots = (case.block_table[0].long()[torch.arange(n, device=DEV) // 16] * 16 + torch.arange(n, device=DEV) % 16)
+    case.kv_pool[slots, :8] = case.kv_pool[slots[0], :8]
+    out = _run(case, num_splits=2)
+    want = case.kv_pool[slots, 8:].float().mean(dim=0).repeat_interleave(2, dim=0)
+    assert float((out[0].float() - want).abs().max()) <= 2e-3
+
+
+def test_stages_can_be_called_separately():
+    print("decode stages", flush=True)
+    case = workloads.make_decode_case("stages", 97, [900, 2000, 100], 64, 8, device=DEV)
+    both = _run(case, max_splits=8, min_pages_per_split=4)
+    ws = ops.decode_workspace(case.batch, 64, 8, DEV)
+    out = torch.zeros_like(both)
+    ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, case.softmax_scale,
+                     max_splits=8, min_pages_per_split=4, out=out, workspace=ws, stage="split")
+    ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, case.softmax_scale,
+                     max_splits=8, min_pages_per_split=4, out=out, workspace=ws, stage="merge")
+    torch.cuda.synchronize()
+    assert torch.equal(out, both)
+
+
+def test_unwritten_tail_slots_do_not_leak():
+    """NaN/Inf bit patterns in slots past the sequence end must not reach the output."""
+    print("decode tail garbage", flush=True)
+    case = workloads.make_decode_case("tail", 98, [20, 37], 16, 8, device=DEV)
+    ref = _oracle(case)
+    for b in range(2):
+        n = int(case.seq_lens[b])
+        page = int(case.block_table[b, (n - 1) // 16])
+        case.kv_pool[page * 16 + n % 16: page * 16 + 16] = float("nan")
+    assert_attention_close(_run(case, num_splits=1), ref, "tail NaN")
+
+
+def test_invalid_arguments_raise():
+    print("decode errors", flush=True)
+    case = workloads.make_decode_case("err", 99, [10], 16, 8, device=DEV)
+    from llama_lite_npu_amd._lib import LiteKVError
+    with pytest.raises(LiteKVError, match="head_dim"):
+        ops.paged_decode(case.q[..., :64].contiguous(), case.kv_pool[..., :64].contiguous(), case.block_table,
+                         case.seq_lens)
+    with pytest.raises(LiteKVError, match="workspace"):
+        ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, max_splits=4,
+                         min_pages_per_split=1, workspace=torch.empty(4, device=DEV))
