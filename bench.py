@@ -1,0 +1,361 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged-KV attention path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--all]
+
+Default workload (config c2): Qwen3-32B attention shape, decode. A step is one
+pass over 64 layers' worth of independent KV pools: per layer one KV append of
+the batch's new tokens followed by paged flash-decoding (split + merge). All
+inputs are resident in HBM before the timed region. One JSON line is printed on
+stdout; `--all` adds one line per other configuration on stderr and in
+gpurun_out/bench_all.jsonl.
+
+`value` is algorithmic bytes of the whole step divided by its wall-clock time.
+`roofline` describes the dominant kernel (the decode split kernel): algorithmic
+bytes of one launch over its mean duration, taken from HIP events recorded
+around every one of its launches inside the timed region, on the stream the
+kernels run on. `cpu_baseline` times the PyTorch-CPU restatement of the
+reference's own torch path (oracle/cpu_ref.py) on this machine's host cores for
+one layer of the same workload.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+
+
+def _median(xs):
+    xs = sorted(xs)
+    n = len(xs)
+    return xs[n // 2] if n % 2 else 0.5 * (xs[n // 2 - 1] + xs[n // 2])
+
+
+class DecodeLayerSet:
+    """`layers` independent KV pools sharing one batch's block tables, with pre-bound launches."""
+
+    def __init__(self, case, layers: int, device: str):
+        import torch
+        from llama_lite_npu_amd import _lib, ops
+
+        self.torch = torch
+        self.case = case
+        self.layers = layers
+        lib = _lib.load()
+        self.lib = lib
+        c = case
+        b, hq, hkv = c.batch, c.num_q_heads, c.num_kv_heads
+        slots = c.num_pages * 16
+        pools = torch.empty((layers, slots, 2 * hkv, 128), dtype=torch.float16, device=device)
+        gen = torch.Generator(device=device).manual_seed(4242)
+        for l in range(layers):
+            pools[l].normal_(generator=gen)
+        self.pools = pools
+        self.q = c.q
+        self.out = torch.empty((layers, b, hq, 128), dtype=torch.float16, device=device)
+        self.max_splits, self.min_pps = ops.decode_split_plan(b, hkv, c.block_table.shape[1], c.num_splits)
+        self.ws = ops.decode_workspace(b, hq, self.max_splits, device)
+        ws_ptr = None if self.ws is None else self.ws.data_ptr()
+        ws_bytes = 0 if self.ws is None else self.ws.numel() * 4
+        self.table = c.block_table.contiguous()
+        self.seq_lens = c.seq_lens.contiguous()
+        self.slot_mapping = c.slot_mapping.contiguous()
+        stream = torch.cuda.current_stream().cuda_stream
+        self.append_args, self.split_args, self.merge_args = [], [], []
+        for l in range(layers):
+            pool_ptr = pools[l].data_ptr()
+            self.append_args.append((c.k_new.data_ptr(), c.v_new.data_ptr(), hkv * 128, hkv * 128,
+                                     self.slot_mapping.data_ptr(), pool_ptr, b, hkv, 128, slots, stream))
+            self.split_args.append((self.q.data_ptr(), hq * 128, pool_ptr, self.table.data_ptr(),
+                                    self.table.stride(0), self.seq_lens.data_ptr(), self.out[l].data_ptr(),
+                                    ws_ptr, ws_bytes, b, hq, hkv, 128, 16, c.num_pages, self.max_splits,
+                                    self.min_pps, c.softmax_scale, stream))
+            self.merge_args.append((self.seq_lens.data_ptr(), self.out[l].data_ptr(), ws_ptr, ws_bytes, b, hq,
+                                    128, 16, self.max_splits, self.min_pps, stream))
+
+    def step(self, events=None):
+        lib = self.lib
+        ap, sp, mg = lib.litekv_kv_append, lib.litekv_paged_decode_split, lib.litekv_paged_decode_merge
+        rc = 0
+        for l in range(self.layers):
+            rc |= ap(*self.append_args[l])
+            if events is not None:
+                e = events[l]
+                e[0].record()
+                rc |= sp(*self.split_args[l])
+                e[1].record()
+                rc |= mg(*self.merge_args[l])
+                e[2].record()
+            else:
+                rc |= sp(*self.split_args[l])
+                rc |= mg(*self.merge_args[l])
+        if rc:
+            raise RuntimeError(f"liblitekv launch failed: {lib.litekv_last_error().decode()}")
+
+
+def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: str) -> dict:
+    import torch
+
+    ls = DecodeLayerSet(case, layers, device)
+    for _ in range(max(1, warmup)):
+        ls.step()
+    torch.cuda.synchronize()
+    events = [[[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(layers)]
+              for _ in range(steps)]
+    # plain wall-clock region: exactly `steps` steps, synchronised on both sides
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(steps):
+        ls.step(events[s])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    split_ms, merge_ms = [], []
+    for s in range(steps):
+        for l in range(layers):
+            e = events[s][l]
+            split_ms.append(e[0].elapsed_time(e[1]))
+            merge_ms.append(e[1].elapsed_time(e[2]))
+    ms_per_step = wall * 1e3 / steps
+    decode_bytes = case.decode_bytes()
+    append_bytes = case.append_bytes()
+    step_bytes = layers * (decode_bytes + append_bytes)
+    split_mean = sum(split_ms) / len(split_ms)
+    achieved = decode_bytes / (split_mean * 1e-3) / 1e9
+    return {
+        "label": label,
+        "ms_per_step": ms_per_step,
+        "value": step_bytes / (ms_per_step * 1e-3) / 1e9,
+        "us_per_layer": ms_per_step * 1e3 / layers,
+        "decode_split_us_mean": split_mean * 1e3,
+        "decode_split_us_median": _median(split_ms) * 1e3,
+        "decode_split_us_min": min(split_ms) * 1e3,
+        "decode_merge_us_mean": sum(merge_ms) / len(merge_ms) * 1e3,
+        "decode_bytes_per_layer": decode_bytes,
+        "append_bytes_per_layer": append_bytes,
+        "layers": layers,
+        "max_splits": ls.max_splits,
+        "min_pages_per_split": ls.min_pps,
+        "roofline": {
+            "kernel": "paged_decode_split_kernel",
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": None,
+        },
+    }
+
+
+def time_append(case_tokens_k, case_tokens_v, slot_mapping, pool, reps: int = 20) -> float:
+    """Mean microseconds of one KV-append launch (HIP events on the launch stream)."""
+    import torch
+    from llama_lite_npu_amd import ops
+
+    for _ in range(3):
+        ops.kv_append(case_tokens_k, case_tokens_v, slot_mapping, pool)
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in ev:
+        a.record()
+        ops.kv_append(case_tokens_k, case_tokens_v, slot_mapping, pool)
+        b.record()
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in ev) / reps * 1e3
+
+
+def run_prefill(case, steps: int, warmup: int, device: str, label: str) -> dict:
+    import torch
+    from llama_lite_npu_amd import ops
+
+    out = torch.empty_like(case.q)
+
+    def step(ev=None):
+        ops.kv_append(case.k, case.v, case.slot_mapping, case.kv_pool)
+        if ev is not None:
+            ev[0].record()
+        ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, None, case.max_q_len,
+                          case.softmax_scale, out=out)
+        if ev is not None:
+            ev[1].record()
+
+    for _ in range(max(1, warmup)):
+        step()
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for s in range(steps):
+        step(events[s])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = [a.elapsed_time(b) for a, b in events]
+    mean_ms = sum(ms) / len(ms)
+    flops = case.flops()
+    tokens = int(case.seq_lens.sum())
+    append_us = time_append(case.k, case.v, case.slot_mapping, case.kv_pool)
+    append_bytes = tokens * (2 * 2 * case.num_kv_heads * 128 * 2 + 4)
+    achieved = flops / (mean_ms * 1e-3) / 1e12
+    return {
+        "label": label,
+        "ms_per_step": wall * 1e3 / steps,
+        "prefill_us_mean": mean_ms * 1e3,
+        "prefill_tflops": achieved,
+        "prefill_min_bytes_gbps": case.min_bytes() / (mean_ms * 1e-3) / 1e9,
+        "append_us": append_us,
+        "append_gbps": append_bytes / (append_us * 1e-6) / 1e9,
+        "tokens": tokens,
+        "flops": flops,
+        "roofline": {
+            "kernel": "varlen_prefill_kernel<paged>",
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": MFMA_FP16_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / MFMA_FP16_PEAK_TFLOPS,
+            "traffic": None,
+        },
+    }
+
+
+def cpu_baseline_decode(case, budget_s: float = 20.0) -> dict:
+    """The reference's torch CPU path (append + gathered fp32 attention) for ONE layer of `case`,
+    on the host cores: 1 warm-up + up to 3 repetitions, min taken."""
+    import torch
+    from oracle import cpu_ref
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    c = case.to("cpu")
+    kv = torch.cat([c.k_new, c.v_new], dim=1)
+    pool = c.kv_pool
+
+    def one():
+        t0 = time.perf_counter()
+        cpu_ref.kv_append_ref(kv, c.slot_mapping, pool)
+        cpu_ref.paged_decode_ref(c.q, pool, c.block_table, c.seq_lens, c.softmax_scale)
+        return time.perf_counter() - t0
+
+    first = one()
+    times = []
+    t_used = first
+    for _ in range(3):
+        if t_used > budget_s:
+            break
+        dt = one()
+        times.append(dt)
+        t_used += dt
+    best = min(times) if times else first
+    nbytes = c.decode_bytes() + c.append_bytes()
+    return {
+        "value": nbytes / best / 1e9,
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"1 of the layers of the same workload (append + decode, {nbytes / 1e6:.1f} MB algorithmic), "
+                  f"torch CPU restatement, min of {max(1, len(times))} reps after 1 warm-up, {best:.3f} s",
+        "seconds_per_layer": best,
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--layers", type=int, default=None, help="independent KV pools per step (c2 default 64)")
+    ap.add_argument("--all", action="store_true", help="also report the other configurations (stderr)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures the path on ONE GPU (one process, one device); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        return 2
+
+    import torch
+    from llama_lite_npu_amd import _lib, workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the path has no CPU implementation", file=sys.stderr)
+        return 2
+    _lib.load()
+    device = "cuda:0"
+    torch.cuda.set_device(0)
+
+    def decode_cfg(name):
+        if name == "c1":
+            return workloads.config_c1(device), (args.layers or 64)
+        if name == "c2":
+            return workloads.config_c2(device), (args.layers or 64)
+        if name == "c4":
+            return workloads.config_c4(device), (args.layers or 16)
+        if name == "c5":
+            return workloads.config_c5(device), (args.layers or 1)
+        raise ValueError(name)
+
+    def run(name):
+        if name == "c3":
+            case = workloads.config_c3(device)
+            return run_prefill(case, args.steps, args.warmup, device, case.name), case
+        case, layers = decode_cfg(name)
+        return run_decode(case, layers, args.steps, args.warmup, device, case.name), case
+
+    res, case = run(args.config)
+    line = {
+        "metric": "paged decode attn HBM GB/s (% of 8 TB/s peak); KV-append GB/s; us/layer",
+        "value": res.get("value", res.get("prefill_tflops")),
+        "unit": "GB/s" if "value" in res else "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": res["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": res["label"], "config": args.config},
+        "roofline": res["roofline"],
+        "detail": {k: v for k, v in res.items() if k not in ("roofline", "label", "value", "ms_per_step")},
+    }
+    if args.config != "c3":
+        line["config"].update(batch=case.batch, num_q_heads=case.num_q_heads, num_kv_heads=case.num_kv_heads,
+                              head_dim=128, page_size=16, layers=res["layers"],
+                              tokens_attended=int(case.seq_lens.sum()))
+        line["pct_of_hbm_peak"] = 100.0 * res["roofline"]["frac"]
+        ap_us = time_append(case.k_new, case.v_new, case.slot_mapping, case.kv_pool)
+        line["detail"]["append_us"] = ap_us
+        line["detail"]["append_gbps"] = case.append_bytes() / (ap_us * 1e-6) / 1e9
+        if not args.no_cpu_baseline:
+            line["cpu_baseline"] = cpu_baseline_decode(case)
+    print(json.dumps(line), flush=True)
+
+    if args.all:
+        out_dir = ROOT / "gpurun_out"
+        out_dir.mkdir(exist_ok=True)
+        with open(out_dir / "bench_all.jsonl", "w") as f:
+            f.write(json.dumps(line) + "\n")
+            for name in ("c1", "c2", "c3", "c4", "c5"):
+                if name == args.config:
+                    continue
+                del res, case
+                torch.cuda.empty_cache()
+                res, case = run(name)
+                f.write(json.dumps(res) + "\n")
+                f.flush()
+                print(json.dumps(res), file=sys.stderr, flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
