@@ -151,6 +151,73 @@ int litekv_paged_decode_merge(const int32_t *seq_lens, void *out,
                               void *stream);
 
 /*
+ * Paged flash-decoding, balanced schedule. Same
+ * result contract as litekv_paged_decode (it replaces the same reference
+ * function, lite_llama/kernels/flashdecoding.py:294-342), other work
+ * decomposition: the pages of all sequences, concatenated in batch order, are
+ * cut into `chunks` equal pieces per kv head; a workgroup of up to 8 wavefronts
+ * (one per kv head) streams one piece and crosses sequence boundaries as
+ * needed, so the launch is evenly loaded whatever the length distribution. The
+ * piece of sequence b inside chunk c is partial slot c + b; a sequence inside a
+ * single chunk is written directly; the others are merged in chunk order by a
+ * small second launch (the reference's stage 2, flashdecoding.py:242-267).
+ *
+ * Step plan. The cuts depend only on (block_table, seq_lens, chunks), which
+ * are the same for every layer of a decode step (the reference builds its
+ * per-step metadata once as well, model_executor.py:893-911), so they are
+ * computed once per step by litekv_decode_plan into `plan`
+ * (litekv_decode_plan_bytes bytes) and consumed by every layer's launch.
+ * Launches sharing a workspace must not overlap in time.
+ *
+ * Optional fused append. With k_new / v_new non-NULL ([B][Hkv][D], batch
+ * strides given) the launch also performs this step's KV append: the rows are
+ * written, bit exact, to logical position seq_lens[b] - 1 of sequence b (the
+ * slot the reference passes as cur_select_index, paged_attention.py:310-317)
+ * and take part in the attention. It replaces
+ * the separate update_kv_buffer launch of Attention.token_forward
+ * (lite_llama/models/qwen3.py:53-75).
+ *
+ *   chunks     pieces per kv head (>= 1); litekv_paged_decode_balanced_chunks()
+ *              returns the count that gives each CU of the current device one
+ *              workgroup
+ *   workspace  litekv_paged_decode_balanced_workspace_bytes(B, Hq, D, chunks):
+ *              fp32 partials [chunks + B][Hq][D], then log-sum-exp
+ *              [chunks + B][Hq]
+ *   block_table_stride, chunks  must equal the values the plan was made with
+ */
+int32_t litekv_paged_decode_balanced_chunks(int32_t num_kv_heads);
+
+size_t litekv_paged_decode_balanced_workspace_bytes(int32_t batch, int32_t num_q_heads,
+                                                    int32_t head_dim, int32_t chunks);
+
+size_t litekv_decode_plan_bytes(int32_t batch, int32_t block_table_stride,
+                                int32_t num_kv_heads, int32_t chunks);
+
+int litekv_decode_plan(const int32_t *block_table, int32_t block_table_stride,
+                       const int32_t *seq_lens, int32_t batch, int32_t num_kv_heads,
+                       int32_t page_size, int64_t num_pages, int32_t chunks,
+                       void *plan, size_t plan_bytes, void *stream);
+
+int litekv_paged_decode_balanced(const void *q, int64_t q_batch_stride, void *kv_pool,
+                                 const int32_t *seq_lens, void *plan, size_t plan_bytes,
+                                 const void *k_new, const void *v_new,
+                                 int64_t k_new_stride, int64_t v_new_stride,
+                                 void *out, void *workspace, size_t workspace_bytes,
+                                 int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                                 int32_t head_dim, int32_t page_size, int64_t num_pages,
+                                 int32_t block_table_stride, int32_t chunks,
+                                 float softmax_scale, void *stream);
+
+/*
+ * Profiling aid (no counterpart in the reference): the next
+ * litekv_paged_decode_balanced launch made by this thread carries the two
+ * hipEvent_t handles as its start and stop events, so its device-side
+ * duration can be read with hipEventElapsedTime without extra packets in the
+ * stream. Pass NULLs to cancel.
+ */
+int litekv_profile_next_decode(void *start_event, void *stop_event);
+
+/*
  * Varlen causal prefill over paged KV. Replaces
  * `paged_chunk_flash_attention(q, k_cache, v_cache, sm_scale, req_token_table,
  * req_ids, q_start_loc, context_lens, q_seq_lens, max_q_len)`

@@ -55,6 +55,21 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_size_t, c_int32, c_int32, c_int32, c_int32, c_int32,
          c_int32, c_void_p],
     ),
+    "litekv_paged_decode_balanced_chunks": (c_int32, [c_int32]),
+    "litekv_paged_decode_balanced_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
+    "litekv_decode_plan_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
+    "litekv_decode_plan": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_int32, c_int32, c_int32, c_int64, c_int32, c_void_p, c_size_t,
+         c_void_p],
+    ),
+    "litekv_paged_decode_balanced": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p, c_int64,
+         c_int64, c_void_p, c_void_p, c_size_t, c_int32, c_int32, c_int32, c_int32, c_int32,
+         c_int64, c_int32, c_int32, c_float, c_void_p],
+    ),
+    "litekv_profile_next_decode": (c_int32, [c_void_p, c_void_p]),
     "litekv_paged_prefill": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,

@@ -1,8 +1,9 @@
-// Paged flash-decoding for gfx950: split kernel + deterministic merge.
+// Paged flash-decoding for gfx950: two schedules over one page kernel, and
+// the deterministic log-sum-exp merge.
 //
-// Split kernel, one wavefront per (kv head, split, sequence). A wavefront
-// walks its pages; for each 16-token page it computes, with all Hq/Hkv query
-// heads of the kv head at once (so K/V bytes are read from HBM exactly once):
+// Page step (shared by both schedules). A wavefront owns one kv head and walks
+// 16-token pages; all Hq/Hkv query heads of that kv head ride in the 16-wide N
+// dimension of the MFMA tiles, so K/V bytes are read from HBM exactly once:
 //
 //   S^T[token][head]  = K_page[16 x 128] . Q^T[128 x 16]      4 x MFMA 16x16x32
 //   online softmax over tokens, per head column (fp32, exp2 domain)
@@ -12,12 +13,23 @@
 // the B-operand layout of the second product, so probabilities never leave
 // their lane. K fragments are loaded straight from the page in A-operand
 // layout (64 contiguous bytes per token per instruction); V rows are loaded
-// as full 256-byte rows, staged in LDS and read back transposed. Softmax row
-// reductions run over the 4 lane groups with wavefront shuffles.
+// as full 256-byte rows, staged in LDS and read back with the transposing LDS
+// read. Softmax reductions over the 4 lane groups use wavefront shuffles.
+// DEPTH pages per wavefront are kept in flight in registers.
 //
-// Split boundaries are a pure function of the sequence length, so the result
-// does not depend on scheduling; the merge kernel combines the fp32 partials
-// in split order with the usual log-sum-exp weights.
+// Schedule "splits" (litekv_paged_decode): grid (kv head, split, sequence),
+// one wavefront each; sequence b is cut into n_b splits at page boundaries
+// floor(s * pages_b / n_b).
+//
+// Schedule "balanced" (litekv_paged_decode_balanced): the pages of all
+// sequences, concatenated, are cut into equal chunks; one workgroup of up to
+// 8 wavefronts (one per kv head) streams one chunk, crossing sequence
+// boundaries as needed, so every CU gets the same number of bytes whatever the
+// length distribution, and the kv heads of a page are fetched together.
+//
+// In both schedules the cuts are a pure function of seq_lens and of host
+// scalars, and the merge adds the fp32 partials in index order: results do not
+// depend on timing.
 #include "common.h"
 
 namespace litekv {
@@ -26,6 +38,21 @@ constexpr int kVPitch = kHeadDim + 8;  // fp16 elements per staged V row (272 by
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
+// Pages a wavefront keeps in flight in registers (K fragments and V rows of DEPTH pages are
+// requested before the oldest one is consumed).
+#ifndef LITEKV_DECODE_DEPTH
+#define LITEKV_DECODE_DEPTH 2
+#endif
+// The running max of a head is only raised when the new page exceeds it by more than this many
+// powers of two; until then probabilities are formed against the older, smaller max (they stay
+// below 2^kMaxSlack, far inside fp16 range) and the accumulator rescale is skipped. The final
+// division by the denominator cancels the choice of max exactly.
+constexpr float kMaxSlack = 8.0f;
+
+__host__ __device__ __forceinline__ int pages_of(int len) {
+  return len > 0 ? (len + kPageSize - 1) / kPageSize : 0;
+}
+
 __host__ __device__ __forceinline__ int splits_for_pages(int pages, int max_splits,
                                                          int min_pages_per_split) {
   int n = (pages + min_pages_per_split - 1) / min_pages_per_split;
@@ -33,6 +60,167 @@ __host__ __device__ __forceinline__ int splits_for_pages(int pages, int max_spli
   return n < max_splits ? n : max_splits;
 }
 
+struct PageRegs {
+  half8_t k[4];  // A-operand fragments of K: token n, d = 32*kk + 8*g .. +7
+  half8_t v[4];  // V rows 4*i + g, 16-byte column n
+};
+
+// Softmax state and output accumulator of the (up to 16) query heads of one kv head.
+// acc[j][i] is O^T[d = 16j + 4g + i][head n]; m is shared by the 4 lanes of a head, d is this
+// lane's share of the denominator.
+struct HeadState {
+  float4_t acc[8];
+  float m;
+  float d;
+  __device__ __forceinline__ void reset() {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    m = -INFINITY;
+    d = 0.f;
+  }
+};
+
+// Orders this wavefront's LDS writes before its later LDS reads (and the reverse) for the
+// compiler; the LDS unit itself executes one wavefront's accesses in issue order.
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Q^T as B operand: lane (n, g) holds q[head n][32*kk + 8*g .. +7]; lanes past the group get 0.
+__device__ __forceinline__ void load_q(half8_t (&qf)[4], const half_t *q_row0, int n, int g,
+                                       int group) {
+  const half_t *qrow = q_row0 + (int64_t)n * kHeadDim + 8 * g;
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    qf[kk] = (n < group) ? *(const half8_t *)(qrow + 32 * kk) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  }
+}
+
+// Requests one page: k_lane / v_lane already point at this lane's row and column of page 0.
+__device__ __forceinline__ void request_page(PageRegs &r, const half_t *k_lane,
+                                             const half_t *v_lane, int64_t page_off,
+                                             int64_t row_stride) {
+  const half_t *kr = k_lane + page_off;
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) r.k[kk] = *(const half8_t *)(kr + 32 * kk);
+  const half_t *vr = v_lane + page_off;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) r.v[i] = *(const half8_t *)(vr + 4 * i * row_stride);
+}
+
+// Folds page `p` (tokens 16p .. 16p+15 of a sequence of `len` tokens) into the state.
+__device__ __forceinline__ void attend_page(HeadState &st, const PageRegs &r,
+                                            const half8_t (&qf)[4], half_t *vstage,
+                                            const half_t *vt_lane, int p, int len, int n, int g,
+                                            float scale_log2) {
+  const bool tail = (p + 1) * kPageSize > len;  // wavefront-uniform: last, partly filled page
+  wave_lds_fence();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    half8_t x = r.v[i];
+    // Slots past the sequence end hold arbitrary bits: keep them out of the MFMA.
+    if (tail && p * kPageSize + 4 * i + g >= len) x = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+    *(half8_t *)(&vstage[(4 * i + g) * kVPitch + 8 * n]) = x;
+  }
+  wave_lds_fence();
+
+  float4_t s = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) s = mfma_16x16x32(r.k[kk], qf[kk], s);
+
+  float sv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) sv[i] = s[i] * scale_log2;
+  if (tail) {
+    const int tok0 = p * kPageSize + 4 * g;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sv[i] = (tok0 + i < len) ? sv[i] : -INFINITY;
+  }
+  float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+  mx = fmaxf(mx, xor_lane(mx, 16));
+  mx = fmaxf(mx, xor_lane(mx, 32));
+  // mx is finite (the page holds at least one valid token). Raise the reference max only when
+  // some head needs it; the branch is wavefront-uniform.
+  if (__builtin_amdgcn_ballot_w64(mx > st.m + kMaxSlack) != 0) {
+    const float m_new = fmaxf(st.m, mx);
+    const float alpha = fast_exp2(st.m - m_new);
+    st.d *= alpha;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      st.acc[j][0] *= alpha;
+      st.acc[j][1] *= alpha;
+      st.acc[j][2] *= alpha;
+      st.acc[j][3] *= alpha;
+    }
+    st.m = m_new;
+  }
+  float pr[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) pr[i] = fast_exp2(sv[i] - st.m);
+  st.d += (pr[0] + pr[1]) + (pr[2] + pr[3]);
+  const half4_t pt = half4_t{(half_t)pr[0], (half_t)pr[1], (half_t)pr[2], (half_t)pr[3]};
+
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    // V^T fragment: lane (n, g) receives V[4g .. 4g+3][16j + n] from the transposing LDS read
+    // (lane i of a 16-lane group passes the address of row i/4, columns 4*(i%4) .. +3).
+    const half4_t vt = __builtin_bit_cast(
+        half4_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                     (__attribute__((address_space(3))) short4_t *)(vt_lane + 16 * j)));
+    st.acc[j] = mfma_16x16x16(vt, pt, st.acc[j]);
+  }
+}
+
+// Writes the normalised state either as the final fp16 row or as an fp32 partial + log-sum-exp.
+// Head n of the group writes out_row + n*D, or part_row + n*part_head_stride and
+// part_lse_cell + n*lse_head_stride.
+__device__ __forceinline__ void store_state(const HeadState &st, bool final_row, half_t *out_row,
+                                            float *part_row, int64_t part_head_stride,
+                                            float *part_lse_cell, int64_t lse_head_stride, int n,
+                                            int g, int group) {
+  float d_tot = st.d + xor_lane(st.d, 16);
+  d_tot += xor_lane(d_tot, 32);
+  const float inv = 1.0f / d_tot;
+  if (n >= group) return;
+  if (final_row) {
+    half_t *o = out_row + (int64_t)n * kHeadDim + 4 * g;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      *(half4_t *)(o + 16 * j) =
+          half4_t{(half_t)(st.acc[j][0] * inv), (half_t)(st.acc[j][1] * inv),
+                  (half_t)(st.acc[j][2] * inv), (half_t)(st.acc[j][3] * inv)};
+    }
+  } else {
+    float *po = part_row + (int64_t)n * part_head_stride + 4 * g;
+    const float lse = (st.m + fast_log2(d_tot)) * kLn2;
+    {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        *(float4_t *)(po + 16 * j) = float4_t{st.acc[j][0] * inv, st.acc[j][1] * inv,
+                                              st.acc[j][2] * inv, st.acc[j][3] * inv};
+      }
+      if (g == 0) part_lse_cell[(int64_t)n * lse_head_stride] = lse;
+    }
+  }
+}
+
+// Waits for every vector memory load this wavefront has in flight (s_waitcnt vmcnt(0), other
+// counters untouched). Used at the end of rarely taken branches that load into registers the
+// main loop reads: without it the compiler must assume those loads are still pending after the
+// branch joins the main path, and would drain the whole prefetch queue on every iteration.
+__device__ __forceinline__ void wait_vector_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+__device__ __forceinline__ int clamp_page(int pid, int num_pages) {
+  return pid < 0 ? 0 : (pid >= num_pages ? num_pages - 1 : pid);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Schedule "splits": one wavefront per (kv head, split, sequence).
+// Partials: part_o[b][hq][split][D], part_lse[b][hq][split].
+// ---------------------------------------------------------------------------------------------
+template <int DEPTH>
 __global__ __launch_bounds__(64) void paged_decode_split_kernel(
     const half_t *__restrict__ q, int64_t q_batch_stride, const half_t *__restrict__ kv,
     const int32_t *__restrict__ block_table, int32_t bt_stride,
@@ -49,170 +237,416 @@ __global__ __launch_bounds__(64) void paged_decode_split_kernel(
   const int b = blockIdx.z;
 
   const int len = seq_lens[b];
-  const int hq = h * group + n;
+  const int hq0 = h * group;
+  half_t *out_row = out + ((int64_t)b * num_q_heads + hq0) * kHeadDim;
   if (len <= 0) {
     if (split == 0 && n < group) {
-      half_t *o = out + ((int64_t)b * num_q_heads + hq) * kHeadDim;
+      half_t *o = out_row + (int64_t)n * kHeadDim;
 #pragma unroll
       for (int j = 0; j < 8; ++j) *(half4_t *)(o + 16 * j + 4 * g) = half4_t{0, 0, 0, 0};
     }
     return;
   }
-  const int pages = (len + kPageSize - 1) / kPageSize;
+  const int pages = pages_of(len);
   const int n_splits = splits_for_pages(pages, max_splits, min_pages_per_split);
   if (split >= n_splits) return;
   const int p0 = (int)(((int64_t)split * pages) / n_splits);
   const int p1 = (int)(((int64_t)(split + 1) * pages) / n_splits);
 
-  // Q^T as B operand: lane (n, g) holds q[head n][32*kk + 8*g .. +7].
   half8_t qf[4];
-  {
-    const half_t *qrow = q + (int64_t)b * q_batch_stride + (int64_t)hq * kHeadDim + 8 * g;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      qf[kk] = (n < group) ? *(const half8_t *)(qrow + 32 * kk) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    }
-  }
+  load_q(qf, q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
 
   const int64_t row_stride = (int64_t)2 * num_kv_heads * kHeadDim;  // elements per slot
-  const half_t *k_base = kv + (int64_t)h * kHeadDim + 8 * g;                     // + slot row n
-  const half_t *v_base = kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n;    // + slot row 4i+g
+  const half_t *k_lane = kv + (int64_t)h * kHeadDim + 8 * g + n * row_stride;
+  const half_t *v_lane = kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
+  const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
   const int32_t *table = block_table + (int64_t)b * bt_stride;
 
-  float4_t acc[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY;  // running max (log2 domain), identical in the 4 lanes of a head
-  float d_run = 0.f;        // this lane's share of the running denominator
+  HeadState st;
+  st.reset();
+  PageRegs buf[DEPTH];
 
-  int table_regs = 0;  // page ids p0 + 64*c + lane of the current 64-page chunk
-  half8_t kf[4], vf[4];
-
-  auto load_page = [&](int p, half8_t (&kd)[4], half8_t (&vd)[4]) {
-    int pid = __builtin_amdgcn_readlane(table_regs, (p - p0) & 63);
-    pid = pid < 0 ? 0 : (pid >= num_pages ? num_pages - 1 : pid);
-    const int64_t slot0 = (int64_t)pid * kPageSize;
-    const half_t *kr = k_base + (slot0 + n) * row_stride;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) kd[kk] = *(const half8_t *)(kr + 32 * kk);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int t = 4 * i + g;
-      half8_t x = *(const half8_t *)(v_base + (slot0 + t) * row_stride);
-      // Slots past the sequence end hold arbitrary bits: keep them out of the MFMA.
-      vd[i] = (p * kPageSize + t < len) ? x : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    }
+  // Page ids are wavefront-uniform: they travel through scalar loads one step ahead of their
+  // use. Requests past the range re-read its last page (a cache hit), which keeps the number of
+  // vector loads in flight a compile-time constant, so each wait names exactly the page it
+  // needs and never drains the younger prefetches.
+  auto page_id = [&](int p) { return clamp_page(table[p < p1 ? p : p1 - 1], num_pages); };
+  int pid_next = page_id(p0);
+  auto request = [&](int p, PageRegs &r) {
+    const int64_t page_off = (int64_t)pid_next * kPageSize * row_stride;
+    pid_next = page_id(p + 1);
+    request_page(r, k_lane, v_lane, page_off, row_stride);
   };
 
-  {
-    const int idx = p0 + lane;
-    table_regs = (idx < p1) ? table[idx] : 0;
-  }
-  load_page(p0, kf, vf);
-
-  for (int p = p0; p < p1; ++p) {
-    // Stage V of page p (rows 4i+g, 16-byte column n).
-    __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *(half8_t *)(&vstage[(4 * i + g) * kVPitch + 8 * n]) = vf[i];
-    __syncthreads();
-
-    half8_t kc[4];
+  for (int dd = 0; dd < DEPTH; ++dd) request(p0 + dd, buf[dd]);
+  for (int p = p0; p < p1; p += DEPTH) {
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) kc[kk] = kf[kk];
-
-    // Prefetch page p+1 while page p is being reduced.
-    if (p + 1 < p1) {
-      if (((p + 1 - p0) & 63) == 0) {
-        const int idx = p + 1 + lane;
-        table_regs = (idx < p1) ? table[idx] : 0;
-      }
-      load_page(p + 1, kf, vf);
-    }
-
-    float4_t st = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) st = mfma_16x16x32(kc[kk], qf[kk], st);
-
-    float sv[4];
-    const int tok0 = p * kPageSize + 4 * g;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) sv[i] = (tok0 + i < len) ? st[i] * scale_log2 : -INFINITY;
-    float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-    mx = fmaxf(mx, xor_lane(mx, 16));
-    mx = fmaxf(mx, xor_lane(mx, 32));
-    const float m_new = fmaxf(m_run, mx);  // finite: every page of the range has a valid token
-    const float alpha = fast_exp2(m_run - m_new);
-    float pr[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) pr[i] = fast_exp2(sv[i] - m_new);
-    d_run = d_run * alpha + ((pr[0] + pr[1]) + (pr[2] + pr[3]));
-    m_run = m_new;
-    const half4_t pt = half4_t{(half_t)pr[0], (half_t)pr[1], (half_t)pr[2], (half_t)pr[3]};
-
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const half_t *vcol = &vstage[(4 * g) * kVPitch + 16 * j + n];
-      const half4_t vt = half4_t{vcol[0], vcol[kVPitch], vcol[2 * kVPitch], vcol[3 * kVPitch]};
-      float4_t a = acc[j];
-      a[0] *= alpha;
-      a[1] *= alpha;
-      a[2] *= alpha;
-      a[3] *= alpha;
-      acc[j] = mfma_16x16x16(vt, pt, a);
+    for (int dd = 0; dd < DEPTH; ++dd) {
+      if (p + dd < p1) attend_page(st, buf[dd], qf, vstage, vt_lane, p + dd, len, n, g, scale_log2);
+      request(p + dd + DEPTH, buf[dd]);
     }
   }
 
-  float d_tot = d_run + xor_lane(d_run, 16);
-  d_tot += xor_lane(d_tot, 32);
-  const float inv = 1.0f / d_tot;
-  if (n < group) {
-    if (n_splits == 1) {
-      half_t *o = out + ((int64_t)b * num_q_heads + hq) * kHeadDim + 4 * g;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        *(half4_t *)(o + 16 * j) = half4_t{(half_t)(acc[j][0] * inv), (half_t)(acc[j][1] * inv),
-                                           (half_t)(acc[j][2] * inv), (half_t)(acc[j][3] * inv)};
-      }
-    } else {
-      const int64_t cell = ((int64_t)b * num_q_heads + hq) * max_splits + split;
-      float *po = part_o + cell * kHeadDim + 4 * g;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        *(float4_t *)(po + 16 * j) =
-            float4_t{acc[j][0] * inv, acc[j][1] * inv, acc[j][2] * inv, acc[j][3] * inv};
-      }
-      if (g == 0) part_lse[cell] = (m_run + fast_log2(d_tot)) * kLn2;
-    }
-  }
+  const int64_t cell = ((int64_t)b * num_q_heads + hq0) * max_splits + split;
+  store_state(st, n_splits == 1, out_row, part_o + cell * kHeadDim, (int64_t)max_splits * kHeadDim,
+              part_lse + cell, max_splits, n, g, group);
 }
 
-// One block per (query head, sequence), one lane per output element.
-__global__ __launch_bounds__(kHeadDim) void paged_decode_merge_kernel(
+// Merges `n_parts` partial rows of one query head into its final fp16 row; run by one whole
+// wavefront. Partial s has log-sum-exp lse[s * lse_stride] and row po[s * po_stride .. +D).
+// Lane s holds the weight of partial s (blocks of 64 partials); each lane accumulates two output
+// elements over the partials in index order, with independent row loads kept in flight.
+__device__ __forceinline__ void merge_row(const float *__restrict__ lse, int64_t lse_stride,
+                                          const float *__restrict__ po, int64_t po_stride,
+                                          int n_parts, half_t *out_row, int lane) {
+  float mx = -INFINITY;
+  for (int s0 = 0; s0 < n_parts; s0 += kWave) {
+    const float l = (s0 + lane < n_parts) ? lse[(int64_t)(s0 + lane) * lse_stride] : -INFINITY;
+    mx = fmaxf(mx, l);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, xor_lane(mx, off));
+  float den = 0.f, num0 = 0.f, num1 = 0.f;
+  const float *col = po + 2 * lane;
+  for (int s0 = 0; s0 < n_parts; s0 += kWave) {
+    const float l = (s0 + lane < n_parts) ? lse[(int64_t)(s0 + lane) * lse_stride] : -INFINITY;
+    const float w = fast_exp2((l - mx) * kLog2e);
+    den += w;
+    const int cnt = (n_parts - s0) < kWave ? (n_parts - s0) : kWave;
+    int s = 0;
+    for (; s + 4 <= cnt; s += 4) {
+      float2 r[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) r[u] = *(const float2 *)(col + (int64_t)(s0 + s + u) * po_stride);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float wu = __shfl(w, s + u, kWave);
+        num0 += wu * r[u].x;
+        num1 += wu * r[u].y;
+      }
+    }
+    for (; s < cnt; ++s) {
+      const float2 r = *(const float2 *)(col + (int64_t)(s0 + s) * po_stride);
+      const float wu = __shfl(w, s, kWave);
+      num0 += wu * r.x;
+      num1 += wu * r.y;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) den += xor_lane(den, off);
+  const float inv = 1.0f / den;
+  typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+  *(half2_t *)(out_row + 2 * lane) = half2_t{(half_t)(num0 * inv), (half_t)(num1 * inv)};
+}
+
+// Schedule "splits" merge: one wavefront per (query head, sequence).
+__global__ __launch_bounds__(kWave) void paged_decode_merge_kernel(
     const int32_t *__restrict__ seq_lens, half_t *__restrict__ out,
     const float *__restrict__ part_o, const float *__restrict__ part_lse, int32_t num_q_heads,
     int32_t max_splits, int32_t min_pages_per_split) {
   const int hq = blockIdx.x;
   const int b = blockIdx.y;
-  const int d = threadIdx.x;
   const int len = seq_lens[b];
   if (len <= 0) return;
-  const int pages = (len + kPageSize - 1) / kPageSize;
-  const int n_splits = splits_for_pages(pages, max_splits, min_pages_per_split);
+  const int n_splits = splits_for_pages(pages_of(len), max_splits, min_pages_per_split);
   if (n_splits == 1) return;  // the split kernel already wrote the final row
   const int64_t cell0 = ((int64_t)b * num_q_heads + hq) * max_splits;
-  const float *lse = part_lse + cell0;
-  const float *po = part_o + cell0 * kHeadDim + d;
-  float mx = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) mx = fmaxf(mx, lse[s]);
-  float num = 0.f, den = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float w = fast_exp2((lse[s] - mx) * kLog2e);
-    num += w * po[(int64_t)s * kHeadDim];
-    den += w;
-  }
-  out[((int64_t)b * num_q_heads + hq) * kHeadDim + d] = (half_t)(num / den);
+  merge_row(part_lse + cell0, 1, part_o + cell0 * kHeadDim, kHeadDim, n_splits,
+            out + ((int64_t)b * num_q_heads + hq) * kHeadDim, threadIdx.x);
 }
+
+// ---------------------------------------------------------------------------------------------
+// Schedule "balanced": the pages of all sequences, concatenated in batch order, form one line
+// of `total` pages per kv head; it is cut into `chunks` equal pieces of C = ceil(total / chunks)
+// pages. Wavefront (head h, chunk c) streams pages [c*C, (c+1)*C), finishing one sequence and
+// starting the next where the line crosses a sequence boundary. A workgroup holds
+// `heads_per_wg` heads of `replicas` consecutive chunks.
+//
+// The cuts are made once per decode step by the plan kernel (block tables and lengths are the
+// same for every layer of a step) and stored as one entry per chunk:
+//   entry[0] first page on the line   entry[1] one past its last page
+//   entry[2] sequence of the first page, entry[3], entry[4] that sequence's [first, last) page
+//   entry[8 ..] the chunk's physical page ids, in line order
+// so a wavefront needs one dependent hop (its entry) before it can request K/V.
+//
+// The piece of sequence b inside chunk c is partial slot c + b (strictly increasing along the
+// line, so slots never collide): part_o[slot][hq][D], part_lse[slot][hq]. A sequence lying
+// inside one chunk is written to `out` directly; the others are merged, in chunk order, by a
+// second small launch (one wavefront per sequence and kv head). Merging inside the decode
+// kernel was measured and rejected: pieces written by other XCDs only become visible through
+// device-scope cache write-back / invalidate or write-through accesses, and either costs far
+// more than the 3 us of a launch boundary.
+// ---------------------------------------------------------------------------------------------
+constexpr int kMaxWavesPerWg = 8;
+constexpr int kPlanMeta = 16;      // int32 words of plan meta data
+constexpr int kEntryHeader = 8;    // int32 words of an entry before its page ids
+// plan meta words
+constexpr int kMetaTotal = 0, kMetaChunkPages = 1, kMetaChunks = 2, kMetaBatch = 3,
+              kMetaEntryStride = 4, kMetaKvHeads = 5;
+
+__host__ __device__ __forceinline__ int round_up(int x, int m) { return (x + m - 1) / m * m; }
+
+// Step metadata that no launch of the decode kernel modifies (plan entries, sequence lengths) is
+// read through the constant address space: with a wavefront-uniform address such a load is
+// always a scalar load, whatever fences and atomics surround it, so it never joins the in-order
+// queue of the vector loads that stream K/V.
+typedef const __attribute__((address_space(4))) int32_t *uniform_i32_ptr;
+__device__ __forceinline__ uniform_i32_ptr as_uniform(const int32_t *p) {
+  return (uniform_i32_ptr)(uintptr_t)p;
+}
+
+// Entry stride (int32 words) that holds the largest possible chunk: no sequence has more than
+// `bt_stride` pages, so total <= batch * bt_stride.
+__host__ __device__ __forceinline__ int plan_entry_stride(int batch, int bt_stride, int chunks) {
+  const int64_t max_total = (int64_t)batch * bt_stride;
+  const int max_chunk_pages = (int)((max_total + chunks - 1) / chunks);
+  return round_up(kEntryHeader + max_chunk_pages, 4);
+}
+// Plan buffer (int32 words): meta[kPlanMeta], then per sequence (first chunk, number of
+// chunks it spans), then the chunk entries.
+__host__ __device__ __forceinline__ int plan_seq_info_offset() { return kPlanMeta; }
+__host__ __device__ __forceinline__ int plan_entries_offset(int batch) {
+  return kPlanMeta + round_up(2 * batch, 4);
+}
+
+// One block per sequence: places the sequence's pages on the line, fills the entries they fall
+// into and records which chunks the sequence spans; block 0 also writes the meta words and
+// marks the chunks past the end of the line as empty.
+__global__ __launch_bounds__(256) void decode_plan_kernel(
+    const int32_t *__restrict__ block_table, int32_t bt_stride,
+    const int32_t *__restrict__ seq_lens, int32_t batch, int32_t num_kv_heads, int32_t chunks,
+    int32_t entry_stride, int32_t num_pages, int32_t *__restrict__ plan) {
+  __shared__ int red[4][2];
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x;
+  int before = 0, total = 0;
+  for (int i = tid; i < batch; i += 256) {
+    int pg = pages_of(seq_lens[i]);
+    pg = pg < bt_stride ? pg : bt_stride;
+    total += pg;
+    before += (i < b) ? pg : 0;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    total += __shfl_xor(total, off, kWave);
+    before += __shfl_xor(before, off, kWave);
+  }
+  if ((tid & 63) == 0) {
+    red[tid >> 6][0] = total;
+    red[tid >> 6][1] = before;
+  }
+  __syncthreads();
+  total = red[0][0] + red[1][0] + red[2][0] + red[3][0];
+  before = red[0][1] + red[1][1] + red[2][1] + red[3][1];
+  const int chunk_pages = total > 0 ? (total + chunks - 1) / chunks : 1;
+  int32_t *entries = plan + plan_entries_offset(batch);
+
+  if (b == 0) {
+    if (tid == 0) {
+      plan[kMetaTotal] = total;
+      plan[kMetaChunkPages] = chunk_pages;
+      plan[kMetaChunks] = chunks;
+      plan[kMetaBatch] = batch;
+      plan[kMetaEntryStride] = entry_stride;
+      plan[kMetaKvHeads] = num_kv_heads;
+    }
+    for (int c = tid; c < chunks; c += 256) {
+      if ((int64_t)c * chunk_pages >= total) {
+        entries[(int64_t)c * entry_stride + 0] = 0;
+        entries[(int64_t)c * entry_stride + 1] = 0;
+      }
+    }
+  }
+  int my_pages = pages_of(seq_lens[b]);
+  my_pages = my_pages < bt_stride ? my_pages : bt_stride;
+  if (tid == 0) {
+    const int c_first = before / chunk_pages;
+    plan[plan_seq_info_offset() + 2 * b] = c_first;
+    plan[plan_seq_info_offset() + 2 * b + 1] =
+        my_pages > 0 ? (before + my_pages - 1) / chunk_pages - c_first + 1 : 0;
+  }
+  const int32_t *row = block_table + (int64_t)b * bt_stride;
+  for (int p = tid; p < my_pages; p += 256) {
+    const int f = before + p;
+    const int c = f / chunk_pages;
+    const int r = f - c * chunk_pages;
+    int32_t *e = entries + (int64_t)c * entry_stride;
+    e[kEntryHeader + r] = clamp_page(row[p], num_pages);
+    if (r == 0) {
+      const int end = f + chunk_pages;
+      e[0] = f;
+      e[1] = end < total ? end : total;
+      e[2] = b;
+      e[3] = before;
+      e[4] = before + my_pages;
+    }
+  }
+}
+
+// Balanced-schedule merge, one wavefront per (query head, sequence): combines the sequence's
+// pieces (partial slots c_first + b, c_first + b + 1, ...) if it spans several chunks.
+__global__ __launch_bounds__(kWave) void paged_decode_balanced_merge_kernel(
+    const int32_t *__restrict__ plan, half_t *__restrict__ out,
+    const float *__restrict__ part_o, const float *__restrict__ part_lse, int32_t num_q_heads) {
+  const int hq = blockIdx.x;
+  const int b = blockIdx.y;
+  const int c_first = plan[plan_seq_info_offset() + 2 * b];
+  const int n_parts = plan[plan_seq_info_offset() + 2 * b + 1];
+  if (n_parts <= 1) return;  // empty, or written directly by the decode kernel
+  const int64_t cell0 = (int64_t)(c_first + b) * num_q_heads + hq;
+  merge_row(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
+            (int64_t)num_q_heads * kHeadDim, n_parts,
+            out + ((int64_t)b * num_q_heads + hq) * kHeadDim, threadIdx.x);
+}
+
+template <int DEPTH>
+__global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_kernel(
+    const half_t *__restrict__ q, int64_t q_batch_stride, half_t *__restrict__ kv,
+    const int32_t *__restrict__ seq_lens, const int32_t *__restrict__ plan,
+    const half_t *__restrict__ k_new, const half_t *__restrict__ v_new, int64_t k_new_stride,
+    int64_t v_new_stride, half_t *__restrict__ out, float *__restrict__ part_o,
+    float *__restrict__ part_lse, int32_t bt_stride, int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t group,
+    int32_t heads_per_wg, int32_t replicas, int32_t chunks, float scale_log2) {
+  __shared__ __attribute__((aligned(16))) half_t vstage_all[kMaxWavesPerWg][kPageSize * kVPitch];
+
+  // readfirstlane tells the compiler the wavefront index is uniform (scalar branches and loads)
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  const int n = lane & 15;
+  const int g = lane >> 4;
+  const int h = blockIdx.y * heads_per_wg + wave % heads_per_wg;
+  const int cidx = blockIdx.x * replicas + wave / heads_per_wg;
+  if (h >= num_kv_heads || cidx >= chunks) return;  // whole wavefront; no workgroup barriers below
+  half_t *vstage = vstage_all[wave];
+
+  // Empty sequences are on no chunk's line: chunk c zeroes the rows of sequences c, c + chunks, ...
+  for (int bz = cidx; bz < batch; bz += chunks) {
+    if (seq_lens[bz] <= 0 && n < group) {
+      half_t *o = out + ((int64_t)bz * num_q_heads + h * group + n) * kHeadDim + 4 * g;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) *(half4_t *)(o + 16 * j) = half4_t{0, 0, 0, 0};
+    }
+  }
+
+  const int entry_stride = plan_entry_stride(batch, bt_stride, chunks);
+  const uniform_i32_ptr lens = as_uniform(seq_lens);
+  const uniform_i32_ptr entry =
+      as_uniform(plan) + plan_entries_offset(batch) + (int64_t)cidx * entry_stride;
+  const int f0 = entry[0];
+  const int f1 = entry[1];
+  if (f1 <= f0) return;
+  int cur_b = entry[2];
+  int cu_lo = entry[3];  // current sequence: [first, last) page on the line
+  int cu_hi = entry[4];
+  const uniform_i32_ptr page_ids = entry + kEntryHeader;
+  int first_ids[DEPTH];
+#pragma unroll
+  for (int dd = 0; dd < DEPTH; ++dd) first_ids[dd] = page_ids[dd < f1 - f0 ? dd : f1 - f0 - 1];
+
+  int len_b = lens[cur_b];
+  int len_after = (cur_b + 1 < batch) ? lens[cur_b + 1] : 0;  // read ahead for the crossing
+
+  const int hq0 = h * group;
+  const int64_t row_stride = (int64_t)2 * num_kv_heads * kHeadDim;
+  half_t *k_lane = kv + (int64_t)h * kHeadDim + 8 * g + n * row_stride;
+  half_t *v_lane = kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
+  const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
+
+  // Requests past the chunk re-read its last page (a cache hit) so the number of vector loads
+  // in flight stays a compile-time constant and every wait names exactly the page it needs.
+  // Page ids travel through scalar loads, one request ahead of their use.
+  int pid_next = 0;
+  auto request = [&](int i, PageRegs &r) {  // i = page index inside the chunk
+    const int64_t page_off = (int64_t)pid_next * kPageSize * row_stride;
+    const int nx = i + 1 < f1 - f0 ? i + 1 : f1 - f0 - 1;
+    pid_next = page_ids[nx];
+    request_page(r, k_lane, v_lane, page_off, row_stride);
+  };
+
+  HeadState st;
+  st.reset();
+  half8_t qf[4];
+  load_q(qf, q + (int64_t)cur_b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
+
+  auto flush = [&]() {
+    const bool whole = cu_lo >= f0 && cu_hi <= f1;  // the sequence lies inside this chunk
+    const int64_t cell = (int64_t)(cidx + cur_b) * num_q_heads + hq0;
+    half_t *out_row = out + ((int64_t)cur_b * num_q_heads + hq0) * kHeadDim;
+    store_state(st, whole, out_row, part_o + cell * kHeadDim, kHeadDim, part_lse + cell, 1, n, g,
+                group);
+  };
+
+  PageRegs buf[DEPTH];
+#pragma unroll
+  for (int dd = 0; dd < DEPTH; ++dd) {
+    pid_next = first_ids[dd];
+    request(dd, buf[dd]);
+  }
+  // after the prologue pid_next holds the id of page DEPTH (clamped), as the loop expects
+  for (int f = f0; f < f1; f += DEPTH) {
+#pragma unroll
+    for (int dd = 0; dd < DEPTH; ++dd) {
+      const int ff = f + dd;
+      if (ff < f1) {
+        if (ff >= cu_hi) {  // the line enters the next non-empty sequence
+          flush();
+          do {
+            ++cur_b;
+            len_b = len_after;
+            len_after = (cur_b + 1 < batch) ? lens[cur_b + 1] : 0;
+            int pg = pages_of(len_b);
+            pg = pg < bt_stride ? pg : bt_stride;
+            cu_lo = cu_hi;
+            cu_hi += pg;
+          } while (ff >= cu_hi);
+          load_q(qf, q + (int64_t)cur_b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
+          st.reset();
+          wait_vector_loads();
+        }
+        const int p = ff - cu_lo;  // page index inside the sequence
+        if (k_new != nullptr && (p + 1) * kPageSize >= len_b) {
+          // Last page of the sequence: the step's new token (logical position len_b - 1) is
+          // appended here. Its K and V rows go to the pool and replace the stale values this
+          // wavefront requested before the write.
+          const int t_new = (len_b - 1) & (kPageSize - 1);
+          const half_t *kn = k_new + (int64_t)cur_b * k_new_stride + (int64_t)h * kHeadDim;
+          const half_t *vn = v_new + (int64_t)cur_b * v_new_stride + (int64_t)h * kHeadDim;
+          const int pid = page_ids[ff - f0];
+          const int64_t slot_off = ((int64_t)pid * kPageSize + t_new) * row_stride;
+          if (n == t_new) {
+            half_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 8 * g;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+              const half8_t x = *(const half8_t *)(kn + 32 * kk + 8 * g);
+              buf[dd].k[kk] = x;
+              *(half8_t *)(dst + 32 * kk) = x;
+            }
+          }
+          if (g == (t_new & 3)) {
+            const half8_t x = *(const half8_t *)(vn + 8 * n);
+            *(half8_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n) = x;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              if (i == (t_new >> 2)) buf[dd].v[i] = x;
+            }
+          }
+          wait_vector_loads();
+        }
+        attend_page(st, buf[dd], qf, vstage, vt_lane, p, len_b, n, g, scale_log2);
+      }
+      request(ff - f0 + DEPTH, buf[dd]);
+    }
+  }
+  flush();
+}
+
+}  // namespace litekv
+
+// ---------------------------------------------------------------------------------------------
+// Host side: argument checks and launches.
+// ---------------------------------------------------------------------------------------------
+namespace litekv {
 
 struct DecodeArgs {
   const void *q;
@@ -226,36 +660,27 @@ struct DecodeArgs {
   size_t workspace_bytes;
   int32_t batch, num_q_heads, num_kv_heads, head_dim, page_size;
   int64_t num_pages;
-  int32_t max_splits, min_pages_per_split;
   float softmax_scale;
   void *stream;
 };
 
-static size_t workspace_bytes_for(int64_t batch, int64_t hq, int64_t d, int64_t s) {
-  if (batch <= 0 || hq <= 0 || d <= 0 || s <= 1) return 0;
-  return (size_t)(batch * hq * s * (d + 1)) * sizeof(float);
-}
-
-static int validate_common(const char *what, const DecodeArgs &a, bool need_inputs) {
-  LITEKV_REQUIRE(a.batch >= 0, "%s: batch %d < 0", what, a.batch);
+// Checks shared by every decode entry point; `need_inputs` is false for the merge-only calls.
+static int validate_decode(const char *what, const DecodeArgs &a, size_t workspace_needed,
+                           bool need_inputs) {
+  LITEKV_REQUIRE(a.batch >= 0 && a.batch <= 65535, "%s: batch %d out of [0, 65535]", what, a.batch);
   LITEKV_REQUIRE(a.head_dim == kHeadDim, "%s: head_dim %d unsupported (only %d)", what, a.head_dim,
                  kHeadDim);
   LITEKV_REQUIRE(a.page_size == kPageSize, "%s: page_size %d unsupported (only %d)", what,
                  a.page_size, kPageSize);
-  LITEKV_REQUIRE(a.num_q_heads > 0, "%s: num_q_heads %d <= 0", what, a.num_q_heads);
-  LITEKV_REQUIRE(a.max_splits >= 1 && a.max_splits <= 65535, "%s: max_splits %d out of [1, 65535]",
-                 what, a.max_splits);
-  LITEKV_REQUIRE(a.min_pages_per_split >= 1, "%s: min_pages_per_split %d < 1", what,
-                 a.min_pages_per_split);
-  LITEKV_REQUIRE(a.batch <= 65535, "%s: batch %d > 65535", what, a.batch);
+  LITEKV_REQUIRE(a.num_q_heads > 0 && a.num_q_heads <= 65535, "%s: num_q_heads %d out of range",
+                 what, a.num_q_heads);
   if (a.batch == 0) return LITEKV_OK;
   LITEKV_REQUIRE(a.seq_lens && a.out, "%s: null pointer", what);
   LITEKV_REQUIRE(aligned16(a.out), "%s: out must be 16-byte aligned", what);
-  if (a.max_splits > 1) {
-    const size_t need = workspace_bytes_for(a.batch, a.num_q_heads, a.head_dim, a.max_splits);
-    LITEKV_REQUIRE(a.workspace != nullptr && a.workspace_bytes >= need,
-                   "%s: workspace of %zu bytes needed for %d splits, got %zu", what, need,
-                   a.max_splits, a.workspace ? a.workspace_bytes : (size_t)0);
+  if (workspace_needed > 0) {
+    LITEKV_REQUIRE(a.workspace != nullptr && a.workspace_bytes >= workspace_needed,
+                   "%s: workspace of %zu bytes needed, got %zu", what, workspace_needed,
+                   a.workspace ? a.workspace_bytes : (size_t)0);
     LITEKV_REQUIRE(aligned16(a.workspace), "%s: workspace must be 16-byte aligned", what);
   }
   if (need_inputs) {
@@ -269,8 +694,8 @@ static int validate_common(const char *what, const DecodeArgs &a, bool need_inpu
     LITEKV_REQUIRE(a.q_batch_stride >= (int64_t)a.num_q_heads * a.head_dim &&
                        a.q_batch_stride % 8 == 0,
                    "%s: q_batch_stride %lld invalid", what, (long long)a.q_batch_stride);
-    LITEKV_REQUIRE(aligned16(a.q) && aligned16(a.kv_pool), "%s: q and kv_pool must be 16-byte aligned",
-                   what);
+    LITEKV_REQUIRE(aligned16(a.q) && aligned16(a.kv_pool),
+                   "%s: q and kv_pool must be 16-byte aligned", what);
     LITEKV_REQUIRE(a.block_table_stride >= 1, "%s: block_table_stride %d < 1", what,
                    a.block_table_stride);
     LITEKV_REQUIRE(a.num_pages >= 1 && a.num_pages <= 0x7fffffffLL / kPageSize,
@@ -279,43 +704,251 @@ static int validate_common(const char *what, const DecodeArgs &a, bool need_inpu
   return LITEKV_OK;
 }
 
-static float *lse_of(const DecodeArgs &a) {
-  return static_cast<float *>(a.workspace) +
-         (size_t)a.batch * a.num_q_heads * a.max_splits * a.head_dim;
+// ---- schedule "splits" ----
+
+static size_t splits_workspace_bytes(int64_t batch, int64_t hq, int64_t d, int64_t s) {
+  if (batch <= 0 || hq <= 0 || d <= 0 || s <= 1) return 0;
+  return (size_t)(batch * hq * s * (d + 1)) * sizeof(float);
 }
 
-static int launch_split(const DecodeArgs &a) {
-  int rc = validate_common("paged_decode_split", a, true);
-  if (rc != LITEKV_OK || a.batch == 0) return rc;
+static int check_split_plan(const char *what, int32_t max_splits, int32_t min_pages_per_split) {
+  LITEKV_REQUIRE(max_splits >= 1 && max_splits <= 65535, "%s: max_splits %d out of [1, 65535]", what,
+                 max_splits);
+  LITEKV_REQUIRE(min_pages_per_split >= 1, "%s: min_pages_per_split %d < 1", what,
+                 min_pages_per_split);
+  return LITEKV_OK;
+}
+
+static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split) {
+  const char *what = "paged_decode_split";
+  int rc = check_split_plan(what, max_splits, min_pages_per_split);
+  if (rc != LITEKV_OK) return rc;
+  rc = validate_decode(what, a,
+                       splits_workspace_bytes(a.batch, a.num_q_heads, a.head_dim, max_splits), true);
+  if (rc != LITEKV_OK) return rc;
+  if (a.batch == 0) {
+    clear_error();
+    return LITEKV_OK;
+  }
+  LITEKV_REQUIRE(a.num_kv_heads <= 65535, "%s: num_kv_heads %d > 65535", what, a.num_kv_heads);
   const int group = a.num_q_heads / a.num_kv_heads;
-  float *part_o = a.max_splits > 1 ? static_cast<float *>(a.workspace) : nullptr;
-  float *part_lse = a.max_splits > 1 ? lse_of(a) : nullptr;
-  hipLaunchKernelGGL(paged_decode_split_kernel,
-                     dim3((unsigned)a.num_kv_heads, (unsigned)a.max_splits, (unsigned)a.batch),
-                     dim3(64), 0, static_cast<hipStream_t>(a.stream),
+  float *part_o = max_splits > 1 ? static_cast<float *>(a.workspace) : nullptr;
+  float *part_lse =
+      max_splits > 1 ? part_o + (size_t)a.batch * a.num_q_heads * max_splits * a.head_dim : nullptr;
+  hipLaunchKernelGGL(paged_decode_split_kernel<LITEKV_DECODE_DEPTH>,
+                     dim3((unsigned)a.num_kv_heads, (unsigned)max_splits, (unsigned)a.batch),
+                     dim3(kWave), 0, static_cast<hipStream_t>(a.stream),
                      static_cast<const half_t *>(a.q), a.q_batch_stride,
                      static_cast<const half_t *>(a.kv_pool), a.block_table, a.block_table_stride,
                      a.seq_lens, static_cast<half_t *>(a.out), part_o, part_lse, a.num_q_heads,
-                     a.num_kv_heads, group, a.max_splits, a.min_pages_per_split,
-                     (int32_t)a.num_pages, a.softmax_scale * kLog2e);
-  return check_launch("paged_decode_split");
+                     a.num_kv_heads, group, max_splits, min_pages_per_split, (int32_t)a.num_pages,
+                     a.softmax_scale * kLog2e);
+  return check_launch(what);
 }
 
-static int launch_merge(const DecodeArgs &a) {
-  int rc = validate_common("paged_decode_merge", a, false);
-  if (rc != LITEKV_OK || a.batch == 0 || a.max_splits == 1) return rc;
+static int launch_merge(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split) {
+  const char *what = "paged_decode_merge";
+  int rc = check_split_plan(what, max_splits, min_pages_per_split);
+  if (rc != LITEKV_OK) return rc;
+  rc = validate_decode(what, a,
+                       splits_workspace_bytes(a.batch, a.num_q_heads, a.head_dim, max_splits),
+                       false);
+  if (rc != LITEKV_OK) return rc;
+  if (a.batch == 0 || max_splits == 1) {
+    clear_error();
+    return LITEKV_OK;
+  }
+  const float *part_o = static_cast<const float *>(a.workspace);
+  const float *part_lse = part_o + (size_t)a.batch * a.num_q_heads * max_splits * a.head_dim;
   hipLaunchKernelGGL(paged_decode_merge_kernel, dim3((unsigned)a.num_q_heads, (unsigned)a.batch),
-                     dim3(kHeadDim), 0, static_cast<hipStream_t>(a.stream), a.seq_lens,
-                     static_cast<half_t *>(a.out), static_cast<const float *>(a.workspace),
-                     lse_of(a), a.num_q_heads, a.max_splits, a.min_pages_per_split);
-  return check_launch("paged_decode_merge");
+                     dim3(kWave), 0, static_cast<hipStream_t>(a.stream), a.seq_lens,
+                     static_cast<half_t *>(a.out), part_o, part_lse, a.num_q_heads, max_splits,
+                     min_pages_per_split);
+  return check_launch(what);
 }
+
+// ---- schedule "balanced" ----
+
+struct BalancedShape {
+  int heads_per_wg;  // kv heads served by one workgroup (one wavefront each)
+  int replicas;      // consecutive chunks served by one workgroup
+  int head_groups;   // grid.y
+};
+
+static BalancedShape balanced_shape(int num_kv_heads) {
+  BalancedShape s;
+  s.heads_per_wg = num_kv_heads < kMaxWavesPerWg ? num_kv_heads : kMaxWavesPerWg;
+  s.replicas = kMaxWavesPerWg / s.heads_per_wg;
+  s.head_groups = (num_kv_heads + s.heads_per_wg - 1) / s.heads_per_wg;
+  return s;
+}
+
+static size_t balanced_workspace_bytes(int64_t batch, int64_t hq, int64_t d, int64_t chunks) {
+  if (batch <= 0 || hq <= 0 || d <= 0 || chunks <= 0) return 0;
+  return (size_t)((chunks + batch) * hq * (d + 1)) * sizeof(float);
+}
+
+static size_t plan_bytes_for(int64_t batch, int64_t bt_stride, int64_t hkv, int64_t chunks) {
+  if (batch <= 0 || bt_stride <= 0 || hkv <= 0 || chunks <= 0) return 0;
+  const int64_t words = plan_entries_offset((int)batch) +
+                        chunks * plan_entry_stride((int)batch, (int)bt_stride, (int)chunks);
+  return (size_t)words * sizeof(int32_t);
+}
+
+// Chunks per kv head that give every CU of the current device one workgroup.
+static int auto_chunks(int num_kv_heads) {
+  static thread_local int cached_device = -1;
+  static thread_local int cached_cus = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (dev != cached_device) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus <= 0) {
+      cus = 256;
+    }
+    cached_device = dev;
+    cached_cus = cus;
+  }
+  const BalancedShape s = balanced_shape(num_kv_heads);
+  const int wgs = (cached_cus + s.head_groups - 1) / s.head_groups;
+  return wgs * s.replicas;
+}
+
+static int check_chunks(const char *what, int32_t batch, int32_t bt_stride, int32_t hkv,
+                        int32_t chunks) {
+  LITEKV_REQUIRE(chunks >= 1 && chunks <= (1 << 20), "%s: chunks %d out of [1, 2^20]", what, chunks);
+  LITEKV_REQUIRE(bt_stride >= 1, "%s: block_table_stride %d < 1", what, bt_stride);
+  LITEKV_REQUIRE(hkv >= 1 && hkv <= 65535, "%s: num_kv_heads %d out of range", what, hkv);
+  LITEKV_REQUIRE((int64_t)batch * bt_stride <= 0x7fffffffLL / 4,
+                 "%s: batch * block_table_stride too large", what);
+  return LITEKV_OK;
+}
+
+// Optional HIP events bracketing the next balanced decode launch of this thread (profiling).
+static thread_local hipEvent_t g_profile_start = nullptr;
+static thread_local hipEvent_t g_profile_stop = nullptr;
 
 }  // namespace litekv
 
+extern "C" int32_t litekv_paged_decode_balanced_chunks(int32_t num_kv_heads) {
+  return num_kv_heads > 0 ? litekv::auto_chunks(num_kv_heads) : 0;
+}
+
+extern "C" size_t litekv_paged_decode_balanced_workspace_bytes(int32_t batch, int32_t num_q_heads,
+                                                               int32_t head_dim, int32_t chunks) {
+  return litekv::balanced_workspace_bytes(batch, num_q_heads, head_dim, chunks);
+}
+
+extern "C" size_t litekv_decode_plan_bytes(int32_t batch, int32_t block_table_stride,
+                                           int32_t num_kv_heads, int32_t chunks) {
+  return litekv::plan_bytes_for(batch, block_table_stride, num_kv_heads, chunks);
+}
+
+extern "C" int litekv_decode_plan(const int32_t *block_table, int32_t block_table_stride,
+                                  const int32_t *seq_lens, int32_t batch, int32_t num_kv_heads,
+                                  int32_t page_size, int64_t num_pages, int32_t chunks, void *plan,
+                                  size_t plan_bytes, void *stream) {
+  using namespace litekv;
+  const char *what = "decode_plan";
+  LITEKV_REQUIRE(batch >= 0 && batch <= 65535, "%s: batch %d out of [0, 65535]", what, batch);
+  LITEKV_REQUIRE(page_size == kPageSize, "%s: page_size %d unsupported (only %d)", what, page_size,
+                 kPageSize);
+  int rc = check_chunks(what, batch, block_table_stride, num_kv_heads, chunks);
+  if (rc != LITEKV_OK) return rc;
+  if (batch == 0) {
+    clear_error();
+    return LITEKV_OK;
+  }
+  LITEKV_REQUIRE(block_table && seq_lens && plan, "%s: null pointer", what);
+  LITEKV_REQUIRE(aligned16(plan), "%s: plan must be 16-byte aligned", what);
+  LITEKV_REQUIRE(num_pages >= 1 && num_pages <= 0x7fffffffLL / kPageSize,
+                 "%s: num_pages %lld out of range", what, (long long)num_pages);
+  const size_t need = plan_bytes_for(batch, block_table_stride, num_kv_heads, chunks);
+  LITEKV_REQUIRE(plan_bytes >= need, "%s: plan buffer of %zu bytes needed, got %zu", what, need,
+                 plan_bytes);
+  hipLaunchKernelGGL(decode_plan_kernel, dim3((unsigned)batch), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), block_table, block_table_stride, seq_lens,
+                     batch, num_kv_heads, chunks,
+                     plan_entry_stride(batch, block_table_stride, chunks), (int32_t)num_pages,
+                     static_cast<int32_t *>(plan));
+  return check_launch(what);
+}
+
+extern "C" int litekv_profile_next_decode(void *start_event, void *stop_event) {
+  litekv::g_profile_start = static_cast<hipEvent_t>(start_event);
+  litekv::g_profile_stop = static_cast<hipEvent_t>(stop_event);
+  return LITEKV_OK;
+}
+
+extern "C" int litekv_paged_decode_balanced(
+    const void *q, int64_t q_batch_stride, void *kv_pool, const int32_t *seq_lens, void *plan,
+    size_t plan_bytes, const void *k_new, const void *v_new, int64_t k_new_stride,
+    int64_t v_new_stride, void *out, void *workspace, size_t workspace_bytes, int32_t batch,
+    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+    int64_t num_pages, int32_t block_table_stride, int32_t chunks, float softmax_scale,
+    void *stream) {
+  using namespace litekv;
+  const char *what = "paged_decode_balanced";
+  int rc = check_chunks(what, batch, block_table_stride, num_kv_heads, chunks);
+  if (rc != LITEKV_OK) return rc;
+  static const int32_t dummy_table = 0;  // the kernel reads page ids from the plan
+  DecodeArgs a{q, q_batch_stride, kv_pool, &dummy_table, block_table_stride, seq_lens, out,
+               workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim, page_size,
+               num_pages, softmax_scale, stream};
+  rc = validate_decode(what, a,
+                       balanced_workspace_bytes(batch, num_q_heads, head_dim, chunks), true);
+  if (rc != LITEKV_OK) return rc;
+  if (batch == 0) {
+    clear_error();
+    return LITEKV_OK;
+  }
+  LITEKV_REQUIRE(plan != nullptr && aligned16(plan), "%s: plan must be a 16-byte aligned buffer",
+                 what);
+  const size_t need = plan_bytes_for(batch, block_table_stride, num_kv_heads, chunks);
+  LITEKV_REQUIRE(plan_bytes >= need, "%s: plan buffer of %zu bytes needed, got %zu", what, need,
+                 plan_bytes);
+  LITEKV_REQUIRE((k_new == nullptr) == (v_new == nullptr), "%s: k_new and v_new go together", what);
+  if (k_new != nullptr) {
+    const int64_t row = (int64_t)num_kv_heads * head_dim;
+    LITEKV_REQUIRE(aligned16(k_new) && aligned16(v_new), "%s: k_new, v_new must be 16-byte aligned",
+                   what);
+    LITEKV_REQUIRE(k_new_stride >= row && v_new_stride >= row && k_new_stride % 8 == 0 &&
+                       v_new_stride % 8 == 0,
+                   "%s: k_new/v_new strides (%lld, %lld) invalid", what, (long long)k_new_stride,
+                   (long long)v_new_stride);
+  }
+  const BalancedShape s = balanced_shape(num_kv_heads);
+  LITEKV_REQUIRE(s.head_groups <= 65535, "%s: num_kv_heads %d too large", what, num_kv_heads);
+  float *part_o = static_cast<float *>(workspace);
+  float *part_lse = part_o + (size_t)(chunks + batch) * num_q_heads * head_dim;
+  const unsigned wgs = (unsigned)((chunks + s.replicas - 1) / s.replicas);
+  hipEvent_t ev0 = g_profile_start, ev1 = g_profile_stop;
+  g_profile_start = g_profile_stop = nullptr;
+  hipExtLaunchKernelGGL(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH>,
+                        dim3(wgs, (unsigned)s.head_groups),
+                        dim3((unsigned)(kWave * s.heads_per_wg * s.replicas)), 0,
+                        static_cast<hipStream_t>(stream), ev0, ev1, 0,
+                        static_cast<const half_t *>(q), q_batch_stride,
+                        static_cast<half_t *>(kv_pool), seq_lens,
+                        static_cast<const int32_t *>(plan),
+                        static_cast<const half_t *>(k_new), static_cast<const half_t *>(v_new),
+                        k_new_stride, v_new_stride, static_cast<half_t *>(out), part_o, part_lse,
+                        block_table_stride, batch, num_q_heads, num_kv_heads,
+                        num_q_heads / num_kv_heads, s.heads_per_wg, s.replicas, chunks,
+                        softmax_scale * kLog2e);
+  rc = check_launch(what);
+  if (rc != LITEKV_OK) return rc;
+  hipLaunchKernelGGL(paged_decode_balanced_merge_kernel,
+                     dim3((unsigned)num_q_heads, (unsigned)batch), dim3(kWave), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const int32_t *>(plan),
+                     static_cast<half_t *>(out), part_o, part_lse, num_q_heads);
+  return check_launch("paged_decode_balanced_merge");
+}
+
 extern "C" size_t litekv_paged_decode_workspace_bytes(int32_t batch, int32_t num_q_heads,
                                                       int32_t head_dim, int32_t max_splits) {
-  return litekv::workspace_bytes_for(batch, num_q_heads, head_dim, max_splits);
+  return litekv::splits_workspace_bytes(batch, num_q_heads, head_dim, max_splits);
 }
 
 extern "C" int litekv_paged_decode_split(const void *q, int64_t q_batch_stride, const void *kv_pool,
@@ -328,8 +961,8 @@ extern "C" int litekv_paged_decode_split(const void *q, int64_t q_batch_stride, 
                                          float softmax_scale, void *stream) {
   litekv::DecodeArgs a{q, q_batch_stride, kv_pool, block_table, block_table_stride, seq_lens, out,
                        workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim,
-                       page_size, num_pages, max_splits, min_pages_per_split, softmax_scale, stream};
-  return litekv::launch_split(a);
+                       page_size, num_pages, softmax_scale, stream};
+  return litekv::launch_split(a, max_splits, min_pages_per_split);
 }
 
 extern "C" int litekv_paged_decode_merge(const int32_t *seq_lens, void *out, const void *workspace,
@@ -339,8 +972,8 @@ extern "C" int litekv_paged_decode_merge(const int32_t *seq_lens, void *out, con
                                          void *stream) {
   litekv::DecodeArgs a{nullptr, 0, nullptr, nullptr, 1, seq_lens, out,
                        const_cast<void *>(workspace), workspace_bytes, batch, num_q_heads, 1,
-                       head_dim, page_size, 1, max_splits, min_pages_per_split, 0.f, stream};
-  return litekv::launch_merge(a);
+                       head_dim, page_size, 1, 0.f, stream};
+  return litekv::launch_merge(a, max_splits, min_pages_per_split);
 }
 
 extern "C" int litekv_paged_decode(const void *q, int64_t q_batch_stride, const void *kv_pool,
@@ -352,8 +985,8 @@ extern "C" int litekv_paged_decode(const void *q, int64_t q_batch_stride, const 
                                    int32_t min_pages_per_split, float softmax_scale, void *stream) {
   litekv::DecodeArgs a{q, q_batch_stride, kv_pool, block_table, block_table_stride, seq_lens, out,
                        workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim,
-                       page_size, num_pages, max_splits, min_pages_per_split, softmax_scale, stream};
-  int rc = litekv::launch_split(a);
+                       page_size, num_pages, softmax_scale, stream};
+  int rc = litekv::launch_split(a, max_splits, min_pages_per_split);
   if (rc != LITEKV_OK) return rc;
-  return litekv::launch_merge(a);
+  return litekv::launch_merge(a, max_splits, min_pages_per_split);
 }

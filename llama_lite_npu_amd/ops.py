@@ -125,49 +125,156 @@ def decode_workspace(batch: int, num_q_heads: int, max_splits: int, device) -> O
     return torch.empty(nbytes // 4, dtype=torch.float32, device=device)
 
 
+def balanced_chunks(num_kv_heads: int) -> int:
+    """Chunks per kv head that give every CU of the current device one workgroup."""
+    return int(_lib.load().litekv_paged_decode_balanced_chunks(int(num_kv_heads)))
+
+
+class DecodePlan:
+    """Per-step cut of the batch's pages into equal chunks (one launch, reused by every layer).
+
+    Built from the block table and lengths of the step; holds the device plan buffer (chunk
+    entries) and the partial-result workspace of the balanced schedule. Launches that share a
+    plan share its workspace and must run one after the other (same stream).
+    """
+
+    def __init__(self, block_table: torch.Tensor, seq_lens: torch.Tensor, num_q_heads: int,
+                 num_kv_heads: int, num_pages: int, chunks: Optional[int] = None,
+                 page_size: int = PAGE_SIZE):
+        lib = _lib.load()
+        _need(block_table.dim() == 2, "block_table must be [B, max_blocks]")
+        self.block_table = _dev_i32("block_table", block_table)
+        self.seq_lens = _dev_i32("seq_lens", seq_lens)
+        self.batch = int(self.block_table.shape[0])
+        _need(self.seq_lens.numel() == self.batch, "seq_lens must be [B]")
+        self.num_q_heads, self.num_kv_heads = int(num_q_heads), int(num_kv_heads)
+        self.num_pages, self.page_size = int(num_pages), int(page_size)
+        self.bt_stride = int(self.block_table.stride(0))
+        self.chunks = int(chunks) if chunks is not None else balanced_chunks(num_kv_heads)
+        dev = self.block_table.device
+        self.plan_bytes = int(lib.litekv_decode_plan_bytes(self.batch, self.bt_stride, self.num_kv_heads,
+                                                           self.chunks))
+        self.buffer = torch.empty(max(4, self.plan_bytes // 4), dtype=torch.int32, device=dev)
+        ws_bytes = int(lib.litekv_paged_decode_balanced_workspace_bytes(self.batch, self.num_q_heads,
+                                                                        HEAD_DIM, self.chunks))
+        self.workspace = torch.empty(max(4, ws_bytes // 4), dtype=torch.float32, device=dev)
+        self.workspace_bytes = ws_bytes
+        self.refresh()
+
+    def refresh(self, block_table: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None) -> None:
+        """Recomputes the cuts after the tables or lengths changed (same shapes)."""
+        if block_table is not None:
+            bt = _dev_i32("block_table", block_table)
+            _need(bt.shape == self.block_table.shape and bt.stride(0) == self.bt_stride, "block_table shape changed")
+            self.block_table = bt
+        if seq_lens is not None:
+            sl = _dev_i32("seq_lens", seq_lens)
+            _need(sl.numel() == self.batch, "seq_lens shape changed")
+            self.seq_lens = sl
+        lib = _lib.load()
+        _lib.check(lib.litekv_decode_plan(_ptr(self.block_table), self.bt_stride, _ptr(self.seq_lens), self.batch,
+                                          self.num_kv_heads, self.page_size, self.num_pages, self.chunks,
+                                          _ptr(self.buffer), self.plan_bytes, _stream()))
+
+
+def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
+                k_new: Optional[torch.Tensor] = None, v_new: Optional[torch.Tensor] = None,
+                softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The balanced schedule for one layer: optional append of k_new / v_new ([B, Hkv, D]) at logical
+    position seq_lens[b] - 1 fused into the attention of q [B, Hq, D] over the planned pages, then the
+    merge of the sequences that span several chunks."""
+    _dev_half("q", q), _dev_half("kv_pool", kv_pool)
+    _need(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2], "q must be [B, Hq, D] with contiguous heads")
+    b, hq, d = q.shape
+    _, hkv, dk, n_pages, _ = pool_geometry(kv_pool, plan.page_size)
+    _need(d == dk, "q and kv_pool differ in head_dim")
+    _need((b, hq, hkv, n_pages) == (plan.batch, plan.num_q_heads, plan.num_kv_heads, plan.num_pages),
+          "plan was made for another batch / head / pool geometry")
+    _need((k_new is None) == (v_new is None), "k_new and v_new go together")
+    kn_stride = vn_stride = 0
+    if k_new is not None:
+        _dev_half("k_new", k_new), _dev_half("v_new", v_new)
+        _need(k_new.shape == (b, hkv, d) and v_new.shape == (b, hkv, d), "k_new / v_new must be [B, Hkv, D]")
+        kn_stride, vn_stride = _rows("k_new", k_new), _rows("v_new", v_new)
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    if out is None:
+        out = torch.empty((b, hq, d), dtype=torch.float16, device=q.device)
+    else:
+        _dev_half("out", out)
+        _need(out.shape == (b, hq, d) and out.is_contiguous(), "out must be contiguous [B, Hq, D]")
+    q_stride = q.stride(0) if b > 1 else max(q.stride(0), hq * d)
+    lib = _lib.load()
+    _lib.check(lib.litekv_paged_decode_balanced(
+        _ptr(q), q_stride, _ptr(kv_pool), _ptr(plan.seq_lens), _ptr(plan.buffer), plan.plan_bytes,
+        _ptr(k_new), _ptr(v_new), kn_stride, vn_stride, _ptr(out), _ptr(plan.workspace), plan.workspace_bytes,
+        b, hq, hkv, d, plan.page_size, n_pages, plan.bt_stride, plan.chunks, float(softmax_scale), _stream()))
+    return out
+
+
+_STAGES = ("both", "split", "merge")
+
+
 def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tensor,
                  seq_lens: torch.Tensor, softmax_scale: Optional[float] = None,
                  num_splits: Optional[int] = None, min_pages_per_split: Optional[int] = None,
                  max_splits: Optional[int] = None, out: Optional[torch.Tensor] = None,
                  workspace: Optional[torch.Tensor] = None, page_size: int = PAGE_SIZE,
-                 stage: str = "both") -> torch.Tensor:
-    """Decode attention of q [B, Hq, D] over the pages named by block_table [B, max_blocks]."""
+                 stage: str = "both", schedule: Optional[str] = None,
+                 chunks: Optional[int] = None, plan: Optional[DecodePlan] = None) -> torch.Tensor:
+    """Decode attention of q [B, Hq, D] over the pages named by block_table [B, max_blocks].
+
+    schedule "balanced" (default): all pages of the batch are cut into `chunks` equal pieces per
+    kv head (default: one workgroup per CU); a DecodePlan is built for the call unless one is
+    passed. schedule "splits" (chosen when num_splits, max_splits or min_pages_per_split is
+    given): every sequence is cut into its own splits; two launches (`stage` selects one).
+    """
     _dev_half("q", q), _dev_half("kv_pool", kv_pool)
     _need(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2], "q must be [B, Hq, D] with contiguous heads")
     b, hq, d = q.shape
     _, hkv, dk, n_pages, _ = pool_geometry(kv_pool, page_size)
     _need(d == dk, "q and kv_pool differ in head_dim")
+    _need(stage in _STAGES, f"unknown stage {stage!r}")
+    if schedule is None:
+        split_args = (num_splits, max_splits, min_pages_per_split)
+        schedule = "splits" if any(x is not None for x in split_args) or stage != "both" else "balanced"
+    _need(schedule in ("balanced", "splits"), f"unknown schedule {schedule!r}")
+
+    if schedule == "balanced":
+        _need(stage == "both", "the balanced schedule is a single launch")
+        if plan is None:
+            plan = DecodePlan(block_table, seq_lens, hq, hkv, n_pages, chunks, page_size)
+        return decode_step(q, kv_pool, plan, None, None, softmax_scale, out)
+
     _need(block_table.dim() == 2 and block_table.shape[0] == b, "block_table must be [B, max_blocks]")
     block_table = _dev_i32("block_table", block_table)
     seq_lens = _dev_i32("seq_lens", seq_lens)
     _need(seq_lens.numel() == b, "seq_lens must be [B]")
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
-    if max_splits is None or min_pages_per_split is None:
-        s, pps = decode_split_plan(b, hkv, block_table.shape[1], num_splits)
-        max_splits = s if max_splits is None else max_splits
-        min_pages_per_split = pps if min_pages_per_split is None else min_pages_per_split
     if out is None:
         out = torch.empty((b, hq, d), dtype=torch.float16, device=q.device)
     else:
         _dev_half("out", out)
         _need(out.shape == (b, hq, d) and out.is_contiguous(), "out must be contiguous [B, Hq, D]")
+    lib = _lib.load()
+    q_stride = q.stride(0) if b > 1 else max(q.stride(0), hq * d)
+    if max_splits is None or min_pages_per_split is None:
+        s, pps = decode_split_plan(b, hkv, block_table.shape[1], num_splits)
+        max_splits = s if max_splits is None else max_splits
+        min_pages_per_split = pps if min_pages_per_split is None else min_pages_per_split
     if workspace is None:
         workspace = decode_workspace(b, hq, max_splits, q.device)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    lib = _lib.load()
-    q_stride = q.stride(0) if b > 1 else max(q.stride(0), hq * d)
     if stage in ("both", "split"):
         fn = lib.litekv_paged_decode if stage == "both" else lib.litekv_paged_decode_split
         _lib.check(fn(_ptr(q), q_stride, _ptr(kv_pool), _ptr(block_table), block_table.stride(0),
                       _ptr(seq_lens), _ptr(out), _ptr(workspace), ws_bytes, b, hq, hkv, d, page_size,
                       n_pages, max_splits, min_pages_per_split, float(softmax_scale), _stream()))
-    elif stage == "merge":
+    else:
         _lib.check(lib.litekv_paged_decode_merge(_ptr(seq_lens), _ptr(out), _ptr(workspace), ws_bytes, b,
                                                  hq, d, page_size, max_splits, min_pages_per_split,
                                                  _stream()))
-    else:
-        raise ValueError(f"unknown stage {stage!r}")
     return out
 
 

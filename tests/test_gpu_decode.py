@@ -29,7 +29,8 @@ def test_c1_append_then_decode():
     case = workloads.config_c1(DEV)
     ops.kv_append(case.k_new, case.v_new, case.slot_mapping, case.kv_pool)
     ref = _oracle(case)
-    for kw in ({}, {"num_splits": 1}, {"num_splits": 4}, {"max_splits": 8, "min_pages_per_split": 8}):
+    for kw in ({}, {"schedule": "balanced", "chunks": 16}, {"num_splits": 1}, {"num_splits": 4},
+               {"max_splits": 8, "min_pages_per_split": 8}):
         print("  ", kw, flush=True)
         assert_attention_close(_run(case, **kw), ref, f"C1 {kw}")
 
@@ -42,6 +43,70 @@ def test_head_layouts_and_ragged_lengths(hq, hkv):
     ref = _oracle(case)
     for kw in ({"num_splits": 1}, {"num_splits": 3}, {"max_splits": 16, "min_pages_per_split": 2}):
         assert_attention_close(_run(case, **kw), ref, f"ragged {hq}/{hkv} {kw}")
+
+
+@pytest.mark.parametrize("hq,hkv", [(64, 8), (32, 4), (16, 1), (6, 3), (32, 16), (24, 12)])
+@pytest.mark.parametrize("chunks", [1, 3, 37, 256, 1000])
+def test_balanced_schedule_any_chunk_count(hq, hkv, chunks):
+    """Equal-share schedule: chunks cut across sequence boundaries, empty sequences in between."""
+    print(f"decode balanced {hq}/{hkv} chunks={chunks}", flush=True)
+    lens = [300, 0, 1, 15, 16, 17, 700, 64, 2, 1200]
+    case = workloads.make_decode_case("balanced", 60 + hq + hkv, lens, hq, hkv, device=DEV)
+    case.seq_lens[1] = 0            # an empty sequence in the middle of the line
+    case.seq_lens[8] = 0
+    ref = _oracle(case)
+    out = _run(case, schedule="balanced", chunks=chunks)
+    assert_attention_close(out, ref, f"balanced {hq}/{hkv} chunks={chunks}")
+    assert float(out[1].abs().max()) == 0.0 and float(out[8].abs().max()) == 0.0
+    again = _run(case, schedule="balanced", chunks=chunks)
+    assert torch.equal(out, again)
+
+
+@pytest.mark.parametrize("hq,hkv,chunks", [(64, 8, None), (32, 4, 7), (16, 8, 64), (8, 1, 3)])
+def test_fused_append_decode_step(hq, hkv, chunks):
+    """One launch = append of the step's token + attention: pool bit exact, output as append->decode."""
+    print(f"decode fused step {hq}/{hkv} chunks={chunks}", flush=True)
+    lens = [37, 128, 511, 1000, 0, 15, 16, 31, 1]      # contexts; 128 -> new page, 15 -> fills a page
+    case = workloads.make_decode_case("fused", 70 + hq, lens, hq, hkv, device=DEV)
+    pool0 = case.kv_pool.clone()
+    ops.kv_append(case.k_new, case.v_new, case.slot_mapping, case.kv_pool)
+    want_out = _run(case, num_splits=1)
+    ref = _oracle(case)
+    pool = pool0.clone()
+    plan = ops.DecodePlan(case.block_table, case.seq_lens, hq, hkv, case.num_pages, chunks)
+    out = ops.decode_step(case.q, pool, plan, case.k_new, case.v_new, case.softmax_scale)
+    torch.cuda.synchronize()
+    assert torch.equal(pool.view(torch.int16), case.kv_pool.view(torch.int16)), "fused append not bit exact"
+    assert_attention_close(out, ref, "fused step vs oracle")
+    assert float((out.float() - want_out.float()).abs().max()) <= 1e-3
+    # the plan is reusable: a second layer (other pool) through the same plan
+    pool2 = pool0.clone()
+    out2 = ops.decode_step(case.q, pool2, plan, case.k_new, case.v_new, case.softmax_scale)
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out) and torch.equal(pool2.view(torch.int16), pool.view(torch.int16))
+
+
+def test_plan_refresh_follows_growing_sequences():
+    """Decode steps: lengths grow by one per step; the plan is refreshed, not rebuilt."""
+    print("decode plan refresh", flush=True)
+    case = workloads.make_decode_case("grow", 71, [14, 300, 47], 16, 8, num_pages=64, device=DEV)
+    plan = ops.DecodePlan(case.block_table, case.seq_lens, 16, 8, case.num_pages, chunks=8)
+    lens = case.seq_lens.clone()
+    for step in range(3):
+        out = ops.decode_step(case.q, case.kv_pool, plan, None, None, case.softmax_scale)
+        torch.cuda.synchronize()
+        ref = _oracle(case, lens)
+        assert_attention_close(out, ref, f"refresh step {step}")
+        lens = lens + 1
+        plan.refresh(seq_lens=lens)
+
+
+def test_balanced_all_sequences_empty():
+    print("decode balanced all empty", flush=True)
+    case = workloads.make_decode_case("empty", 61, [5, 9], 16, 8, device=DEV)
+    case.seq_lens[:] = 0
+    out = _run(case, schedule="balanced")
+    assert float(out.abs().max()) == 0.0
 
 
 def test_zero_length_sequence_gives_zeros():
