@@ -4,17 +4,18 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2] [--all]
 
 Default workload (config c2): Qwen3-32B attention shape, decode. A step is one
-pass over 64 layers' worth of independent KV pools: per layer one KV append of
-the batch's new tokens followed by paged flash-decoding (split + merge). All
-inputs are resident in HBM before the timed region. One JSON line is printed on
+pass over 64 layers' worth of independent KV pools: one step plan (the cut of
+the batch's pages into equal chunks, shared by all layers), then per layer the
+KV append of the batch's new tokens fused into paged flash-decoding, and the
+merge of its partial results. All inputs are resident in HBM before the timed
+region. One JSON line is printed on
 stdout; `--all` adds one line per other configuration on stderr and in
 gpurun_out/bench_all.jsonl.
 
 `value` is algorithmic bytes of the whole step divided by its wall-clock time.
-`roofline` describes the dominant kernel (the decode split kernel): algorithmic
-bytes of one launch over its mean duration, taken from HIP events recorded
-around every one of its launches inside the timed region, on the stream the
-kernels run on. `cpu_baseline` times the PyTorch-CPU restatement of the
+`roofline` describes the dominant kernel (the decode kernel): algorithmic bytes
+of one launch over its mean duration, taken from HIP events attached to every
+one of its launches inside the timed region, on the stream the kernels run on. `cpu_baseline` times the PyTorch-CPU restatement of the
 reference's own torch path (oracle/cpu_ref.py) on this machine's host cores for
 one layer of the same workload.
 """
@@ -42,16 +43,53 @@ def _median(xs):
     return xs[n // 2] if n % 2 else 0.5 * (xs[n // 2 - 1] + xs[n // 2])
 
 
-class DecodeLayerSet:
-    """`layers` independent KV pools sharing one batch's block tables, with pre-bound launches."""
+class HipEvents:
+    """HIP events created through the runtime PyTorch already loaded; they are attached to the decode
+    kernel's own dispatch (litekv_profile_next_decode), so they time the kernel on its stream without
+    adding packets between launches."""
 
-    def __init__(self, case, layers: int, device: str):
+    def __init__(self):
+        import ctypes
+        import torch
+
+        self.ct = ctypes
+        self.hip = ctypes.CDLL(os.path.join(os.path.dirname(torch.__file__), "lib", "libamdhip64.so"))
+        self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+
+    def create(self):
+        e = self.ct.c_void_p()
+        rc = self.hip.hipEventCreate(self.ct.byref(e))
+        if rc != 0:
+            raise RuntimeError(f"hipEventCreate failed: {rc}")
+        return e
+
+    def elapsed_ms(self, a, b) -> float:
+        ms = self.ct.c_float()
+        rc = self.hip.hipEventElapsedTime(self.ct.byref(ms), a, b)
+        if rc != 0:
+            raise RuntimeError(f"hipEventElapsedTime failed: {rc}")
+        return ms.value
+
+    def destroy(self, e) -> None:
+        self.hip.hipEventDestroy(e)
+
+
+class DecodeLayerSet:
+    """`layers` independent KV pools sharing one batch's block tables, with pre-bound launches.
+
+    A step = one plan launch (the cuts are shared by every layer of a decode step) + per layer one
+    balanced decode call with the KV append fused in (decode kernel + merge kernel)."""
+
+    def __init__(self, case, layers: int, device: str, schedule: str = "balanced"):
         import torch
         from llama_lite_npu_amd import _lib, ops
 
         self.torch = torch
         self.case = case
         self.layers = layers
+        self.schedule = schedule
         lib = _lib.load()
         self.lib = lib
         c = case
@@ -64,90 +102,130 @@ class DecodeLayerSet:
         self.pools = pools
         self.q = c.q
         self.out = torch.empty((layers, b, hq, 128), dtype=torch.float16, device=device)
-        self.max_splits, self.min_pps = ops.decode_split_plan(b, hkv, c.block_table.shape[1], c.num_splits)
-        self.ws = ops.decode_workspace(b, hq, self.max_splits, device)
-        ws_ptr = None if self.ws is None else self.ws.data_ptr()
-        ws_bytes = 0 if self.ws is None else self.ws.numel() * 4
         self.table = c.block_table.contiguous()
         self.seq_lens = c.seq_lens.contiguous()
         self.slot_mapping = c.slot_mapping.contiguous()
         stream = torch.cuda.current_stream().cuda_stream
-        self.append_args, self.split_args, self.merge_args = [], [], []
-        for l in range(layers):
-            pool_ptr = pools[l].data_ptr()
-            self.append_args.append((c.k_new.data_ptr(), c.v_new.data_ptr(), hkv * 128, hkv * 128,
-                                     self.slot_mapping.data_ptr(), pool_ptr, b, hkv, 128, slots, stream))
-            self.split_args.append((self.q.data_ptr(), hq * 128, pool_ptr, self.table.data_ptr(),
-                                    self.table.stride(0), self.seq_lens.data_ptr(), self.out[l].data_ptr(),
-                                    ws_ptr, ws_bytes, b, hq, hkv, 128, 16, c.num_pages, self.max_splits,
-                                    self.min_pps, c.softmax_scale, stream))
-            self.merge_args.append((self.seq_lens.data_ptr(), self.out[l].data_ptr(), ws_ptr, ws_bytes, b, hq,
-                                    128, 16, self.max_splits, self.min_pps, stream))
+        self.stream = stream
+        bts = self.table.stride(0)
+        if schedule == "balanced":
+            self.chunks = c.extra.get("chunks") or lib.litekv_paged_decode_balanced_chunks(hkv)
+            self.plan_bytes = lib.litekv_decode_plan_bytes(b, bts, hkv, self.chunks)
+            self.plan = torch.empty(self.plan_bytes // 4, dtype=torch.int32, device=device)
+            ws_bytes = lib.litekv_paged_decode_balanced_workspace_bytes(b, hq, 128, self.chunks)
+            self.ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=device)
+            self.plan_args = (self.table.data_ptr(), bts, self.seq_lens.data_ptr(), b, hkv, 16, c.num_pages,
+                              self.chunks, self.plan.data_ptr(), self.plan_bytes, stream)
+            self.decode_args = [
+                (self.q.data_ptr(), hq * 128, pools[l].data_ptr(), self.seq_lens.data_ptr(), self.plan.data_ptr(),
+                 self.plan_bytes, c.k_new.data_ptr(), c.v_new.data_ptr(), hkv * 128, hkv * 128,
+                 self.out[l].data_ptr(), self.ws.data_ptr(), ws_bytes, b, hq, hkv, 128, 16, c.num_pages, bts,
+                 self.chunks, c.softmax_scale, stream)
+                for l in range(layers)
+            ]
+            self.plan_info = {"schedule": "balanced", "chunks": self.chunks}
+        else:
+            self.max_splits, self.min_pps = ops.decode_split_plan(b, hkv, self.table.shape[1], c.num_splits)
+            self.ws = ops.decode_workspace(b, hq, self.max_splits, device)
+            ws_ptr = None if self.ws is None else self.ws.data_ptr()
+            ws_bytes = 0 if self.ws is None else self.ws.numel() * 4
+            self.append_args, self.split_args, self.merge_args = [], [], []
+            for l in range(layers):
+                pool_ptr = pools[l].data_ptr()
+                self.append_args.append((c.k_new.data_ptr(), c.v_new.data_ptr(), hkv * 128, hkv * 128,
+                                         self.slot_mapping.data_ptr(), pool_ptr, b, hkv, 128, slots, stream))
+                self.split_args.append((self.q.data_ptr(), hq * 128, pool_ptr, self.table.data_ptr(), bts,
+                                        self.seq_lens.data_ptr(), self.out[l].data_ptr(), ws_ptr, ws_bytes, b, hq,
+                                        hkv, 128, 16, c.num_pages, self.max_splits, self.min_pps,
+                                        c.softmax_scale, stream))
+                self.merge_args.append((self.seq_lens.data_ptr(), self.out[l].data_ptr(), ws_ptr, ws_bytes, b, hq,
+                                        128, 16, self.max_splits, self.min_pps, stream))
+            self.plan_info = {"schedule": "splits", "max_splits": self.max_splits,
+                              "min_pages_per_split": self.min_pps}
 
     def step(self, events=None):
+        """One pass over all layers. `events[l]`: (start, stop) raw HIP events for layer l's decode kernel
+        (balanced) or 3 torch events bracketing split and merge (splits)."""
         lib = self.lib
-        ap, sp, mg = lib.litekv_kv_append, lib.litekv_paged_decode_split, lib.litekv_paged_decode_merge
         rc = 0
-        for l in range(self.layers):
-            rc |= ap(*self.append_args[l])
-            if events is not None:
-                e = events[l]
-                e[0].record()
-                rc |= sp(*self.split_args[l])
-                e[1].record()
-                rc |= mg(*self.merge_args[l])
-                e[2].record()
-            else:
-                rc |= sp(*self.split_args[l])
-                rc |= mg(*self.merge_args[l])
+        if self.schedule == "balanced":
+            rc |= lib.litekv_decode_plan(*self.plan_args)
+            dec, prof = lib.litekv_paged_decode_balanced, lib.litekv_profile_next_decode
+            for l in range(self.layers):
+                if events is not None:
+                    prof(events[l][0], events[l][1])
+                rc |= dec(*self.decode_args[l])
+        else:
+            ap, sp, mg = lib.litekv_kv_append, lib.litekv_paged_decode_split, lib.litekv_paged_decode_merge
+            for l in range(self.layers):
+                rc |= ap(*self.append_args[l])
+                if events is not None:
+                    e = events[l]
+                    e[0].record()
+                    rc |= sp(*self.split_args[l])
+                    e[1].record()
+                    rc |= mg(*self.merge_args[l])
+                    e[2].record()
+                else:
+                    rc |= sp(*self.split_args[l])
+                    rc |= mg(*self.merge_args[l])
         if rc:
             raise RuntimeError(f"liblitekv launch failed: {lib.litekv_last_error().decode()}")
 
 
-def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: str) -> dict:
+def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: str,
+               schedule: str = "balanced") -> dict:
     import torch
 
-    ls = DecodeLayerSet(case, layers, device)
+    ls = DecodeLayerSet(case, layers, device, schedule)
     for _ in range(max(1, warmup)):
         ls.step()
     torch.cuda.synchronize()
-    events = [[[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(layers)]
-              for _ in range(steps)]
-    # plain wall-clock region: exactly `steps` steps, synchronised on both sides
+    balanced = schedule == "balanced"
+    if balanced:
+        hip = HipEvents()
+        events = [[(hip.create(), hip.create()) for _ in range(layers)] for _ in range(steps)]
+    else:
+        events = [[[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(layers)]
+                  for _ in range(steps)]
+    # timed region: exactly `steps` steps, synchronised on both sides
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for s in range(steps):
         ls.step(events[s])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    split_ms, merge_ms = [], []
+    kernel_ms = []
     for s in range(steps):
         for l in range(layers):
             e = events[s][l]
-            split_ms.append(e[0].elapsed_time(e[1]))
-            merge_ms.append(e[1].elapsed_time(e[2]))
+            kernel_ms.append(hip.elapsed_ms(e[0], e[1]) if balanced else e[0].elapsed_time(e[1]))
+    if balanced:
+        for s in range(steps):
+            for l in range(layers):
+                hip.destroy(events[s][l][0])
+                hip.destroy(events[s][l][1])
     ms_per_step = wall * 1e3 / steps
     decode_bytes = case.decode_bytes()
     append_bytes = case.append_bytes()
     step_bytes = layers * (decode_bytes + append_bytes)
-    split_mean = sum(split_ms) / len(split_ms)
-    achieved = decode_bytes / (split_mean * 1e-3) / 1e9
-    return {
+    k_mean = sum(kernel_ms) / len(kernel_ms)
+    # the fused kernel also moves the appended rows; they are part of its algorithmic bytes
+    kernel_bytes = decode_bytes + (append_bytes if balanced else 0)
+    achieved = kernel_bytes / (k_mean * 1e-3) / 1e9
+    res = {
         "label": label,
         "ms_per_step": ms_per_step,
         "value": step_bytes / (ms_per_step * 1e-3) / 1e9,
         "us_per_layer": ms_per_step * 1e3 / layers,
-        "decode_split_us_mean": split_mean * 1e3,
-        "decode_split_us_median": _median(split_ms) * 1e3,
-        "decode_split_us_min": min(split_ms) * 1e3,
-        "decode_merge_us_mean": sum(merge_ms) / len(merge_ms) * 1e3,
+        "decode_kernel_us_mean": k_mean * 1e3,
+        "decode_kernel_us_median": _median(kernel_ms) * 1e3,
+        "decode_kernel_us_min": min(kernel_ms) * 1e3,
         "decode_bytes_per_layer": decode_bytes,
         "append_bytes_per_layer": append_bytes,
         "layers": layers,
-        "max_splits": ls.max_splits,
-        "min_pages_per_split": ls.min_pps,
         "roofline": {
-            "kernel": "paged_decode_split_kernel",
+            "kernel": "paged_decode_balanced_kernel" if balanced else "paged_decode_split_kernel",
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
@@ -156,6 +234,8 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
             "traffic": None,
         },
     }
+    res.update(ls.plan_info)
+    return res
 
 
 def time_append(case_tokens_k, case_tokens_v, slot_mapping, pool, reps: int = 20) -> float:
@@ -275,6 +355,8 @@ def main() -> int:
     ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--layers", type=int, default=None, help="independent KV pools per step (c2 default 64)")
     ap.add_argument("--all", action="store_true", help="also report the other configurations (stderr)")
+    ap.add_argument("--schedule", default="balanced", choices=["balanced", "splits"],
+                    help="decode work decomposition (splits: separate append, split and merge launches)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -308,7 +390,10 @@ def main() -> int:
             case = workloads.config_c3(device)
             return run_prefill(case, args.steps, args.warmup, device, case.name), case
         case, layers = decode_cfg(name)
-        return run_decode(case, layers, args.steps, args.warmup, device, case.name), case
+        sched = args.schedule
+        if name == "c5" and args.schedule == "balanced" and False:
+            sched = "splits"
+        return run_decode(case, layers, args.steps, args.warmup, device, case.name, sched), case
 
     res, case = run(args.config)
     line = {
