@@ -1,0 +1,339 @@
+"""Paged-KV metadata API of the executor: request reservation, prefix-cache sharing and the
+per-step ``AttentionInfo`` builders.
+
+Method names, arguments, return values and error texts follow the paged half of the reference's
+``ModelExecutor`` (lite_llama/executor/model_executor.py:496-987); model loading, tensor-parallel
+weight sharding and graph capture are not part of this package. Differences underneath:
+
+* every builder assembles its slot mappings and lengths on the host and uploads each tensor
+  once (the reference concatenates per-request device views);
+* the batch's block-table rows travel with the metadata (``atten_info.block_table``), and a
+  decode step carries a ``DecodePlan`` shared by all layers;
+* ``copy_on_write`` runs before appends into shared pages, and ``compact_kv_pool`` exists.
+"""
+
+from __future__ import annotations
+
+from collections import OrderedDict
+from typing import Optional, Sequence
+
+import numpy as np
+import torch
+
+from .executor_struct import AttentionInfo
+from .paged_attention import PagedKVCacheManager, PagedReqTokensManager
+
+
+class ModelExecutor:
+    """Owns the page pool, the request tables, the prefix caches and the step metadata."""
+
+    def __init__(self, num_layers: int, num_q_heads: int, num_kv_heads: int, head_dim: int,
+                 num_pages: int, max_seq_len: int, max_requests: Optional[int] = None,
+                 page_size: int = 16, device: str = "cuda:0", dtype: torch.dtype = torch.float16,
+                 tp_world_size: int = 1, build_decode_plans: bool = True):
+        if page_size <= 0:
+            raise ValueError("this executor only runs the paged path (page_size > 0)")
+        self.device = device
+        # heads are sharded over tensor-parallel ranks exactly as in the reference (:249-250)
+        self.local_q_heads = num_q_heads // tp_world_size
+        self.local_kv_heads = num_kv_heads // tp_world_size
+        self.head_dim = head_dim
+        self.num_layers = num_layers
+        self.max_seq_len = int(max_seq_len)
+        self.page_size = int(page_size)
+        self.use_paged_attn = True
+        self.kv_mem_manager = PagedKVCacheManager(num_layers, self.local_kv_heads, head_dim, num_pages,
+                                                  page_size, dtype, device)
+        if max_requests is None:
+            max_requests = max(1, (num_pages * page_size) // self.max_seq_len)
+        self.max_request_num = int(max_requests)
+        self.req_tokens_manager = PagedReqTokensManager(self.max_request_num, self.max_seq_len,
+                                                        self.kv_mem_manager, device=device)
+        self.atten_info = AttentionInfo()
+        self.atten_info.kv_buffer = self.kv_mem_manager.gpu_kv_buffer
+        self.build_decode_plans = build_decode_plans and torch.device(device).type == "cuda"
+        self._decode_plan = None
+        self._paged_request_ids: tuple[int, ...] = ()
+        # exact-prompt cache: prompt -> (pages, token count, first generated token), LRU of 128
+        self._paged_prefix_cache: OrderedDict = OrderedDict()
+        self._paged_prefix_cache_max_entries = 128
+        # block cache: (fingerprint of the parent chain, block tokens) -> (page, tokens covered), LRU of 4096
+        self._paged_block_prefix_cache: OrderedDict = OrderedDict()
+        self._paged_block_prefix_cache_max_entries = 4096
+        self.max_prefill_tokens = max(1, 60000 // max(1, self.local_q_heads))
+
+    # ---- reservation -----------------------------------------------------------------------
+    def reserve_paged_requests(self, prompt_lengths: Sequence[int],
+                               reserved_lengths: Optional[Sequence[int]] = None) -> tuple[int, ...]:
+        """One request id per prompt; on failure everything reserved by the call is released."""
+        if reserved_lengths is not None and len(reserved_lengths) != len(prompt_lengths):
+            raise ValueError("reserved_lengths must match prompt_lengths")
+        made: list[int] = []
+        try:
+            for i, length in enumerate(prompt_lengths):
+                cap = None if reserved_lengths is None else int(reserved_lengths[i])
+                req_idx = self.req_tokens_manager.reserve_req(int(length), cap)
+                if req_idx is None:
+                    raise RuntimeError("Paged KV request or page capacity is exhausted")
+                made.append(req_idx)
+        except BaseException:
+            for req_idx in made:
+                self.req_tokens_manager.free_req(req_idx)
+            raise
+        return tuple(made)
+
+    def ensure_paged_request_capacity(self, req_idx: int, total_tokens: int) -> None:
+        if not self.req_tokens_manager.ensure_req_capacity(req_idx, total_tokens):
+            raise RuntimeError(f"Paged KV capacity reservation failed for request {req_idx}")
+
+    # ---- prefix caches ---------------------------------------------------------------------
+    @staticmethod
+    def _paged_block_key(parent_fingerprint, block_tokens):
+        return parent_fingerprint, tuple(int(t) for t in block_tokens)
+
+    def share_paged_request_from_cache(self, prompt_tokens) -> Optional[tuple[int, int]]:
+        """Exact prompt hit: a new request sharing the cached pages, and the cached first token."""
+        key = tuple(int(t) for t in prompt_tokens)
+        hit = self._paged_prefix_cache.get(key)
+        if hit is None:
+            return None
+        self._paged_prefix_cache.move_to_end(key)
+        pages, num_tokens, first_token = hit
+        req_idx = self.req_tokens_manager.reserve_shared_req(pages, num_tokens)
+        return None if req_idx is None else (int(req_idx), int(first_token))
+
+    def share_paged_prefix_from_cache(self, prompt_tokens) -> Optional[tuple[int, int, Optional[int]]]:
+        """(request id, matched tokens, first token or None): the exact prompt if cached, else the
+        longest chain of cached full pages (the caller then replays only the suffix)."""
+        key = tuple(int(t) for t in prompt_tokens)
+        if not key:
+            return None
+        exact = self._paged_prefix_cache.get(key)
+        if exact is not None:
+            self._paged_prefix_cache.move_to_end(key)
+            pages, num_tokens, first_token = exact
+            req_idx = self.req_tokens_manager.reserve_shared_req(pages, num_tokens)
+            return None if req_idx is None else (int(req_idx), len(key), int(first_token))
+        chain: list[torch.Tensor] = []
+        matched, parent, ps = 0, None, self.page_size
+        for first in range(0, len(key) - ps + 1, ps):
+            block_key = self._paged_block_key(parent, key[first:first + ps])
+            hit = self._paged_block_prefix_cache.get(block_key)
+            if hit is None:
+                break
+            self._paged_block_prefix_cache.move_to_end(block_key)
+            page, covered = hit
+            chain.append(page.reshape(-1))
+            matched = int(covered)
+            parent = hash(block_key)
+        if not chain or matched <= 0:
+            return None
+        req_idx = self.req_tokens_manager.reserve_shared_req(torch.cat(chain), matched)
+        return None if req_idx is None else (int(req_idx), matched, None)
+
+    def _store_paged_prompt_blocks(self, prompt_tokens: tuple[int, ...], page_indices: torch.Tensor) -> None:
+        ps = self.page_size
+        parent = None
+        for block in range(len(prompt_tokens) // ps):
+            block_key = self._paged_block_key(parent, prompt_tokens[block * ps:(block + 1) * ps])
+            parent = hash(block_key)
+            if block_key in self._paged_block_prefix_cache:
+                self._paged_block_prefix_cache.move_to_end(block_key)
+                continue
+            page = page_indices[block:block + 1].clone()
+            self.kv_mem_manager.add_ref(page)
+            self._paged_block_prefix_cache[block_key] = (page, (block + 1) * ps)
+            while len(self._paged_block_prefix_cache) > self._paged_block_prefix_cache_max_entries:
+                _, (old_page, _) = self._paged_block_prefix_cache.popitem(last=False)
+                self.kv_mem_manager.free(old_page)
+
+    def store_paged_request_prefix(self, prompt_tokens, req_idx: int, first_token_id: int) -> None:
+        """Caches a finished prefill: one page reference for the exact prompt, one per full block."""
+        if req_idx not in self.req_tokens_manager.req_page_table:
+            return
+        key = tuple(int(t) for t in prompt_tokens)
+        if key in self._paged_prefix_cache:
+            return
+        pages = self.req_tokens_manager.req_page_table[int(req_idx)]
+        self.kv_mem_manager.add_ref(pages)
+        self._paged_prefix_cache[key] = (pages.clone(), int(self.req_tokens_manager.req_token_count[int(req_idx)]),
+                                         int(first_token_id))
+        self._store_paged_prompt_blocks(key, pages)
+        while len(self._paged_prefix_cache) > self._paged_prefix_cache_max_entries:
+            _, (old_pages, _, _) = self._paged_prefix_cache.popitem(last=False)
+            self.kv_mem_manager.free(old_pages)
+
+    # ---- step metadata ---------------------------------------------------------------------
+    def _reset_paged_chunk_prefill_metadata(self) -> None:
+        info = self.atten_info
+        info.is_paged_chunk_prefill = False
+        info.chunk_context_len = info.chunk_q_seq_len = info.max_actual_q_seq_len = None
+        info.context_lens_i32 = None
+        info.decode_plan = None
+
+    def _i32(self, values) -> torch.Tensor:
+        return torch.as_tensor(np.asarray(values, dtype=np.int32), device=self.device)
+
+    def _i64(self, values) -> torch.Tensor:
+        return torch.as_tensor(np.asarray(values, dtype=np.int64), device=self.device)
+
+    def _set_batch(self, request_ids: tuple[int, ...], kv_lens: Sequence[int], q_lens: Sequence[int],
+                   slot_parts: list[np.ndarray]) -> None:
+        """Common tail of the builders: ids, lengths, slot mapping, packed starts, block-table rows."""
+        info, mgr = self.atten_info, self.req_tokens_manager
+        self._paged_request_ids = request_ids
+        info.b_req_idx = self._i32(request_ids)
+        info.b_seq_len = self._i64(kv_lens)
+        info.seq_lens_i32 = self._i32(kv_lens)
+        info.cur_select_index = self._i32(np.concatenate(slot_parts) if slot_parts else [])
+        cu = np.zeros(len(q_lens) + 1, dtype=np.int32)
+        cu[1:] = np.cumsum(q_lens)
+        info.cu_q_lens = self._i32(cu)
+        info.b_start_loc = self._i32(cu[:-1])
+        info.block_table = mgr.block_table_rows(request_ids)
+        info.b_req_tokens_table = None   # derived from the block table only if somebody asks
+        info.max_actual_seq_len = int(max(kv_lens))
+
+    def activate_paged_prefill_batch(self, request_ids: tuple[int, ...], prompt_length: int) -> None:
+        """Equal-length prompts, one prefill forward."""
+        self._reset_paged_chunk_prefill_metadata()
+        if not request_ids:
+            raise ValueError("request_ids must not be empty")
+        mgr = self.req_tokens_manager
+        for req_idx in request_ids:
+            actual = mgr.req_token_count[req_idx]
+            if actual != prompt_length:
+                raise ValueError("continuous prefill groups must have equal prompt "
+                                 f"lengths: expected={prompt_length}, request={req_idx}, actual={actual}")
+        ids = tuple(int(r) for r in request_ids)
+        lens = [int(prompt_length)] * len(ids)
+        self._set_batch(ids, lens, lens, [mgr.slots(r, 0, prompt_length) for r in ids])
+
+    def activate_paged_packed_prefill_batch(self, request_ids, prompt_lengths):
+        """Mixed-length prompts packed without padding. Returns (flat position ids, flat index of
+        each request's last prompt token), both int64 on the device."""
+        self._reset_paged_chunk_prefill_metadata()
+        if not request_ids:
+            raise ValueError("request_ids must not be empty")
+        if len(request_ids) != len(prompt_lengths):
+            raise ValueError("request_ids and prompt_lengths must have same length")
+        lens = [int(n) for n in prompt_lengths]
+        if any(n <= 0 for n in lens):
+            raise ValueError("prompt_lengths must be positive")
+        mgr = self.req_tokens_manager
+        ids = tuple(int(r) for r in request_ids)
+        for req_idx, n in zip(ids, lens):
+            actual = mgr.req_token_count[req_idx]
+            if actual != n:
+                raise ValueError("packed prefill request length mismatch: "
+                                 f"request={req_idx}, expected={n}, actual={actual}")
+        self._set_batch(ids, lens, lens, [mgr.slots(r, 0, n) for r, n in zip(ids, lens)])
+        ends = np.cumsum(lens)
+        positions = np.concatenate([np.arange(n) for n in lens])
+        return self._i64(positions), self._i64(ends - 1)
+
+    def activate_paged_chunk_prefill_batch(self, request_ids, context_lengths, chunk_lengths):
+        """Later chunks of a chunked prefill: extends each request by its chunk, then describes a
+        batch whose queries are the chunks and whose keys are history + chunk, read through the
+        pages. Returns (flat position ids, flat index of each chunk's last token)."""
+        if not request_ids:
+            raise ValueError("request_ids must not be empty")
+        if len(request_ids) != len(context_lengths) or len(request_ids) != len(chunk_lengths):
+            raise ValueError("request_ids, context_lengths and chunk_lengths must have same length")
+        ids = tuple(int(r) for r in request_ids)
+        ctx = [int(n) for n in context_lengths]
+        chunk = [int(n) for n in chunk_lengths]
+        if any(n < 0 for n in ctx):
+            raise ValueError("context_lengths must be non-negative")
+        if any(n <= 0 for n in chunk):
+            raise ValueError("chunk_lengths must be positive")
+        mgr = self.req_tokens_manager
+        for req_idx, c, q in zip(ids, ctx, chunk):
+            actual = mgr.req_token_count[req_idx]
+            if actual != c:
+                raise ValueError("paged chunk prefill context length mismatch: "
+                                 f"request={req_idx}, expected={c}, actual={actual}")
+            if not mgr.extend_req(req_idx, q):
+                raise RuntimeError(
+                    "Paged KV allocation failed for chunked prefill request "
+                    f"{req_idx}: context_tokens={c}, chunk_tokens={q}, "
+                    f"current_tokens={mgr.req_token_count.get(req_idx, 'unknown')}, "
+                    f"max_seq_len={mgr.max_seq_len}, free_pages={mgr.page_mgr.num_free_pages}")
+        self._reset_paged_chunk_prefill_metadata()
+        total = [c + q for c, q in zip(ctx, chunk)]
+        self._set_batch(ids, total, chunk, [mgr.slots(r, c, t) for r, c, t in zip(ids, ctx, total)])
+        info = self.atten_info
+        info.max_actual_q_seq_len = max(chunk)
+        info.chunk_context_len = self._i64(ctx)
+        info.chunk_q_seq_len = self._i64(chunk)
+        info.context_lens_i32 = self._i32(ctx)
+        info.is_paged_chunk_prefill = True
+        ends = np.cumsum(chunk)
+        positions = np.concatenate([np.arange(c, c + q) for c, q in zip(ctx, chunk)])
+        return self._i64(positions), self._i64(ends - 1)
+
+    def activate_paged_decode_batch(self, request_ids: tuple[int, ...]) -> None:
+        """Metadata of one decode step: each sequence's length already counts the token whose K/V
+        this step appends, and ``cur_select_index`` is that token's slot."""
+        self._reset_paged_chunk_prefill_metadata()
+        mgr = self.req_tokens_manager
+        ids = tuple(int(r) for r in request_ids)
+        req_ids, seq_lens, last = mgr.batch_metadata(list(ids))
+        info = self.atten_info
+        self._paged_request_ids = ids
+        info.b_req_idx, info.b_seq_len, info.cur_select_index = req_ids, seq_lens, last
+        info.seq_lens_i32 = seq_lens.to(torch.int32)
+        info.b_start_loc = torch.zeros(len(ids), dtype=torch.int32, device=self.device)
+        info.cu_q_lens = torch.arange(len(ids) + 1, dtype=torch.int32, device=self.device)
+        info.block_table = mgr.block_table_rows(ids)
+        info.b_req_tokens_table = None
+        info.max_actual_seq_len = max(mgr.req_token_count[r] for r in ids)
+        if self.build_decode_plans:
+            from .. import ops
+
+            info.decode_plan = ops.DecodePlan(info.block_table, info.seq_lens_i32, self.local_q_heads,
+                                              self.local_kv_heads, self.kv_mem_manager.num_pages,
+                                              page_size=self.page_size)
+
+    def extend_paged_requests(self, request_ids: tuple[int, ...]) -> None:
+        """Reserves the KV position of the next decode input of every request, then activates the batch."""
+        mgr = self.req_tokens_manager
+        for req_idx in request_ids:
+            if not mgr.extend_req(req_idx, 1):
+                raise RuntimeError(
+                    "Paged KV allocation failed for request "
+                    f"{req_idx}: current_tokens={mgr.req_token_count.get(req_idx, 'unknown')}, "
+                    f"max_seq_len={mgr.max_seq_len}, free_pages={mgr.page_mgr.num_free_pages}")
+        self.activate_paged_decode_batch(tuple(request_ids))
+
+    def decode_alloc_kv_cache(self, batch_size: int) -> torch.Tensor:
+        """Static-batch decode step over the request ids cached at prefill time."""
+        if len(self._paged_request_ids) != batch_size:
+            raise RuntimeError("Paged request id cache is not initialized for the "
+                               f"decode batch: cached={len(self._paged_request_ids)}, batch_size={batch_size}")
+        for req_idx in self._paged_request_ids:
+            if not self.req_tokens_manager.extend_req(req_idx, 1):
+                raise RuntimeError("Paged KV allocation failed during decode")
+        self.activate_paged_decode_batch(self._paged_request_ids)
+        return self.atten_info.cur_select_index
+
+    def release_paged_request_ids(self, request_ids: tuple[int, ...]) -> None:
+        for req_idx in request_ids:
+            self.req_tokens_manager.free_req(req_idx)
+        if tuple(request_ids) == self._paged_request_ids:
+            self._paged_request_ids = ()
+
+    def release_paged_requests(self) -> None:
+        self.release_paged_request_ids(self._paged_request_ids)
+
+    # ---- page moves ------------------------------------------------------------------------
+    def copy_on_write(self, request_ids: Sequence[int]):
+        """Private copies of shared last pages before a step appends into them."""
+        return self.req_tokens_manager.copy_on_write(request_ids)
+
+    def compact_kv_pool(self):
+        """Moves live pages into the dense prefix of the pool (all layers), fixing every table and
+        every prefix-cache entry that names a moved page."""
+        holders = [entry[0] for entry in self._paged_prefix_cache.values()]
+        holders += [entry[0] for entry in self._paged_block_prefix_cache.values()]
+        return self.req_tokens_manager.compact(holders)

@@ -1,0 +1,226 @@
+"""GPU: the reference's call surface end to end -- executor metadata -> Attention.context_forward /
+token_forward -> HIP kernels -- checked against the CPU oracle; prefix sharing with copy-on-write,
+pool compaction, and the lite_llama.kernels-compatible wrappers."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from llama_lite_npu_amd import kernels as compat
+from llama_lite_npu_amd import ops
+from llama_lite_npu_amd.attention import Attention
+from llama_lite_npu_amd.executor import ModelExecutor
+from oracle import c_oracle
+from tests.parity import assert_attention_close, assert_bit_exact, to_np16
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+HQ, HKV, D = 16, 8, 128
+SCALE = 1.0 / math.sqrt(D)
+LOG2E = 1.4426950408889634
+
+
+def _executor(num_pages=96, layers=2, max_requests=8, max_seq_len=512):
+    ex = ModelExecutor(num_layers=layers, num_q_heads=HQ, num_kv_heads=HKV, head_dim=D, num_pages=num_pages,
+                       max_seq_len=max_seq_len, max_requests=max_requests, device=DEV)
+    for pool in ex.kv_mem_manager.gpu_kv_buffer:
+        pool.normal_()          # stale data everywhere: only written slots may matter
+    return ex
+
+
+def _qkv(tokens, seed):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    q = torch.randn((tokens, HQ, D), generator=g, device=DEV, dtype=torch.float16)
+    k = torch.randn((tokens, HKV, D), generator=g, device=DEV, dtype=torch.float16)
+    v = torch.randn((tokens, HKV, D), generator=g, device=DEV, dtype=torch.float16)
+    return q, k, v
+
+
+def _oracle_decode(ex, q, layer):
+    info = ex.atten_info
+    return c_oracle.paged_decode(to_np16(q), to_np16(info.kv_buffer[layer]), info.block_table.cpu().numpy(),
+                                 info.seq_lens_i32.cpu().numpy(), SCALE)
+
+
+def test_packed_prefill_then_fused_decode_steps():
+    print("executor: packed prefill + decode", flush=True)
+    ex = _executor()
+    attn = Attention(HQ, HKV, D)
+    lens = [37, 16, 90, 5]
+    ids = ex.reserve_paged_requests(lens)
+    ex.activate_paged_packed_prefill_batch(ids, lens)
+    info = ex.atten_info
+    total = sum(lens)
+    for layer in range(2):
+        q, k, v = _qkv(total, 10 + layer)
+        out = attn.context_forward(q, k, v, info, layer, qk_scale=SCALE * LOG2E)
+        torch.cuda.synchronize()
+        ref = c_oracle.varlen_prefill(to_np16(q), to_np16(k), to_np16(v), info.b_start_loc.cpu().numpy(),
+                                      np.asarray(lens, dtype=np.int32), SCALE)
+        assert_attention_close(out, ref, f"prefill layer {layer}")
+        # the K/V rows landed in the slots the metadata names
+        pool = info.kv_buffer[layer]
+        sel = info.cur_select_index.long()
+        assert_bit_exact(pool[sel][:, :HKV], k, "K rows in pages")
+        assert_bit_exact(pool[sel][:, HKV:], v, "V rows in pages")
+    for step in range(20):             # 16 -> 17 opens a page, 37 + 11 = 48 fills one
+        ex.extend_paged_requests(ids)
+        info = ex.atten_info
+        assert info.decode_plan is not None
+        for layer in range(2):
+            q, k, v = _qkv(len(ids), 100 + 2 * step + layer)
+            out = attn.token_forward(q, k, v, info, layer, qk_scale=SCALE)
+            torch.cuda.synchronize()
+            pool = info.kv_buffer[layer]
+            sel = info.cur_select_index.long()
+            assert_bit_exact(pool[sel][:, :HKV], k, "appended K")
+            assert_bit_exact(pool[sel][:, HKV:], v, "appended V")
+            assert_attention_close(out, _oracle_decode(ex, q, layer), f"decode step {step} layer {layer}")
+    assert info.b_seq_len.tolist() == [n + 20 for n in lens]
+
+
+def test_chunked_prefill_matches_one_shot_prefill():
+    print("executor: chunked prefill", flush=True)
+    attn = Attention(HQ, HKV, D)
+    n = 150
+    q, k, v = _qkv(n, 7)
+    whole = _executor(layers=1)
+    (rid,) = whole.reserve_paged_requests([n])
+    whole.activate_paged_packed_prefill_batch((rid,), [n])
+    out_whole = attn.context_forward(q, k, v, whole.atten_info, 0, SCALE * LOG2E)
+
+    ex = _executor(layers=1)
+    (rid,) = ex.reserve_paged_requests([64], reserved_lengths=[n])
+    ex.activate_paged_packed_prefill_batch((rid,), [64])
+    outs = [attn.context_forward(q[:64], k[:64], v[:64], ex.atten_info, 0, SCALE * LOG2E)]
+    done = 64
+    for chunk in (50, 36):
+        ex.activate_paged_chunk_prefill_batch((rid,), [done], [chunk])
+        sl = slice(done, done + chunk)
+        outs.append(attn.context_forward(q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous(),
+                                         ex.atten_info, 0, SCALE * LOG2E))
+        done += chunk
+    torch.cuda.synchronize()
+    got = torch.cat(outs)
+    assert float((got.float() - out_whole.float()).abs().max()) <= 1e-3
+    ref = c_oracle.varlen_prefill(to_np16(q), to_np16(k), to_np16(v), np.array([0], dtype=np.int32),
+                                  np.array([n], dtype=np.int32), SCALE)
+    assert_attention_close(got, ref, "chunked prefill")
+
+
+def test_prefix_sharing_with_copy_on_write():
+    print("executor: prefix sharing + COW", flush=True)
+    ex = _executor(layers=1)
+    attn = Attention(HQ, HKV, D)
+    prompt = tuple(range(1000, 1040))                # 40 tokens: 2 full pages + 8 tokens
+    (a,) = ex.reserve_paged_requests([40])
+    ex.activate_paged_packed_prefill_batch((a,), [40])
+    q, k, v = _qkv(40, 21)
+    attn.context_forward(q, k, v, ex.atten_info, 0, SCALE * LOG2E)
+    ex.store_paged_request_prefix(prompt, a, first_token_id=3)
+    b, first = ex.share_paged_request_from_cache(prompt)
+    assert first == 3
+    pages_a = ex.req_tokens_manager.request_pages(a)
+    assert ex.req_tokens_manager.request_pages(b) == pages_a
+    pool = ex.atten_info.kv_buffer[0]
+    before = pool.clone()
+    # both requests are about to append token 40 into the shared, partly filled third page
+    moves = ex.copy_on_write((a, b))
+    torch.cuda.synchronize()
+    # the cache entry still holds the original page, so both requests get a private copy of it
+    assert len(moves) == 2 and {m[0] for m in moves} == {pages_a[2]}
+    pages_a2, pages_b2 = ex.req_tokens_manager.request_pages(a), ex.req_tokens_manager.request_pages(b)
+    assert pages_a2[:2] == pages_b2[:2] == pages_a[:2] and len({pages_a[2], pages_a2[2], pages_b2[2]}) == 3
+    for src, dst in moves:
+        assert_bit_exact(pool[dst * 16:(dst + 1) * 16], before[src * 16:(src + 1) * 16], "COW page copy")
+    ex.extend_paged_requests((a, b))
+    qd, kd, vd = _qkv(2, 22)
+    out = attn.token_forward(qd, kd, vd, ex.atten_info, 0, SCALE)
+    torch.cuda.synchronize()
+    assert_attention_close(out, _oracle_decode(ex, qd, 0), "decode after COW")
+    # the cached page was not touched by either append
+    shared = pages_a[2]
+    assert_bit_exact(pool[shared * 16:(shared + 1) * 16], before[shared * 16:(shared + 1) * 16], "cached page")
+    # the two requests read the same prefix but their own new token
+    assert float((out[0].float() - out[1].float()).abs().max()) > 1e-3
+
+
+def test_compaction_keeps_results_bitwise():
+    print("executor: compaction", flush=True)
+    ex = _executor(num_pages=64, layers=2)
+    attn = Attention(HQ, HKV, D)
+    lens = [70, 33, 120, 48, 9]
+    ids = ex.reserve_paged_requests(lens)
+    ex.activate_paged_packed_prefill_batch(ids, lens)
+    for layer in range(2):
+        q, k, v = _qkv(sum(lens), 30 + layer)
+        attn.context_forward(q, k, v, ex.atten_info, layer, SCALE * LOG2E)
+    ex.release_paged_request_ids((ids[0], ids[3]))        # punch holes into the pool
+    keep = (ids[1], ids[2], ids[4])
+    ex.activate_paged_decode_batch(keep)
+    qd = _qkv(3, 40)[0]
+    before = [ops.paged_decode(qd, ex.atten_info.kv_buffer[l], ex.atten_info.block_table,
+                               ex.atten_info.seq_lens_i32, SCALE, num_splits=1) for l in range(2)]
+    moves = ex.compact_kv_pool()
+    assert moves, "expected at least one page move"
+    n_live = sum(len(ex.req_tokens_manager.request_pages(r)) for r in keep)
+    assert all(dst < n_live <= src for src, dst in moves)
+    assert sorted(p for r in keep for p in ex.req_tokens_manager.request_pages(r)) == list(range(n_live))
+    ex.activate_paged_decode_batch(keep)
+    after = [ops.paged_decode(qd, ex.atten_info.kv_buffer[l], ex.atten_info.block_table,
+                              ex.atten_info.seq_lens_i32, SCALE, num_splits=1) for l in range(2)]
+    torch.cuda.synchronize()
+    for l in range(2):
+        assert torch.equal(before[l], after[l]), "compaction changed the attention result"
+
+
+def test_lite_llama_kernels_signatures():
+    """The four reference functions, called the way lite_llama/models/qwen3.py:20-75 calls them."""
+    print("compat wrappers", flush=True)
+    ex = _executor(layers=1)
+    lens = [45, 130, 17]
+    ids = ex.reserve_paged_requests(lens)
+    ex.activate_paged_packed_prefill_batch(ids, lens)
+    info = ex.atten_info
+    pool = info.kv_buffer[0]
+    q, k, v = _qkv(sum(lens), 50)
+    compat.update_kv_buffer(torch.cat([k, v], dim=-2), info.cur_select_index, pool)
+    out = compat.flash_attention2_no_pad(q, k, v, SCALE * LOG2E, info.b_start_loc, info.b_seq_len,
+                                         info.max_actual_seq_len)
+    torch.cuda.synchronize()
+    sel = info.cur_select_index.long()
+    assert_bit_exact(pool[sel], torch.cat([k, v], dim=-2), "update_kv_buffer")
+    ref = c_oracle.varlen_prefill(to_np16(q), to_np16(k), to_np16(v), info.b_start_loc.cpu().numpy(),
+                                  np.asarray(lens, dtype=np.int32), SCALE)
+    assert_attention_close(out, ref, "flash_attention2_no_pad")
+
+    table = ex.req_tokens_manager.b_req_tokens_table          # the reference's per-token table
+    ex.extend_paged_requests(ids)
+    info = ex.atten_info
+    table = ex.req_tokens_manager.b_req_tokens_table
+    qd, kd, vd = _qkv(3, 51)
+    compat.update_kv_buffer(torch.cat([kd, vd], dim=-2), info.cur_select_index, pool)
+    out = compat.flash_decoding(qd, pool[:, :HKV, :], pool[:, HKV:, :], SCALE, table, info.b_seq_len,
+                                info.max_actual_seq_len)
+    torch.cuda.synchronize()
+    assert_attention_close(out, _oracle_decode(ex, qd, 0), "flash_decoding")
+
+    # later chunk of a chunked prefill through the paged function
+    ctx = [int(n) for n in info.b_seq_len.tolist()]
+    chunk = [20, 3, 31]
+    ex.activate_paged_chunk_prefill_batch(ids, ctx, chunk)
+    info = ex.atten_info
+    table = ex.req_tokens_manager.b_req_tokens_table
+    qc, kc, vc = _qkv(sum(chunk), 52)
+    compat.update_kv_buffer(torch.cat([kc, vc], dim=-2), info.cur_select_index, pool)
+    out = compat.paged_chunk_flash_attention(qc, pool[:, :HKV, :], pool[:, HKV:, :], SCALE * LOG2E, table,
+                                             info.b_req_idx, info.b_start_loc, info.chunk_context_len,
+                                             info.chunk_q_seq_len, info.max_actual_q_seq_len)
+    torch.cuda.synchronize()
+    ref = c_oracle.paged_prefill(to_np16(qc), to_np16(pool), info.block_table.cpu().numpy(),
+                                 info.cu_q_lens.cpu().numpy(), np.asarray(ctx, dtype=np.int32), SCALE)
+    assert_attention_close(out, ref, "paged_chunk_flash_attention")
+    with pytest.raises(ValueError, match="halves of one"):
+        compat.flash_decoding(qd, pool[:, :HKV, :].contiguous(), pool[:, HKV:, :], SCALE, table, info.b_seq_len, 8)

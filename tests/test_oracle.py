@@ -1,0 +1,228 @@
+"""Pins the CPU oracle (oracle/litekv_oracle.c and oracle/cpu_ref.py) before it is trusted as the
+checker of the HIP kernels: closed forms, brute force on tiny inputs, library routines, invariants.
+A dropped term, a wrong GQA map, a transposed K/V half or an off-by-one in the causal mask fails
+at least one of these."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from llama_lite_npu_amd import workloads
+from oracle import c_oracle, cpu_ref
+
+
+def test_half_conversion_matches_numpy_for_every_bit_pattern():
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([c_oracle.half_to_float(int(b)) for b in bits[::97]], dtype=np.float32)
+    w = want[::97]
+    both_nan = np.isnan(w) & np.isnan(got)
+    assert np.array_equal(got[~both_nan], w[~both_nan])
+    for special in (0x0000, 0x8000, 0x0001, 0x03ff, 0x0400, 0x7bff, 0x7c00, 0xfc00, 0x3c00):
+        assert c_oracle.half_to_float(special) == np.uint16(special).view(np.float16).astype(np.float32)
+
+
+def _random_half(shape, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(-32768, 32767, shape, generator=g, dtype=torch.int16).view(torch.float16)
+
+
+def test_kv_append_is_index_assignment():
+    pool = _random_half((64, 6, 8), 1)
+    kv = _random_half((5, 6, 8), 2)
+    idx = torch.tensor([9, 0, 63, 17, 33], dtype=torch.int32)
+    want = pool.clone()
+    for i, s in enumerate(idx.tolist()):
+        want[s] = kv[i]
+    got_c = pool.clone().numpy()
+    c_oracle.kv_append(kv.numpy(), idx.numpy(), got_c)
+    got_t = pool.clone()
+    cpu_ref.kv_append_ref(kv, idx, got_t)
+    assert np.array_equal(got_c.view(np.int16), want.numpy().view(np.int16))
+    assert torch.equal(got_t.view(torch.int16), want.view(torch.int16))
+    untouched = np.setdiff1d(np.arange(64), idx.numpy())
+    assert np.array_equal(got_c.view(np.int16)[untouched], pool.numpy().view(np.int16)[untouched])
+    # idempotent
+    again = got_c.copy()
+    c_oracle.kv_append(kv.numpy(), idx.numpy(), again)
+    assert np.array_equal(again.view(np.int16), got_c.view(np.int16))
+
+
+def test_page_gather_scatter_round_trip():
+    n_pages, ps = 12, 4
+    pool = _random_half((n_pages * ps, 2, 8), 3)
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(4)).to(torch.int32)
+    scattered = np.zeros_like(pool.numpy())
+    c_oracle.page_gather(pool.numpy(), scattered, np.arange(n_pages), perm.numpy(), page_size=ps)
+    back = np.zeros_like(scattered)
+    c_oracle.page_gather(scattered, back, perm.numpy(), None, page_size=ps)
+    assert np.array_equal(back.view(np.int16), pool.numpy().view(np.int16))
+    paged = pool.view(n_pages, ps, 2, 8)
+    want = torch.zeros_like(paged)
+    want[perm.long()] = paged
+    assert np.array_equal(scattered.view(np.int16), want.view(n_pages * ps, 2, 8).numpy().view(np.int16))
+    t = torch.zeros_like(pool)
+    cpu_ref.page_gather_ref(pool, t, torch.arange(n_pages), perm, page_size=ps)
+    assert torch.equal(t.view(torch.int16), want.view(n_pages * ps, 2, 8).view(torch.int16))
+
+
+def _brute_decode(q, pool, table, lens, scale, ps):
+    """Plain Python loops, one (sequence, head) at a time; GQA map h // (Hq / Hkv); K heads are
+    pool[:, :Hkv], V heads pool[:, Hkv:]."""
+    b, hq, d = q.shape
+    hkv = pool.shape[1] // 2
+    out = np.zeros((b, hq, d))
+    for i in range(b):
+        for h in range(hq):
+            kvh = h // (hq // hkv)
+            scores, values = [], []
+            for t in range(int(lens[i])):
+                slot = int(table[i][t // ps]) * ps + t % ps
+                k = pool[slot, kvh].astype(np.float64)
+                scores.append(float(np.dot(q[i, h].astype(np.float64), k)) * scale)
+                values.append(pool[slot, hkv + kvh].astype(np.float64))
+            if not scores:
+                continue
+            m = max(scores)
+            w = [math.exp(s - m) for s in scores]
+            out[i, h] = sum(wi * vi for wi, vi in zip(w, values)) / sum(w)
+    return out
+
+
+def test_decode_against_brute_force_tiny():
+    ps, hq, hkv, d = 4, 4, 2, 8
+    g = torch.Generator().manual_seed(5)
+    pool = torch.randn((10 * ps, 2 * hkv, d), generator=g).half()
+    q = torch.randn((3, hq, d), generator=g).half()
+    table = torch.tensor([[7, 2, 9], [0, 0, 0], [4, 1, 0]], dtype=torch.int32)
+    lens = torch.tensor([11, 1, 8], dtype=torch.int32)
+    want = _brute_decode(q.numpy(), pool.numpy(), table.tolist(), lens.tolist(), 0.37, ps)
+    for wide in (False, True):
+        got = c_oracle.paged_decode(q.numpy(), pool.numpy(), table.numpy(), lens.numpy(), 0.37, page_size=ps,
+                                    wide=wide)
+        assert np.abs(got - want).max() < (1e-6 if wide else 2e-6)
+    got_t = cpu_ref.paged_decode_ref(q, pool, table, lens, 0.37, page_size=ps, dtype=torch.float64).numpy()
+    assert np.abs(got_t - want).max() < 1e-12
+
+
+def test_decode_closed_forms():
+    case = workloads.make_decode_case("cf", 6, [0, 30], 8, 4)
+    # one token: out == v of that token (GQA: heads 2k, 2k+1 share kv head k)
+    out = c_oracle.paged_decode(case.q.numpy(), case.kv_pool.numpy(), case.block_table.numpy(),
+                                case.seq_lens.numpy(), case.softmax_scale)
+    slot = int(case.block_table[0, 0]) * 16
+    v = case.kv_pool[slot, 4:].float().numpy()
+    assert np.array_equal(out[0], np.repeat(v, 2, axis=0))
+    # equal keys: out == mean of V over the sequence
+    n = int(case.seq_lens[1])
+    slots = cpu_ref.slots_of(case.block_table[1], n, 16)
+    pool = case.kv_pool.clone()
+    pool[slots, :4] = pool[slots[0], :4]
+    out = c_oracle.paged_decode(case.q.numpy(), pool.numpy(), case.block_table.numpy(), case.seq_lens.numpy(),
+                                case.softmax_scale, wide=True)
+    want = np.repeat(pool[slots, 4:].double().mean(dim=0).numpy(), 2, axis=0)
+    assert np.abs(out[1] - want).max() < 1e-6
+
+
+def test_c_and_torch_oracles_agree_on_c1_and_lse_is_logsumexp():
+    case = workloads.config_c1()
+    a, lse = c_oracle.paged_decode(case.q.numpy(), case.kv_pool.numpy(), case.block_table.numpy(),
+                                   case.seq_lens.numpy(), case.softmax_scale, return_lse=True)
+    b = cpu_ref.paged_decode_ref(case.q, case.kv_pool, case.block_table, case.seq_lens, case.softmax_scale)
+    assert np.abs(a - b.numpy()).max() < 5e-6
+    i, h = 2, 5
+    slots = cpu_ref.slots_of(case.block_table[i], int(case.seq_lens[i]), 16)
+    s = (case.kv_pool[slots, h // 2].double() @ case.q[i, h].double()) * case.softmax_scale
+    assert abs(float(torch.logsumexp(s, 0)) - float(lse[i, h])) < 1e-5
+
+
+def test_partitioned_decode_equals_one_pass_for_any_partition():
+    case = workloads.make_decode_case("part", 8, [100, 257, 15], 8, 2)
+    one = c_oracle.paged_decode(case.q.numpy(), case.kv_pool.numpy(), case.block_table.numpy(),
+                                case.seq_lens.numpy(), case.softmax_scale, wide=True)
+    for part in (16, 128, 4096):
+        out, mid_o, mid_lse = c_oracle.decode_partitioned(case.q.numpy(), case.kv_pool.numpy(),
+                                                          case.block_table.numpy(), case.seq_lens.numpy(),
+                                                          case.softmax_scale, partition=part)
+        assert np.abs(out - one).max() < 2e-6, part
+    t_out, t_mid, t_lse = cpu_ref.flash_decoding_ref(case.q, case.kv_pool, case.block_table, case.seq_lens,
+                                                      case.softmax_scale, partition=128)
+    out, mid_o, mid_lse = c_oracle.decode_partitioned(case.q.numpy(), case.kv_pool.numpy(),
+                                                      case.block_table.numpy(), case.seq_lens.numpy(),
+                                                      case.softmax_scale, partition=128)
+    assert np.abs(t_out.numpy() - one).max() < 5e-6
+    valid = np.isfinite(mid_lse)
+    assert np.abs(t_lse.numpy()[valid] - mid_lse[valid]).max() < 1e-5
+    assert np.abs(t_mid.numpy() - mid_o).max() < 5e-6
+
+
+def test_lse_merge_is_associative_and_order_free():
+    rng = np.random.default_rng(9)
+    o = rng.standard_normal((6, 16)).astype(np.float32)
+    lse = rng.standard_normal(6).astype(np.float32) * 3
+    full = c_oracle.lse_merge(o, lse)
+    w = np.exp(lse.astype(np.float64) - lse.max())
+    want = (w[:, None] * o).sum(0) / w.sum()
+    assert np.abs(full - want).max() < 1e-6
+    left = c_oracle.lse_merge(o[:3], lse[:3])
+    right = c_oracle.lse_merge(o[3:], lse[3:])
+    lse_l = np.log(np.exp(lse[:3].astype(np.float64)).sum())
+    lse_r = np.log(np.exp(lse[3:].astype(np.float64)).sum())
+    two = c_oracle.lse_merge(np.stack([left, right]), np.array([lse_l, lse_r], dtype=np.float32))
+    assert np.abs(two - full).max() < 1e-6
+    assert np.abs(c_oracle.lse_merge(o[::-1].copy(), lse[::-1].copy()) - full).max() < 1e-6
+
+
+def test_prefill_matches_sdpa_and_brute_force_mask():
+    case = workloads.make_prefill_case("pf", 10, [5, 33, 1, 17], 4, 2)
+    pool = case.kv_pool.clone()
+    cpu_ref.kv_append_ref(torch.cat([case.k, case.v], 1), case.slot_mapping, pool)
+    got = c_oracle.paged_prefill(case.q.numpy(), pool.numpy(), case.block_table.numpy(), case.cu_q_lens.numpy(),
+                                 None, case.softmax_scale)
+    sdpa = cpu_ref.varlen_prefill_ref(case.q, case.k, case.v, case.cu_q_lens[:-1], case.seq_lens,
+                                      case.softmax_scale).numpy()
+    assert np.abs(got - sdpa).max() < 5e-6
+    packed = c_oracle.varlen_prefill(case.q.numpy(), case.k.numpy(), case.v.numpy(), case.cu_q_lens[:-1].numpy(),
+                                     case.seq_lens.numpy(), case.softmax_scale)
+    assert np.abs(packed - got).max() < 1e-6
+    torch_paged = cpu_ref.paged_prefill_ref(case.q, pool, case.block_table, case.cu_q_lens, None,
+                                            case.softmax_scale).numpy()
+    assert np.abs(torch_paged - got).max() < 5e-6
+    # row m of a sequence == decode over its first m + 1 tokens
+    b, m = 1, 20
+    row = int(case.cu_q_lens[b]) + m
+    dec = c_oracle.paged_decode(case.q[row:row + 1].numpy(), pool.numpy(), case.block_table[b:b + 1].numpy(),
+                                np.array([m + 1]), case.softmax_scale)
+    assert np.abs(dec[0] - got[row]).max() < 1e-6
+
+
+def test_chunked_prefill_equals_rows_of_full_prefill():
+    full = workloads.make_prefill_case("full", 11, [40, 23], 4, 2)
+    pool = full.kv_pool.clone()
+    cpu_ref.kv_append_ref(torch.cat([full.k, full.v], 1), full.slot_mapping, pool)
+    whole = c_oracle.paged_prefill(full.q.numpy(), pool.numpy(), full.block_table.numpy(), full.cu_q_lens.numpy(),
+                                   None, full.softmax_scale)
+    ctx = np.array([25, 0], dtype=np.int32)
+    chunk = full.seq_lens.numpy() - ctx
+    cu = np.concatenate([[0], np.cumsum(chunk)]).astype(np.int32)
+    rows = np.concatenate([np.arange(int(full.cu_q_lens[i]) + ctx[i], int(full.cu_q_lens[i + 1])) for i in range(2)])
+    part = c_oracle.paged_prefill(full.q.numpy()[rows], pool.numpy(), full.block_table.numpy(), cu, ctx,
+                                  full.softmax_scale)
+    assert np.abs(part - whole[rows]).max() < 1e-6
+    part_t = cpu_ref.paged_prefill_ref(full.q[torch.from_numpy(rows)], pool, full.block_table,
+                                       torch.from_numpy(cu), torch.from_numpy(ctx), full.softmax_scale).numpy()
+    assert np.abs(part_t - whole[rows]).max() < 5e-6
+
+
+def test_workload_generators_are_seeded_and_consistent():
+    a, b = workloads.config_c1(), workloads.config_c1()
+    assert torch.equal(a.block_table, b.block_table) and torch.equal(a.q, b.q)
+    assert a.seq_lens.tolist() == [38, 129, 512, 1001] and a.num_pages == 512
+    pages = sorted(p for i in range(4) for p in a.block_table[i, :(int(a.seq_lens[i]) + 15) // 16].tolist())
+    assert len(set(pages)) == len(pages)                      # no page is assigned twice
+    c4 = workloads.config_c4(batch=4, prefix=64, lo=5, hi=40)
+    n = c4.extra["n_shared"]
+    assert all(torch.equal(c4.block_table[i, :n], c4.block_table[0, :n]) for i in range(4))
+    assert c4.decode_bytes() > 0 and c4.append_bytes() == 4 * (2 * 4096 + 4)
