@@ -34,6 +34,10 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+# HBM bytes per launch of the decode kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by a 1 GiB
+# copy kernel); summary and commands in profiles/paged_decode_balanced_c2_pmc.txt. Only meaningful for
+# the workload it was measured on.
+MEASURED_TRAFFIC_BYTES = {("c2", "balanced"): 314.2e6}
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 
 
@@ -358,6 +362,9 @@ def main() -> int:
     ap.add_argument("--schedule", default="balanced", choices=["balanced", "splits"],
                     help="decode work decomposition (splits: separate append, split and merge launches)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one page_gather of exactly 1 GiB (read) + 1 GiB (write): a plain copy of "
+                         "known size against which profiler byte counters can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures the path on ONE GPU (one process, one device); "
@@ -395,7 +402,23 @@ def main() -> int:
             sched = "splits"
         return run_decode(case, layers, args.steps, args.warmup, device, case.name, sched), case
 
+    if args.calibrate_copy:
+        from llama_lite_npu_amd import ops
+        n_cal = 16384                                   # pages of 64 KiB = 1 GiB
+        src = torch.empty((n_cal * 16, 16, 128), dtype=torch.float16, device=device).normal_()
+        dst = torch.empty_like(src)
+        ids = torch.randperm(n_cal, device=device).to(torch.int32)
+        ops.page_gather(src, dst, ids, None)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
+
     res, case = run(args.config)
+    traffic = MEASURED_TRAFFIC_BYTES.get((args.config, args.schedule))
+    if traffic is not None and args.config != "c3":
+        res["roofline"]["traffic"] = traffic / (res["decode_kernel_us_mean"] * 1e-6) / 1e9
+        res["roofline"]["traffic_bytes_per_launch"] = traffic
+        res["roofline"]["algorithmic_bytes_per_launch"] = res["decode_bytes_per_layer"] + res["append_bytes_per_layer"]
     line = {
         "metric": "paged decode attn HBM GB/s (% of 8 TB/s peak); KV-append GB/s; us/layer",
         "value": res.get("value", res.get("prefill_tflops")),
