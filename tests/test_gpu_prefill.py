@@ -27,6 +27,10 @@ def _oracle_paged(case):
     (64, 8, [128, 77, 200]),
     (32, 4, [300, 5]),
     (8, 8, [65]),
+    (16, 1, [130, 40]),        # 16 query heads per kv head: two workgroups per kv head
+    (28, 4, [260, 31]),        # 7 heads per kv head: one idle column tile
+    (4, 4, [520, 129]),        # no grouping: 128 query rows per workgroup
+    (64, 8, [700, 333]),       # long enough for tiles wholly below the diagonal
 ])
 def test_paged_prefill_context_zero(hq, hkv, lens):
     print(f"prefill paged {hq}/{hkv} {lens}", flush=True)
@@ -76,3 +80,39 @@ def test_decode_equals_prefill_of_one_row():
                             case.softmax_scale)
     torch.cuda.synchronize()
     assert float((dec.float() - pre.float()).abs().max()) <= 1e-3
+
+
+def test_prefill_running_maximum_keeps_growing():
+    """Scores rise steadily along the keys, so every tile moves the running maximum by far more
+    than the slack the lazy rescale allows."""
+    print("prefill growing maximum", flush=True)
+    case = workloads.make_prefill_case("g", 420, [600, 190], 16, 2, device=DEV)
+    gen = torch.Generator().manual_seed(421)
+    direction = torch.randn(workloads.HEAD_DIM, generator=gen)
+    direction = direction / direction.norm()
+    t_total = case.q.shape[0]
+    pos = torch.cat([torch.arange(int(n)) for n in case.seq_lens.tolist()]).float()
+    noise_q = 0.1 * torch.randn(case.q.shape, generator=gen)
+    noise_k = 0.1 * torch.randn(case.k.shape, generator=gen)
+    case.q.copy_((8.0 * direction + noise_q).half())
+    # score ~ 8 * 0.3 * pos: about +0.3 in log2 units per key after scaling, +10 per 32 keys
+    case.k.copy_((direction * (0.3 * pos)[:, None, None] + noise_k).half())
+    assert case.k.shape[0] == t_total
+    _append(case)
+    out = ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, None, case.max_q_len,
+                            case.softmax_scale)
+    torch.cuda.synchronize()
+    assert_attention_close(out, _oracle_paged(case), "growing maximum")
+
+
+def test_prefill_never_reads_values_past_the_sequence_end():
+    """Slots after the last token of a page (and unowned pages) hold NaN: they must not leak."""
+    print("prefill NaN in unused slots", flush=True)
+    case = workloads.make_prefill_case("n", 430, [70, 17, 100, 1], 16, 8, device=DEV)
+    case.kv_pool.fill_(float("nan"))
+    _append(case)
+    out = ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, None, case.max_q_len,
+                            case.softmax_scale)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    assert_attention_close(out, _oracle_paged(case), "NaN outside the sequences")
