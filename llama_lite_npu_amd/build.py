@@ -41,6 +41,14 @@ HIPCC_FLAGS = (
 )
 
 
+# Extra flags per source. The prefill kernel takes maxima of MFMA results: without NaN
+# semantics to honour, the compiler drops the self-max that quiets each operand and fuses the
+# rest into v_max3_f32. Nothing in that file relies on NaN propagation (masking uses -inf).
+PER_FILE_FLAGS = {
+    "paged_prefill.hip": ("-fno-honor-nans",),
+}
+
+
 def _hipcc() -> str:
     found = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(found):
@@ -80,7 +88,7 @@ def build_library(force: bool = False, extra_flags: tuple[str, ...] = ()) -> Pat
     objs = [OBJ_DIR / (Path(s).stem + ".o") for s in SOURCES]
     with ThreadPoolExecutor(max_workers=min(len(SOURCES), 8)) as pool:
         jobs = [
-            pool.submit(_compile, hipcc, CSRC / s, o, tuple(extra_flags))
+            pool.submit(_compile, hipcc, CSRC / s, o, PER_FILE_FLAGS.get(s, ()) + tuple(extra_flags))
             for s, o in zip(SOURCES, objs)
         ]
         for j in jobs:

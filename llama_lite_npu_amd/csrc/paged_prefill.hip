@@ -4,7 +4,7 @@
 //
 // A workgroup of 4 wavefronts owns 128 score columns: up to 8 query heads of one KV head (the
 // GQA group) times 16 * row_tiles query rows, 32 columns per wavefront. It walks the keys the
-// block may see in tiles of 64. Per tile and wavefront:
+// block may see in tiles of 64 (two halves of 32 for the softmax). Per tile and wavefront:
 //
 //   S^T[key][col]  = K_tile[64 x 128] . Q^T[128 x 32]         32 x MFMA 16x16x32
 //   causal mask, online softmax per column (fp32, exp2 domain, lazy rescale)
@@ -25,11 +25,18 @@
 // rows are unpadded (256 bytes) and the 16-byte chunks of a row are XOR-swizzled instead: the
 // lane that fills slot p of row r fetches chunk p ^ f(r) from memory. f differs for K (read
 // back as 16-byte rows by 16 lanes of different rows) and V (read back transposed, 8 rows x
-// 32 bytes at a time); both reads are then conflict free.
+// 32 bytes at a time); both reads are then free of bank conflicts.
 //
-// 256 registers per lane leave two wavefronts per SIMD: two workgroups share a compute unit and
-// drift apart, so one's softmax (vector ALU) overlaps the other's MFMAs and a finishing block's
-// prologue/epilogue hides behind its neighbour.
+// The accumulators are only ever rescaled in straight-line code (general_tile): a conditional
+// rescale inside the key loop makes the compiler copy all 72 accumulator registers at the join
+// on every tile. Tiles below the diagonal run in a loop that leaves as soon as a column maximum
+// grows by more than 8 and otherwise touches the accumulators with MFMAs only.
+//
+// About 216 registers per lane leave two wavefronts per SIMD: two workgroups share a compute
+// unit and drift apart, so one's softmax (vector ALU) overlaps the other's MFMAs and a
+// finishing block's prologue/epilogue hides behind its neighbour. Grid: x = kv head (times the
+// head split), y = row block (long blocks first), z = sequence; with 8 kv heads a head's blocks
+// all land on one XCD and share its L2.
 #include <type_traits>
 
 #include "common.h"
@@ -59,21 +66,19 @@ constexpr int kTiledWaves = 4;
 constexpr int kWgColTiles = kColTiles * kTiledWaves;
 constexpr int kTileHalfs = kKvTile * kHeadDim;  // one staged tile: 64 rows of 256 bytes
 
-typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(3))) half_t lds_half_t;
+typedef __attribute__((address_space(3))) half8_t lds_half8_t;
 typedef __attribute__((address_space(3))) short4_t lds_short4_t;
 typedef short short8_t __attribute__((ext_vector_type(8)));
 
-// max without the NaN-quieting self-max the compiler adds around llvm.maxnum of MFMA results.
+// Plain maxima. This file is compiled with -fno-honor-nans, so the compiler does not wrap every
+// operand in a NaN-quieting self-max and fuses pairs into v_max3_f32. (They must stay compiler
+// instructions: an asm v_max3 reading an MFMA result gets none of the wait states that the
+// compiler inserts between an MFMA and the first use of its result.)
 __device__ __forceinline__ float vmax3(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
+  return __builtin_fmaxf(__builtin_fmaxf(a, b), c);
 }
-__device__ __forceinline__ float vmax2(float a, float b) {
-  float r;
-  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
+__device__ __forceinline__ float vmax2(float a, float b) { return __builtin_fmaxf(a, b); }
 // Maximum over the four lanes that hold one column (lanes l, l^16, l^32, l^48). The swaps
 // exchange 16- and 32-lane halves between their two operands, so max(first, second) of the
 // swapped pair is the pairwise maximum, without a trip through LDS.
@@ -93,18 +98,19 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     const int32_t *__restrict__ q_lens_or_null, const int32_t *__restrict__ context_lens,
     int32_t group, int32_t head_splits, int32_t heads_per_wg, int32_t row_tiles,
     float scale_log2) {
-  __shared__ __attribute__((aligned(1024))) half_t kbuf0[kTileHalfs];
-  __shared__ __attribute__((aligned(1024))) half_t kbuf1[kTileHalfs];
-  __shared__ __attribute__((aligned(1024))) half_t vbuf0[kTileHalfs];
-  __shared__ __attribute__((aligned(1024))) half_t vbuf1[kTileHalfs];
+  // Two tiles of K and two of V: tile t sits in half t % 2.
+  __shared__ __attribute__((aligned(1024))) half_t kbuf[2 * kTileHalfs];
+  __shared__ __attribute__((aligned(1024))) half_t vbuf[2 * kTileHalfs];
+  const uint32_t k_lds = (uint32_t)(uintptr_t)(lds_half_t *)kbuf;  // LDS byte addresses
+  const uint32_t v_lds = (uint32_t)(uintptr_t)(lds_half_t *)vbuf;
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int n = lane & 15;
   const int g = lane >> 4;
-  const int h = (int)blockIdx.y / head_splits;  // kv head
-  const int head0 = ((int)blockIdx.y - h * head_splits) * heads_per_wg;
+  const int h = (int)blockIdx.x / head_splits;  // kv head
+  const int head0 = ((int)blockIdx.x - h * head_splits) * heads_per_wg;
   const int heads_here = (group - head0) < heads_per_wg ? (group - head0) : heads_per_wg;
   const int b = blockIdx.z;
 
@@ -117,7 +123,8 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     q_len = q_lens_or_null[b];
   }
   const int block_rows = 16 * row_tiles;
-  const int m0 = ((int)gridDim.x - 1 - (int)blockIdx.x) * block_rows;  // long blocks first
+  // Long blocks first, all heads of a row block next to each other.
+  const int m0 = ((int)gridDim.y - 1 - (int)blockIdx.y) * block_rows;
   if (m0 >= q_len) return;
   const int ctx = (PAGED && context_lens) ? context_lens[b] : 0;
   const int kv_len = ctx + q_len;
@@ -146,7 +153,10 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   const int32_t *table = PAGED ? paged.block_table + (int64_t)b * paged.bt_stride : nullptr;
   const int last_page = last_key >> 4;
 
-  auto issue_tile = [&](int kt, half_t *kb, half_t *vb) {
+  // Starts the loads of tile kt into its LDS half. The instruction is written as asm so that the
+  // compiler does not make later LDS reads of the *other* half wait for it; the wait is the
+  // explicit vmcnt(0) before the barrier that publishes the tile.
+  auto issue_tile = [&](int kt) {
     const int row0 = kt * kKvTile + 16 * wave;  // first key of this wavefront's 16 rows
     const char *kbase, *vbase;
     int src0;  // key index the bases point at
@@ -164,36 +174,36 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       vbase = (const char *)packed.v + (int64_t)(q_start + first) * v_pitch;
       src0 = first;
     }
+    const uint32_t dst = (uint32_t)((kt & 1) * kTileHalfs + 16 * wave * kHeadDim) * 2u;
+    auto load_rows = [&](uint32_t i, uint32_t ko, uint32_t vo) {
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                   :
+                   : "s"(k_lds + dst + 1024u * i), "v"(ko), "s"(kbase)
+                   : "memory");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                   :
+                   : "s"(v_lds + dst + 1024u * i), "v"(vo), "s"(vbase)
+                   : "memory");
+    };
     if (row0 + 15 <= last_key) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        __builtin_amdgcn_global_load_lds(kbase + koff[i],
-                                         (lds_void_t *)(kb + (16 * wave + 4 * i) * kHeadDim), 16,
-                                         0, 0);
-        __builtin_amdgcn_global_load_lds(vbase + voff[i],
-                                         (lds_void_t *)(vb + (16 * wave + 4 * i) * kHeadDim), 16,
-                                         0, 0);
-      }
+      for (int i = 0; i < 4; ++i) load_rows(i, koff[i], voff[i]);
     } else {
-      // Rows past the last key re-read it: finite values the zero probabilities multiply.
+      // Only in the last tile of a sequence. Rows past the last key re-read it: finite values
+      // that zero probabilities multiply.
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int rip = 4 * i + r_loc;
         int tok = row0 + rip;
         tok = tok < last_key ? tok : last_key;
         const uint32_t back = (uint32_t)(row0 + rip - tok) - (uint32_t)(row0 - src0);
-        // source row = rip - back (0 <= . < 16 inside the page / at the clamped packed row)
-        __builtin_amdgcn_global_load_lds(kbase + (koff[i] - back * k_pitch),
-                                         (lds_void_t *)(kb + (16 * wave + 4 * i) * kHeadDim), 16,
-                                         0, 0);
-        __builtin_amdgcn_global_load_lds(vbase + (voff[i] - back * v_pitch),
-                                         (lds_void_t *)(vb + (16 * wave + 4 * i) * kHeadDim), 16,
-                                         0, 0);
+        // source row = rip - back: inside the page / at the clamped packed row
+        load_rows(i, koff[i] - back * k_pitch, voff[i] - back * v_pitch);
       }
     }
   };
 
-  issue_tile(0, kbuf0, vbuf0);
+  issue_tile(0);
 
   // ---- this wavefront's columns: tile t = head (t / row_tiles), rows 16 * (t % row_tiles) ..
   half8_t qf[kColTiles][4];
@@ -231,18 +241,35 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   }
   const half8_t ones = half8_t{1, 1, 1, 1, 1, 1, 1, 1};
 
-  // Swizzled read offsets (in halfs) inside a tile.
-  // K, A operand of S^T: row 16m + n, chunk (4kk + g) ^ n  ==  base ^ (4kk << 3 halfs).
-  const int k_read = n * kHeadDim + 8 * (g ^ (n & 3)) + 32 * (n >> 2);
+  // Swizzled read addresses (LDS bytes) for the tile half in use; they flip between the halves
+  // once per tile.
+  // K, A operand of S^T: row 16m + n, chunk (4kk + g) ^ n.
+  uint32_t k_addr[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    k_addr[kk] = k_lds + 2u * (uint32_t)(n * kHeadDim + 8 * ((4 * kk + g) ^ n));
+  }
   // V^T, A operand of O^T: row 32 s2 + 4g + n/4 (+16), halfs 16j + 4(n%4); chunk pair j ^ (r%8).
   const int v_row = 4 * g + (n >> 2);
-  const int v_read = v_row * kHeadDim + 16 * (v_row & 7) + 4 * (n & 3);
+  uint32_t v_addr[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    v_addr[j] = v_lds + 2u * (uint32_t)(v_row * kHeadDim + 16 * (j ^ (v_row & 7)) + 4 * (n & 3));
+  }
+  int flip = kTileHalfs * 2;  // bytes to the other half
+  auto flip_halves = [&]() {
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) k_addr[kk] += flip;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v_addr[j] += flip;
+    flip = -flip;
+  };
 
   float4_t st[2][kColTiles];
   half8_t pk[kColTiles];
 
   // S^T of 32 keys (rows 32 s2 .. +31 of the staged K tile) against this wavefront's columns.
-  auto scores_sub = [&](const half_t *kb, int s2) {
+  auto scores_into = [&](float4_t (&st)[2][kColTiles], int s2) {
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
 #pragma unroll
@@ -250,14 +277,25 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
         const half8_t a =
-            *(const half8_t *)(&kb[(32 * s2 + 16 * m) * kHeadDim + (k_read ^ (32 * kk))]);
+            *(const lds_half8_t *)(uintptr_t)(k_addr[kk] + 2u * (32 * s2 + 16 * m) * kHeadDim);
 #pragma unroll
         for (int u = 0; u < kColTiles; ++u) st[m][u] = mfma_16x16x32(a, qf[u][kk], st[m][u]);
       }
     }
   };
+  // -inf on the keys column u may not see; key0 = first key of the sub-tile.
+  auto mask_sub = [&](int u, int key0) {
+    const int lim = q_pos[u] - key0 - 4 * g;  // key offset 16m + i is visible iff <= lim
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (16 * m + i > lim) st[m][u][i] = -INFINITY;
+      }
+    }
+  };
   // Column maxima of `st`, in scaled (log2) units.
-  auto column_max = [&](int u) {
+  auto column_max_of = [&](const float4_t (&st)[2][kColTiles], int u) {
     float mx = vmax3(st[0][u][0], st[0][u][1], st[0][u][2]);
     mx = vmax3(mx, st[0][u][3], st[1][u][0]);
     mx = vmax3(mx, st[1][u][1], st[1][u][2]);
@@ -265,7 +303,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     return max_across_groups(mx) * scale_log2;  // scale > 0: max and scaling commute
   };
   // p = 2^(s * scale - m), cast to fp16, in B-operand order.
-  auto exponentials = [&](int u) {
+  auto exponentials_of = [&](const float4_t (&st)[2][kColTiles], half8_t (&pk)[kColTiles], int u) {
     const float neg_m = -m_run[u];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -276,51 +314,49 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     }
   };
   // O^T += V^T . P^T,  l += 1^T . P^T for keys 32 s2 .. +31 of the staged V tile.
-  auto accumulate_sub = [&](const half_t *vb, int s2) {
+  auto accumulate_with = [&](const half8_t (&pk)[kColTiles], int s2) {
 #pragma unroll
     for (int u = 0; u < kColTiles; ++u) dsum[u] = mfma_16x16x32(ones, pk[u], dsum[u]);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const half_t *vlo = &vb[32 * s2 * kHeadDim + (v_read ^ (16 * j))];
-      const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t *)vlo);
-      const short4_t hi =
-          __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t *)(vlo + 16 * kHeadDim));
+      const uint32_t at = v_addr[j] + 2u * 32 * s2 * kHeadDim;
+      const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t *)(uintptr_t)at);
+      const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (lds_short4_t *)(uintptr_t)(at + 2u * 16 * kHeadDim));
       const short8_t both = short8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       const half8_t a = __builtin_bit_cast(half8_t, both);
 #pragma unroll
       for (int u = 0; u < kColTiles; ++u) acc[j][u] = mfma_16x16x32(a, pk[u], acc[j][u]);
     }
   };
-  auto sync_and_prefetch = [&](int kt, half_t *k_next, half_t *v_next) {
+  auto scores_sub = [&](int s2) { scores_into(st, s2); };
+  auto column_max = [&](int u) { return column_max_of(st, u); };
+  auto exponentials = [&](int u) { exponentials_of(st, pk, u); };
+  auto accumulate_sub = [&](int s2) { accumulate_with(pk, s2); };
+  float4_t st1[2][kColTiles];  // scores of the second half of a fast tile
+  half8_t pk1[kColTiles];
+
+  // Publishes tile kt (already requested) and requests tile kt + 1 into the other half.
+  auto sync_and_prefetch = [&](int kt) {
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's part of tile kt is in LDS
     __syncthreads();                     // ... and everyone's; everyone is done with tile kt-1
-    if (kt + 1 < n_tiles) issue_tile(kt + 1, k_next, v_next);
+    if (kt + 1 < n_tiles) issue_tile(kt + 1);
   };
 
-  // General tile: causal mask, and the accumulators are rescaled to the new running maximum
-  // unconditionally (straight-line code: a branch around the rescale makes the compiler copy
-  // every accumulator at the join, on every tile). Used for the first tiles, the diagonal and
-  // wherever a fast tile saw a maximum grow. Starts at sub-tile `first`; `synced` says that the
-  // barrier and prefetch of this tile are already done.
-  auto general_tile = [&](int kt, int first, bool synced, auto buf_tag) {
-    constexpr int BUF = decltype(buf_tag)::value;
-    if (!synced) sync_and_prefetch(kt, BUF ? kbuf0 : kbuf1, BUF ? vbuf0 : vbuf1);
+  // General sub-tiles of tile kt from `first` on: causal mask, and the accumulators are rescaled
+  // to the new running maximum unconditionally (straight-line code: a branch around the
+  // rescale makes the compiler copy every accumulator at the join, on every tile). Used for the
+  // first tile and wherever the fast loop saw a maximum grow.
+  auto general_tile = [&](int kt, int first) {
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2) {
       const int key0 = kt * kKvTile + 32 * s2;
       if (s2 < first) continue;
       if (key0 >= kv_end) break;  // nothing visible in the second half
-      scores_sub(BUF ? kbuf1 : kbuf0, s2);
+      scores_sub(s2);
 #pragma unroll
       for (int u = 0; u < kColTiles; ++u) {
-        const int lim = q_pos[u] - key0 - 4 * g;  // key offset 16m + i is visible iff <= lim
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            if (16 * m + i > lim) st[m][u][i] = -INFINITY;
-          }
-        }
+        mask_sub(u, key0);
         const float m_new = vmax2(m_run[u], column_max(u));
         const float alpha = fast_exp2(m_run[u] - m_new);
         m_run[u] = m_new;
@@ -329,58 +365,79 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
         for (int j = 0; j < 8; ++j) acc[j][u] *= alpha;
         exponentials(u);
       }
-      accumulate_sub(BUF ? vbuf1 : vbuf0, s2);
+      accumulate_sub(s2);
     }
   };
 
-  // Fast tile: entirely below the diagonal, and it only proceeds while no column maximum exceeds
-  // the running one by more than 8 (p stays below 2^8: far inside fp16 and fp32 range), so the
-  // accumulators are never touched outside the MFMAs. Returns 0 when the tile is done, else
-  // 1 + the sub-tile at which a maximum grew; that sub-tile has not been accumulated.
-  auto fast_tile = [&](int kt, auto buf_tag) -> int {
-    constexpr int BUF = decltype(buf_tag)::value;
-    sync_and_prefetch(kt, BUF ? kbuf0 : kbuf1, BUF ? vbuf0 : vbuf1);
+  // Fast tiles kt .. kt_end-1: they proceed only while no column maximum exceeds the running one
+  // by more than 8 (p stays below 2^8: far inside fp16 and fp32 range), so the accumulators are
+  // touched by nothing but MFMAs. Returns 0 at kt_end, else 1 + the sub-tile of tile kt that
+  // has to be redone with a rescale.
+  int kt = 1;
+  auto fast_tiles = [&](int kt_end, auto masked_tag) -> int {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    for (; kt < kt_end; ++kt) {
+      sync_and_prefetch(kt);
+      flip_halves();
 #pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-      scores_sub(BUF ? kbuf1 : kbuf0, s2);
-      const float mx0 = column_max(0), mx1 = column_max(1);
-      if (__builtin_amdgcn_ballot_w64(mx0 > m_run[0] + 8.0f || mx1 > m_run[1] + 8.0f) != 0) {
-        return 1 + s2;
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const int key0 = kt * kKvTile + 32 * s2;
+        if (MASKED && key0 >= kv_end) break;
+        scores_sub(s2);
+        if (MASKED) {
+          mask_sub(0, key0);
+          mask_sub(1, key0);
+        }
+        const float mx0 = column_max(0), mx1 = column_max(1);
+        if (__builtin_amdgcn_ballot_w64(mx0 > m_run[0] + 8.0f || mx1 > m_run[1] + 8.0f) != 0) {
+          return 1 + s2;
+        }
+        exponentials(0);
+        exponentials(1);
+        accumulate_sub(s2);
       }
-      exponentials(0);
-      exponentials(1);
-      accumulate_sub(BUF ? vbuf1 : vbuf0, s2);
+    }
+    return 0;
+  };
+
+  // Fast tiles below the diagonal: both halves' scores first, one growth check, then the halves'
+  // exponentials and second products, so that in each basic block MFMAs of one half can run
+  // beside the vector ALU work of the other. Returns like fast_tiles (a grown tile is redone
+  // from its first half).
+  auto fast_plain_tiles = [&](int kt_end) -> int {
+    for (; kt < kt_end; ++kt) {
+      sync_and_prefetch(kt);
+      flip_halves();
+      scores_into(st, 0);
+      scores_into(st1, 1);
+      const float a0 = column_max_of(st, 0), a1 = column_max_of(st, 1);
+      const float b0 = column_max_of(st1, 0), b1 = column_max_of(st1, 1);
+      const float lim0 = m_run[0] + 8.0f, lim1 = m_run[1] + 8.0f;
+      if (__builtin_amdgcn_ballot_w64(a0 > lim0 || a1 > lim1 || b0 > lim0 || b1 > lim1) != 0) {
+        return 1;
+      }
+      exponentials_of(st, pk, 0);
+      exponentials_of(st, pk, 1);
+      accumulate_with(pk, 0);
+      exponentials_of(st1, pk1, 0);
+      exponentials_of(st1, pk1, 1);
+      accumulate_with(pk1, 1);
     }
     return 0;
   };
 
   {
-    const std::integral_constant<int, 0> even;
-    const std::integral_constant<int, 1> odd;
-    const int diag = ctx + m0;  // tiles whose last key is <= diag are unmasked
-    int kt = 0, first = 0;
-    bool synced = false;
+    // Tiles whose last key is at or below the block's first row need no mask.
+    int n_plain = (ctx + m0 + 1) / kKvTile;
+    n_plain = n_plain < n_tiles ? n_plain : n_tiles;
+    sync_and_prefetch(0);
+    general_tile(0, 0);
     while (kt < n_tiles) {
-      if (kt & 1) general_tile(kt, first, synced, odd);
-      else general_tile(kt, first, synced, even);
-      ++kt;
-      first = 0;
-      synced = false;
-      if (kt & 1) continue;  // the fast loop starts on buffer 0
-      while (kt * kKvTile + kKvTile - 1 <= diag) {  // implies kt + 1 < n_tiles
-        int r = fast_tile(kt, even);
-        if (r == 0) {
-          ++kt;
-          if (kt * kKvTile + kKvTile - 1 > diag) break;
-          r = fast_tile(kt, odd);
-          if (r == 0) {
-            ++kt;
-            continue;
-          }
-        }
-        first = r - 1;
-        synced = true;
-        break;
+      int grew = fast_plain_tiles(n_plain);
+      if (grew == 0) grew = fast_tiles(n_tiles, std::true_type{});
+      if (grew != 0) {
+        general_tile(kt, grew - 1);
+        ++kt;
       }
     }
   }
@@ -466,8 +523,9 @@ extern "C" int litekv_paged_prefill(const void *q, int64_t q_token_stride, const
   PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
   const int group = num_q_heads / num_kv_heads;
   const PrefillShape s = prefill_shape(group, max_q_len);
+  LITEKV_REQUIRE(s.row_blocks <= 65535u, "paged_prefill: max_q_len %d too large", max_q_len);
   hipLaunchKernelGGL(varlen_prefill_tiled_kernel<true>,
-                     dim3(s.row_blocks, (unsigned)(num_kv_heads * s.head_splits), (unsigned)batch),
+                     dim3((unsigned)(num_kv_heads * s.head_splits), s.row_blocks, (unsigned)batch),
                      dim3(kTiledWaves * kWave), 0, static_cast<hipStream_t>(stream),
                      static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
                      out_token_stride, paged, packed, cu_q_lens, (const int32_t *)nullptr,
@@ -505,8 +563,9 @@ extern "C" int litekv_varlen_prefill(const void *q, int64_t q_token_stride, cons
                       k_token_stride, v_token_stride, seq_starts};
   const int group = num_q_heads / num_kv_heads;
   const PrefillShape s = prefill_shape(group, max_seq_len);
+  LITEKV_REQUIRE(s.row_blocks <= 65535u, "varlen_prefill: max_seq_len %d too large", max_seq_len);
   hipLaunchKernelGGL(varlen_prefill_tiled_kernel<false>,
-                     dim3(s.row_blocks, (unsigned)(num_kv_heads * s.head_splits), (unsigned)batch),
+                     dim3((unsigned)(num_kv_heads * s.head_splits), s.row_blocks, (unsigned)batch),
                      dim3(kTiledWaves * kWave), 0, static_cast<hipStream_t>(stream),
                      static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
                      out_token_stride, paged, packed, seq_starts, seq_lens,

@@ -116,3 +116,17 @@ def test_prefill_never_reads_values_past_the_sequence_end():
     torch.cuda.synchronize()
     assert bool(torch.isfinite(out).all())
     assert_attention_close(out, _oracle_paged(case), "NaN outside the sequences")
+
+
+def test_prefill_repeats_bit_for_bit():
+    """Same inputs, same bits: nothing in the kernel may depend on wavefront timing."""
+    print("prefill repeatability", flush=True)
+    case = workloads.make_prefill_case("r", 440, [700, 333], 64, 8, device=DEV)
+    _append(case)
+    outs = []
+    for _ in range(6):
+        outs.append(ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, None,
+                                      case.max_q_len, case.softmax_scale))
+    torch.cuda.synchronize()
+    for o in outs[1:]:
+        assert torch.equal(outs[0], o)
