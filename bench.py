@@ -263,12 +263,13 @@ def run_prefill(case, steps: int, warmup: int, device: str, label: str) -> dict:
     from llama_lite_npu_amd import ops
 
     out = torch.empty_like(case.q)
+    max_q_len = case.max_q_len  # one host read, outside the timed steps
 
     def step(ev=None):
         ops.kv_append(case.k, case.v, case.slot_mapping, case.kv_pool)
         if ev is not None:
             ev[0].record()
-        ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, None, case.max_q_len,
+        ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, None, max_q_len,
                           case.softmax_scale, out=out)
         if ev is not None:
             ev[1].record()
@@ -300,7 +301,7 @@ def run_prefill(case, steps: int, warmup: int, device: str, label: str) -> dict:
         "tokens": tokens,
         "flops": flops,
         "roofline": {
-            "kernel": "varlen_prefill_kernel<paged>",
+            "kernel": "varlen_prefill_tiled_kernel<paged>",
             "bound": "mfma",
             "achieved": achieved,
             "peak": MFMA_FP16_PEAK_TFLOPS,
