@@ -238,8 +238,104 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
             "traffic": None,
         },
     }
+    unique = case.unique_decode_bytes() + (append_bytes if balanced else 0)
+    if unique < kernel_bytes:
+        # Pages shared between block tables: the roofline fraction is taken on the bytes that must
+        # come from HBM at least once; the logical rate (every reader counted) is kept beside it.
+        res["roofline"].update(achieved=unique / (k_mean * 1e-3) / 1e9,
+                               frac=unique / (k_mean * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                               logical_gbps=achieved, unique_bytes_per_launch=unique,
+                               logical_bytes_per_launch=kernel_bytes)
     res.update(ls.plan_info)
     return res
+
+
+def _time_us(fn, reps: int = 10, warm: int = 2) -> float:
+    import torch
+
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in ev:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return sum(a.elapsed_time(b) for a, b in ev) / reps * 1e3
+
+
+def cow_step(case) -> dict:
+    """C4: the copy-on-write move before a step appends into a shared last page: every sequence's
+    last page is copied into its spare page (page_copy, one launch)."""
+    import torch
+    from llama_lite_npu_amd import ops
+
+    n_last = (case.seq_lens.cpu().to(torch.int64) - 1) // 16
+    src = case.block_table.cpu().gather(1, n_last[:, None])[:, 0].to(torch.int32).to(case.kv_pool.device)
+    dst = case.extra["spare_pages"].to(case.kv_pool.device)
+    us = _time_us(lambda: ops.page_copy(case.kv_pool, src, dst))
+    nbytes = 2 * src.numel() * case.tok_bytes * 16 + 8 * src.numel()
+    return {"cow_pages": int(src.numel()), "cow_us": us, "cow_gbps": nbytes / (us * 1e-6) / 1e9}
+
+
+def compaction_step(case) -> dict:
+    """C5: out-of-place compaction. Every live page is gathered into the dense prefix of a second
+    pool, the block table is rewritten, and the decode result must not change by a bit."""
+    import torch
+    from llama_lite_npu_amd import ops
+
+    dev = case.kv_pool.device
+    lens = case.seq_lens.cpu().to(torch.int64)
+    n_pages = ((lens + 15) // 16).tolist()
+    table = case.block_table.cpu()
+    live = torch.cat([table[b, :n] for b, n in enumerate(n_pages)])
+    new_table = torch.zeros_like(table)
+    cur = 0
+    for b, n in enumerate(n_pages):
+        new_table[b, :n] = torch.arange(cur, cur + n, dtype=torch.int32)
+        cur += n
+    dense = torch.empty((cur * 16,) + tuple(case.kv_pool.shape[1:]), dtype=case.kv_pool.dtype, device=dev)
+    src = live.to(torch.int32).to(dev)
+    us = _time_us(lambda: ops.page_gather(case.kv_pool, dense, src, None), reps=5, warm=1)
+    nbytes = 2 * cur * case.tok_bytes * 16 + 4 * cur
+    before = ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, case.softmax_scale)
+    after = ops.paged_decode(case.q, dense, new_table.to(dev), case.seq_lens, case.softmax_scale)
+    again = ops.paged_decode(case.q, dense, new_table.to(dev), case.seq_lens, case.softmax_scale)
+    torch.cuda.synchronize()
+    return {"gather_pages": cur, "gather_us": us, "gather_gbps": nbytes / (us * 1e-6) / 1e9,
+            "decode_same_bits_after_compaction": bool(torch.equal(before, after)),
+            "decode_repeat_same_bits": bool(torch.equal(after, again))}
+
+
+def cpu_baseline_prefill(case, budget_s: float = 10.0) -> dict:
+    """Per-sequence causal attention of the whole C3 workload in torch on the host cores
+    (restates flashattention2_nopad.py:250-274), min over repetitions for about `budget_s` s."""
+    import torch
+    from oracle import cpu_ref
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    c = case.to("cpu")
+    starts = c.cu_q_lens[:-1]
+
+    def one():
+        t0 = time.perf_counter()
+        cpu_ref.varlen_prefill_ref(c.q, c.k, c.v, starts, c.seq_lens, c.softmax_scale)
+        return time.perf_counter() - t0
+
+    first = one()
+    times, used = [], first
+    for _ in range(64):
+        if used > budget_s:
+            break
+        dt = one()
+        times.append(dt)
+        used += dt
+    best = min(times) if times else first
+    return {"value": case.flops() / best / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"the whole workload ({case.flops() / 1e12:.3f} TFLOP causal), torch CPU restatement, "
+                      f"min of {max(1, len(times))} reps after 1 warm-up, {best:.3f} s"}
 
 
 def time_append(case_tokens_k, case_tokens_v, slot_mapping, pool, reps: int = 20) -> float:
@@ -355,8 +451,8 @@ def cpu_baseline_decode(case, budget_s: float = 10.0) -> dict:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (default 10; 30 for c3)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps first (default 3; 10 for c3)")
     ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--layers", type=int, default=None, help="independent KV pools per step (c2 default 64)")
     ap.add_argument("--all", action="store_true", help="also report the other configurations (stderr)")
@@ -367,6 +463,11 @@ def main() -> int:
                     help="also launch one page_gather of exactly 1 GiB (read) + 1 GiB (write): a plain copy of "
                          "known size against which profiler byte counters can be scaled")
     args = ap.parse_args()
+    # A prefill step is ~0.4 ms: the part needs more of them to settle at its sustained clock.
+    if args.steps is None:
+        args.steps = 30 if args.config == "c3" else 10
+    if args.warmup is None:
+        args.warmup = 10 if args.config == "c3" else 3
     if args.gpus != 1:
         print("bench.py: this build measures the path on ONE GPU (one process, one device); "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
@@ -445,8 +546,14 @@ def main() -> int:
         ap_us = time_append(case.k_new, case.v_new, case.slot_mapping, case.kv_pool)
         line["detail"]["append_us"] = ap_us
         line["detail"]["append_gbps"] = case.append_bytes() / (ap_us * 1e-6) / 1e9
+        if args.config == "c4":
+            line["detail"].update(cow_step(case))
+        if args.config == "c5":
+            line["detail"].update(compaction_step(case))
         if not args.no_cpu_baseline:
             line["cpu_baseline"] = cpu_baseline_decode(case)
+    elif not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline_prefill(case)
     print(json.dumps(line), flush=True)
 
     if args.all:

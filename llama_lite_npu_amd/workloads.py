@@ -71,6 +71,25 @@ class DecodeCase:
     def append_bytes(self) -> int:
         return self.batch * (2 * self.tok_bytes + 4)
 
+    def unique_decode_bytes(self) -> int:
+        """decode_bytes() with every physical page counted once (pages shared between block tables
+        are fetched from HBM once if the cache keeps them): the conservative figure for C4."""
+        lens = self.seq_lens.cpu().tolist()
+        table = self.block_table.cpu()
+        fill = {}
+        pages = 0
+        for b, n in enumerate(lens):
+            n_pages = (n + PAGE_SIZE - 1) // PAGE_SIZE
+            pages += n_pages
+            ids = table[b, :n_pages].tolist()
+            for j, pid in enumerate(ids):
+                used = min(PAGE_SIZE, n - j * PAGE_SIZE)
+                if used > fill.get(pid, 0):
+                    fill[pid] = used
+        toks = sum(fill.values())
+        return (toks * self.tok_bytes + 2 * self.batch * self.num_q_heads * HEAD_DIM * 2
+                + pages * 4 + self.batch * 4)
+
     def to(self, device) -> "DecodeCase":
         kw = dict(self.__dict__)
         for key in ("context_lens", "seq_lens", "block_table", "slot_mapping", "q", "k_new", "v_new", "kv_pool"):
