@@ -86,7 +86,7 @@ class DecodeLayerSet:
     A step = one plan launch (the cuts are shared by every layer of a decode step) + per layer one
     balanced decode call with the KV append fused in (decode kernel + merge kernel)."""
 
-    def __init__(self, case, layers: int, device: str, schedule: str = "balanced"):
+    def __init__(self, case, layers: int, device: str, schedule: str = "balanced", shared_pages: int = 0):
         import torch
         from llama_lite_npu_amd import _lib, ops
 
@@ -113,21 +113,22 @@ class DecodeLayerSet:
         self.stream = stream
         bts = self.table.stride(0)
         if schedule == "balanced":
+            self.shared_pages = shared_pages
             self.chunks = c.extra.get("chunks") or lib.litekv_paged_decode_balanced_chunks(hkv)
             self.plan_bytes = lib.litekv_decode_plan_bytes(b, bts, hkv, self.chunks)
             self.plan = torch.empty(self.plan_bytes // 4, dtype=torch.int32, device=device)
-            ws_bytes = lib.litekv_paged_decode_balanced_workspace_bytes(b, hq, 128, self.chunks)
+            ws_bytes = lib.litekv_paged_decode_prefix_workspace_bytes(b, hq, 128, self.chunks)
             self.ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=device)
             self.plan_args = (self.table.data_ptr(), bts, self.seq_lens.data_ptr(), b, hkv, 16, c.num_pages,
-                              self.chunks, self.plan.data_ptr(), self.plan_bytes, stream)
+                              self.chunks, shared_pages, self.plan.data_ptr(), self.plan_bytes, stream)
             self.decode_args = [
-                (self.q.data_ptr(), hq * 128, pools[l].data_ptr(), self.seq_lens.data_ptr(), self.plan.data_ptr(),
-                 self.plan_bytes, c.k_new.data_ptr(), c.v_new.data_ptr(), hkv * 128, hkv * 128,
-                 self.out[l].data_ptr(), self.ws.data_ptr(), ws_bytes, b, hq, hkv, 128, 16, c.num_pages, bts,
-                 self.chunks, c.softmax_scale, stream)
+                (self.q.data_ptr(), hq * 128, pools[l].data_ptr(), self.table.data_ptr(), self.seq_lens.data_ptr(),
+                 self.plan.data_ptr(), self.plan_bytes, c.k_new.data_ptr(), c.v_new.data_ptr(), hkv * 128,
+                 hkv * 128, self.out[l].data_ptr(), self.ws.data_ptr(), ws_bytes, b, hq, hkv, 128, 16,
+                 c.num_pages, bts, self.chunks, shared_pages, c.softmax_scale, stream)
                 for l in range(layers)
             ]
-            self.plan_info = {"schedule": "balanced", "chunks": self.chunks}
+            self.plan_info = {"schedule": "balanced", "chunks": self.chunks, "shared_pages": shared_pages}
         else:
             self.max_splits, self.min_pps = ops.decode_split_plan(b, hkv, self.table.shape[1], c.num_splits)
             self.ws = ops.decode_workspace(b, hq, self.max_splits, device)
@@ -153,8 +154,8 @@ class DecodeLayerSet:
         lib = self.lib
         rc = 0
         if self.schedule == "balanced":
-            rc |= lib.litekv_decode_plan(*self.plan_args)
-            dec, prof = lib.litekv_paged_decode_balanced, lib.litekv_profile_next_decode
+            rc |= lib.litekv_decode_plan_prefix(*self.plan_args)
+            dec, prof = lib.litekv_paged_decode_prefix, lib.litekv_profile_next_decode
             for l in range(self.layers):
                 if events is not None:
                     prof(events[l][0], events[l][1])
@@ -178,10 +179,10 @@ class DecodeLayerSet:
 
 
 def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: str,
-               schedule: str = "balanced") -> dict:
+               schedule: str = "balanced", shared_pages: int = 0) -> dict:
     import torch
 
-    ls = DecodeLayerSet(case, layers, device, schedule)
+    ls = DecodeLayerSet(case, layers, device, schedule, shared_pages)
     for _ in range(max(1, warmup)):
         ls.step()
     torch.cuda.synchronize()
@@ -238,6 +239,12 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
             "traffic": None,
         },
     }
+    if shared_pages > 0:
+        # three launches share the work (prefix kernel, decode kernel, merge): the rate is taken over
+        # the layer's wall-clock share of the step instead of one kernel's duration
+        k_mean = ms_per_step / layers
+        res["roofline"]["kernel"] = "shared prefix (varlen_prefill_tiled_kernel<2>) + paged_decode_balanced_kernel + merge"
+        res["roofline"]["duration_us"] = k_mean * 1e3
     unique = case.unique_decode_bytes() + (append_bytes if balanced else 0)
     if unique < kernel_bytes:
         # Pages shared between block tables: the roofline fraction is taken on the bytes that must
@@ -459,6 +466,10 @@ def main() -> int:
     ap.add_argument("--schedule", default="balanced", choices=["balanced", "splits"],
                     help="decode work decomposition (splits: separate append, split and merge launches)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--chunks", type=int, default=None,
+                    help="balanced schedule: pieces per kv head (default: one workgroup per compute unit)")
+    ap.add_argument("--no-shared-prefix", action="store_true",
+                    help="c4: read the shared prefix pages once per sequence like any other page")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one page_gather of exactly 1 GiB (read) + 1 GiB (write): a plain copy of "
                          "known size against which profiler byte counters can be scaled")
@@ -499,10 +510,15 @@ def main() -> int:
             case = workloads.config_c3(device)
             return run_prefill(case, args.steps, args.warmup, device, case.name), case
         case, layers = decode_cfg(name)
+        if args.chunks:
+            case.extra["chunks"] = args.chunks
         sched = args.schedule
         if name == "c5" and args.schedule == "balanced" and False:
             sched = "splits"
-        return run_decode(case, layers, args.steps, args.warmup, device, case.name, sched), case
+        shared = 0
+        if sched == "balanced" and not args.no_shared_prefix and not case.extra.get("private_prefix"):
+            shared = int(case.extra.get("n_shared", 0))
+        return run_decode(case, layers, args.steps, args.warmup, device, case.name, sched, shared), case
 
     if args.calibrate_copy:
         from llama_lite_npu_amd import ops

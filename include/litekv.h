@@ -209,6 +209,47 @@ int litekv_paged_decode_balanced(const void *q, int64_t q_batch_stride, void *kv
                                  float softmax_scale, void *stream);
 
 /*
+ * Balanced paged decode for a batch whose sequences all start with the same
+ * `shared_pages` physical pages (block_table[b][0 .. shared_pages) identical
+ * for every b): a cached system prompt or few-shot prefix, which the
+ * reference maps into every request's table by reference
+ * (ModelExecutor.share_paged_prefix_from_cache, model_executor.py:570-620;
+ * PagedReqTokensManager.share_req_from_pages, paged_attention.py:252-274) and
+ * then reads once per sequence and query head (flashdecoding.py:84-94). Here
+ * the shared pages are attended once for the whole batch: the (sequence, query
+ * head) pairs of one kv head form the columns of an MFMA-tiled kernel over the
+ * prefix keys, whose partial rows join the log-sum-exp merge of the private
+ * pages. Result contract as litekv_paged_decode_balanced (same tolerance; not
+ * bit-identical to it, the summation order differs).
+ *
+ *   litekv_decode_plan_prefix   as litekv_decode_plan, over the pages after
+ *                the first shared_pages of every sequence
+ *   shared_pages must equal the value the plan was made with; 0 gives
+ *                litekv_paged_decode_balanced. Every sequence with
+ *                seq_lens[b] > 0 must hold at least shared_pages full pages.
+ *   block_table  [B][block_table_stride]; only row 0's first shared_pages
+ *                entries are read by this call (the rest is in the plan)
+ *   workspace    litekv_paged_decode_prefix_workspace_bytes(B, Hq, D, chunks)
+ */
+size_t litekv_paged_decode_prefix_workspace_bytes(int32_t batch, int32_t num_q_heads,
+                                                  int32_t head_dim, int32_t chunks);
+
+int litekv_decode_plan_prefix(const int32_t *block_table, int32_t block_table_stride,
+                              const int32_t *seq_lens, int32_t batch, int32_t num_kv_heads,
+                              int32_t page_size, int64_t num_pages, int32_t chunks,
+                              int32_t shared_pages, void *plan, size_t plan_bytes, void *stream);
+
+int litekv_paged_decode_prefix(const void *q, int64_t q_batch_stride, void *kv_pool,
+                               const int32_t *block_table, const int32_t *seq_lens, void *plan,
+                               size_t plan_bytes, const void *k_new, const void *v_new,
+                               int64_t k_new_stride, int64_t v_new_stride, void *out,
+                               void *workspace, size_t workspace_bytes, int32_t batch,
+                               int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                               int32_t page_size, int64_t num_pages, int32_t block_table_stride,
+                               int32_t chunks, int32_t shared_pages, float softmax_scale,
+                               void *stream);
+
+/*
  * Profiling aid (no counterpart in the reference): the next
  * litekv_paged_decode_balanced launch made by this thread carries the two
  * hipEvent_t handles as its start and stop events, so its device-side

@@ -38,6 +38,19 @@ int check_launch(const char *what);
     if (!(cond)) return ::litekv::fail(LITEKV_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
   } while (0)
 
+// Most key slices the shared-prefix kernel may cut the prefix into (bounds its workspace).
+constexpr int kMaxPrefixSplits = 8;
+
+// Attention of every (sequence, query head) of a decode step over the first `shared_pages`
+// pages of block-table row 0 (which all sequences share), as normalised fp32 partial rows
+// part_o[split][batch][Hq][128] and log-sum-exps part_lse[split][batch][Hq]; *splits_out
+// receives the number of key slices written. Defined beside the prefill kernel it reuses.
+int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_pool,
+                         const int32_t *block_table, int32_t batch, int32_t num_q_heads,
+                         int32_t num_kv_heads, int64_t num_pages, int32_t shared_pages,
+                         float *part_o, float *part_lse, float softmax_scale, hipStream_t stream,
+                         int *splits_out);
+
 // ---- device side ---------------------------------------------------------
 
 // 2^x on the transcendental unit (v_exp_f32); exp2(-inf) == 0.

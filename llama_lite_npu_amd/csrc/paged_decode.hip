@@ -293,24 +293,33 @@ __global__ __launch_bounds__(64) void paged_decode_split_kernel(
               part_lse + cell, max_splits, n, g, group);
 }
 
-// Merges `n_parts` partial rows of one query head into its final fp16 row; run by one whole
-// wavefront. Partial s has log-sum-exp lse[s * lse_stride] and row po[s * po_stride .. +D).
-// Lane s holds the weight of partial s (blocks of 64 partials); each lane accumulates two output
-// elements over the partials in index order, with independent row loads kept in flight.
-__device__ __forceinline__ void merge_row(const float *__restrict__ lse, int64_t lse_stride,
-                                          const float *__restrict__ po, int64_t po_stride,
-                                          int n_parts, half_t *out_row, int lane) {
+// Merges partial rows of one query head into its final fp16 row; run by one whole wavefront.
+// The partials come in two runs: n1 of them at lse1[s * lse1_stride], po1[s * po1_stride .. +D),
+// then n2 more at lse2 / po2 (n2 may be 0). Lane s holds the weight of partial s (blocks of 64
+// partials); each lane accumulates two output elements over the partials in index order, with
+// independent row loads kept in flight.
+__device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_t lse1_stride,
+                                          const float *__restrict__ po1, int64_t po1_stride, int n1,
+                                          const float *__restrict__ lse2, int64_t lse2_stride,
+                                          const float *__restrict__ po2, int64_t po2_stride, int n2,
+                                          half_t *out_row, int lane) {
+  const int n_parts = n1 + n2;
+  auto lse_of = [&](int s) {
+    return s < n1 ? lse1[(int64_t)s * lse1_stride] : lse2[(int64_t)(s - n1) * lse2_stride];
+  };
+  auto row_of = [&](int s) {
+    return s < n1 ? po1 + (int64_t)s * po1_stride : po2 + (int64_t)(s - n1) * po2_stride;
+  };
   float mx = -INFINITY;
   for (int s0 = 0; s0 < n_parts; s0 += kWave) {
-    const float l = (s0 + lane < n_parts) ? lse[(int64_t)(s0 + lane) * lse_stride] : -INFINITY;
+    const float l = (s0 + lane < n_parts) ? lse_of(s0 + lane) : -INFINITY;
     mx = fmaxf(mx, l);
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, xor_lane(mx, off));
   float den = 0.f, num0 = 0.f, num1 = 0.f;
-  const float *col = po + 2 * lane;
   for (int s0 = 0; s0 < n_parts; s0 += kWave) {
-    const float l = (s0 + lane < n_parts) ? lse[(int64_t)(s0 + lane) * lse_stride] : -INFINITY;
+    const float l = (s0 + lane < n_parts) ? lse_of(s0 + lane) : -INFINITY;
     const float w = fast_exp2((l - mx) * kLog2e);
     den += w;
     const int cnt = (n_parts - s0) < kWave ? (n_parts - s0) : kWave;
@@ -318,7 +327,7 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse, int64_t
     for (; s + 4 <= cnt; s += 4) {
       float2 r[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) r[u] = *(const float2 *)(col + (int64_t)(s0 + s + u) * po_stride);
+      for (int u = 0; u < 4; ++u) r[u] = *(const float2 *)(row_of(s0 + s + u) + 2 * lane);
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const float wu = __shfl(w, s + u, kWave);
@@ -327,7 +336,7 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse, int64_t
       }
     }
     for (; s < cnt; ++s) {
-      const float2 r = *(const float2 *)(col + (int64_t)(s0 + s) * po_stride);
+      const float2 r = *(const float2 *)(row_of(s0 + s) + 2 * lane);
       const float wu = __shfl(w, s, kWave);
       num0 += wu * r.x;
       num1 += wu * r.y;
@@ -352,8 +361,8 @@ __global__ __launch_bounds__(kWave) void paged_decode_merge_kernel(
   const int n_splits = splits_for_pages(pages_of(len), max_splits, min_pages_per_split);
   if (n_splits == 1) return;  // the split kernel already wrote the final row
   const int64_t cell0 = ((int64_t)b * num_q_heads + hq) * max_splits;
-  merge_row(part_lse + cell0, 1, part_o + cell0 * kHeadDim, kHeadDim, n_splits,
-            out + ((int64_t)b * num_q_heads + hq) * kHeadDim, threadIdx.x);
+  merge_row(part_lse + cell0, 1, part_o + cell0 * kHeadDim, kHeadDim, n_splits, nullptr, 0, nullptr,
+            0, 0, out + ((int64_t)b * num_q_heads + hq) * kHeadDim, threadIdx.x);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -373,7 +382,13 @@ __global__ __launch_bounds__(kWave) void paged_decode_merge_kernel(
 // The piece of sequence b inside chunk c is partial slot c + b (strictly increasing along the
 // line, so slots never collide): part_o[slot][hq][D], part_lse[slot][hq]. A sequence lying
 // inside one chunk is written to `out` directly; the others are merged, in chunk order, by a
-// second small launch (one wavefront per sequence and kv head). Merging inside the decode
+// second small launch (one wavefront per sequence and kv head).
+//
+// Shared prefix: when every sequence of the step starts with the same `skip` physical pages
+// (a cached system prompt), the line holds only the pages after them, and those `skip` pages are
+// attended once for all sequences by the MFMA-tiled kernel of paged_prefill.hip, whose columns
+// are the (sequence, query head) pairs. Its per-key-slice partials join the merge as a second
+// run of pieces; no sequence is then written directly. Merging inside the decode
 // kernel was measured and rejected: pieces written by other XCDs only become visible through
 // device-scope cache write-back / invalidate or write-through accesses, and either costs far
 // more than the 3 us of a launch boundary.
@@ -383,7 +398,7 @@ constexpr int kPlanMeta = 16;      // int32 words of plan meta data
 constexpr int kEntryHeader = 8;    // int32 words of an entry before its page ids
 // plan meta words
 constexpr int kMetaTotal = 0, kMetaChunkPages = 1, kMetaChunks = 2, kMetaBatch = 3,
-              kMetaEntryStride = 4, kMetaKvHeads = 5;
+              kMetaEntryStride = 4, kMetaKvHeads = 5, kMetaSkip = 6;
 
 __host__ __device__ __forceinline__ int round_up(int x, int m) { return (x + m - 1) / m * m; }
 
@@ -416,14 +431,15 @@ __host__ __device__ __forceinline__ int plan_entries_offset(int batch) {
 __global__ __launch_bounds__(256) void decode_plan_kernel(
     const int32_t *__restrict__ block_table, int32_t bt_stride,
     const int32_t *__restrict__ seq_lens, int32_t batch, int32_t num_kv_heads, int32_t chunks,
-    int32_t entry_stride, int32_t num_pages, int32_t *__restrict__ plan) {
+    int32_t entry_stride, int32_t num_pages, int32_t skip, int32_t *__restrict__ plan) {
   __shared__ int red[4][2];
   const int b = blockIdx.x;
   const int tid = threadIdx.x;
   int before = 0, total = 0;
   for (int i = tid; i < batch; i += 256) {
     int pg = pages_of(seq_lens[i]);
-    pg = pg < bt_stride ? pg : bt_stride;
+    pg = (pg < bt_stride ? pg : bt_stride) - skip;
+    pg = pg > 0 ? pg : 0;
     total += pg;
     before += (i < b) ? pg : 0;
   }
@@ -450,6 +466,7 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
       plan[kMetaBatch] = batch;
       plan[kMetaEntryStride] = entry_stride;
       plan[kMetaKvHeads] = num_kv_heads;
+      plan[kMetaSkip] = skip;
     }
     for (int c = tid; c < chunks; c += 256) {
       if ((int64_t)c * chunk_pages >= total) {
@@ -459,14 +476,15 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
     }
   }
   int my_pages = pages_of(seq_lens[b]);
-  my_pages = my_pages < bt_stride ? my_pages : bt_stride;
+  my_pages = (my_pages < bt_stride ? my_pages : bt_stride) - skip;
+  my_pages = my_pages > 0 ? my_pages : 0;
   if (tid == 0) {
     const int c_first = before / chunk_pages;
     plan[plan_seq_info_offset() + 2 * b] = c_first;
     plan[plan_seq_info_offset() + 2 * b + 1] =
         my_pages > 0 ? (before + my_pages - 1) / chunk_pages - c_first + 1 : 0;
   }
-  const int32_t *row = block_table + (int64_t)b * bt_stride;
+  const int32_t *row = block_table + (int64_t)b * bt_stride + skip;
   for (int p = tid; p < my_pages; p += 256) {
     const int f = before + p;
     const int c = f / chunk_pages;
@@ -485,18 +503,25 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
 }
 
 // Balanced-schedule merge, one wavefront per (query head, sequence): combines the sequence's
-// pieces (partial slots c_first + b, c_first + b + 1, ...) if it spans several chunks.
+// pieces (partial slots c_first + b, c_first + b + 1, ...) if it spans several chunks, and the
+// `pre_splits` partials of the shared prefix if there is one.
 __global__ __launch_bounds__(kWave) void paged_decode_balanced_merge_kernel(
-    const int32_t *__restrict__ plan, half_t *__restrict__ out,
-    const float *__restrict__ part_o, const float *__restrict__ part_lse, int32_t num_q_heads) {
+    const int32_t *__restrict__ plan, const int32_t *__restrict__ seq_lens,
+    half_t *__restrict__ out, const float *__restrict__ part_o,
+    const float *__restrict__ part_lse, const float *__restrict__ pre_o,
+    const float *__restrict__ pre_lse, int32_t pre_splits, int32_t batch, int32_t num_q_heads) {
   const int hq = blockIdx.x;
   const int b = blockIdx.y;
   const int c_first = plan[plan_seq_info_offset() + 2 * b];
   const int n_parts = plan[plan_seq_info_offset() + 2 * b + 1];
-  if (n_parts <= 1) return;  // empty, or written directly by the decode kernel
+  if (pre_splits == 0 && n_parts <= 1) return;  // empty, or written directly by the decode kernel
+  if (seq_lens[b] <= 0) return;                 // the decode kernel zeroed the row
   const int64_t cell0 = (int64_t)(c_first + b) * num_q_heads + hq;
+  const int64_t pre0 = (int64_t)b * num_q_heads + hq;
+  const int64_t pre_step = (int64_t)batch * num_q_heads;
   merge_row(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
-            (int64_t)num_q_heads * kHeadDim, n_parts,
+            (int64_t)num_q_heads * kHeadDim, n_parts, pre_lse + pre0, pre_step,
+            pre_o + pre0 * kHeadDim, pre_step * kHeadDim, pre_splits,
             out + ((int64_t)b * num_q_heads + hq) * kHeadDim, threadIdx.x);
 }
 
@@ -507,7 +532,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     const half_t *__restrict__ k_new, const half_t *__restrict__ v_new, int64_t k_new_stride,
     int64_t v_new_stride, half_t *__restrict__ out, float *__restrict__ part_o,
     float *__restrict__ part_lse, int32_t bt_stride, int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t group,
-    int32_t heads_per_wg, int32_t replicas, int32_t chunks, float scale_log2) {
+    int32_t heads_per_wg, int32_t replicas, int32_t chunks, int32_t skip, float scale_log2) {
   __shared__ __attribute__((aligned(16))) half_t vstage_all[kMaxWavesPerWg][kPageSize * kVPitch];
 
   // readfirstlane tells the compiler the wavefront index is uniform (scalar branches and loads)
@@ -570,7 +595,8 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   load_q(qf, q + (int64_t)cur_b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
 
   auto flush = [&]() {
-    const bool whole = cu_lo >= f0 && cu_hi <= f1;  // the sequence lies inside this chunk
+    // the sequence lies inside this chunk and has no shared-prefix partials to merge with
+    const bool whole = cu_lo >= f0 && cu_hi <= f1 && skip == 0;
     const int64_t cell = (int64_t)(cidx + cur_b) * num_q_heads + hq0;
     half_t *out_row = out + ((int64_t)cur_b * num_q_heads + hq0) * kHeadDim;
     store_state(st, whole, out_row, part_o + cell * kHeadDim, kHeadDim, part_lse + cell, 1, n, g,
@@ -596,7 +622,8 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
             len_b = len_after;
             len_after = (cur_b + 1 < batch) ? lens[cur_b + 1] : 0;
             int pg = pages_of(len_b);
-            pg = pg < bt_stride ? pg : bt_stride;
+            pg = (pg < bt_stride ? pg : bt_stride) - skip;
+            pg = pg > 0 ? pg : 0;
             cu_lo = cu_hi;
             cu_hi += pg;
           } while (ff >= cu_hi);
@@ -604,7 +631,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
           st.reset();
           wait_vector_loads();
         }
-        const int p = ff - cu_lo;  // page index inside the sequence
+        const int p = ff - cu_lo + skip;  // page index inside the sequence
         if (k_new != nullptr && (p + 1) * kPageSize >= len_b) {
           // Last page of the sequence: the step's new token (logical position len_b - 1) is
           // appended here. Its K and V rows go to the pool and replace the stale values this
@@ -787,6 +814,13 @@ static size_t balanced_workspace_bytes(int64_t batch, int64_t hq, int64_t d, int
   if (batch <= 0 || hq <= 0 || d <= 0 || chunks <= 0) return 0;
   return (size_t)((chunks + batch) * hq * (d + 1)) * sizeof(float);
 }
+// With a shared prefix: the pieces of the private pages, then the prefix partials of up to
+// kMaxPrefixSplits key slices.
+static size_t prefix_workspace_bytes(int64_t batch, int64_t hq, int64_t d, int64_t chunks) {
+  if (batch <= 0 || hq <= 0 || d <= 0 || chunks <= 0) return 0;
+  return balanced_workspace_bytes(batch, hq, d, chunks) +
+         (size_t)(kMaxPrefixSplits * batch * hq * (d + 1)) * sizeof(float);
+}
 
 static size_t plan_bytes_for(int64_t batch, int64_t bt_stride, int64_t hkv, int64_t chunks) {
   if (batch <= 0 || bt_stride <= 0 || hkv <= 0 || chunks <= 0) return 0;
@@ -845,17 +879,19 @@ extern "C" size_t litekv_decode_plan_bytes(int32_t batch, int32_t block_table_st
   return litekv::plan_bytes_for(batch, block_table_stride, num_kv_heads, chunks);
 }
 
-extern "C" int litekv_decode_plan(const int32_t *block_table, int32_t block_table_stride,
-                                  const int32_t *seq_lens, int32_t batch, int32_t num_kv_heads,
-                                  int32_t page_size, int64_t num_pages, int32_t chunks, void *plan,
-                                  size_t plan_bytes, void *stream) {
-  using namespace litekv;
-  const char *what = "decode_plan";
+namespace litekv {
+static int launch_plan(const char *what, const int32_t *block_table, int32_t block_table_stride,
+                       const int32_t *seq_lens, int32_t batch, int32_t num_kv_heads,
+                       int32_t page_size, int64_t num_pages, int32_t chunks, int32_t shared_pages,
+                       void *plan, size_t plan_bytes, void *stream) {
   LITEKV_REQUIRE(batch >= 0 && batch <= 65535, "%s: batch %d out of [0, 65535]", what, batch);
   LITEKV_REQUIRE(page_size == kPageSize, "%s: page_size %d unsupported (only %d)", what, page_size,
                  kPageSize);
   int rc = check_chunks(what, batch, block_table_stride, num_kv_heads, chunks);
   if (rc != LITEKV_OK) return rc;
+  LITEKV_REQUIRE(shared_pages >= 0 && shared_pages <= block_table_stride,
+                 "%s: shared_pages %d out of [0, block_table_stride %d]", what, shared_pages,
+                 block_table_stride);
   if (batch == 0) {
     clear_error();
     return LITEKV_OK;
@@ -871,8 +907,28 @@ extern "C" int litekv_decode_plan(const int32_t *block_table, int32_t block_tabl
                      static_cast<hipStream_t>(stream), block_table, block_table_stride, seq_lens,
                      batch, num_kv_heads, chunks,
                      plan_entry_stride(batch, block_table_stride, chunks), (int32_t)num_pages,
-                     static_cast<int32_t *>(plan));
+                     shared_pages, static_cast<int32_t *>(plan));
   return check_launch(what);
+}
+}  // namespace litekv
+
+extern "C" int litekv_decode_plan(const int32_t *block_table, int32_t block_table_stride,
+                                  const int32_t *seq_lens, int32_t batch, int32_t num_kv_heads,
+                                  int32_t page_size, int64_t num_pages, int32_t chunks, void *plan,
+                                  size_t plan_bytes, void *stream) {
+  return litekv::launch_plan("decode_plan", block_table, block_table_stride, seq_lens, batch,
+                             num_kv_heads, page_size, num_pages, chunks, 0, plan, plan_bytes,
+                             stream);
+}
+
+extern "C" int litekv_decode_plan_prefix(const int32_t *block_table, int32_t block_table_stride,
+                                         const int32_t *seq_lens, int32_t batch,
+                                         int32_t num_kv_heads, int32_t page_size, int64_t num_pages,
+                                         int32_t chunks, int32_t shared_pages, void *plan,
+                                         size_t plan_bytes, void *stream) {
+  return litekv::launch_plan("decode_plan_prefix", block_table, block_table_stride, seq_lens, batch,
+                             num_kv_heads, page_size, num_pages, chunks, shared_pages, plan,
+                             plan_bytes, stream);
 }
 
 extern "C" int litekv_profile_next_decode(void *start_event, void *stop_event) {
@@ -881,24 +937,30 @@ extern "C" int litekv_profile_next_decode(void *start_event, void *stop_event) {
   return LITEKV_OK;
 }
 
-extern "C" int litekv_paged_decode_balanced(
-    const void *q, int64_t q_batch_stride, void *kv_pool, const int32_t *seq_lens, void *plan,
-    size_t plan_bytes, const void *k_new, const void *v_new, int64_t k_new_stride,
-    int64_t v_new_stride, void *out, void *workspace, size_t workspace_bytes, int32_t batch,
-    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
-    int64_t num_pages, int32_t block_table_stride, int32_t chunks, float softmax_scale,
-    void *stream) {
-  using namespace litekv;
-  const char *what = "paged_decode_balanced";
+namespace litekv {
+// The balanced decode step; with shared_pages > 0 preceded by the shared-prefix launch.
+static int launch_balanced(const char *what, const void *q, int64_t q_batch_stride, void *kv_pool,
+                           const int32_t *block_table, const int32_t *seq_lens, void *plan,
+                           size_t plan_bytes, const void *k_new, const void *v_new,
+                           int64_t k_new_stride, int64_t v_new_stride, void *out, void *workspace,
+                           size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+                           int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                           int64_t num_pages, int32_t block_table_stride, int32_t chunks,
+                           int32_t shared_pages, float softmax_scale, void *stream) {
   int rc = check_chunks(what, batch, block_table_stride, num_kv_heads, chunks);
   if (rc != LITEKV_OK) return rc;
-  static const int32_t dummy_table = 0;  // the kernel reads page ids from the plan
-  DecodeArgs a{q, q_batch_stride, kv_pool, &dummy_table, block_table_stride, seq_lens, out,
-               workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim, page_size,
-               num_pages, softmax_scale, stream};
-  rc = validate_decode(what, a,
-                       balanced_workspace_bytes(batch, num_q_heads, head_dim, chunks), true);
+  static const int32_t dummy_table = 0;  // the decode kernel reads page ids from the plan
+  DecodeArgs a{q, q_batch_stride, kv_pool, block_table ? block_table : &dummy_table,
+               block_table_stride, seq_lens, out, workspace, workspace_bytes, batch, num_q_heads,
+               num_kv_heads, head_dim, page_size, num_pages, softmax_scale, stream};
+  const size_t ws_need = shared_pages > 0
+                             ? prefix_workspace_bytes(batch, num_q_heads, head_dim, chunks)
+                             : balanced_workspace_bytes(batch, num_q_heads, head_dim, chunks);
+  rc = validate_decode(what, a, ws_need, true);
   if (rc != LITEKV_OK) return rc;
+  LITEKV_REQUIRE(shared_pages >= 0 && shared_pages <= block_table_stride,
+                 "%s: shared_pages %d out of [0, block_table_stride %d]", what, shared_pages,
+                 block_table_stride);
   if (batch == 0) {
     clear_error();
     return LITEKV_OK;
@@ -922,6 +984,16 @@ extern "C" int litekv_paged_decode_balanced(
   LITEKV_REQUIRE(s.head_groups <= 65535, "%s: num_kv_heads %d too large", what, num_kv_heads);
   float *part_o = static_cast<float *>(workspace);
   float *part_lse = part_o + (size_t)(chunks + batch) * num_q_heads * head_dim;
+  float *pre_o = part_lse + (size_t)(chunks + batch) * num_q_heads;
+  float *pre_lse = pre_o + (size_t)kMaxPrefixSplits * batch * num_q_heads * head_dim;
+  int pre_splits = 0;
+  if (shared_pages > 0) {
+    LITEKV_REQUIRE(block_table != nullptr, "%s: block_table is null", what);
+    rc = launch_shared_prefix(q, q_batch_stride, kv_pool, block_table, batch, num_q_heads,
+                              num_kv_heads, num_pages, shared_pages, pre_o, pre_lse, softmax_scale,
+                              static_cast<hipStream_t>(stream), &pre_splits);
+    if (rc != LITEKV_OK) return rc;
+  }
   const unsigned wgs = (unsigned)((chunks + s.replicas - 1) / s.replicas);
   hipEvent_t ev0 = g_profile_start, ev1 = g_profile_stop;
   g_profile_start = g_profile_stop = nullptr;
@@ -936,14 +1008,49 @@ extern "C" int litekv_paged_decode_balanced(
                         k_new_stride, v_new_stride, static_cast<half_t *>(out), part_o, part_lse,
                         block_table_stride, batch, num_q_heads, num_kv_heads,
                         num_q_heads / num_kv_heads, s.heads_per_wg, s.replicas, chunks,
-                        softmax_scale * kLog2e);
+                        shared_pages, softmax_scale * kLog2e);
   rc = check_launch(what);
   if (rc != LITEKV_OK) return rc;
   hipLaunchKernelGGL(paged_decode_balanced_merge_kernel,
                      dim3((unsigned)num_q_heads, (unsigned)batch), dim3(kWave), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const int32_t *>(plan),
-                     static_cast<half_t *>(out), part_o, part_lse, num_q_heads);
+                     static_cast<hipStream_t>(stream), static_cast<const int32_t *>(plan), seq_lens,
+                     static_cast<half_t *>(out), part_o, part_lse, pre_o, pre_lse, pre_splits,
+                     batch, num_q_heads);
   return check_launch("paged_decode_balanced_merge");
+}
+}  // namespace litekv
+
+extern "C" int litekv_paged_decode_balanced(
+    const void *q, int64_t q_batch_stride, void *kv_pool, const int32_t *seq_lens, void *plan,
+    size_t plan_bytes, const void *k_new, const void *v_new, int64_t k_new_stride,
+    int64_t v_new_stride, void *out, void *workspace, size_t workspace_bytes, int32_t batch,
+    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+    int64_t num_pages, int32_t block_table_stride, int32_t chunks, float softmax_scale,
+    void *stream) {
+  return litekv::launch_balanced("paged_decode_balanced", q, q_batch_stride, kv_pool, nullptr,
+                                 seq_lens, plan, plan_bytes, k_new, v_new, k_new_stride,
+                                 v_new_stride, out, workspace, workspace_bytes, batch, num_q_heads,
+                                 num_kv_heads, head_dim, page_size, num_pages, block_table_stride,
+                                 chunks, 0, softmax_scale, stream);
+}
+
+extern "C" size_t litekv_paged_decode_prefix_workspace_bytes(int32_t batch, int32_t num_q_heads,
+                                                             int32_t head_dim, int32_t chunks) {
+  return litekv::prefix_workspace_bytes(batch, num_q_heads, head_dim, chunks);
+}
+
+extern "C" int litekv_paged_decode_prefix(
+    const void *q, int64_t q_batch_stride, void *kv_pool, const int32_t *block_table,
+    const int32_t *seq_lens, void *plan, size_t plan_bytes, const void *k_new, const void *v_new,
+    int64_t k_new_stride, int64_t v_new_stride, void *out, void *workspace, size_t workspace_bytes,
+    int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+    int64_t num_pages, int32_t block_table_stride, int32_t chunks, int32_t shared_pages,
+    float softmax_scale, void *stream) {
+  return litekv::launch_balanced("paged_decode_prefix", q, q_batch_stride, kv_pool, block_table,
+                                 seq_lens, plan, plan_bytes, k_new, v_new, k_new_stride,
+                                 v_new_stride, out, workspace, workspace_bytes, batch, num_q_heads,
+                                 num_kv_heads, head_dim, page_size, num_pages, block_table_stride,
+                                 chunks, shared_pages, softmax_scale, stream);
 }
 
 extern "C" size_t litekv_paged_decode_workspace_bytes(int32_t batch, int32_t num_q_heads,

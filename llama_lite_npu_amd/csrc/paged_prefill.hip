@@ -53,6 +53,18 @@ struct PagedSource {
   int32_t num_kv_heads;
   int32_t num_pages;
 };
+// Shared-prefix decode (mode kSharedPrefix): the columns are (sequence, query head) pairs of one
+// decode step, the keys are a slice of the pages every sequence starts with, and the result is
+// a normalised fp32 partial row + log-sum-exp per column, for the decode merge.
+struct PrefixTask {
+  float *part_o;            // [splits][batch][Hq][128]
+  float *part_lse;          // [splits][batch][Hq]
+  int64_t q_batch_stride;   // elements between the q rows of consecutive sequences
+  int32_t batch;
+  int32_t num_q_heads;
+  int32_t prefix_keys;      // shared pages * 16
+  int32_t keys_per_split;   // multiple of the key tile
+};
 struct PackedSource {
   const half_t *k;              // [T][Hkv][128]
   const half_t *v;
@@ -91,13 +103,16 @@ __device__ __forceinline__ float max_across_groups(float x) {
   s = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
   return vmax2(__builtin_bit_cast(float, s[0]), __builtin_bit_cast(float, s[1]));
 }
-template <bool PAGED>
+constexpr int kPagedPrefill = 0, kPackedPrefill = 1, kSharedPrefix = 2;
+
+template <int MODE>
 __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_kernel(
     const half_t *__restrict__ q, int64_t q_stride, half_t *__restrict__ out, int64_t out_stride,
-    PagedSource paged, PackedSource packed, const int32_t *__restrict__ q_starts_or_cu,
-    const int32_t *__restrict__ q_lens_or_null, const int32_t *__restrict__ context_lens,
-    int32_t group, int32_t head_splits, int32_t heads_per_wg, int32_t row_tiles,
-    float scale_log2) {
+    PagedSource paged, PackedSource packed, PrefixTask prefix,
+    const int32_t *__restrict__ q_starts_or_cu, const int32_t *__restrict__ q_lens_or_null,
+    const int32_t *__restrict__ context_lens, int32_t group, int32_t head_splits,
+    int32_t heads_per_wg, int32_t row_tiles, float scale_log2) {
+  constexpr bool PAGED = MODE != kPackedPrefill;
   // Two tiles of K and two of V: tile t sits in half t % 2.
   __shared__ __attribute__((aligned(1024))) half_t kbuf[2 * kTileHalfs];
   __shared__ __attribute__((aligned(1024))) half_t vbuf[2 * kTileHalfs];
@@ -114,24 +129,39 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   const int heads_here = (group - head0) < heads_per_wg ? (group - head0) : heads_per_wg;
   const int b = blockIdx.z;
 
-  int q_start, q_len;
-  if (PAGED) {
-    q_start = q_starts_or_cu[b];
-    q_len = q_starts_or_cu[b + 1] - q_start;
+  // What the block works on: query rows m0.. of sequence b (prefill), or the column block
+  // blockIdx.y of all (sequence, head) pairs against key slice blockIdx.z (shared prefix).
+  //   kv_end  one past the last key the block may see      diag  last key every column sees
+  //   tile0   first key tile (tiles are counted from it)   last_key  last key that exists
+  int q_start = 0, q_len = 0, m0 = 0, ctx = 0, kv_end, diag, last_key;
+  int tile0 = 0;
+  if constexpr (MODE == kSharedPrefix) {
+    const int key_begin = (int)blockIdx.z * prefix.keys_per_split;
+    if (key_begin >= prefix.prefix_keys) return;
+    kv_end = key_begin + prefix.keys_per_split;
+    kv_end = kv_end < prefix.prefix_keys ? kv_end : prefix.prefix_keys;
+    diag = kv_end - 1;
+    last_key = prefix.prefix_keys - 1;
+    tile0 = key_begin / kKvTile;
   } else {
-    q_start = packed.seq_starts[b];
-    q_len = q_lens_or_null[b];
+    if (PAGED) {
+      q_start = q_starts_or_cu[b];
+      q_len = q_starts_or_cu[b + 1] - q_start;
+    } else {
+      q_start = packed.seq_starts[b];
+      q_len = q_lens_or_null[b];
+    }
+    const int block_rows = 16 * row_tiles;
+    // Long blocks first, all heads of a row block next to each other.
+    m0 = ((int)gridDim.y - 1 - (int)blockIdx.y) * block_rows;
+    if (m0 >= q_len) return;
+    ctx = (PAGED && context_lens) ? context_lens[b] : 0;
+    const int rows = (q_len - m0) < block_rows ? (q_len - m0) : block_rows;
+    kv_end = ctx + m0 + rows;
+    diag = ctx + m0;
+    last_key = ctx + q_len - 1;
   }
-  const int block_rows = 16 * row_tiles;
-  // Long blocks first, all heads of a row block next to each other.
-  const int m0 = ((int)gridDim.y - 1 - (int)blockIdx.y) * block_rows;
-  if (m0 >= q_len) return;
-  const int ctx = (PAGED && context_lens) ? context_lens[b] : 0;
-  const int kv_len = ctx + q_len;
-  const int rows = (q_len - m0) < block_rows ? (q_len - m0) : block_rows;
-  const int kv_end = ctx + m0 + rows;  // keys the block may see
-  const int last_key = kv_len - 1;
-  const int n_tiles = (kv_end + kKvTile - 1) / kKvTile;
+  const int n_tiles = (kv_end + kKvTile - 1) / kKvTile - tile0;
 
   // ---- staging addresses -------------------------------------------------------------------
   // Direct-load instruction i of wavefront w fills tile rows 16w + 4i .. +3 (one page per
@@ -150,18 +180,19 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     voff[i] = rip * v_pitch +
               (uint32_t)(((PAGED ? paged.num_kv_heads : 0) + h) * kHeadDim + 8 * cv) * 2u;
   }
-  const int32_t *table = PAGED ? paged.block_table + (int64_t)b * paged.bt_stride : nullptr;
+  const int32_t *table =
+      PAGED ? paged.block_table + (MODE == kSharedPrefix ? 0 : (int64_t)b * paged.bt_stride) : nullptr;
   const int last_page = last_key >> 4;
 
   // Starts the loads of tile kt into its LDS half. The instruction is written as asm so that the
   // compiler does not make later LDS reads of the *other* half wait for it; the wait is the
   // explicit vmcnt(0) before the barrier that publishes the tile.
   auto issue_tile = [&](int kt) {
-    const int row0 = kt * kKvTile + 16 * wave;  // first key of this wavefront's 16 rows
+    const int row0 = (tile0 + kt) * kKvTile + 16 * wave;  // first key of this wavefront's 16 rows
     const char *kbase, *vbase;
     int src0;  // key index the bases point at
     if (PAGED) {
-      int pidx = kt * 4 + wave;
+      int pidx = (tile0 + kt) * 4 + wave;
       pidx = pidx < last_page ? pidx : last_page;
       int pid = table[pidx];
       pid = pid < 0 ? 0 : (pid >= paged.num_pages ? paged.num_pages - 1 : pid);
@@ -213,16 +244,28 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
 #pragma unroll
   for (int u = 0; u < kColTiles; ++u) {
     const int t = wave * kColTiles + u;
-    const int head = t / row_tiles;
-    const int row = m0 + (t - head * row_tiles) * 16 + n;
-    const bool ok = head < heads_here && row < q_len;
-    const int hq = h * group + head0 + (head < heads_here ? head : 0);
-    const int last = q_len - 1;
-    q_pos[u] = ctx + (row < last ? row : last);
-    out_row[u] = ok ? q_start + row : -1;
+    bool ok;
+    int hq;
+    const half_t *qrow;
+    if constexpr (MODE == kSharedPrefix) {
+      const int col = (int)blockIdx.y * (16 * kWgColTiles) + 16 * t + n;  // (sequence, head) pair
+      ok = col < prefix.batch * group;
+      const int seq = ok ? col / group : 0;
+      hq = h * group + (ok ? col - seq * group : 0);
+      q_pos[u] = kv_end - 1;
+      out_row[u] = ok ? seq : -1;
+      qrow = q + (int64_t)seq * prefix.q_batch_stride + (int64_t)hq * kHeadDim + 8 * g;
+    } else {
+      const int head = t / row_tiles;
+      const int row = m0 + (t - head * row_tiles) * 16 + n;
+      ok = head < heads_here && row < q_len;
+      hq = h * group + head0 + (head < heads_here ? head : 0);
+      const int last = q_len - 1;
+      q_pos[u] = ctx + (row < last ? row : last);
+      out_row[u] = ok ? q_start + row : -1;
+      qrow = q + (int64_t)(q_start + (ok ? row : 0)) * q_stride + (int64_t)hq * kHeadDim + 8 * g;
+    }
     out_head[u] = hq;
-    const half_t *qrow =
-        q + (int64_t)(q_start + (ok ? row : 0)) * q_stride + (int64_t)hq * kHeadDim + 8 * g;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
       qf[u][kk] = ok ? *(const half8_t *)(qrow + 32 * kk) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
@@ -350,7 +393,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   auto general_tile = [&](int kt, int first) {
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2) {
-      const int key0 = kt * kKvTile + 32 * s2;
+      const int key0 = (tile0 + kt) * kKvTile + 32 * s2;
       if (s2 < first) continue;
       if (key0 >= kv_end) break;  // nothing visible in the second half
       scores_sub(s2);
@@ -381,7 +424,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       flip_halves();
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
-        const int key0 = kt * kKvTile + 32 * s2;
+        const int key0 = (tile0 + kt) * kKvTile + 32 * s2;
         if (MASKED && key0 >= kv_end) break;
         scores_sub(s2);
         if (MASKED) {
@@ -428,7 +471,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
 
   {
     // Tiles whose last key is at or below the block's first row need no mask.
-    int n_plain = (ctx + m0 + 1) / kKvTile;
+    int n_plain = (diag + 1) / kKvTile - tile0;
     n_plain = n_plain < n_tiles ? n_plain : n_tiles;
     sync_and_prefetch(0);
     general_tile(0, 0);
@@ -445,6 +488,20 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
 #pragma unroll
   for (int u = 0; u < kColTiles; ++u) {
     const float inv = 1.0f / dsum[u][0];
+    if constexpr (MODE == kSharedPrefix) {
+      if (out_row[u] >= 0) {
+        const int64_t cell =
+            ((int64_t)blockIdx.z * prefix.batch + out_row[u]) * prefix.num_q_heads + out_head[u];
+        float *po = prefix.part_o + cell * kHeadDim + 4 * g;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          *(float4_t *)(po + 16 * j) = float4_t{acc[j][u][0] * inv, acc[j][u][1] * inv,
+                                                acc[j][u][2] * inv, acc[j][u][3] * inv};
+        }
+        if (g == 0) prefix.part_lse[cell] = (m_run[u] + fast_log2(dsum[u][0])) * 0.6931471805599453f;
+      }
+      continue;
+    }
     if (out_row[u] >= 0) {
       half_t *o = out + (int64_t)out_row[u] * out_stride + (int64_t)out_head[u] * kHeadDim + 4 * g;
 #pragma unroll
@@ -492,6 +549,42 @@ static PrefillShape prefill_shape(int group, int max_q_len) {
   return s;
 }
 
+int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_pool,
+                         const int32_t *block_table, int32_t batch, int32_t num_q_heads,
+                         int32_t num_kv_heads, int64_t num_pages, int32_t shared_pages,
+                         float *part_o, float *part_lse, float softmax_scale, hipStream_t stream,
+                         int *splits_out) {
+  const char *what = "shared_prefix";
+  const int group = num_q_heads / num_kv_heads;
+  LITEKV_REQUIRE(group >= 1 && group <= 16, "%s: %d query heads per kv head unsupported", what, group);
+  LITEKV_REQUIRE(num_kv_heads <= 1024, "%s: num_kv_heads %d > 1024", what, num_kv_heads);
+  LITEKV_REQUIRE(shared_pages >= 1 && shared_pages <= (1 << 24), "%s: shared_pages %d out of range",
+                 what, shared_pages);
+  const int prefix_keys = shared_pages * kPageSize;
+  const int col_blocks = (batch * group + 16 * kWgColTiles - 1) / (16 * kWgColTiles);
+  LITEKV_REQUIRE(col_blocks <= 65535, "%s: batch %d too large", what, batch);
+  // Enough key slices for about one workgroup per compute unit, at least 128 keys each.
+  int splits = 256 / (num_kv_heads * col_blocks);
+  splits = splits < 1 ? 1 : (splits > kMaxPrefixSplits ? kMaxPrefixSplits : splits);
+  const int max_by_keys = (prefix_keys + 127) / 128;
+  splits = splits < max_by_keys ? splits : max_by_keys;
+  int keys_per_split = (prefix_keys + splits - 1) / splits;
+  keys_per_split = (keys_per_split + kKvTile - 1) / kKvTile * kKvTile;
+  splits = (prefix_keys + keys_per_split - 1) / keys_per_split;
+  PagedSource paged{static_cast<const half_t *>(kv_pool), block_table, 0, num_kv_heads,
+                    (int32_t)num_pages};
+  PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
+  PrefixTask task{part_o, part_lse, q_batch_stride, batch, num_q_heads, prefix_keys, keys_per_split};
+  hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kSharedPrefix>,
+                     dim3((unsigned)num_kv_heads, (unsigned)col_blocks, (unsigned)splits),
+                     dim3(kTiledWaves * kWave), 0, stream, static_cast<const half_t *>(q),
+                     (int64_t)0, (half_t *)nullptr, (int64_t)0, paged, packed, task,
+                     (const int32_t *)nullptr, (const int32_t *)nullptr, (const int32_t *)nullptr,
+                     group, 1, group, 1, softmax_scale * kLog2eP);
+  *splits_out = splits;
+  return check_launch(what);
+}
+
 }  // namespace litekv
 
 extern "C" int litekv_paged_prefill(const void *q, int64_t q_token_stride, const void *kv_pool,
@@ -524,11 +617,11 @@ extern "C" int litekv_paged_prefill(const void *q, int64_t q_token_stride, const
   const int group = num_q_heads / num_kv_heads;
   const PrefillShape s = prefill_shape(group, max_q_len);
   LITEKV_REQUIRE(s.row_blocks <= 65535u, "paged_prefill: max_q_len %d too large", max_q_len);
-  hipLaunchKernelGGL(varlen_prefill_tiled_kernel<true>,
+  hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kPagedPrefill>,
                      dim3((unsigned)(num_kv_heads * s.head_splits), s.row_blocks, (unsigned)batch),
                      dim3(kTiledWaves * kWave), 0, static_cast<hipStream_t>(stream),
                      static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
-                     out_token_stride, paged, packed, cu_q_lens, (const int32_t *)nullptr,
+                     out_token_stride, paged, packed, PrefixTask{}, cu_q_lens, (const int32_t *)nullptr,
                      context_lens, group, s.head_splits, s.heads_per_wg, s.row_tiles,
                      softmax_scale * kLog2eP);
   return check_launch("paged_prefill");
@@ -564,11 +657,11 @@ extern "C" int litekv_varlen_prefill(const void *q, int64_t q_token_stride, cons
   const int group = num_q_heads / num_kv_heads;
   const PrefillShape s = prefill_shape(group, max_seq_len);
   LITEKV_REQUIRE(s.row_blocks <= 65535u, "varlen_prefill: max_seq_len %d too large", max_seq_len);
-  hipLaunchKernelGGL(varlen_prefill_tiled_kernel<false>,
+  hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kPackedPrefill>,
                      dim3((unsigned)(num_kv_heads * s.head_splits), s.row_blocks, (unsigned)batch),
                      dim3(kTiledWaves * kWave), 0, static_cast<hipStream_t>(stream),
                      static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
-                     out_token_stride, paged, packed, seq_starts, seq_lens,
+                     out_token_stride, paged, packed, PrefixTask{}, seq_starts, seq_lens,
                      (const int32_t *)nullptr, group, s.head_splits, s.heads_per_wg, s.row_tiles,
                      softmax_scale * kLog2eP);
   return check_launch("varlen_prefill");

@@ -140,8 +140,12 @@ class DecodePlan:
 
     def __init__(self, block_table: torch.Tensor, seq_lens: torch.Tensor, num_q_heads: int,
                  num_kv_heads: int, num_pages: int, chunks: Optional[int] = None,
-                 page_size: int = PAGE_SIZE):
+                 page_size: int = PAGE_SIZE, shared_pages: int = 0):
+        """``shared_pages``: leading block-table entries that are the same physical pages in every
+        row (a shared cached prefix); they are then attended once for the whole batch."""
         lib = _lib.load()
+        self.shared_pages = int(shared_pages)
+        _need(0 <= self.shared_pages <= block_table.shape[1], "shared_pages out of range")
         _need(block_table.dim() == 2, "block_table must be [B, max_blocks]")
         self.block_table = _dev_i32("block_table", block_table)
         self.seq_lens = _dev_i32("seq_lens", seq_lens)
@@ -155,8 +159,9 @@ class DecodePlan:
         self.plan_bytes = int(lib.litekv_decode_plan_bytes(self.batch, self.bt_stride, self.num_kv_heads,
                                                            self.chunks))
         self.buffer = torch.empty(max(4, self.plan_bytes // 4), dtype=torch.int32, device=dev)
-        ws_bytes = int(lib.litekv_paged_decode_balanced_workspace_bytes(self.batch, self.num_q_heads,
-                                                                        HEAD_DIM, self.chunks))
+        ws_fn = (lib.litekv_paged_decode_prefix_workspace_bytes if self.shared_pages > 0
+                 else lib.litekv_paged_decode_balanced_workspace_bytes)
+        ws_bytes = int(ws_fn(self.batch, self.num_q_heads, HEAD_DIM, self.chunks))
         self.workspace = torch.empty(max(4, ws_bytes // 4), dtype=torch.float32, device=dev)
         self.workspace_bytes = ws_bytes
         self.refresh()
@@ -172,9 +177,10 @@ class DecodePlan:
             _need(sl.numel() == self.batch, "seq_lens shape changed")
             self.seq_lens = sl
         lib = _lib.load()
-        _lib.check(lib.litekv_decode_plan(_ptr(self.block_table), self.bt_stride, _ptr(self.seq_lens), self.batch,
-                                          self.num_kv_heads, self.page_size, self.num_pages, self.chunks,
-                                          _ptr(self.buffer), self.plan_bytes, _stream()))
+        _lib.check(lib.litekv_decode_plan_prefix(_ptr(self.block_table), self.bt_stride, _ptr(self.seq_lens),
+                                                 self.batch, self.num_kv_heads, self.page_size, self.num_pages,
+                                                 self.chunks, self.shared_pages, _ptr(self.buffer),
+                                                 self.plan_bytes, _stream()))
 
 
 def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
@@ -205,6 +211,13 @@ def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
         _need(out.shape == (b, hq, d) and out.is_contiguous(), "out must be contiguous [B, Hq, D]")
     q_stride = q.stride(0) if b > 1 else max(q.stride(0), hq * d)
     lib = _lib.load()
+    if plan.shared_pages > 0:
+        _lib.check(lib.litekv_paged_decode_prefix(
+            _ptr(q), q_stride, _ptr(kv_pool), _ptr(plan.block_table), _ptr(plan.seq_lens), _ptr(plan.buffer),
+            plan.plan_bytes, _ptr(k_new), _ptr(v_new), kn_stride, vn_stride, _ptr(out), _ptr(plan.workspace),
+            plan.workspace_bytes, b, hq, hkv, d, plan.page_size, n_pages, plan.bt_stride, plan.chunks,
+            plan.shared_pages, float(softmax_scale), _stream()))
+        return out
     _lib.check(lib.litekv_paged_decode_balanced(
         _ptr(q), q_stride, _ptr(kv_pool), _ptr(plan.seq_lens), _ptr(plan.buffer), plan.plan_bytes,
         _ptr(k_new), _ptr(v_new), kn_stride, vn_stride, _ptr(out), _ptr(plan.workspace), plan.workspace_bytes,
@@ -221,8 +234,12 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
                  max_splits: Optional[int] = None, out: Optional[torch.Tensor] = None,
                  workspace: Optional[torch.Tensor] = None, page_size: int = PAGE_SIZE,
                  stage: str = "both", schedule: Optional[str] = None,
-                 chunks: Optional[int] = None, plan: Optional[DecodePlan] = None) -> torch.Tensor:
+                 chunks: Optional[int] = None, plan: Optional[DecodePlan] = None,
+                 shared_pages: int = 0) -> torch.Tensor:
     """Decode attention of q [B, Hq, D] over the pages named by block_table [B, max_blocks].
+
+    ``shared_pages`` (balanced schedule): the first that many entries of every block-table row are
+    the same physical pages; they are attended once for the whole batch.
 
     schedule "balanced" (default): all pages of the batch are cut into `chunks` equal pieces per
     kv head (default: one workgroup per CU); a DecodePlan is built for the call unless one is
@@ -243,7 +260,7 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
     if schedule == "balanced":
         _need(stage == "both", "the balanced schedule is a single launch")
         if plan is None:
-            plan = DecodePlan(block_table, seq_lens, hq, hkv, n_pages, chunks, page_size)
+            plan = DecodePlan(block_table, seq_lens, hq, hkv, n_pages, chunks, page_size, shared_pages)
         return decode_step(q, kv_pool, plan, None, None, softmax_scale, out)
 
     _need(block_table.dim() == 2 and block_table.shape[0] == b, "block_table must be [B, max_blocks]")

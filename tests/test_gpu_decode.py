@@ -205,3 +205,57 @@ def test_invalid_arguments_raise():
     with pytest.raises(LiteKVError, match="workspace"):
         ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, max_splits=4,
                          min_pages_per_split=1, workspace=torch.empty(4, device=DEV))
+
+
+def _shared_prefix_case(seed, hq, hkv, shared_pages, suffix_ctx):
+    """Every block-table row starts with the same `shared_pages` pages; context = prefix + suffix."""
+    ctx = [shared_pages * 16 + s for s in suffix_ctx]
+    priv = [(c + 1 + 15) // 16 - shared_pages for c in ctx]
+    num_pages = shared_pages + sum(priv) + 7
+    perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(seed)).to(torch.int32)
+    shared, cur, lists = perm[:shared_pages], shared_pages, []
+    for n in priv:
+        lists.append(torch.cat([shared, perm[cur:cur + n]]))
+        cur += n
+    return workloads.make_decode_case("shared", seed, ctx, hq, hkv, num_pages=num_pages, device=DEV,
+                                      page_lists=lists)
+
+
+@pytest.mark.parametrize("hq,hkv,shared_pages,suffix", [
+    (64, 8, 13, [0, 5, 15, 16, 40, 300]),          # 208 prefix keys: not a multiple of the key tile
+    (16, 8, 1, [3, 0, 90]),                        # one shared page
+    (32, 4, 40, list(range(0, 170, 10))),          # 17 sequences x 8 heads: two column blocks
+    (16, 1, 64, [1, 2, 3, 500]),                   # 16 query heads per kv head
+    (28, 4, 9, [7, 0, 33, 64, 65]),                # 7 heads per kv head
+])
+def test_shared_prefix_decode(hq, hkv, shared_pages, suffix):
+    """Pages common to all sequences attended once for the batch == the plain decode."""
+    print(f"decode shared prefix {hq}/{hkv} pages={shared_pages}", flush=True)
+    case = _shared_prefix_case(700 + hq + shared_pages, hq, hkv, shared_pages, suffix)
+    ref = _oracle(case)
+    for chunks in (None, 5):
+        out = _run(case, schedule="balanced", chunks=chunks, shared_pages=shared_pages)
+        assert_attention_close(out, ref, f"shared prefix {hq}/{hkv} chunks={chunks}")
+    # fewer pages declared shared than really are: still the same attention
+    out = _run(case, schedule="balanced", shared_pages=max(1, shared_pages // 2))
+    assert_attention_close(out, ref, "shared prefix, half declared")
+
+
+def test_shared_prefix_fused_append_and_empty_rows():
+    """The fused append writes the same bits with a shared prefix; empty sequences give zero rows."""
+    print("decode shared prefix + fused append", flush=True)
+    case = _shared_prefix_case(760, 64, 8, 6, [0, 14, 15, 16, 31, 100, 7])
+    pool_ref = case.kv_pool.clone()
+    ops.kv_append(case.k_new, case.v_new, case.slot_mapping, pool_ref)
+    lens = case.seq_lens.clone()
+    lens[2] = 0
+    plan = ops.DecodePlan(case.block_table, lens, 64, 8, case.num_pages, shared_pages=6)
+    out = ops.decode_step(case.q, case.kv_pool, plan, case.k_new, case.v_new, case.softmax_scale)
+    torch.cuda.synchronize()
+    keep = torch.ones(case.kv_pool.shape[0], dtype=torch.bool, device=DEV)
+    keep[case.slot_mapping[2].long()] = False       # sequence 2 is empty: its row is not appended
+    assert torch.equal(case.kv_pool[keep], pool_ref[keep])
+    ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool_ref), case.block_table.cpu().numpy(),
+                                lens.cpu().numpy(), case.softmax_scale)
+    assert_attention_close(out, ref, "shared prefix + fused append")
+    assert float(out[2].abs().max()) == 0.0
