@@ -52,6 +52,7 @@ class ModelExecutor:
         self.atten_info = AttentionInfo()
         self.atten_info.kv_buffer = self.kv_mem_manager.gpu_kv_buffer
         self.build_decode_plans = build_decode_plans and torch.device(device).type == "cuda"
+        self.shared_prefix_min_pages = 4  # below that the two extra launches cost more than they save
         self._decode_plan = None
         self._paged_request_ids: tuple[int, ...] = ()
         # exact-prompt cache: prompt -> (pages, token count, first generated token), LRU of 128
@@ -293,7 +294,27 @@ class ModelExecutor:
 
             info.decode_plan = ops.DecodePlan(info.block_table, info.seq_lens_i32, self.local_q_heads,
                                               self.local_kv_heads, self.kv_mem_manager.num_pages,
-                                              page_size=self.page_size)
+                                              page_size=self.page_size,
+                                              shared_pages=self.shared_prefix_pages(ids))
+
+    def shared_prefix_pages(self, request_ids: Sequence[int]) -> int:
+        """Leading pages that are the same physical pages, and full, in every request of the batch
+        (prefix-cache hits map one page list into many requests, :547-620): the decode step then
+        attends them once for the whole batch. 0 when the batch shares fewer than
+        ``shared_prefix_min_pages`` pages."""
+        mgr = self.req_tokens_manager
+        ids = list(request_ids)
+        if len(ids) < 2:
+            return 0
+        lists = [mgr.request_pages(r) for r in ids]
+        # the page that receives this step's token, and everything after it, is private
+        limit = min((mgr.req_token_count[r] - 1) // self.page_size for r in ids)
+        limit = min(limit, min(len(p) for p in lists))
+        first = lists[0]
+        n = 0
+        while n < limit and all(p[n] == first[n] for p in lists[1:]):
+            n += 1
+        return n if n >= self.shared_prefix_min_pages else 0
 
     def extend_paged_requests(self, request_ids: tuple[int, ...]) -> None:
         """Reserves the KV position of the next decode input of every request, then activates the batch."""

@@ -147,6 +147,38 @@ def test_prefix_sharing_with_copy_on_write():
     assert float((out[0].float() - out[1].float()).abs().max()) > 1e-3
 
 
+def test_cached_system_prompt_is_attended_once_for_the_batch():
+    """Three requests share a 96-token prompt prefix through the block cache; each replays its own
+    suffix; the decode step then runs with a shared-prefix plan and matches the oracle."""
+    print("executor: shared prefix decode", flush=True)
+    ex = _executor(num_pages=128, layers=1)
+    attn = Attention(HQ, HKV, D)
+    system = tuple(range(2000, 2096))               # 6 full pages
+    (a,) = ex.reserve_paged_requests([96])
+    ex.activate_paged_packed_prefill_batch((a,), [96])
+    q, k, v = _qkv(96, 31)
+    attn.context_forward(q, k, v, ex.atten_info, 0, SCALE * LOG2E)
+    ex.store_paged_request_prefix(system, a, first_token_id=5)
+    others = []
+    for i, extra in enumerate((20, 3)):
+        prompt = system + tuple(range(3000 + 100 * i, 3000 + 100 * i + extra))
+        req, matched, first = ex.share_paged_prefix_from_cache(prompt)
+        assert matched == 96 and first is None
+        ex.ensure_paged_request_capacity(req, 96 + extra + 8)
+        ex.activate_paged_chunk_prefill_batch((req,), [96], [extra])
+        qs, ks, vs = _qkv(extra, 40 + i)
+        attn.context_forward(qs, ks, vs, ex.atten_info, 0, SCALE * LOG2E)
+        others.append(req)
+    batch = (a, *others)
+    assert ex.shared_prefix_pages(batch) == 5       # not extended yet: page 5 still ends request a
+    ex.extend_paged_requests(batch)
+    assert ex.atten_info.decode_plan.shared_pages == 6
+    qd, kd, vd = _qkv(3, 50)
+    out = attn.token_forward(qd, kd, vd, ex.atten_info, 0, SCALE)
+    torch.cuda.synchronize()
+    assert_attention_close(out, _oracle_decode(ex, qd, 0), "decode over a shared system prompt")
+
+
 def test_compaction_keeps_results_bitwise():
     print("executor: compaction", flush=True)
     ex = _executor(num_pages=64, layers=2)

@@ -222,7 +222,6 @@ def test_prefix_cache_exact_and_block_hits_hold_page_references():
 def test_compaction_plan_moves_high_pages_into_holes(monkeypatch):
     ex = _executor(num_pages=8, max_requests=4)
     ids = ex.reserve_paged_requests([4, 4, 4, 4, ][:4])   # pages 0..3
-    more = ex.reserve_paged_requests([]) if False else ()
     ex.req_tokens_manager.extend_req(ids[3], 8)           # request 3 now owns pages 3, 4, 5
     ex.release_paged_request_ids((ids[0], ids[2]))        # holes at 0 and 2; live = {1, 3, 4, 5}
     moved = []
@@ -235,3 +234,26 @@ def test_compaction_plan_moves_high_pages_into_holes(monkeypatch):
     assert mgr.page_free.tolist() == [False, False, False, False, True, True, True, True]
     assert mgr.alloc(4).tolist() == [4]
     assert ex.req_tokens_manager.block_table[ids[3], :3].tolist() == [3, 0, 2]
+
+
+def test_shared_prefix_pages_counts_full_common_pages():
+    """Requests that map the same cached pages (block prefix cache) share them in a decode step;
+    the page receiving a request's next token never counts."""
+    ex = _executor(num_pages=32, max_seq_len=64, max_requests=4, page_size=4)
+    ex.shared_prefix_min_pages = 2
+    system = tuple(range(100, 112))                      # 3 full pages of 4 tokens
+    (a,) = ex.reserve_paged_requests([12])
+    ex.activate_paged_packed_prefill_batch((a,), [12])
+    ex.store_paged_request_prefix(system, a, first_token_id=1)
+    b, matched, first = ex.share_paged_prefix_from_cache(system + (7, 8, 9))
+    assert (matched, first) == (12, None)
+    ex.ensure_paged_request_capacity(b, 20)
+    ex.activate_paged_chunk_prefill_batch((b,), [12], [3])
+    pages_a, pages_b = ex.req_tokens_manager.request_pages(a), ex.req_tokens_manager.request_pages(b)
+    assert pages_a[:3] == pages_b[:3]
+    assert ex.shared_prefix_pages((a,)) == 0             # nothing to share with
+    assert ex.shared_prefix_pages((a, b)) == 2           # a holds 12 tokens: its page 2 takes no part yet
+    ex.extend_paged_requests((a, b))                     # a -> 13 tokens on a private 4th page
+    assert ex.shared_prefix_pages((a, b)) == 3
+    ex.shared_prefix_min_pages = 4
+    assert ex.shared_prefix_pages((a, b)) == 0           # too short to pay for the extra launches
