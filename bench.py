@@ -272,6 +272,24 @@ def _time_us(fn, reps: int = 10, warm: int = 2) -> float:
     return sum(a.elapsed_time(b) for a, b in ev) / reps * 1e3
 
 
+def time_qk_epilogue(tokens: int, hq: int, hkv: int, slot_mapping, pool) -> dict:
+    """The fused QK-norm + RoPE + append launch on `tokens` rows of the workload's head layout."""
+    import torch
+    from llama_lite_npu_amd import ops
+
+    dev = pool.device
+    g = torch.Generator(device=dev).manual_seed(99)
+    q = torch.randn((tokens, hq, 128), generator=g, device=dev, dtype=torch.float16)
+    k = torch.randn((tokens, hkv, 128), generator=g, device=dev, dtype=torch.float16)
+    v = torch.randn((tokens, hkv, 128), generator=g, device=dev, dtype=torch.float16)
+    w = torch.ones(128, device=dev, dtype=torch.float16)
+    ang = torch.rand((tokens, 128), generator=g, device=dev) * 6.28
+    cos, sin = ang.cos().half(), ang.sin().half()
+    us = _time_us(lambda: ops.qk_norm_rope_append(q, k, v, slot_mapping, pool, w, w, cos, sin, 1e-6), reps=20)
+    nbytes = tokens * ((2 * hq + 4 * hkv) * 256 + 2 * 128 + 4)
+    return {"qk_epilogue_us": us, "qk_epilogue_gbps": nbytes / (us * 1e-6) / 1e9, "qk_epilogue_bytes": nbytes}
+
+
 def cow_step(case) -> dict:
     """C4: the copy-on-write move before a step appends into a shared last page: every sequence's
     last page is copied into its spare page (page_copy, one launch)."""
@@ -562,14 +580,19 @@ def main() -> int:
         ap_us = time_append(case.k_new, case.v_new, case.slot_mapping, case.kv_pool)
         line["detail"]["append_us"] = ap_us
         line["detail"]["append_gbps"] = case.append_bytes() / (ap_us * 1e-6) / 1e9
+        line["detail"].update(time_qk_epilogue(case.batch, case.num_q_heads, case.num_kv_heads,
+                                               case.slot_mapping, case.kv_pool))
         if args.config == "c4":
             line["detail"].update(cow_step(case))
         if args.config == "c5":
             line["detail"].update(compaction_step(case))
         if not args.no_cpu_baseline:
             line["cpu_baseline"] = cpu_baseline_decode(case)
-    elif not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline_prefill(case)
+    else:
+        line["detail"].update(time_qk_epilogue(int(case.seq_lens.sum()), case.num_q_heads, case.num_kv_heads,
+                                               case.slot_mapping, case.kv_pool))
+        if not args.no_cpu_baseline:
+            line["cpu_baseline"] = cpu_baseline_prefill(case)
     print(json.dumps(line), flush=True)
 
     if args.all:

@@ -67,6 +67,40 @@ int litekv_kv_append(const void *k, const void *v,
                      int64_t num_slots, void *stream);
 
 /*
+ * Fused epilogue of the QKV projection, the step before the KV append on the
+ * reference's path (Qwen3Attention._get_qkv, lite_llama/models/qwen3.py:109-130,
+ * followed by Attention.context_forward / token_forward :29, :62): per-head
+ * RMSNorm of q and k (skip_rmsnorm with residual None ->
+ * rms_norm_kernel, lite_llama/kernels/skip_rmsnorm.py:117-146), rotary
+ * embedding of q and k (rope_emb_forward, lite_llama/kernels/rope_emb.py:6-131;
+ * first-half / second-half pairing, the first head_dim/2 entries of each cos /
+ * sin row are used), `torch.cat([xk, xv])` and `update_kv_buffer`, in one
+ * launch:
+ *     q[t][h]                             = rope(norm(q[t][h]) * q_norm_weight)      in place
+ *     kv_pool[slot_mapping[t]][h]         = rope(norm(k[t][h]) * k_norm_weight)
+ *     kv_pool[slot_mapping[t]][Hkv + h]   = v[t][h]                                   bit exact
+ * norm(x) = x / sqrt(mean(x^2) + rms_eps) in fp32, rounded to fp16 before the
+ * weight multiply, the product rounded to fp16 (as the reference); the
+ * rotation is evaluated in fp32 from those fp16 values and rounded once.
+ *   q_norm_weight, k_norm_weight   [head_dim] fp16, or both NULL (models
+ *                                  without QK norm: llama.py, qwen2.py)
+ *   cos_rows, sin_rows             [num_tokens][cos_sin_token_stride] fp16, the
+ *                                  row of each token's position (what
+ *                                  RotaryEmbedding.forward returns,
+ *                                  RotaryEmbedding.py:183-200), or both NULL
+ *   slot outside [0, num_slots)    k / v of that token are not stored; q is
+ *                                  still processed
+ */
+int litekv_qk_norm_rope_append(void *q, int64_t q_token_stride, const void *k,
+                               int64_t k_token_stride, const void *v, int64_t v_token_stride,
+                               const void *q_norm_weight, const void *k_norm_weight,
+                               const void *cos_rows, const void *sin_rows,
+                               int64_t cos_sin_token_stride, const int32_t *slot_mapping,
+                               void *kv_pool, int32_t num_tokens, int32_t num_q_heads,
+                               int32_t num_kv_heads, int32_t head_dim, int64_t num_slots,
+                               float rms_eps, void *stream);
+
+/*
  * Page gather / page copy. The reference has no page-move operation (its
  * allocator never moves KV: lite_llama/executor/paged_attention.py:1-11);
  * these serve copy-on-write of a shared page and pool compaction:

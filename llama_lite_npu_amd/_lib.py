@@ -29,6 +29,11 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_int32, c_int32, c_int32,
          c_int64, c_void_p],
     ),
+    "litekv_qk_norm_rope_append": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int64, c_float, c_void_p],
+    ),
     "litekv_page_gather": (
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p],

@@ -298,17 +298,20 @@ __global__ __launch_bounds__(64) void paged_decode_split_kernel(
 // then n2 more at lse2 / po2 (n2 may be 0). Lane s holds the weight of partial s (blocks of 64
 // partials); each lane accumulates two output elements over the partials in index order, with
 // independent row loads kept in flight.
+template <bool TWO_RUNS>
 __device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_t lse1_stride,
                                           const float *__restrict__ po1, int64_t po1_stride, int n1,
                                           const float *__restrict__ lse2, int64_t lse2_stride,
                                           const float *__restrict__ po2, int64_t po2_stride, int n2,
                                           half_t *out_row, int lane) {
-  const int n_parts = n1 + n2;
+  const int n_parts = TWO_RUNS ? n1 + n2 : n1;
   auto lse_of = [&](int s) {
-    return s < n1 ? lse1[(int64_t)s * lse1_stride] : lse2[(int64_t)(s - n1) * lse2_stride];
+    if (!TWO_RUNS || s < n1) return lse1[(int64_t)s * lse1_stride];
+    return lse2[(int64_t)(s - n1) * lse2_stride];
   };
   auto row_of = [&](int s) {
-    return s < n1 ? po1 + (int64_t)s * po1_stride : po2 + (int64_t)(s - n1) * po2_stride;
+    if (!TWO_RUNS || s < n1) return po1 + (int64_t)s * po1_stride;
+    return po2 + (int64_t)(s - n1) * po2_stride;
   };
   float mx = -INFINITY;
   for (int s0 = 0; s0 < n_parts; s0 += kWave) {
@@ -361,8 +364,8 @@ __global__ __launch_bounds__(kWave) void paged_decode_merge_kernel(
   const int n_splits = splits_for_pages(pages_of(len), max_splits, min_pages_per_split);
   if (n_splits == 1) return;  // the split kernel already wrote the final row
   const int64_t cell0 = ((int64_t)b * num_q_heads + hq) * max_splits;
-  merge_row(part_lse + cell0, 1, part_o + cell0 * kHeadDim, kHeadDim, n_splits, nullptr, 0, nullptr,
-            0, 0, out + ((int64_t)b * num_q_heads + hq) * kHeadDim, threadIdx.x);
+  merge_row<false>(part_lse + cell0, 1, part_o + cell0 * kHeadDim, kHeadDim, n_splits, nullptr, 0,
+                   nullptr, 0, 0, out + ((int64_t)b * num_q_heads + hq) * kHeadDim, threadIdx.x);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -515,14 +518,20 @@ __global__ __launch_bounds__(kWave) void paged_decode_balanced_merge_kernel(
   const int c_first = plan[plan_seq_info_offset() + 2 * b];
   const int n_parts = plan[plan_seq_info_offset() + 2 * b + 1];
   if (pre_splits == 0 && n_parts <= 1) return;  // empty, or written directly by the decode kernel
-  if (seq_lens[b] <= 0) return;                 // the decode kernel zeroed the row
+  if (pre_splits != 0 && seq_lens[b] <= 0) return;  // the decode kernel zeroed the row
   const int64_t cell0 = (int64_t)(c_first + b) * num_q_heads + hq;
   const int64_t pre0 = (int64_t)b * num_q_heads + hq;
   const int64_t pre_step = (int64_t)batch * num_q_heads;
-  merge_row(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
-            (int64_t)num_q_heads * kHeadDim, n_parts, pre_lse + pre0, pre_step,
-            pre_o + pre0 * kHeadDim, pre_step * kHeadDim, pre_splits,
-            out + ((int64_t)b * num_q_heads + hq) * kHeadDim, threadIdx.x);
+  half_t *out_row = out + ((int64_t)b * num_q_heads + hq) * kHeadDim;
+  if (pre_splits == 0) {
+    merge_row<false>(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
+                     (int64_t)num_q_heads * kHeadDim, n_parts, nullptr, 0, nullptr, 0, 0, out_row,
+                     threadIdx.x);
+  } else {
+    merge_row<true>(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
+                    (int64_t)num_q_heads * kHeadDim, n_parts, pre_lse + pre0, pre_step,
+                    pre_o + pre0 * kHeadDim, pre_step * kHeadDim, pre_splits, out_row, threadIdx.x);
+  }
 }
 
 template <int DEPTH>

@@ -1,0 +1,156 @@
+// Fused epilogue of the QKV projection: per-head RMSNorm of q and k, rotary position embedding
+// of both, and the KV append -- the rotated k row and the v row of each token go straight into
+// the token's page slot, q is updated in place. One launch instead of the reference's five
+// (skip_rmsnorm x2, rope_emb_forward, torch.cat, update_kv_buffer: lite_llama/models/qwen3.py:109-130,
+// 29, 62), and k/v are read once and written once.
+//
+// A head row (128 fp16) is held by 16 lanes, 8 elements each; a wavefront works on 4 rows. The
+// sum of squares is reduced across the 16 lanes; the rotation pairs element i with i + 64, which
+// lives 8 lanes away. Rounding follows the reference where it is specified: the normalised value
+// is rounded to fp16 before the weight multiply, and that product to fp16
+// (`(x * rrms).to(fp16) * w`, lite_llama/kernels/skip_rmsnorm.py:137-145); the rotation
+// x1*cos - x2*sin, x2*cos + x1*sin (lite_llama/kernels/rope_emb.py:79-87) is evaluated in fp32
+// from fp16 inputs and rounded once.
+#include "common.h"
+
+namespace litekv {
+
+constexpr int kLanesPerRow = 16;
+
+__device__ __forceinline__ float row_sum(float v) {
+  v += __shfl_xor(v, 1, kLanesPerRow);
+  v += __shfl_xor(v, 2, kLanesPerRow);
+  v += __shfl_xor(v, 4, kLanesPerRow);
+  v += __shfl_xor(v, 8, kLanesPerRow);
+  return v;
+}
+
+__global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
+    half_t *__restrict__ q, int64_t q_stride, const half_t *__restrict__ k, int64_t k_stride,
+    const half_t *__restrict__ v, int64_t v_stride, const half_t *__restrict__ q_weight,
+    const half_t *__restrict__ k_weight, const half_t *__restrict__ cos_rows,
+    const half_t *__restrict__ sin_rows, int64_t cs_stride, const int32_t *__restrict__ slot_mapping,
+    half_t *__restrict__ pool, int64_t total_rows, int32_t num_q_heads, int32_t num_kv_heads,
+    int64_t num_slots, float eps) {
+  const int l16 = threadIdx.x & 15;
+  const int64_t row = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+  if (row >= total_rows) return;  // whole 16-lane groups leave together
+  const int rows_per_token = num_q_heads + 2 * num_kv_heads;
+  const int64_t token = row / rows_per_token;
+  const int r = (int)(row - token * rows_per_token);
+  const int64_t slot = slot_mapping[token];
+  const bool slot_ok = slot >= 0 && slot < num_slots;
+  half_t *slot_row = pool + slot * (int64_t)(2 * num_kv_heads * kHeadDim);
+
+  if (r >= num_q_heads + num_kv_heads) {  // a v row: plain copy into the slot
+    const int head = r - num_q_heads - num_kv_heads;
+    if (slot_ok) {
+      const half8_t x = *(const half8_t *)(v + token * v_stride + (int64_t)head * kHeadDim + 8 * l16);
+      *(half8_t *)(slot_row + (int64_t)(num_kv_heads + head) * kHeadDim + 8 * l16) = x;
+    }
+    return;
+  }
+  const bool is_q = r < num_q_heads;
+  const int head = is_q ? r : r - num_q_heads;
+  const half_t *src = is_q ? q + token * q_stride + (int64_t)head * kHeadDim
+                           : k + token * k_stride + (int64_t)head * kHeadDim;
+  const half_t *weight = is_q ? q_weight : k_weight;
+  half8_t x = *(const half8_t *)(src + 8 * l16);
+
+  if (weight != nullptr) {
+    float xf[8], ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      xf[i] = (float)x[i];
+      ss += xf[i] * xf[i];
+    }
+    ss = row_sum(ss);
+    const float rrms = 1.0f / sqrtf(ss * (1.0f / kHeadDim) + eps);
+    const half8_t w = *(const half8_t *)(weight + 8 * l16);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const half_t y = (half_t)(xf[i] * rrms);
+      x[i] = (half_t)((float)y * (float)w[i]);
+    }
+  }
+
+  if (cos_rows != nullptr) {
+    // partner: element i + 64 for the first half of the row, i - 64 for the second
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 bits = __builtin_bit_cast(u32x4, x);
+    u32x4 other;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) other[i] = __shfl_xor(bits[i], 8, kLanesPerRow);
+    const half8_t p = __builtin_bit_cast(half8_t, other);
+    const int j = 8 * (l16 & 7);  // index into the first 64 entries of the cos / sin row
+    const half8_t c = *(const half8_t *)(cos_rows + token * cs_stride + j);
+    const half8_t s = *(const half8_t *)(sin_rows + token * cs_stride + j);
+    const float sign = l16 < 8 ? -1.0f : 1.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      x[i] = (half_t)((float)x[i] * (float)c[i] + sign * ((float)p[i] * (float)s[i]));
+    }
+  }
+
+  if (is_q) {
+    *(half8_t *)(q + token * q_stride + (int64_t)head * kHeadDim + 8 * l16) = x;
+  } else if (slot_ok) {
+    *(half8_t *)(slot_row + (int64_t)head * kHeadDim + 8 * l16) = x;
+  }
+}
+
+}  // namespace litekv
+
+extern "C" int litekv_qk_norm_rope_append(void *q, int64_t q_token_stride, const void *k,
+                                          int64_t k_token_stride, const void *v,
+                                          int64_t v_token_stride, const void *q_norm_weight,
+                                          const void *k_norm_weight, const void *cos_rows,
+                                          const void *sin_rows, int64_t cos_sin_token_stride,
+                                          const int32_t *slot_mapping, void *kv_pool,
+                                          int32_t num_tokens, int32_t num_q_heads,
+                                          int32_t num_kv_heads, int32_t head_dim, int64_t num_slots,
+                                          float rms_eps, void *stream) {
+  using namespace litekv;
+  const char *what = "qk_norm_rope_append";
+  LITEKV_REQUIRE(num_tokens >= 0, "%s: num_tokens %d < 0", what, num_tokens);
+  LITEKV_REQUIRE(head_dim == kHeadDim, "%s: head_dim %d unsupported (only %d)", what, head_dim,
+                 kHeadDim);
+  LITEKV_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads <= 65535 && num_kv_heads <= 65535,
+                 "%s: num_q_heads %d / num_kv_heads %d invalid", what, num_q_heads, num_kv_heads);
+  if (num_tokens == 0) {
+    clear_error();
+    return LITEKV_OK;
+  }
+  LITEKV_REQUIRE(q && k && v && slot_mapping && kv_pool, "%s: null pointer", what);
+  LITEKV_REQUIRE((q_norm_weight == nullptr) == (k_norm_weight == nullptr),
+                 "%s: q_norm_weight and k_norm_weight go together", what);
+  LITEKV_REQUIRE((cos_rows == nullptr) == (sin_rows == nullptr), "%s: cos and sin go together", what);
+  LITEKV_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(kv_pool) &&
+                     aligned16(q_norm_weight) && aligned16(k_norm_weight) && aligned16(cos_rows) &&
+                     aligned16(sin_rows),
+                 "%s: all tensors must be 16-byte aligned", what);
+  LITEKV_REQUIRE(q_token_stride >= (int64_t)num_q_heads * head_dim && q_token_stride % 8 == 0 &&
+                     k_token_stride >= (int64_t)num_kv_heads * head_dim && k_token_stride % 8 == 0 &&
+                     v_token_stride >= (int64_t)num_kv_heads * head_dim && v_token_stride % 8 == 0,
+                 "%s: token strides (%lld, %lld, %lld) invalid", what, (long long)q_token_stride,
+                 (long long)k_token_stride, (long long)v_token_stride);
+  if (cos_rows != nullptr) {
+    LITEKV_REQUIRE(cos_sin_token_stride >= head_dim / 2 && cos_sin_token_stride % 8 == 0,
+                   "%s: cos/sin token stride %lld invalid (>= %d, multiple of 8)", what,
+                   (long long)cos_sin_token_stride, head_dim / 2);
+  }
+  LITEKV_REQUIRE(num_slots > 0, "%s: num_slots %lld <= 0", what, (long long)num_slots);
+  LITEKV_REQUIRE(rms_eps >= 0.f, "%s: rms_eps %g < 0", what, (double)rms_eps);
+  const int64_t total_rows = (int64_t)num_tokens * (num_q_heads + 2 * num_kv_heads);
+  const int64_t blocks = (total_rows * kLanesPerRow + 255) / 256;
+  LITEKV_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many tokens", what);
+  hipLaunchKernelGGL(qk_norm_rope_append_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<half_t *>(q), q_token_stride,
+                     static_cast<const half_t *>(k), k_token_stride, static_cast<const half_t *>(v),
+                     v_token_stride, static_cast<const half_t *>(q_norm_weight),
+                     static_cast<const half_t *>(k_norm_weight), static_cast<const half_t *>(cos_rows),
+                     static_cast<const half_t *>(sin_rows), cos_sin_token_stride, slot_mapping,
+                     static_cast<half_t *>(kv_pool), total_rows, num_q_heads, num_kv_heads, num_slots,
+                     rms_eps);
+  return check_launch(what);
+}

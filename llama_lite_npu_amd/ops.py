@@ -73,6 +73,43 @@ def kv_append(k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor, kv_p
                                     _ptr(kv_pool), t, hkv, d, slots, _stream()))
 
 
+def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor,
+                        kv_pool: torch.Tensor, q_norm_weight: Optional[torch.Tensor] = None,
+                        k_norm_weight: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
+                        sin: Optional[torch.Tensor] = None, rms_eps: float = 1e-6) -> torch.Tensor:
+    """Per-head RMSNorm (optional) and rotary embedding (optional) of q [T, Hq, D] in place and of
+    k [T, Hkv, D] on its way into the pool, plus the append of v: one launch for the reference's
+    skip_rmsnorm x2 + rope_emb_forward + cat + update_kv_buffer. cos / sin are [T, >= D/2] rows of
+    each token's position. Returns q."""
+    _dev_half("q", q), _dev_half("k", k), _dev_half("v", v), _dev_half("kv_pool", kv_pool)
+    slots, hkv, d, _, _ = pool_geometry(kv_pool, 1)
+    t, hq = q.shape[0], q.shape[1]
+    _need(q.dim() == 3 and q.shape[2] == d, "q must be [T, Hq, D]")
+    _need(k.shape == (t, hkv, d) and v.shape == (t, hkv, d), "k / v must be [T, Hkv, D] matching the pool")
+    _need((q_norm_weight is None) == (k_norm_weight is None), "q_norm_weight and k_norm_weight go together")
+    _need((cos is None) == (sin is None), "cos and sin go together")
+    if q_norm_weight is not None:
+        _dev_half("q_norm_weight", q_norm_weight), _dev_half("k_norm_weight", k_norm_weight)
+        _need(q_norm_weight.numel() == d and k_norm_weight.numel() == d and q_norm_weight.is_contiguous()
+              and k_norm_weight.is_contiguous(), "norm weights must be contiguous [D]")
+    cs_stride = 0
+    if cos is not None:
+        _dev_half("cos", cos), _dev_half("sin", sin)
+        cos, sin = cos.reshape(-1, cos.shape[-1]), sin.reshape(-1, sin.shape[-1])
+        _need(cos.shape == sin.shape and cos.shape[0] == t and cos.shape[1] >= d // 2, "cos / sin must be [T, >= D/2]")
+        _need(cos.stride(1) == 1 and sin.stride(1) == 1 and cos.stride(0) == sin.stride(0),
+              "cos / sin rows must be contiguous with equal row strides")
+        cs_stride = cos.stride(0)
+    slot_mapping = _dev_i32("slot_mapping", slot_mapping)
+    _need(slot_mapping.numel() == t, "slot_mapping must hold one slot per token")
+    lib = _lib.load()
+    _lib.check(lib.litekv_qk_norm_rope_append(
+        _ptr(q), _rows("q", q), _ptr(k), _rows("k", k), _ptr(v), _rows("v", v), _ptr(q_norm_weight),
+        _ptr(k_norm_weight), _ptr(cos), _ptr(sin), cs_stride, _ptr(slot_mapping), _ptr(kv_pool), t, hq, hkv, d,
+        slots, float(rms_eps), _stream()))
+    return q
+
+
 def page_gather(src_pool: torch.Tensor, dst_pool: torch.Tensor, src_ids: torch.Tensor,
                 dst_ids: Optional[torch.Tensor] = None, page_size: int = PAGE_SIZE) -> None:
     """dst_pool[page dst_ids[i]] = src_pool[page src_ids[i]]; dst_ids None means page i."""

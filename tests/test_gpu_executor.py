@@ -256,3 +256,43 @@ def test_lite_llama_kernels_signatures():
     assert_attention_close(out, ref, "paged_chunk_flash_attention")
     with pytest.raises(ValueError, match="halves of one"):
         compat.flash_decoding(qd, pool[:, :HKV, :].contiguous(), pool[:, HKV:, :], SCALE, table, info.b_seq_len, 8)
+
+
+def test_qkv_epilogue_then_attention_equals_separate_steps():
+    """Executor flow with the fused QK-norm + RoPE + append in front of prefill and decode."""
+    print("executor: fused qkv epilogue", flush=True)
+    from oracle import qk_epilogue
+
+    ex = _executor(layers=1)
+    attn = Attention(HQ, HKV, D)
+    g = torch.Generator(device=DEV).manual_seed(77)
+    wq = (1.0 + 0.1 * torch.randn(D, generator=g, device=DEV)).half()
+    wk = (1.0 + 0.1 * torch.randn(D, generator=g, device=DEV)).half()
+
+    def rows(positions):
+        pos = torch.tensor(positions, device=DEV, dtype=torch.float64)
+        inv = 10000.0 ** (-torch.arange(0, D, 2, device=DEV, dtype=torch.float64) / D)
+        emb = torch.cat([pos[:, None] * inv[None, :]] * 2, dim=1)
+        return emb.cos().half(), emb.sin().half()
+
+    ids = ex.reserve_paged_requests([21, 40])
+    ex.activate_paged_packed_prefill_batch(ids, [21, 40])
+    q, k, v = _qkv(61, 60)
+    cos, sin = rows(list(range(21)) + list(range(40)))
+    q_ref = torch.from_numpy(qk_epilogue.rope(qk_epilogue.rms_norm(to_np16(q), to_np16(wq), 1e-6),
+                                             to_np16(cos), to_np16(sin))).to(DEV)
+    attn.qkv_epilogue(q, k, v, ex.atten_info, 0, wq, wk, (cos, sin), 1e-6)
+    out = attn.context_forward(q, None, None, ex.atten_info, 0, SCALE * LOG2E)
+    torch.cuda.synchronize()
+    assert float((q.float() - q_ref.float()).abs().max()) <= 4e-3
+    info = ex.atten_info
+    ref = c_oracle.paged_prefill(to_np16(q), to_np16(info.kv_buffer[0]), info.block_table.cpu().numpy(),
+                                 info.cu_q_lens.cpu().numpy(), np.zeros(2, np.int32), SCALE)
+    assert_attention_close(out, ref, "prefill after fused epilogue")
+    ex.extend_paged_requests(ids)
+    qd, kd, vd = _qkv(2, 61)
+    cos, sin = rows([21, 40])
+    attn.qkv_epilogue(qd, kd, vd, ex.atten_info, 0, wq, wk, (cos, sin), 1e-6)
+    out = attn.token_forward(qd, None, None, ex.atten_info, 0, SCALE)
+    torch.cuda.synchronize()
+    assert_attention_close(out, _oracle_decode(ex, qd, 0), "decode after fused epilogue")

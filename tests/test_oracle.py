@@ -226,3 +226,101 @@ def test_workload_generators_are_seeded_and_consistent():
     n = c4.extra["n_shared"]
     assert all(torch.equal(c4.block_table[i, :n], c4.block_table[0, :n]) for i in range(4))
     assert c4.decode_bytes() > 0 and c4.append_bytes() == 4 * (2 * 4096 + 4)
+
+
+# ---- QK-norm + RoPE + append (oracle/qk_epilogue.py) ---------------------------------------------
+
+def _rows(seed, t, h, d=128):
+    rng = np.random.default_rng(seed)
+    return rng.standard_normal((t, h, d)).astype(np.float16)
+
+
+def _angles(seed, t, d=128):
+    """cos / sin rows the way RotaryEmbedding.forward builds them: theta_i = pos * base^(-2i/d),
+    both halves of the row equal (RotaryEmbedding.py:190-200)."""
+    rng = np.random.default_rng(seed)
+    pos = rng.integers(0, 4096, size=t).astype(np.float64)
+    inv = 10000.0 ** (-np.arange(0, d, 2, dtype=np.float64) / d)
+    theta = pos[:, None] * inv[None, :]
+    emb = np.concatenate([theta, theta], axis=1)
+    return theta, np.cos(emb).astype(np.float16), np.sin(emb).astype(np.float16)
+
+
+def test_rms_norm_is_the_closed_form():
+    from oracle import qk_epilogue
+
+    x = _rows(1, 5, 3) * np.float16(3.0)
+    w = (1.0 + 0.1 * np.random.default_rng(2).standard_normal(128)).astype(np.float16)
+    got = qk_epilogue.rms_norm(x, w, 1e-6).astype(np.float64)
+    xd = x.astype(np.float64)
+    want = xd / np.sqrt((xd * xd).mean(axis=-1, keepdims=True) + 1e-6) * w.astype(np.float64)
+    assert np.abs(got - want).max() <= 2.5e-3          # two fp16 roundings of O(1..4) values
+    # unit weight and a row of equal entries: every output is +-1
+    ones = np.full((1, 1, 128), 2.5, dtype=np.float16)
+    assert np.all(qk_epilogue.rms_norm(ones, np.ones(128, np.float16), 0.0) == np.float16(1.0))
+    # a missing term (no mean: sum instead) would scale by sqrt(128)
+    assert abs(float(np.abs(got).mean()) / float(np.abs(want).mean()) - 1.0) < 1e-2
+
+
+def test_rope_is_complex_multiplication():
+    from oracle import qk_epilogue
+
+    t, h = 7, 4
+    x = _rows(3, t, h)
+    theta, cos, sin = _angles(4, t)
+    got = qk_epilogue.rope(x, cos, sin).astype(np.float64)
+    # (x1 + i x2) * exp(i theta) with the cos / sin the kernel sees (fp16-rounded)
+    z = x[..., :64].astype(np.float64) + 1j * x[..., 64:].astype(np.float64)
+    rot = cos[:, None, :64].astype(np.float64) + 1j * sin[:, None, :64].astype(np.float64)
+    want = np.concatenate([(z * rot).real, (z * rot).imag], axis=-1)
+    assert np.abs(got - want).max() <= 2e-3            # one fp16 rounding of |x| < 4
+    # pair norms survive the rotation (up to the rounding of cos / sin and of the result)
+    n_in = np.abs(z)
+    n_out = np.hypot(got[..., :64], got[..., 64:])
+    assert np.abs(n_in - n_out).max() <= 6e-3
+    # position 0: cos 1, sin 0 -> identity, bit for bit
+    one, zero = np.ones((t, 128), np.float16), np.zeros((t, 128), np.float16)
+    assert np.array_equal(qk_epilogue.rope(x, one, zero), x)
+
+
+def test_rope_angles_add():
+    from oracle import qk_epilogue
+
+    x = _rows(5, 3, 2)
+    inv = 10000.0 ** (-np.arange(0, 128, 2, dtype=np.float64) / 128)
+
+    def rows(pos):
+        th = np.asarray(pos, dtype=np.float64)[:, None] * inv[None, :]
+        e = np.concatenate([th, th], axis=1)
+        return np.cos(e).astype(np.float16), np.sin(e).astype(np.float16)
+
+    c1, s1 = rows([3, 10, 100])
+    c2, s2 = rows([4, 1, 28])
+    c3, s3 = rows([7, 11, 128])
+    twice = qk_epilogue.rope(qk_epilogue.rope(x, c1, s1), c2, s2).astype(np.float64)
+    once = qk_epilogue.rope(x, c3, s3).astype(np.float64)
+    assert np.abs(twice - once).max() <= 1.5e-2        # fp16 cos / sin and two result roundings
+
+
+def test_qk_epilogue_append_is_index_assignment():
+    from oracle import qk_epilogue
+
+    t, hq, hkv = 6, 4, 2
+    q, k, v = _rows(6, t, hq), _rows(7, t, hkv), _rows(8, t, hkv)
+    _, cos, sin = _angles(9, t)
+    w = np.ones(128, np.float16)
+    pool = np.full((32, 2 * hkv, 128), 7.0, dtype=np.float16)
+    slots = np.array([5, 31, -1, 0, 40, 17], dtype=np.int32)       # two out of range
+    q_out, new_pool = qk_epilogue.qk_norm_rope_append(q, k, v, slots, pool, w, w, cos, sin, 1e-6)
+    k_out = qk_epilogue.rope(qk_epilogue.rms_norm(k, w, 1e-6), cos, sin)
+    assert np.array_equal(q_out, qk_epilogue.rope(qk_epilogue.rms_norm(q, w, 1e-6), cos, sin))
+    for i, s in enumerate(slots):
+        if 0 <= s < 32:
+            assert np.array_equal(new_pool[s, :hkv], k_out[i]) and np.array_equal(new_pool[s, hkv:], v[i])
+    untouched = np.setdiff1d(np.arange(32), slots)
+    assert np.all(new_pool[untouched] == np.float16(7.0))
+    # no norm, no rope: plain KV append (same result as the append oracle)
+    _, plain = qk_epilogue.qk_norm_rope_append(q, k, v, slots, pool)
+    want = pool.copy()
+    c_oracle.kv_append(np.concatenate([k, v], axis=1), slots, want)
+    assert np.array_equal(plain, want)
