@@ -3,7 +3,8 @@
 // blockIdx.x is the move index, blockIdx.y walks the page in tiles of
 // 256 lanes x UNROLL x 16 bytes. All loads of a tile are issued before its
 // stores so each lane keeps UNROLL 16-byte transactions in flight; a page is a
-// contiguous run of bytes, so accesses are fully coalesced. Bit exact.
+// contiguous run of bytes, so accesses are fully coalesced. Bit exact. Loads and stores carry the
+// streaming (non-temporal) hint: nothing moved here is read again soon.
 #include "common.h"
 
 namespace litekv {
@@ -25,12 +26,12 @@ __global__ __launch_bounds__(256) void page_gather_kernel(
 #pragma unroll
   for (int u = 0; u < kGatherUnroll; ++u) {
     const int64_t c = base + u * 256;
-    if (c < page_items) regs[u] = src[c];
+    if (c < page_items) regs[u] = __builtin_nontemporal_load(src + c);
   }
 #pragma unroll
   for (int u = 0; u < kGatherUnroll; ++u) {
     const int64_t c = base + u * 256;
-    if (c < page_items) dst[c] = regs[u];
+    if (c < page_items) __builtin_nontemporal_store(regs[u], dst + c);
   }
 }
 
