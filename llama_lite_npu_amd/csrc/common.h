@@ -60,6 +60,20 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 // Value held by lane (lane ^ mask) of the same wavefront.
 __device__ __forceinline__ float xor_lane(float v, int mask) { return __shfl_xor(v, mask, kWave); }
 
+// Maximum over the four lanes l, l^16, l^32, l^48 (the lane groups that share a column of an
+// MFMA accumulator). The swaps exchange 16- and 32-lane halves between their two operands, so
+// max(first, second) of the swapped pair is the pairwise maximum: two vector ALU instructions
+// per step instead of a round trip through the LDS crossbar.
+__device__ __forceinline__ float max_over_lane_groups(float x) {
+  typedef unsigned uint2_t __attribute__((ext_vector_type(2)));
+  unsigned bits = __builtin_bit_cast(unsigned, x);
+  uint2_t s = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+  const float y = fmaxf(__builtin_bit_cast(float, s[0]), __builtin_bit_cast(float, s[1]));
+  bits = __builtin_bit_cast(unsigned, y);
+  s = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+  return fmaxf(__builtin_bit_cast(float, s[0]), __builtin_bit_cast(float, s[1]));
+}
+
 // D(16x16) += A(16x32) * B(32x16), fp16 inputs, fp32 accumulate.
 // Lane l supplies A[l % 16][8*(l/16) .. +7] and B[8*(l/16) .. +7][l % 16];
 // it receives D[4*(l/16) + i][l % 16] in element i.

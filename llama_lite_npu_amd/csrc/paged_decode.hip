@@ -128,21 +128,22 @@ __device__ __forceinline__ void attend_page(HeadState &st, const PageRegs &r,
   }
   wave_lds_fence();
 
-  float4_t s = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int kk = 0; kk < 4; ++kk) s = mfma_16x16x32(r.k[kk], qf[kk], s);
+  // two accumulators: the dependent MFMA chain is two deep instead of four
+  float4_t s = mfma_16x16x32(r.k[0], qf[0], float4_t{0.f, 0.f, 0.f, 0.f});
+  float4_t s1 = mfma_16x16x32(r.k[2], qf[2], float4_t{0.f, 0.f, 0.f, 0.f});
+  s = mfma_16x16x32(r.k[1], qf[1], s);
+  s1 = mfma_16x16x32(r.k[3], qf[3], s1);
 
   float sv[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) sv[i] = s[i] * scale_log2;
+  for (int i = 0; i < 4; ++i) sv[i] = (s[i] + s1[i]) * scale_log2;
   if (tail) {
     const int tok0 = p * kPageSize + 4 * g;
 #pragma unroll
     for (int i = 0; i < 4; ++i) sv[i] = (tok0 + i < len) ? sv[i] : -INFINITY;
   }
   float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
-  mx = fmaxf(mx, xor_lane(mx, 16));
-  mx = fmaxf(mx, xor_lane(mx, 32));
+  mx = max_over_lane_groups(mx);
   // mx is finite (the page holds at least one valid token). Raise the reference max only when
   // some head needs it; the branch is wavefront-uniform.
   if (__builtin_amdgcn_ballot_w64(mx > st.m + kMaxSlack) != 0) {
@@ -576,9 +577,15 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   int cu_lo = entry[3];  // current sequence: [first, last) page on the line
   int cu_hi = entry[4];
   const uniform_i32_ptr page_ids = entry + kEntryHeader;
+  // The first DEPTH ids are read at fixed offsets (an entry always has room for them), in the
+  // same round trip as the header, and clamped afterwards: one dependent hop less before the
+  // first K/V request.
+  static_assert(DEPTH <= 4, "an entry is only guaranteed to hold kEntryHeader + 4 words");
   int first_ids[DEPTH];
 #pragma unroll
-  for (int dd = 0; dd < DEPTH; ++dd) first_ids[dd] = page_ids[dd < f1 - f0 ? dd : f1 - f0 - 1];
+  for (int dd = 0; dd < DEPTH; ++dd) first_ids[dd] = page_ids[dd];
+#pragma unroll
+  for (int dd = 1; dd < DEPTH; ++dd) first_ids[dd] = dd < f1 - f0 ? first_ids[dd] : first_ids[dd - 1];
 
   int len_b = lens[cur_b];
   int len_after = (cur_b + 1 < batch) ? lens[cur_b + 1] : 0;  // read ahead for the crossing
@@ -622,6 +629,11 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   }
   // after the prologue pid_next holds the id of page DEPTH (clamped), as the loop expects
   for (int f = f0; f < f1; f += DEPTH) {
+    // Keep the wavefronts of the workgroup (the kv heads of one chunk) in step: the hardware
+    // favours the older wavefront of each SIMD, the favoured half would finish a third earlier
+    // and leave the memory system half loaded for the rest of the launch. A wavefront that has
+    // left the kernel no longer counts at the barrier, so unequal chunk lengths are harmless.
+    __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int dd = 0; dd < DEPTH; ++dd) {
       const int ff = f + dd;
