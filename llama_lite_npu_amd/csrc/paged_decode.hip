@@ -101,15 +101,21 @@ __device__ __forceinline__ void load_q(half8_t (&qf)[4], const half_t *q_row0, i
 // Requests one page: k_lane / v_lane already point at this lane's row and column of page 0.
 // K/V bytes are used once per launch: the loads carry the streaming (non-temporal) hint, which
 // keeps the step metadata and q rows in L2 and measured 2 % (C2) to 7 % (C5) faster.
+// `dummy` (wavefront-uniform) marks a request past the end of the chunk, issued only to keep the
+// number of loads in flight constant: every lane then reads the same 16 bytes of the page
+// (streaming loads do not stay in L2, so re-reading the whole last page would cost HBM traffic).
 __device__ __forceinline__ void request_page(PageRegs &r, const half_t *k_lane,
                                              const half_t *v_lane, int64_t page_off,
-                                             int64_t row_stride) {
-  const half_t *kr = k_lane + page_off;
+                                             int64_t row_stride, bool dummy = false,
+                                             const half_t *pool = nullptr) {
+  const half_t *kr = dummy ? pool + page_off : k_lane + page_off;
+  const int64_t k_step = dummy ? 0 : 32;
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) r.k[kk] = __builtin_nontemporal_load((const half8_t *)(kr + 32 * kk));
-  const half_t *vr = v_lane + page_off;
+  for (int kk = 0; kk < 4; ++kk) r.k[kk] = __builtin_nontemporal_load((const half8_t *)(kr + kk * k_step));
+  const half_t *vr = dummy ? pool + page_off : v_lane + page_off;
+  const int64_t v_step = dummy ? 0 : 4 * row_stride;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) r.v[i] = __builtin_nontemporal_load((const half8_t *)(vr + 4 * i * row_stride));
+  for (int i = 0; i < 4; ++i) r.v[i] = __builtin_nontemporal_load((const half8_t *)(vr + i * v_step));
 }
 
 // Folds page `p` (tokens 16p .. 16p+15 of a sequence of `len` tokens) into the state.
@@ -596,15 +602,16 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   half_t *v_lane = kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
   const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
 
-  // Requests past the chunk re-read its last page (a cache hit) so the number of vector loads
-  // in flight stays a compile-time constant and every wait names exactly the page it needs.
+  // Requests past the chunk still issue their loads (16 bytes of its last page) so the number of
+  // vector loads in flight stays a compile-time constant and every wait names exactly the page
+  // it needs.
   // Page ids travel through scalar loads, one request ahead of their use.
   int pid_next = 0;
   auto request = [&](int i, PageRegs &r) {  // i = page index inside the chunk
     const int64_t page_off = (int64_t)pid_next * kPageSize * row_stride;
     const int nx = i + 1 < f1 - f0 ? i + 1 : f1 - f0 - 1;
     pid_next = page_ids[nx];
-    request_page(r, k_lane, v_lane, page_off, row_stride);
+    request_page(r, k_lane, v_lane, page_off, row_stride, i >= f1 - f0, kv);
   };
 
   HeadState st;
