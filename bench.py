@@ -37,7 +37,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 # HBM bytes per launch of the decode kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by a 1 GiB
 # copy kernel); summary and commands in profiles/paged_decode_balanced_c2_pmc.txt. Only meaningful for
 # the workload it was measured on.
-MEASURED_TRAFFIC_BYTES = {("c2", "balanced"): 314.2e6}
+MEASURED_TRAFFIC_BYTES = {("c2", "balanced"): 317.0e6}
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 
 

@@ -276,15 +276,15 @@ __global__ __launch_bounds__(64) void paged_decode_split_kernel(
   PageRegs buf[DEPTH];
 
   // Page ids are wavefront-uniform: they travel through scalar loads one step ahead of their
-  // use. Requests past the range re-read its last page (a cache hit), which keeps the number of
-  // vector loads in flight a compile-time constant, so each wait names exactly the page it
-  // needs and never drains the younger prefetches.
+  // use. Requests past the range still issue their loads (16 bytes of its last page), which keeps
+  // the number of vector loads in flight a compile-time constant, so each wait names exactly the
+  // page it needs and never drains the younger prefetches.
   auto page_id = [&](int p) { return clamp_page(table[p < p1 ? p : p1 - 1], num_pages); };
   int pid_next = page_id(p0);
   auto request = [&](int p, PageRegs &r) {
     const int64_t page_off = (int64_t)pid_next * kPageSize * row_stride;
     pid_next = page_id(p + 1);
-    request_page(r, k_lane, v_lane, page_off, row_stride);
+    request_page(r, k_lane, v_lane, page_off, row_stride, p >= p1, kv);
   };
 
 #pragma unroll
