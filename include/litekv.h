@@ -284,6 +284,42 @@ int litekv_paged_decode_prefix(const void *q, int64_t q_batch_stride, void *kv_p
                                void *stream);
 
 /*
+ * Advances the metadata of a decode batch by one token on the device, so that
+ * a captured graph of a decode step replays without host work. Replaces, per
+ * step, PagedReqTokensManager.extend_req + batch_metadata
+ * (lite_llama/executor/paged_attention.py:287-359), update_kv_index
+ * (lite_llama/kernels/update_kv_index.py:41-74) and the host-to-device copies
+ * of cur_select_index / b_seq_len / b_req_idx in NpuGraphRunner.replay
+ * (lite_llama/executor/npu_graph.py:183-197). Pages must have been reserved
+ * ahead by the host (ensure_req_capacity, paged_attention.py:222-250): the
+ * kernel only reads page lists.
+ *
+ *   request_tables [max_requests][request_table_stride] int32: the page list
+ *                  of every request slot (the executor's device block table)
+ *   request_ids    [B] int32: request slot of each batch row
+ *   capacity       [B] int32 or NULL: tokens each row may grow to (its
+ *                  reserved pages * page_size); NULL: width * page_size
+ *   seq_lens       [B] int32, in/out: += increment (0 recomputes the outputs
+ *                  for the lengths as they are, 1 is a decode step)
+ *   seq_lens_i64   [B] int64 or NULL: copy of seq_lens (b_seq_len)
+ *   slot_mapping   [B] int32 out: slot of logical token seq_lens[b] - 1
+ *                  (cur_select_index); -1 when the row is empty or invalid
+ *   position_ids   [B] int64 or NULL: seq_lens[b] - 1
+ *   block_table    [B][block_table_stride] int32 out: first `width` entries
+ *                  of each row's page list, in batch order
+ *   overflow       int32[1] or NULL: set to 1 (never cleared here) when a row
+ *                  could not advance (bad request id, capacity reached); that
+ *                  row keeps its length
+ */
+int litekv_decode_advance(const int32_t *request_tables, int64_t request_table_stride,
+                          int32_t max_requests, const int32_t *request_ids,
+                          const int32_t *capacity, int32_t *seq_lens, int64_t *seq_lens_i64,
+                          int32_t *slot_mapping, int64_t *position_ids, int32_t *block_table,
+                          int64_t block_table_stride, int32_t width, int32_t *overflow,
+                          int32_t batch, int32_t page_size, int64_t num_pages,
+                          int32_t increment, void *stream);
+
+/*
  * Profiling aid (no counterpart in the reference): the next
  * litekv_paged_decode_balanced launch made by this thread carries the two
  * hipEvent_t handles as its start and stop events, so its device-side

@@ -86,6 +86,11 @@ SIGNATURES = {
          c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_int32, c_int32, c_int32, c_int32, c_int32,
          c_int64, c_int32, c_int32, c_int32, c_float, c_void_p],
     ),
+    "litekv_decode_advance": (
+        c_int32,
+        [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_int32, c_void_p, c_int32, c_int32, c_int64, c_int32, c_void_p],
+    ),
     "litekv_profile_next_decode": (c_int32, [c_void_p, c_void_p]),
     "litekv_paged_prefill": (
         c_int32,

@@ -25,6 +25,7 @@ SOURCES = (
     "qk_rope_append.hip",
     "page_ops.hip",
     "paged_decode.hip",
+    "decode_advance.hip",
     "paged_prefill.hip",
 )
 

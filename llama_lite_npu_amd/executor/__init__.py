@@ -3,5 +3,7 @@
 from .executor_struct import AttentionInfo
 from .paged_attention import PagedKVCacheManager, PagedReqTokensManager
 from .model_executor import ModelExecutor
+from .decode_graph import DecodeGraphRunner, DeviceDecodeBatch, supports_decode_graph
 
-__all__ = ["AttentionInfo", "PagedKVCacheManager", "PagedReqTokensManager", "ModelExecutor"]
+__all__ = ["AttentionInfo", "PagedKVCacheManager", "PagedReqTokensManager", "ModelExecutor",
+           "DecodeGraphRunner", "DeviceDecodeBatch", "supports_decode_graph"]

@@ -33,3 +33,4 @@ class AttentionInfo:
     cu_q_lens: Optional[torch.Tensor] = None             # [B+1] int32 packed-row offsets (prefill)
     context_lens_i32: Optional[torch.Tensor] = None      # chunk_context_len as int32
     decode_plan: Any = None                              # ops.DecodePlan of the step (decode only)
+    device_decode: Any = None                            # DeviceDecodeBatch that owns the tensors above, if any

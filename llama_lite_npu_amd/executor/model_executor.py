@@ -55,6 +55,10 @@ class ModelExecutor:
         self.shared_prefix_min_pages = 4  # below that the two extra launches cost more than they save
         self._decode_plan = None
         self._paged_request_ids: tuple[int, ...] = ()
+        self._device_batch = None            # DeviceDecodeBatch in charge of the running decode batch
+        self._device_batches: dict = {}      # (batch size, shared pages) -> DeviceDecodeBatch
+        self.model = None
+        self.graph_runner = None
         # exact-prompt cache: prompt -> (pages, token count, first generated token), LRU of 128
         self._paged_prefix_cache: OrderedDict = OrderedDict()
         self._paged_prefix_cache_max_entries = 128
@@ -171,6 +175,8 @@ class ModelExecutor:
         info.chunk_context_len = info.chunk_q_seq_len = info.max_actual_q_seq_len = None
         info.context_lens_i32 = None
         info.decode_plan = None
+        info.device_decode = None
+        self._device_batch = None
 
     def _i32(self, values) -> torch.Tensor:
         return torch.as_tensor(np.asarray(values, dtype=np.int32), device=self.device)
@@ -297,28 +303,64 @@ class ModelExecutor:
                                               page_size=self.page_size,
                                               shared_pages=self.shared_prefix_pages(ids))
 
-    def shared_prefix_pages(self, request_ids: Sequence[int]) -> int:
-        """Leading pages that are the same physical pages, and full, in every request of the batch
-        (prefix-cache hits map one page list into many requests, :547-620): the decode step then
-        attends them once for the whole batch. 0 when the batch shares fewer than
-        ``shared_prefix_min_pages`` pages."""
+    def common_leading_pages(self, request_ids: Sequence[int], upcoming_tokens: int = 0) -> int:
+        """How many leading pages are the same physical pages, and full, in every request of the
+        batch. ``upcoming_tokens``: tokens the next step will add to each request before it attends
+        (0 when ``extend_req`` has already booked them)."""
         mgr = self.req_tokens_manager
         ids = list(request_ids)
         if len(ids) < 2:
             return 0
         lists = [mgr.request_pages(r) for r in ids]
         # the page that receives this step's token, and everything after it, is private
-        limit = min((mgr.req_token_count[r] - 1) // self.page_size for r in ids)
+        limit = min((mgr.req_token_count[r] + int(upcoming_tokens) - 1) // self.page_size for r in ids)
         limit = min(limit, min(len(p) for p in lists))
         first = lists[0]
         n = 0
         while n < limit and all(p[n] == first[n] for p in lists[1:]):
             n += 1
+        return n
+
+    def shared_prefix_pages(self, request_ids: Sequence[int], upcoming_tokens: int = 0) -> int:
+        """Leading pages the decode step attends once for the whole batch (prefix-cache hits map one
+        page list into many requests, :547-620). 0 when the batch shares fewer than
+        ``shared_prefix_min_pages`` pages."""
+        n = self.common_leading_pages(request_ids, upcoming_tokens)
         return n if n >= self.shared_prefix_min_pages else 0
+
+    def activate_device_decode_batch(self, request_ids: Sequence[int], reserve_tokens: int = 0):
+        """Decode metadata that steps on the device (see ``DeviceDecodeBatch``): call once when the
+        set of running requests changes, instead of ``activate_paged_decode_batch`` every step.
+        Afterwards ``extend_paged_requests`` with the same ids only books the token on the host;
+        the device half runs with the step (``forward``, a ``DecodeGraphRunner``, or
+        ``device_batch.enqueue_advance()``). Batches are kept per (size, shared pages) so that
+        graphs captured on their tensors stay valid."""
+        from .decode_graph import DeviceDecodeBatch
+
+        self._reset_paged_chunk_prefill_metadata()
+        ids = tuple(int(r) for r in request_ids)
+        shared = self.shared_prefix_pages(ids, upcoming_tokens=1)
+        batch = self._device_batches.get((len(ids), shared))
+        if batch is None:
+            batch = DeviceDecodeBatch(self, ids, reserve_tokens, shared_pages=shared)
+            self._device_batches[(len(ids), shared)] = batch
+        else:
+            batch.load(ids, reserve_tokens)
+        batch.bind(self.atten_info)
+        self._paged_request_ids = ids
+        self._device_batch = batch
+        return batch
 
     def extend_paged_requests(self, request_ids: tuple[int, ...]) -> None:
         """Reserves the KV position of the next decode input of every request, then activates the batch."""
         mgr = self.req_tokens_manager
+        batch = self._device_batch
+        if batch is not None and batch.request_ids == tuple(int(r) for r in request_ids):
+            batch.host_advance()
+            self.atten_info.max_actual_seq_len = batch.max_actual_seq_len
+            return
+        self._device_batch = None
+        self.atten_info.device_decode = None
         for req_idx in request_ids:
             if not mgr.extend_req(req_idx, 1):
                 raise RuntimeError(
@@ -346,6 +388,36 @@ class ModelExecutor:
 
     def release_paged_requests(self) -> None:
         self.release_paged_request_ids(self._paged_request_ids)
+
+    # ---- the step itself -------------------------------------------------------------------
+    def attach_model(self, model, model_type: str = "unknown", use_graph: bool = True,
+                     moe_parallel_mode: str = "tp") -> None:
+        """``model.forward(input_ids, position_ids, atten_info)`` is what ``forward`` runs; decode
+        steps go through a graph runner when the model family allows it (:306-314, :380-386)."""
+        from .decode_graph import DecodeGraphRunner, supports_decode_graph
+
+        self.model = model
+        self.graph_runner = None
+        if use_graph and supports_decode_graph(model_type, moe_parallel_mode):
+            self.graph_runner = DecodeGraphRunner(model, model_type,
+                                                  max_blocks=self.req_tokens_manager.max_pages_per_req)
+
+    def forward(self, input_ids, position_ids=None, **kwargs):
+        """One model step on the active batch (:977-987). Decode steps (one token per sequence)
+        take the graph runner; with a device decode batch ``position_ids`` may be None (the batch
+        computes them) and the device half of the step's metadata is enqueued here."""
+        if self.model is None:
+            raise RuntimeError("no model attached (attach_model)")
+        batch = self._device_batch
+        is_decode = input_ids.dim() == 2 and input_ids.shape[1] == 1
+        if batch is not None and not is_decode:
+            raise ValueError("a device decode batch is active: forward takes one token per sequence")
+        if self.graph_runner is not None and is_decode and not kwargs:
+            return self.graph_runner(input_ids, position_ids, self.atten_info)
+        if batch is not None:
+            batch.enqueue_advance()
+            position_ids = batch.position_ids
+        return self.model.forward(input_ids, position_ids, self.atten_info, **kwargs)
 
     # ---- page moves ------------------------------------------------------------------------
     def copy_on_write(self, request_ids: Sequence[int]):

@@ -220,6 +220,46 @@ class DecodePlan:
                                                  self.plan_bytes, _stream()))
 
 
+def _fixed(name: str, t: Optional[torch.Tensor], dtype: torch.dtype, numel: Optional[int] = None) -> None:
+    """An output (or in/out) tensor must already have its final form: nothing is cast or copied."""
+    if t is None:
+        return
+    _need(t.is_cuda and t.dtype == dtype and t.is_contiguous(), f"{name} must be a contiguous {dtype} GPU tensor")
+    _need(numel is None or t.numel() == numel, f"{name} must hold {numel} elements")
+
+
+def decode_advance(request_tables: torch.Tensor, request_ids: torch.Tensor, seq_lens: torch.Tensor,
+                   slot_mapping: torch.Tensor, block_table: torch.Tensor, num_pages: int,
+                   capacity: Optional[torch.Tensor] = None, seq_lens_i64: Optional[torch.Tensor] = None,
+                   position_ids: Optional[torch.Tensor] = None, overflow: Optional[torch.Tensor] = None,
+                   page_size: int = PAGE_SIZE, increment: int = 1) -> None:
+    """One decode step of metadata on the device, in place: seq_lens += increment, slot_mapping[b] =
+    slot of logical token seq_lens[b] - 1 in request request_ids[b]'s page list (a row of
+    request_tables [max_requests, max_pages]), position_ids[b] = seq_lens[b] - 1, and block_table
+    [B, width] = the batch's page lists. Rows that cannot advance (capacity reached, bad request id)
+    keep their length and raise the overflow flag."""
+    _need(request_tables.dim() == 2 and request_tables.stride(1) == 1, "request_tables must be [max_requests, max_pages]")
+    _fixed("request_tables", request_tables, torch.int32)
+    b = request_ids.numel()
+    _fixed("request_ids", request_ids, torch.int32)
+    _fixed("seq_lens", seq_lens, torch.int32, b)
+    _fixed("slot_mapping", slot_mapping, torch.int32, b)
+    _fixed("capacity", capacity, torch.int32, b)
+    _fixed("seq_lens_i64", seq_lens_i64, torch.int64, b)
+    _fixed("position_ids", position_ids, torch.int64, b)
+    _fixed("overflow", overflow, torch.int32, 1)
+    _need(block_table.is_cuda and block_table.dtype == torch.int32 and block_table.dim() == 2
+          and block_table.shape[0] == b and block_table.stride(1) == 1, "block_table must be int32 [B, width] on the GPU")
+    width = int(block_table.shape[1])
+    _need(width <= request_tables.shape[1], "block_table is wider than request_tables")
+    lib = _lib.load()
+    _lib.check(lib.litekv_decode_advance(
+        _ptr(request_tables), request_tables.stride(0), request_tables.shape[0], _ptr(request_ids), _ptr(capacity),
+        _ptr(seq_lens), _ptr(seq_lens_i64), _ptr(slot_mapping), _ptr(position_ids), _ptr(block_table),
+        block_table.stride(0) if b > 1 else max(block_table.stride(0), width), width, _ptr(overflow), b,
+        int(page_size), int(num_pages), int(increment), _stream()))
+
+
 def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
                 k_new: Optional[torch.Tensor] = None, v_new: Optional[torch.Tensor] = None,
                 softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -324,3 +324,60 @@ def test_qk_epilogue_append_is_index_assignment():
     want = pool.copy()
     c_oracle.kv_append(np.concatenate([k, v], axis=1), slots, want)
     assert np.array_equal(plain, want)
+
+
+# ---- decode metadata (integer arithmetic) -------------------------------------------------------
+
+def test_token_slots_reference_docstring_example():
+    from oracle import decode_metadata
+
+    # worked example of build_token_table (lite_llama/executor/paged_attention.py:125-129)
+    got = decode_metadata.token_slots([3, 7, 12], 10, page_size=4)
+    assert got.tolist() == [12, 13, 14, 15, 28, 29, 30, 31, 48, 49]
+
+
+def test_decode_advance_walks_the_per_token_table():
+    from oracle import decode_metadata
+
+    rng = np.random.default_rng(11)
+    ps, width, num_pages, max_req = 4, 6, 64, 5
+    tables = np.zeros((max_req, width), dtype=np.int32)
+    for r in range(max_req):
+        tables[r] = rng.choice(num_pages, size=width, replace=False)
+    # explicit per-token table, built page by page as the reference does
+    per_token = np.zeros((max_req, width * ps), dtype=np.int64)
+    for r in range(max_req):
+        for p in range(width):
+            for o in range(ps):
+                per_token[r, p * ps + o] = int(tables[r, p]) * ps + o
+    ids = np.array([4, 0, 2], dtype=np.int32)
+    lens = np.array([1, 7, 12], dtype=np.int32)
+    for step in range(8):
+        new_lens, slots, pos, rows, overflow = decode_metadata.decode_advance(tables, ids, lens, None, width, ps,
+                                                                              num_pages)
+        assert overflow == 0
+        assert new_lens.tolist() == (lens + 1).tolist()
+        assert pos.tolist() == lens.tolist()                       # position of the new token = old length
+        assert slots.tolist() == [per_token[r, n] for r, n in zip(ids, lens)]
+        assert np.array_equal(rows, tables[ids])
+        lens = new_lens
+    # increment 0 recomputes for the lengths as they are
+    same, slots0, pos0, _, _ = decode_metadata.decode_advance(tables, ids, lens, None, width, ps, num_pages, 0)
+    assert same.tolist() == lens.tolist() and pos0.tolist() == (lens - 1).tolist()
+    assert slots0.tolist() == [per_token[r, n - 1] for r, n in zip(ids, lens)]
+
+
+def test_decode_advance_refusals_leave_the_length():
+    from oracle import decode_metadata
+
+    ps, width, num_pages = 4, 3, 16
+    tables = np.array([[1, 2, 3], [4, 5, 6]], dtype=np.int32)
+    ids = np.array([0, 1, 7, 1], dtype=np.int32)            # 7: no such request
+    lens = np.array([12, 8, 3, 0], dtype=np.int32)          # row 0 is at the table's end
+    cap = np.array([12, 8, 12, 12], dtype=np.int32)         # row 1 has reached its reserved pages
+    new_lens, slots, pos, rows, overflow = decode_metadata.decode_advance(tables, ids, lens, cap, width, ps, num_pages)
+    assert overflow == 1
+    assert new_lens.tolist() == [12, 8, 3, 1]
+    assert slots.tolist() == [3 * 4 + 3, 5 * 4 + 3, -1, 4 * 4 + 0]
+    assert pos.tolist() == [11, 7, 2, 0]
+    assert rows[2].tolist() == [0, 0, 0]
