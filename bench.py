@@ -37,7 +37,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 # HBM bytes per launch of the decode kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by a 1 GiB
 # copy kernel); summary and commands in profiles/paged_decode_balanced_c2_pmc.txt. Only meaningful for
 # the workload it was measured on.
-MEASURED_TRAFFIC_BYTES = {("c2", "balanced"): 317.0e6}
+MEASURED_TRAFFIC_BYTES = {("c2", "balanced"): 317.9e6}
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 
 
@@ -119,10 +119,21 @@ class DecodeLayerSet:
             self.plan = torch.empty(self.plan_bytes // 4, dtype=torch.int32, device=device)
             ws_bytes = lib.litekv_paged_decode_prefix_workspace_bytes(b, hq, 128, self.chunks)
             self.ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=device)
-            self.plan_args = (self.table.data_ptr(), bts, self.seq_lens.data_ptr(), b, hkv, 16, c.num_pages,
+            # per-step metadata on the device: the batch's rows are gathered from the request tables
+            # (here request i is batch row i) and slots / positions recomputed; increment 0 keeps the
+            # workload's lengths fixed from step to step
+            self.req_ids = torch.arange(b, dtype=torch.int32, device=device)
+            self.batch_table = torch.zeros_like(self.table)
+            self.slot_out = torch.empty(b, dtype=torch.int32, device=device)
+            self.pos_out = torch.empty(b, dtype=torch.int64, device=device)
+            self.advance_args = (self.table.data_ptr(), bts, b, self.req_ids.data_ptr(), None,
+                                 self.seq_lens.data_ptr(), None, self.slot_out.data_ptr(), self.pos_out.data_ptr(),
+                                 self.batch_table.data_ptr(), bts, self.table.shape[1], None, b, 16, c.num_pages,
+                                 0, stream)
+            self.plan_args = (self.batch_table.data_ptr(), bts, self.seq_lens.data_ptr(), b, hkv, 16, c.num_pages,
                               self.chunks, shared_pages, self.plan.data_ptr(), self.plan_bytes, stream)
             self.decode_args = [
-                (self.q.data_ptr(), hq * 128, pools[l].data_ptr(), self.table.data_ptr(), self.seq_lens.data_ptr(),
+                (self.q.data_ptr(), hq * 128, pools[l].data_ptr(), self.batch_table.data_ptr(), self.seq_lens.data_ptr(),
                  self.plan.data_ptr(), self.plan_bytes, c.k_new.data_ptr(), c.v_new.data_ptr(), hkv * 128,
                  hkv * 128, self.out[l].data_ptr(), self.ws.data_ptr(), ws_bytes, b, hq, hkv, 128, 16,
                  c.num_pages, bts, self.chunks, shared_pages, c.softmax_scale, stream)
@@ -148,18 +159,21 @@ class DecodeLayerSet:
             self.plan_info = {"schedule": "splits", "max_splits": self.max_splits,
                               "min_pages_per_split": self.min_pps}
 
-    def step(self, events=None):
+    def step(self, events=None, stream=None):
         """One pass over all layers. `events[l]`: (start, stop) raw HIP events for layer l's decode kernel
-        (balanced) or 3 torch events bracketing split and merge (splits)."""
+        (balanced) or 3 torch events bracketing split and merge (splits). `stream`: launch there
+        instead of the stream the set was built on (balanced only; used under graph capture)."""
         lib = self.lib
         rc = 0
         if self.schedule == "balanced":
-            rc |= lib.litekv_decode_plan_prefix(*self.plan_args)
+            on = (lambda a: a) if stream is None else (lambda a: a[:-1] + (stream,))
+            rc |= lib.litekv_decode_advance(*on(self.advance_args))
+            rc |= lib.litekv_decode_plan_prefix(*on(self.plan_args))
             dec, prof = lib.litekv_paged_decode_prefix, lib.litekv_profile_next_decode
             for l in range(self.layers):
                 if events is not None:
                     prof(events[l][0], events[l][1])
-                rc |= dec(*self.decode_args[l])
+                rc |= dec(*on(self.decode_args[l]))
         else:
             ap, sp, mg = lib.litekv_kv_append, lib.litekv_paged_decode_split, lib.litekv_paged_decode_merge
             for l in range(self.layers):
@@ -177,9 +191,17 @@ class DecodeLayerSet:
         if rc:
             raise RuntimeError(f"liblitekv launch failed: {lib.litekv_last_error().decode()}")
 
+    def capture(self):
+        """The whole step (metadata, plan, every layer) recorded once as a HIP graph."""
+        torch = self.torch
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            self.step(stream=torch.cuda.current_stream().cuda_stream)
+        return graph
+
 
 def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: str,
-               schedule: str = "balanced", shared_pages: int = 0) -> dict:
+               schedule: str = "balanced", shared_pages: int = 0, graph: bool = True) -> dict:
     import torch
 
     ls = DecodeLayerSet(case, layers, device, schedule, shared_pages)
@@ -214,6 +236,20 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
     decode_bytes = case.decode_bytes()
     append_bytes = case.append_bytes()
     step_bytes = layers * (decode_bytes + append_bytes)
+    replay = None
+    if balanced and graph:
+        # the same step replayed as one HIP graph (how the executor runs decode steps by default)
+        g = ls.capture()
+        for _ in range(max(1, warmup)):
+            g.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            g.replay()
+        torch.cuda.synchronize()
+        replay_ms = (time.perf_counter() - t0) * 1e3 / steps
+        replay = {"ms_per_step": replay_ms, "us_per_layer": replay_ms * 1e3 / layers,
+                  "value": step_bytes / (replay_ms * 1e-3) / 1e9}
     k_mean = sum(kernel_ms) / len(kernel_ms)
     # the fused kernel also moves the appended rows; they are part of its algorithmic bytes
     kernel_bytes = decode_bytes + (append_bytes if balanced else 0)
@@ -254,6 +290,24 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
                                logical_gbps=achieved, unique_bytes_per_launch=unique,
                                logical_bytes_per_launch=kernel_bytes)
     res.update(ls.plan_info)
+    res["launch"] = "eager"
+    if replay is not None:
+        # Both ways of issuing the same step are timed; the reported step is the faster one (a graph
+        # wins when launches are short against their issue cost, eager launches win for a step of one
+        # long kernel, where a graph launch's fixed cost is not spread over many nodes).
+        res["eager_launch"] = {"ms_per_step": res["ms_per_step"], "us_per_layer": res["us_per_layer"],
+                               "value": res["value"]}
+        res["graph_replay"] = replay
+        if replay["ms_per_step"] < res["ms_per_step"]:
+            res.update(replay)
+            res["launch"] = "hipgraph replay"
+            if shared_pages > 0:
+                k = replay["ms_per_step"] / layers
+                scale = res["roofline"]["duration_us"] / (k * 1e3)
+                res["roofline"]["duration_us"] = k * 1e3
+                for key in ("achieved", "frac", "logical_gbps"):
+                    if key in res["roofline"]:
+                        res["roofline"][key] *= scale
     return res
 
 
@@ -488,6 +542,8 @@ def main() -> int:
                     help="balanced schedule: pieces per kv head (default: one workgroup per compute unit)")
     ap.add_argument("--no-shared-prefix", action="store_true",
                     help="c4: read the shared prefix pages once per sequence like any other page")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="skip the leg that replays the decode step as one HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one page_gather of exactly 1 GiB (read) + 1 GiB (write): a plain copy of "
                          "known size against which profiler byte counters can be scaled")
@@ -536,7 +592,8 @@ def main() -> int:
         shared = 0
         if sched == "balanced" and not args.no_shared_prefix and not case.extra.get("private_prefix"):
             shared = int(case.extra.get("n_shared", 0))
-        return run_decode(case, layers, args.steps, args.warmup, device, case.name, sched, shared), case
+        return run_decode(case, layers, args.steps, args.warmup, device, case.name, sched, shared,
+                          graph=not args.no_graph), case
 
     if args.calibrate_copy:
         from llama_lite_npu_amd import ops
@@ -568,9 +625,9 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": res["label"], "config": args.config},
+        "config": {"workload": res["label"], "config": args.config, "launch": res.get("launch", "eager")},
         "roofline": res["roofline"],
-        "detail": {k: v for k, v in res.items() if k not in ("roofline", "label", "value", "ms_per_step")},
+        "detail": {k: v for k, v in res.items() if k not in ("roofline", "label", "value", "ms_per_step", "launch")},
     }
     if args.config != "c3":
         line["config"].update(batch=case.batch, num_q_heads=case.num_q_heads, num_kv_heads=case.num_kv_heads,

@@ -379,9 +379,9 @@ __global__ __launch_bounds__(kWave) void paged_decode_merge_kernel(
 
 // ---------------------------------------------------------------------------------------------
 // Schedule "balanced": the pages of all sequences, concatenated in batch order, form one line
-// of `total` pages per kv head; it is cut into `chunks` equal pieces of C = ceil(total / chunks)
-// pages. Wavefront (head h, chunk c) streams pages [c*C, (c+1)*C), finishing one sequence and
-// starting the next where the line crosses a sequence boundary. A workgroup holds
+// of `total` pages per kv head; it is cut into `chunks` pieces of floor(total / chunks) or one
+// more pages. Wavefront (head h, chunk c) streams the pages of its piece, finishing one sequence
+// and starting the next where the line crosses a sequence boundary. A workgroup holds
 // `heads_per_wg` heads of `replicas` consecutive chunks.
 //
 // The cuts are made once per decode step by the plan kernel (block tables and lengths are the
@@ -467,13 +467,24 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
   __syncthreads();
   total = red[0][0] + red[1][0] + red[2][0] + red[3][0];
   before = red[0][1] + red[1][1] + red[2][1] + red[3][1];
-  const int chunk_pages = total > 0 ? (total + chunks - 1) / chunks : 1;
+  // The line of `total` pages is cut into `chunks` pieces whose sizes differ by at most one page:
+  // the first `rem` chunks hold quot + 1 pages, the others quot (none when quot == 0). With a
+  // fixed ceil(total / chunks) pages per chunk the last chunks would stay empty whenever total is
+  // just above a multiple of chunks (5 % of the compute units idle at 18.004 pages per chunk).
+  const int quot = total / chunks;
+  const int rem = total - quot * chunks;
+  const int big_end = rem * (quot + 1);  // pages covered by the larger chunks
+  auto chunk_start = [&](int c) { return c * quot + (c < rem ? c : rem); };
+  auto chunk_of = [&](int f) {
+    if (f < big_end) return f / (quot + 1);
+    return quot > 0 ? rem + (f - big_end) / quot : rem;
+  };
   int32_t *entries = plan + plan_entries_offset(batch);
 
   if (b == 0) {
     if (tid == 0) {
       plan[kMetaTotal] = total;
-      plan[kMetaChunkPages] = chunk_pages;
+      plan[kMetaChunkPages] = quot + (rem > 0 ? 1 : 0);
       plan[kMetaChunks] = chunks;
       plan[kMetaBatch] = batch;
       plan[kMetaEntryStride] = entry_stride;
@@ -481,7 +492,7 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
       plan[kMetaSkip] = skip;
     }
     for (int c = tid; c < chunks; c += 256) {
-      if ((int64_t)c * chunk_pages >= total) {
+      if (quot == 0 && c >= rem) {  // a chunk without pages
         entries[(int64_t)c * entry_stride + 0] = 0;
         entries[(int64_t)c * entry_stride + 1] = 0;
       }
@@ -491,22 +502,21 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
   my_pages = (my_pages < bt_stride ? my_pages : bt_stride) - skip;
   my_pages = my_pages > 0 ? my_pages : 0;
   if (tid == 0) {
-    const int c_first = before / chunk_pages;
+    const int c_first = chunk_of(before);
     plan[plan_seq_info_offset() + 2 * b] = c_first;
     plan[plan_seq_info_offset() + 2 * b + 1] =
-        my_pages > 0 ? (before + my_pages - 1) / chunk_pages - c_first + 1 : 0;
+        my_pages > 0 ? chunk_of(before + my_pages - 1) - c_first + 1 : 0;
   }
   const int32_t *row = block_table + (int64_t)b * bt_stride + skip;
   for (int p = tid; p < my_pages; p += 256) {
     const int f = before + p;
-    const int c = f / chunk_pages;
-    const int r = f - c * chunk_pages;
+    const int c = chunk_of(f);
+    const int first = chunk_start(c);
     int32_t *e = entries + (int64_t)c * entry_stride;
-    e[kEntryHeader + r] = clamp_page(row[p], num_pages);
-    if (r == 0) {
-      const int end = f + chunk_pages;
+    e[kEntryHeader + (f - first)] = clamp_page(row[p], num_pages);
+    if (f == first) {
       e[0] = f;
-      e[1] = end < total ? end : total;
+      e[1] = chunk_start(c + 1);
       e[2] = b;
       e[3] = before;
       e[4] = before + my_pages;
