@@ -54,7 +54,7 @@ class DeviceDecodeBatch:
     """
 
     def __init__(self, executor, request_ids: Sequence[int], reserve_tokens: int = 0,
-                 shared_pages: Optional[int] = None):
+                 shared_pages: Optional[int] = None, host_ahead: bool = False):
         from .. import ops
 
         self.executor = executor
@@ -80,12 +80,12 @@ class DeviceDecodeBatch:
         self.steps = 0
         self._capacity_host = np.zeros(b, dtype=np.int32)
         if shared_pages is None:
-            shared_pages = executor.shared_prefix_pages(request_ids, upcoming_tokens=1)
+            shared_pages = executor.shared_prefix_pages(request_ids, upcoming_tokens=0 if host_ahead else 1)
         self.shared_pages = int(shared_pages)
         self.decode_plan = ops.DecodePlan(self.block_table, self.seq_lens_i32, executor.local_q_heads,
                                           executor.local_kv_heads, executor.kv_mem_manager.num_pages,
                                           page_size=executor.page_size, shared_pages=self.shared_pages)
-        self.load(request_ids, reserve_tokens)
+        self.load(request_ids, reserve_tokens, host_ahead)
 
     # ---- host side -------------------------------------------------------------------------
     def _upload_capacity(self) -> None:
@@ -97,11 +97,13 @@ class DeviceDecodeBatch:
             self._capacity_host = cap
             self.capacity.copy_(torch.from_numpy(cap))
 
-    def load(self, request_ids: Sequence[int], reserve_tokens: int = 0) -> None:
+    def load(self, request_ids: Sequence[int], reserve_tokens: int = 0, host_ahead: bool = False) -> None:
         """Points the batch at ``request_ids`` (same count): uploads ids and current lengths, then
-        recomputes slots, positions, table rows and the plan on the device for those lengths."""
-        from .. import ops
-
+        recomputes slots, positions, table rows and the plan on the device for those lengths.
+        ``host_ahead``: the host has already booked the next step's token for every request (the
+        reference's order: ``extend_paged_requests`` follows each forward, model_executor.py:913-933,
+        continuous_batching.py:1574-1595), so the device starts one token behind and the first
+        step needs no ``host_advance()``."""
         mgr = self.executor.req_tokens_manager
         ids = tuple(int(r) for r in request_ids)
         if len(ids) != self.batch:
@@ -109,15 +111,18 @@ class DeviceDecodeBatch:
         for r in ids:
             if r not in mgr.req_token_count:
                 raise KeyError(f"request {r} is not allocated")
-        if self.shared_pages and self.executor.common_leading_pages(ids, upcoming_tokens=1) < self.shared_pages:
+        ahead = 1 if host_ahead else 0
+        if any(mgr.req_token_count[r] - ahead < 1 for r in ids):
+            raise ValueError("every request needs at least one token in the cache before it decodes")
+        if self.shared_pages and self.executor.common_leading_pages(ids, upcoming_tokens=1 - ahead) < self.shared_pages:
             raise ValueError(f"requests do not share the {self.shared_pages} leading pages this batch was built for")
         self.request_ids = ids
         self.b_req_idx.copy_(torch.tensor(ids, dtype=torch.int32))
-        self.seq_lens_i32.copy_(torch.tensor([mgr.req_token_count[r] for r in ids], dtype=torch.int32))
+        self.seq_lens_i32.copy_(torch.tensor([mgr.req_token_count[r] - ahead for r in ids], dtype=torch.int32))
         self._capacity_host = np.zeros(self.batch, dtype=np.int32)
         self.reserve(reserve_tokens)
         self.overflow.zero_()
-        self.pending = False
+        self.pending = bool(host_ahead)
         self._launch_advance(0)
 
     def reserve(self, tokens_ahead: int) -> None:

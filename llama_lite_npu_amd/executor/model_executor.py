@@ -328,24 +328,28 @@ class ModelExecutor:
         n = self.common_leading_pages(request_ids, upcoming_tokens)
         return n if n >= self.shared_prefix_min_pages else 0
 
-    def activate_device_decode_batch(self, request_ids: Sequence[int], reserve_tokens: int = 0):
+    def activate_device_decode_batch(self, request_ids: Sequence[int], reserve_tokens: int = 0,
+                                     host_ahead: bool = False):
         """Decode metadata that steps on the device (see ``DeviceDecodeBatch``): call once when the
         set of running requests changes, instead of ``activate_paged_decode_batch`` every step.
         Afterwards ``extend_paged_requests`` with the same ids only books the token on the host;
         the device half runs with the step (``forward``, a ``DecodeGraphRunner``, or
         ``device_batch.enqueue_advance()``). Batches are kept per (size, shared pages) so that
-        graphs captured on their tensors stay valid."""
+        graphs captured on their tensors stay valid. ``host_ahead``: the requests' lengths already
+        count the token of the first step (``extend_paged_requests`` was called after the previous
+        forward, as the reference's backend does); each later step is then forward first,
+        ``extend_paged_requests`` afterwards."""
         from .decode_graph import DeviceDecodeBatch
 
         self._reset_paged_chunk_prefill_metadata()
         ids = tuple(int(r) for r in request_ids)
-        shared = self.shared_prefix_pages(ids, upcoming_tokens=1)
+        shared = self.shared_prefix_pages(ids, upcoming_tokens=0 if host_ahead else 1)
         batch = self._device_batches.get((len(ids), shared))
         if batch is None:
-            batch = DeviceDecodeBatch(self, ids, reserve_tokens, shared_pages=shared)
+            batch = DeviceDecodeBatch(self, ids, reserve_tokens, shared_pages=shared, host_ahead=host_ahead)
             self._device_batches[(len(ids), shared)] = batch
         else:
-            batch.load(ids, reserve_tokens)
+            batch.load(ids, reserve_tokens, host_ahead)
         batch.bind(self.atten_info)
         self._paged_request_ids = ids
         self._device_batch = batch
@@ -381,6 +385,10 @@ class ModelExecutor:
         return self.atten_info.cur_select_index
 
     def release_paged_request_ids(self, request_ids: tuple[int, ...]) -> None:
+        batch = self._device_batch
+        if batch is not None and any(int(r) in batch.request_ids for r in request_ids):
+            self._device_batch = None            # its tensors describe a request that is gone
+            self.atten_info.device_decode = None
         for req_idx in request_ids:
             self.req_tokens_manager.free_req(req_idx)
         if tuple(request_ids) == self._paged_request_ids:
