@@ -103,6 +103,19 @@ def sample_next_token(logits: torch.Tensor, temperature: Sequence[float], top_p:
     return torch.where(is_greedy, greedy, drawn)
 
 
+class _TokenRows(dict):
+    """request id -> its last sampled token as a 0-d device tensor. Entries are kept as (batch
+    tensor, row) and sliced only when somebody asks, so remembering a step's samples costs no
+    device work per request."""
+
+    def remember(self, req_idx: int, sampled: torch.Tensor, row: int) -> None:
+        dict.__setitem__(self, req_idx, (sampled, row))
+
+    def __getitem__(self, req_idx: int) -> torch.Tensor:
+        sampled, row = dict.__getitem__(self, req_idx)
+        return sampled[row].reshape(())
+
+
 class ContinuousBatchModelBackend:
     """Paged-KV model adapter between a continuous-batching scheduler and ``ModelExecutor``."""
 
@@ -121,7 +134,7 @@ class ContinuousBatchModelBackend:
         self.device_decode = bool(device_decode) and hasattr(self.executor, "activate_device_decode_batch")
         self.decode_reserve_tokens = int(decode_reserve_tokens)
         self._sampler = sampler if sampler is not None else sample_next_token
-        self._device_tokens: dict[int, torch.Tensor] = {}     # last sampled token of each request (0-d)
+        self._device_tokens = _TokenRows()                    # last sampled token of each request (0-d)
         self._positions: dict[int, int] = {}                  # position of that token
         self._step_ids: tuple[int, ...] = ()                  # requests of the last decode step ...
         self._step_tokens: Optional[torch.Tensor] = None      # ... and what it sampled, [B]
@@ -169,7 +182,7 @@ class ContinuousBatchModelBackend:
                   positions: Optional[Sequence[int]] = None) -> None:
         for row, request in enumerate(requests):
             req_idx = int(request.model_request_id)
-            self._device_tokens[req_idx] = sampled[row].reshape(())
+            self._device_tokens.remember(req_idx, sampled, row)
             if positions is not None:
                 self._positions[req_idx] = int(positions[row])
 

@@ -78,6 +78,7 @@ class DeviceDecodeBatch:
         self.request_ids: tuple[int, ...] = ()
         self.pending = False      # host_advance() done, enqueue_advance() (or a replay) still due
         self.steps = 0
+        self.look_ahead = 0       # tokens of page reserve taken again whenever a request runs out
         self._capacity_host = np.zeros(b, dtype=np.int32)
         if shared_pages is None:
             shared_pages = executor.shared_prefix_pages(request_ids, upcoming_tokens=0 if host_ahead else 1)
@@ -91,7 +92,7 @@ class DeviceDecodeBatch:
     def _upload_capacity(self) -> None:
         mgr = self.executor.req_tokens_manager
         ps = self.executor.page_size
-        cap = np.asarray([min(len(mgr.req_page_table[r]) * ps, mgr.max_seq_len) for r in self.request_ids],
+        cap = np.asarray([min(mgr.req_page_count[r] * ps, mgr.max_seq_len) for r in self.request_ids],
                          dtype=np.int32)
         if not np.array_equal(cap, self._capacity_host):
             self._capacity_host = cap
@@ -117,6 +118,7 @@ class DeviceDecodeBatch:
         if self.shared_pages and self.executor.common_leading_pages(ids, upcoming_tokens=1 - ahead) < self.shared_pages:
             raise ValueError(f"requests do not share the {self.shared_pages} leading pages this batch was built for")
         self.request_ids = ids
+        self.look_ahead = int(reserve_tokens)
         self.b_req_idx.copy_(torch.tensor(ids, dtype=torch.int32))
         self.seq_lens_i32.copy_(torch.tensor([mgr.req_token_count[r] - ahead for r in ids], dtype=torch.int32))
         self._capacity_host = np.zeros(self.batch, dtype=np.int32)
@@ -140,13 +142,20 @@ class DeviceDecodeBatch:
         if self.pending:
             raise RuntimeError("the previous host_advance() has not been followed by a device step")
         mgr = self.executor.req_tokens_manager
-        for r in self.request_ids:
+        counts, reserved = mgr.req_token_count, self._capacity_host
+        grew = False
+        for i, r in enumerate(self.request_ids):
+            if counts[r] >= reserved[i]:                  # this token needs a page beyond the reserve:
+                grew = True                               # take the look-ahead again in one go
+                if self.look_ahead > 0:
+                    mgr.ensure_req_capacity(r, min(counts[r] + 1 + self.look_ahead, mgr.max_seq_len))
             if not mgr.extend_req(r, 1):
                 raise RuntimeError(
                     "Paged KV allocation failed for request "
                     f"{r}: current_tokens={mgr.req_token_count.get(r, 'unknown')}, "
                     f"max_seq_len={mgr.max_seq_len}, free_pages={mgr.page_mgr.num_free_pages}")
-        self._upload_capacity()
+        if grew:
+            self._upload_capacity()
         self.pending = True
         self.steps += 1
 

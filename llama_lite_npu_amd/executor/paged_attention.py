@@ -152,6 +152,7 @@ class PagedReqTokensManager:
         self.block_table = torch.zeros((self.max_requests, self.max_pages_per_req), dtype=torch.int32,
                                        device=device)
         self.req_page_table: dict[int, torch.Tensor] = {}
+        self.req_page_count: dict[int, int] = {}      # len(req_page_table[r]) without touching the tensor
         self.req_token_count: dict[int, int] = {}
         self.req_active = torch.zeros(self.max_requests, dtype=torch.bool, device="cpu")
         self.free_req_indices = list(range(self.max_requests))
@@ -176,7 +177,7 @@ class PagedReqTokensManager:
 
     def block_table_rows(self, req_indices: Sequence[int]) -> torch.Tensor:
         """Block-table rows of a batch, in batch order, trimmed to the longest page list."""
-        width = max(1, max(len(self.req_page_table[r]) for r in req_indices))
+        width = max(1, max(self.req_page_count[r] for r in req_indices))
         rows = np.ascontiguousarray(self._table_host[list(req_indices), :width])
         return torch.from_numpy(rows).to(self.device)
 
@@ -199,6 +200,7 @@ class PagedReqTokensManager:
     def _bind(self, req_idx: int, pages: torch.Tensor, num_tokens: int) -> None:
         self.free_req_indices.remove(req_idx)
         self.req_page_table[req_idx] = pages
+        self.req_page_count[req_idx] = len(pages)
         self.req_token_count[req_idx] = num_tokens
         self.req_active[req_idx] = True
         self._publish_pages(req_idx)
@@ -222,13 +224,14 @@ class PagedReqTokensManager:
         return self._grow(req_idx, self.page_mgr.pages_for(total_tokens))
 
     def _grow(self, req_idx: int, pages_needed: int) -> bool:
-        have = len(self.req_page_table[req_idx])
+        have = self.req_page_count[req_idx]
         if pages_needed <= have:
             return True
         extra = self.page_mgr.alloc((pages_needed - have) * self.page_mgr.page_size)
         if extra is None:
             return False
         self.req_page_table[req_idx] = torch.cat([self.req_page_table[req_idx], extra])
+        self.req_page_count[req_idx] = pages_needed
         self._publish_pages(req_idx, have)
         return True
 
@@ -261,7 +264,8 @@ class PagedReqTokensManager:
         new_total = self.req_token_count[req_idx] + int(num_new_tokens)
         if new_total > self.max_seq_len:
             return False
-        if not self._grow(req_idx, self.page_mgr.pages_for(new_total)):
+        ps = self.page_mgr.page_size
+        if new_total > self.req_page_count[req_idx] * ps and not self._grow(req_idx, (new_total + ps - 1) // ps):
             return False
         self.req_token_count[req_idx] = new_total
         return True
@@ -270,6 +274,7 @@ class PagedReqTokensManager:
         if req_idx in self.req_page_table:
             self.page_mgr.free(self.req_page_table.pop(req_idx))
             del self.req_token_count[req_idx]
+            del self.req_page_count[req_idx]
         self.req_active[req_idx] = False
         if req_idx not in self.free_req_indices:
             self.free_req_indices.append(req_idx)
@@ -300,7 +305,8 @@ class PagedReqTokensManager:
                 raise KeyError(f"request {req_idx} is not allocated")
         ps = self.page_mgr.page_size
         lens = [self.req_token_count[r] for r in req_indices]
-        last = [int(self.req_page_table[r][(n - 1) // ps]) * ps + (n - 1) % ps for r, n in zip(req_indices, lens)]
+        table = self._table_host
+        last = [int(table[r, (n - 1) // ps]) * ps + (n - 1) % ps for r, n in zip(req_indices, lens)]
         return (torch.tensor(req_indices, dtype=torch.int32, device=self.device),
                 torch.tensor(lens, dtype=torch.long, device=self.device),
                 torch.tensor(last, dtype=torch.int32, device=self.device))
