@@ -284,6 +284,56 @@ int litekv_paged_decode_prefix(const void *q, int64_t q_batch_stride, void *kv_p
                                void *stream);
 
 /*
+ * FP8 KV pool (no counterpart in the reference: its README lists FP8 as "not
+ * yet stabilized", README.md:89, and its only low-precision KV code is the
+ * unused int8 prefill kernel lite_llama/kernels/others/
+ * context_flashattention_nopad.py:374-553; the layout and call shape follow
+ * the fp16 entry points above). The pool is
+ *     kv_pool_fp8[num_pages * page_size][2 * num_kv_heads][head_dim]  bytes
+ * of OCP E4M3FN codes (bias 7, largest finite value 448, no infinities), K
+ * heads then V heads, with one fp32 scale per head, scales[2 * num_kv_heads]
+ * (K heads, then V heads):
+ *     code  = e4m3(clamp(x * (1 / scale), -448, 448)), round to nearest even
+ *     value = decode(code) * scale
+ * A page is one contiguous run of page_size * 2 * Hkv * head_dim bytes, so
+ * litekv_page_copy / litekv_page_gather move fp8 pages as they are.
+ *
+ * litekv_kv_append_fp8: litekv_kv_append into an fp8 pool (k, v fp16 rows).
+ * The stored codes are a pure function of the row and the scale.
+ *
+ * litekv_page_dequant: dst_pool[page dst_ids[i]] = fp16(value) of page
+ * src_ids[i], for the prefill entry points, which read fp16 pools (a chunk
+ * that attends to cached fp8 history first turns the pages it needs into a
+ * scratch fp16 pool). dst_ids NULL means page i; ids out of range are skipped.
+ *
+ * litekv_paged_decode_balanced_fp8: litekv_paged_decode_balanced over an fp8
+ * pool, same plan, workspace and result contract. Decoding E4M3 to fp16 is
+ * exact, so the result is fp16 attention over the decoded values: the K scale
+ * joins the softmax scale, the V scale the final normalisation. k_new / v_new
+ * (fp16) are quantised as by litekv_kv_append_fp8 and attended as stored.
+ */
+int litekv_kv_append_fp8(const void *k, const void *v, int64_t k_token_stride,
+                         int64_t v_token_stride, const int32_t *slot_mapping,
+                         void *kv_pool_fp8, const float *scales, int32_t num_tokens,
+                         int32_t num_kv_heads, int32_t head_dim, int64_t num_slots,
+                         void *stream);
+
+int litekv_page_dequant(const void *kv_pool_fp8, void *dst_pool, const int32_t *src_ids,
+                        const int32_t *dst_ids, int32_t n, const float *scales,
+                        int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                        int64_t num_src_pages, int64_t num_dst_pages, void *stream);
+
+int litekv_paged_decode_balanced_fp8(const void *q, int64_t q_batch_stride, void *kv_pool_fp8,
+                                     const float *scales, const int32_t *seq_lens, void *plan,
+                                     size_t plan_bytes, const void *k_new, const void *v_new,
+                                     int64_t k_new_stride, int64_t v_new_stride, void *out,
+                                     void *workspace, size_t workspace_bytes, int32_t batch,
+                                     int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                     int32_t page_size, int64_t num_pages,
+                                     int32_t block_table_stride, int32_t chunks,
+                                     float softmax_scale, void *stream);
+
+/*
  * Advances the metadata of a decode batch by one token on the device, so that
  * a captured graph of a decode step replays without host work. Replaces, per
  * step, PagedReqTokensManager.extend_req + batch_metadata

@@ -22,6 +22,7 @@ OBJ_DIR = CSRC / "build"
 SOURCES = (
     "status.hip",
     "kv_append.hip",
+    "kv_fp8.hip",
     "qk_rope_append.hip",
     "page_ops.hip",
     "paged_decode.hip",

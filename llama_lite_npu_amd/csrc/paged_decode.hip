@@ -31,6 +31,7 @@
 // scalars, and the merge adds the fp32 partials in index order: results do not
 // depend on timing.
 #include "common.h"
+#include "kv_fp8.h"
 
 namespace litekv {
 
@@ -60,10 +61,29 @@ __host__ __device__ __forceinline__ int splits_for_pages(int pages, int max_spli
   return n < max_splits ? n : max_splits;
 }
 
-struct PageRegs {
-  half8_t k[4];  // A-operand fragments of K: token n, d = 32*kk + 8*g .. +7
-  half8_t v[4];  // V rows 4*i + g, 16-byte column n
+// One page as this lane requested it: Frag holds 8 elements, half8_t for an fp16 pool, a pair of
+// dwords (8 E4M3 codes) for an fp8 pool.
+template <typename Frag>
+struct RawPage {
+  Frag k[4];  // A-operand fragments of K: token n, d = 32*kk + 8*g .. +7
+  Frag v[4];  // V rows 4*i + g, 8-element column n
 };
+typedef RawPage<half8_t> PageRegs;
+
+// Storage of the pool a kernel reads: element type and the 8-element fragment a lane loads.
+template <bool FP8> struct KvStore;
+template <> struct KvStore<false> { typedef half_t elem; typedef half8_t frag; };
+template <> struct KvStore<true> { typedef uint8_t elem; typedef uint2_t frag; };
+
+__device__ __forceinline__ PageRegs decoded(const RawPage<uint2_t> &r) {
+  PageRegs x;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    x.k[i] = fp8x8_to_half(r.k[i]);
+    x.v[i] = fp8x8_to_half(r.v[i]);
+  }
+  return x;
+}
 
 // Softmax state and output accumulator of the (up to 16) query heads of one kv head.
 // acc[j][i] is O^T[d = 16j + 4g + i][head n]; m is shared by the 4 lanes of a head, d is this
@@ -104,18 +124,19 @@ __device__ __forceinline__ void load_q(half8_t (&qf)[4], const half_t *q_row0, i
 // `dummy` (wavefront-uniform) marks a request past the end of the chunk, issued only to keep the
 // number of loads in flight constant: every lane then reads the same 16 bytes of the page
 // (streaming loads do not stay in L2, so re-reading the whole last page would cost HBM traffic).
-__device__ __forceinline__ void request_page(PageRegs &r, const half_t *k_lane,
-                                             const half_t *v_lane, int64_t page_off,
+template <typename Elem, typename Frag>
+__device__ __forceinline__ void request_page(RawPage<Frag> &r, const Elem *k_lane,
+                                             const Elem *v_lane, int64_t page_off,
                                              int64_t row_stride, bool dummy = false,
-                                             const half_t *pool = nullptr) {
-  const half_t *kr = dummy ? pool + page_off : k_lane + page_off;
+                                             const Elem *pool = nullptr) {
+  const Elem *kr = dummy ? pool + page_off : k_lane + page_off;
   const int64_t k_step = dummy ? 0 : 32;
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) r.k[kk] = __builtin_nontemporal_load((const half8_t *)(kr + kk * k_step));
-  const half_t *vr = dummy ? pool + page_off : v_lane + page_off;
+  for (int kk = 0; kk < 4; ++kk) r.k[kk] = __builtin_nontemporal_load((const Frag *)(kr + kk * k_step));
+  const Elem *vr = dummy ? pool + page_off : v_lane + page_off;
   const int64_t v_step = dummy ? 0 : 4 * row_stride;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) r.v[i] = __builtin_nontemporal_load((const half8_t *)(vr + i * v_step));
+  for (int i = 0; i < 4; ++i) r.v[i] = __builtin_nontemporal_load((const Frag *)(vr + i * v_step));
 }
 
 // Folds page `p` (tokens 16p .. 16p+15 of a sequence of `len` tokens) into the state.
@@ -188,10 +209,10 @@ __device__ __forceinline__ void attend_page(HeadState &st, const PageRegs &r,
 __device__ __forceinline__ void store_state(const HeadState &st, bool final_row, half_t *out_row,
                                             float *part_row, int64_t part_head_stride,
                                             float *part_lse_cell, int64_t lse_head_stride, int n,
-                                            int g, int group) {
+                                            int g, int group, float out_scale = 1.0f) {
   float d_tot = st.d + xor_lane(st.d, 16);
   d_tot += xor_lane(d_tot, 32);
-  const float inv = 1.0f / d_tot;
+  const float inv = out_scale / d_tot;  // out_scale: the V scale of an fp8 pool
   if (n >= group) return;
   if (final_row) {
     half_t *o = out_row + (int64_t)n * kHeadDim + 4 * g;
@@ -553,9 +574,10 @@ __global__ __launch_bounds__(kWave) void paged_decode_balanced_merge_kernel(
   }
 }
 
-template <int DEPTH>
+template <int DEPTH, bool FP8>
 __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_kernel(
-    const half_t *__restrict__ q, int64_t q_batch_stride, half_t *__restrict__ kv,
+    const half_t *__restrict__ q, int64_t q_batch_stride,
+    typename KvStore<FP8>::elem *__restrict__ kv, const float *__restrict__ scales,
     const int32_t *__restrict__ seq_lens, const int32_t *__restrict__ plan,
     const half_t *__restrict__ k_new, const half_t *__restrict__ v_new, int64_t k_new_stride,
     int64_t v_new_stride, half_t *__restrict__ out, float *__restrict__ part_o,
@@ -606,10 +628,23 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   int len_b = lens[cur_b];
   int len_after = (cur_b + 1 < batch) ? lens[cur_b + 1] : 0;  // read ahead for the crossing
 
+  typedef typename KvStore<FP8>::elem Elem;
+  typedef typename KvStore<FP8>::frag Frag;
+  // fp8 pool: the K scale joins the softmax scale, the V scale the final normalisation, and the
+  // step's new rows are quantised with the reciprocals
+  float k_inv = 1.0f, v_inv = 1.0f, v_scale = 1.0f;
+  if constexpr (FP8) {
+    const float ks = scales[h];
+    v_scale = scales[num_kv_heads + h];
+    scale_log2 *= ks;
+    k_inv = 1.0f / ks;
+    v_inv = 1.0f / v_scale;
+  }
+
   const int hq0 = h * group;
   const int64_t row_stride = (int64_t)2 * num_kv_heads * kHeadDim;
-  half_t *k_lane = kv + (int64_t)h * kHeadDim + 8 * g + n * row_stride;
-  half_t *v_lane = kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
+  Elem *k_lane = kv + (int64_t)h * kHeadDim + 8 * g + n * row_stride;
+  Elem *v_lane = kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
   const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
 
   // Requests past the chunk still issue their loads (16 bytes of its last page) so the number of
@@ -617,11 +652,11 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   // it needs.
   // Page ids travel through scalar loads, one request ahead of their use.
   int pid_next = 0;
-  auto request = [&](int i, PageRegs &r) {  // i = page index inside the chunk
+  auto request = [&](int i, RawPage<Frag> &r) {  // i = page index inside the chunk
     const int64_t page_off = (int64_t)pid_next * kPageSize * row_stride;
     const int nx = i + 1 < f1 - f0 ? i + 1 : f1 - f0 - 1;
     pid_next = page_ids[nx];
-    request_page(r, k_lane, v_lane, page_off, row_stride, i >= f1 - f0, kv);
+    request_page<Elem, Frag>(r, k_lane, v_lane, page_off, row_stride, i >= f1 - f0, kv);
   };
 
   HeadState st;
@@ -635,10 +670,10 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     const int64_t cell = (int64_t)(cidx + cur_b) * num_q_heads + hq0;
     half_t *out_row = out + ((int64_t)cur_b * num_q_heads + hq0) * kHeadDim;
     store_state(st, whole, out_row, part_o + cell * kHeadDim, kHeadDim, part_lse + cell, 1, n, g,
-                group);
+                group, v_scale);
   };
 
-  PageRegs buf[DEPTH];
+  RawPage<Frag> buf[DEPTH];
 #pragma unroll
   for (int dd = 0; dd < DEPTH; ++dd) {
     pid_next = first_ids[dd];
@@ -681,18 +716,25 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
           const half_t *vn = v_new + (int64_t)cur_b * v_new_stride + (int64_t)h * kHeadDim;
           const int pid = page_ids[ff - f0];
           const int64_t slot_off = ((int64_t)pid * kPageSize + t_new) * row_stride;
+          auto stored = [&](half8_t x, float inv) {  // the row as the pool holds it
+            if constexpr (FP8) {
+              return half8_to_fp8(x, inv);
+            } else {
+              return x;
+            }
+          };
           if (n == t_new) {
-            half_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 8 * g;
+            Elem *dst = kv + slot_off + (int64_t)h * kHeadDim + 8 * g;
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
-              const half8_t x = *(const half8_t *)(kn + 32 * kk + 8 * g);
+              const Frag x = stored(*(const half8_t *)(kn + 32 * kk + 8 * g), k_inv);
               buf[dd].k[kk] = x;
-              *(half8_t *)(dst + 32 * kk) = x;
+              *(Frag *)(dst + 32 * kk) = x;
             }
           }
           if (g == (t_new & 3)) {
-            const half8_t x = *(const half8_t *)(vn + 8 * n);
-            *(half8_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n) = x;
+            const Frag x = stored(*(const half8_t *)(vn + 8 * n), v_inv);
+            *(Frag *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n) = x;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               if (i == (t_new >> 2)) buf[dd].v[i] = x;
@@ -700,7 +742,11 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
           }
           wait_vector_loads();
         }
-        attend_page(st, buf[dd], qf, vstage, vt_lane, p, len_b, n, g, scale_log2);
+        if constexpr (FP8) {
+          attend_page(st, decoded(buf[dd]), qf, vstage, vt_lane, p, len_b, n, g, scale_log2);
+        } else {
+          attend_page(st, buf[dd], qf, vstage, vt_lane, p, len_b, n, g, scale_log2);
+        }
       }
       request(ff - f0 + DEPTH, buf[dd]);
     }
@@ -980,7 +1026,8 @@ extern "C" int litekv_profile_next_decode(void *start_event, void *stop_event) {
 namespace litekv {
 // The balanced decode step; with shared_pages > 0 preceded by the shared-prefix launch.
 static int launch_balanced(const char *what, const void *q, int64_t q_batch_stride, void *kv_pool,
-                           const int32_t *block_table, const int32_t *seq_lens, void *plan,
+                           const float *fp8_scales, const int32_t *block_table,
+                           const int32_t *seq_lens, void *plan,
                            size_t plan_bytes, const void *k_new, const void *v_new,
                            int64_t k_new_stride, int64_t v_new_stride, void *out, void *workspace,
                            size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
@@ -1037,18 +1084,29 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   const unsigned wgs = (unsigned)((chunks + s.replicas - 1) / s.replicas);
   hipEvent_t ev0 = g_profile_start, ev1 = g_profile_stop;
   g_profile_start = g_profile_stop = nullptr;
-  hipExtLaunchKernelGGL(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH>,
-                        dim3(wgs, (unsigned)s.head_groups),
-                        dim3((unsigned)(kWave * s.heads_per_wg * s.replicas)), 0,
-                        static_cast<hipStream_t>(stream), ev0, ev1, 0,
-                        static_cast<const half_t *>(q), q_batch_stride,
-                        static_cast<half_t *>(kv_pool), seq_lens,
-                        static_cast<const int32_t *>(plan),
-                        static_cast<const half_t *>(k_new), static_cast<const half_t *>(v_new),
-                        k_new_stride, v_new_stride, static_cast<half_t *>(out), part_o, part_lse,
-                        block_table_stride, batch, num_q_heads, num_kv_heads,
-                        num_q_heads / num_kv_heads, s.heads_per_wg, s.replicas, chunks,
-                        shared_pages, softmax_scale * kLog2e);
+  const dim3 grid(wgs, (unsigned)s.head_groups);
+  const dim3 block((unsigned)(kWave * s.heads_per_wg * s.replicas));
+  if (fp8_scales != nullptr) {
+    hipExtLaunchKernelGGL((paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, true>), grid, block, 0,
+                          static_cast<hipStream_t>(stream), ev0, ev1, 0,
+                          static_cast<const half_t *>(q), q_batch_stride,
+                          static_cast<uint8_t *>(kv_pool), fp8_scales, seq_lens,
+                          static_cast<const int32_t *>(plan), static_cast<const half_t *>(k_new),
+                          static_cast<const half_t *>(v_new), k_new_stride, v_new_stride,
+                          static_cast<half_t *>(out), part_o, part_lse, block_table_stride, batch,
+                          num_q_heads, num_kv_heads, num_q_heads / num_kv_heads, s.heads_per_wg,
+                          s.replicas, chunks, shared_pages, softmax_scale * kLog2e);
+  } else {
+    hipExtLaunchKernelGGL((paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, false>), grid, block, 0,
+                          static_cast<hipStream_t>(stream), ev0, ev1, 0,
+                          static_cast<const half_t *>(q), q_batch_stride,
+                          static_cast<half_t *>(kv_pool), fp8_scales, seq_lens,
+                          static_cast<const int32_t *>(plan), static_cast<const half_t *>(k_new),
+                          static_cast<const half_t *>(v_new), k_new_stride, v_new_stride,
+                          static_cast<half_t *>(out), part_o, part_lse, block_table_stride, batch,
+                          num_q_heads, num_kv_heads, num_q_heads / num_kv_heads, s.heads_per_wg,
+                          s.replicas, chunks, shared_pages, softmax_scale * kLog2e);
+  }
   rc = check_launch(what);
   if (rc != LITEKV_OK) return rc;
   hipLaunchKernelGGL(paged_decode_balanced_merge_kernel,
@@ -1067,8 +1125,25 @@ extern "C" int litekv_paged_decode_balanced(
     int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
     int64_t num_pages, int32_t block_table_stride, int32_t chunks, float softmax_scale,
     void *stream) {
-  return litekv::launch_balanced("paged_decode_balanced", q, q_batch_stride, kv_pool, nullptr,
+  return litekv::launch_balanced("paged_decode_balanced", q, q_batch_stride, kv_pool, nullptr, nullptr,
                                  seq_lens, plan, plan_bytes, k_new, v_new, k_new_stride,
+                                 v_new_stride, out, workspace, workspace_bytes, batch, num_q_heads,
+                                 num_kv_heads, head_dim, page_size, num_pages, block_table_stride,
+                                 chunks, 0, softmax_scale, stream);
+}
+
+extern "C" int litekv_paged_decode_balanced_fp8(
+    const void *q, int64_t q_batch_stride, void *kv_pool_fp8, const float *scales,
+    const int32_t *seq_lens, void *plan, size_t plan_bytes, const void *k_new, const void *v_new,
+    int64_t k_new_stride, int64_t v_new_stride, void *out, void *workspace, size_t workspace_bytes,
+    int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+    int64_t num_pages, int32_t block_table_stride, int32_t chunks, float softmax_scale,
+    void *stream) {
+  if (scales == nullptr && batch > 0) {
+    return litekv::fail(LITEKV_ERR_INVALID_ARGUMENT, "paged_decode_balanced_fp8: scales is null");
+  }
+  return litekv::launch_balanced("paged_decode_balanced_fp8", q, q_batch_stride, kv_pool_fp8, scales,
+                                 nullptr, seq_lens, plan, plan_bytes, k_new, v_new, k_new_stride,
                                  v_new_stride, out, workspace, workspace_bytes, batch, num_q_heads,
                                  num_kv_heads, head_dim, page_size, num_pages, block_table_stride,
                                  chunks, 0, softmax_scale, stream);
@@ -1086,7 +1161,7 @@ extern "C" int litekv_paged_decode_prefix(
     int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
     int64_t num_pages, int32_t block_table_stride, int32_t chunks, int32_t shared_pages,
     float softmax_scale, void *stream) {
-  return litekv::launch_balanced("paged_decode_prefix", q, q_batch_stride, kv_pool, block_table,
+  return litekv::launch_balanced("paged_decode_prefix", q, q_batch_stride, kv_pool, nullptr, block_table,
                                  seq_lens, plan, plan_bytes, k_new, v_new, k_new_stride,
                                  v_new_stride, out, workspace, workspace_bytes, batch, num_q_heads,
                                  num_kv_heads, head_dim, page_size, num_pages, block_table_stride,

@@ -36,6 +36,26 @@ def _dev_half(name: str, t: torch.Tensor) -> None:
     _need(t.dtype == torch.float16, f"{name} must be float16, got {t.dtype}")
 
 
+FP8_DTYPES = (torch.uint8, torch.float8_e4m3fn)
+
+
+def _dev_pool(name: str, t: torch.Tensor) -> None:
+    _need(t.is_cuda, f"{name} must live on the GPU")
+    _need(t.dtype == torch.float16 or t.dtype in FP8_DTYPES, f"{name} must be float16 or fp8, got {t.dtype}")
+
+
+def is_fp8_pool(kv_pool: torch.Tensor) -> bool:
+    """An fp8 pool holds one E4M3 code per element (a uint8 or float8_e4m3fn tensor)."""
+    return kv_pool.dtype in FP8_DTYPES
+
+
+def _dev_fp8_pool(kv_pool: torch.Tensor, scales: Optional[torch.Tensor], num_kv_heads: int) -> None:
+    _need(kv_pool.is_cuda and is_fp8_pool(kv_pool), f"kv_pool must be an fp8 (uint8 / float8_e4m3fn) GPU tensor, got {kv_pool.dtype}")
+    _need(scales is not None, "an fp8 pool needs its per-head scales")
+    _need(scales.is_cuda and scales.dtype == torch.float32 and scales.is_contiguous()
+          and scales.numel() == 2 * num_kv_heads, "scales must be float32 [2 * Hkv] on the GPU (K heads, then V heads)")
+
+
 def _dev_i32(name: str, t: torch.Tensor) -> torch.Tensor:
     _need(t.is_cuda, f"{name} must live on the GPU")
     if t.dtype != torch.int32:
@@ -71,6 +91,39 @@ def kv_append(k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor, kv_p
     lib = _lib.load()
     _lib.check(lib.litekv_kv_append(_ptr(k), _ptr(v), _rows("k", k), _rows("v", v), _ptr(slot_mapping),
                                     _ptr(kv_pool), t, hkv, d, slots, _stream()))
+
+
+def kv_append_fp8(k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor, kv_pool: torch.Tensor,
+                  scales: torch.Tensor) -> None:
+    """kv_pool[slot_mapping[t]] = e4m3(concat(k[t], v[t]) / scale of the head) for every token t;
+    scales is float32 [2 * Hkv]: K-head scales, then V-head scales."""
+    _dev_half("k", k), _dev_half("v", v)
+    slots, hkv, d, _, _ = pool_geometry(kv_pool, 1)
+    _dev_fp8_pool(kv_pool, scales, hkv)
+    _need(k.shape == v.shape and k.shape[1] == hkv and k.shape[2] == d, "k / v must be [T, Hkv, D] matching the pool")
+    slot_mapping = _dev_i32("slot_mapping", slot_mapping)
+    t = k.shape[0]
+    _need(slot_mapping.numel() == t, "slot_mapping must hold one slot per token")
+    lib = _lib.load()
+    _lib.check(lib.litekv_kv_append_fp8(_ptr(k), _ptr(v), _rows("k", k), _rows("v", v), _ptr(slot_mapping),
+                                        _ptr(kv_pool), _ptr(scales), t, hkv, d, slots, _stream()))
+
+
+def page_dequant(kv_pool: torch.Tensor, dst_pool: torch.Tensor, src_ids: torch.Tensor,
+                 dst_ids: Optional[torch.Tensor], scales: torch.Tensor, page_size: int = PAGE_SIZE) -> None:
+    """dst_pool[page dst_ids[i]] (fp16) = decoded page src_ids[i] of the fp8 pool; dst_ids None means page i."""
+    _dev_half("dst_pool", dst_pool)
+    _, hkv, d, n_src, _ = pool_geometry(kv_pool, page_size)
+    _, hkv_d, d_d, n_dst, _ = pool_geometry(dst_pool, page_size)
+    _dev_fp8_pool(kv_pool, scales, hkv)
+    _need((hkv, d) == (hkv_d, d_d), "pools differ in head geometry")
+    src_ids = _dev_i32("src_ids", src_ids)
+    if dst_ids is not None:
+        dst_ids = _dev_i32("dst_ids", dst_ids)
+        _need(dst_ids.numel() == src_ids.numel(), "src_ids and dst_ids differ in length")
+    lib = _lib.load()
+    _lib.check(lib.litekv_page_dequant(_ptr(kv_pool), _ptr(dst_pool), _ptr(src_ids), _ptr(dst_ids), src_ids.numel(),
+                                       _ptr(scales), hkv, d, page_size, n_src, n_dst, _stream()))
 
 
 def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor,
@@ -112,8 +165,10 @@ def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_
 
 def page_gather(src_pool: torch.Tensor, dst_pool: torch.Tensor, src_ids: torch.Tensor,
                 dst_ids: Optional[torch.Tensor] = None, page_size: int = PAGE_SIZE) -> None:
-    """dst_pool[page dst_ids[i]] = src_pool[page src_ids[i]]; dst_ids None means page i."""
-    _dev_half("src_pool", src_pool), _dev_half("dst_pool", dst_pool)
+    """dst_pool[page dst_ids[i]] = src_pool[page src_ids[i]]; dst_ids None means page i. Pages are
+    moved as bytes: fp16 pools or fp8 pools, both of the same kind."""
+    _dev_pool("src_pool", src_pool), _dev_pool("dst_pool", dst_pool)
+    _need(src_pool.element_size() == dst_pool.element_size(), "pools differ in element size")
     _, hs, ds, n_src, page_bytes = pool_geometry(src_pool, page_size)
     _, hd, dd, n_dst, page_bytes_d = pool_geometry(dst_pool, page_size)
     _need((hs, ds) == (hd, dd) and page_bytes == page_bytes_d, "pools differ in page geometry")
@@ -128,8 +183,8 @@ def page_gather(src_pool: torch.Tensor, dst_pool: torch.Tensor, src_ids: torch.T
 
 def page_copy(kv_pool: torch.Tensor, src_ids: torch.Tensor, dst_ids: torch.Tensor,
               page_size: int = PAGE_SIZE) -> None:
-    """kv_pool[page dst_ids[i]] = kv_pool[page src_ids[i]] (copy-on-write move inside one pool)."""
-    _dev_half("kv_pool", kv_pool)
+    """kv_pool[page dst_ids[i]] = kv_pool[page src_ids[i]] (copy-on-write move inside one pool, fp16 or fp8)."""
+    _dev_pool("kv_pool", kv_pool)
     _, _, _, n_pages, page_bytes = pool_geometry(kv_pool, page_size)
     src_ids = _dev_i32("src_ids", src_ids)
     dst_ids = _dev_i32("dst_ids", dst_ids)
@@ -262,11 +317,16 @@ def decode_advance(request_tables: torch.Tensor, request_ids: torch.Tensor, seq_
 
 def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
                 k_new: Optional[torch.Tensor] = None, v_new: Optional[torch.Tensor] = None,
-                softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
+                kv_scales: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The balanced schedule for one layer: optional append of k_new / v_new ([B, Hkv, D]) at logical
     position seq_lens[b] - 1 fused into the attention of q [B, Hq, D] over the planned pages, then the
-    merge of the sequences that span several chunks."""
-    _dev_half("q", q), _dev_half("kv_pool", kv_pool)
+    merge of the sequences that span several chunks. An fp8 pool (uint8 / float8_e4m3fn) comes with
+    its per-head ``kv_scales``."""
+    _dev_half("q", q)
+    fp8 = is_fp8_pool(kv_pool)
+    if not fp8:
+        _dev_half("kv_pool", kv_pool)
     _need(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2], "q must be [B, Hq, D] with contiguous heads")
     b, hq, d = q.shape
     _, hkv, dk, n_pages, _ = pool_geometry(kv_pool, plan.page_size)
@@ -288,6 +348,15 @@ def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
         _need(out.shape == (b, hq, d) and out.is_contiguous(), "out must be contiguous [B, Hq, D]")
     q_stride = q.stride(0) if b > 1 else max(q.stride(0), hq * d)
     lib = _lib.load()
+    if fp8:
+        _dev_fp8_pool(kv_pool, kv_scales, hkv)
+        _need(plan.shared_pages == 0, "the shared-prefix decode reads fp16 pools only")
+        _lib.check(lib.litekv_paged_decode_balanced_fp8(
+            _ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(plan.seq_lens), _ptr(plan.buffer),
+            plan.plan_bytes, _ptr(k_new), _ptr(v_new), kn_stride, vn_stride, _ptr(out), _ptr(plan.workspace),
+            plan.workspace_bytes, b, hq, hkv, d, plan.page_size, n_pages, plan.bt_stride, plan.chunks,
+            float(softmax_scale), _stream()))
+        return out
     if plan.shared_pages > 0:
         _lib.check(lib.litekv_paged_decode_prefix(
             _ptr(q), q_stride, _ptr(kv_pool), _ptr(plan.block_table), _ptr(plan.seq_lens), _ptr(plan.buffer),
@@ -312,7 +381,7 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
                  workspace: Optional[torch.Tensor] = None, page_size: int = PAGE_SIZE,
                  stage: str = "both", schedule: Optional[str] = None,
                  chunks: Optional[int] = None, plan: Optional[DecodePlan] = None,
-                 shared_pages: int = 0) -> torch.Tensor:
+                 shared_pages: int = 0, kv_scales: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Decode attention of q [B, Hq, D] over the pages named by block_table [B, max_blocks].
 
     ``shared_pages`` (balanced schedule): the first that many entries of every block-table row are
@@ -322,8 +391,11 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
     kv head (default: one workgroup per CU); a DecodePlan is built for the call unless one is
     passed. schedule "splits" (chosen when num_splits, max_splits or min_pages_per_split is
     given): every sequence is cut into its own splits; two launches (`stage` selects one).
+    An fp8 pool (with its ``kv_scales``) is read by the balanced schedule only.
     """
-    _dev_half("q", q), _dev_half("kv_pool", kv_pool)
+    _dev_half("q", q)
+    if not is_fp8_pool(kv_pool):
+        _dev_half("kv_pool", kv_pool)
     _need(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2], "q must be [B, Hq, D] with contiguous heads")
     b, hq, d = q.shape
     _, hkv, dk, n_pages, _ = pool_geometry(kv_pool, page_size)
@@ -338,8 +410,9 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
         _need(stage == "both", "the balanced schedule is a single launch")
         if plan is None:
             plan = DecodePlan(block_table, seq_lens, hq, hkv, n_pages, chunks, page_size, shared_pages)
-        return decode_step(q, kv_pool, plan, None, None, softmax_scale, out)
+        return decode_step(q, kv_pool, plan, None, None, softmax_scale, out, kv_scales)
 
+    _need(not is_fp8_pool(kv_pool), "fp8 pools are read by the balanced schedule only")
     _need(block_table.dim() == 2 and block_table.shape[0] == b, "block_table must be [B, max_blocks]")
     block_table = _dev_i32("block_table", block_table)
     seq_lens = _dev_i32("seq_lens", seq_lens)

@@ -381,3 +381,80 @@ def test_decode_advance_refusals_leave_the_length():
     assert slots.tolist() == [3 * 4 + 3, 5 * 4 + 3, -1, 4 * 4 + 0]
     assert pos.tolist() == [11, 7, 2, 0]
     assert rows[2].tolist() == [0, 0, 0]
+
+
+# ---- fp8 (E4M3FN) storage ----------------------------------------------------------------------
+
+def test_fp8_code_values_closed_form():
+    from oracle import fp8
+
+    vals = fp8.code_values()
+    assert vals[0x00] == 0.0 and vals[0x80] == 0.0 and np.signbit(vals[0x80])
+    assert vals[0x01] == 2.0 ** -9 and vals[0x07] == 7 * 2.0 ** -9          # subnormals
+    assert vals[0x08] == 2.0 ** -6 and vals[0x38] == 1.0 and vals[0x3C] == 1.5
+    assert vals[0x7E] == 448.0 and vals[0xFE] == -448.0                      # largest finite values
+    assert np.isnan(vals[0x7F]) and np.isnan(vals[0xFF])
+    finite = vals[:0x7F]
+    assert np.all(np.diff(finite) > 0)                                       # codes order like their values
+    assert np.array_equal(vals[0x80:0xFF], -finite)
+
+
+def test_fp8_encode_decode_against_torch_float8():
+    import torch
+    from oracle import fp8
+
+    # every finite fp16 value in range, as the kernels see them (fp16 -> fp32)
+    halves = np.arange(0x10000, dtype=np.uint16).view(np.float16)
+    x = halves[np.isfinite(halves) & (np.abs(halves.astype(np.float32)) <= 448.0)].astype(np.float32)
+    want = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = fp8.encode(x)
+    zero = x == 0
+    assert np.array_equal(got[~zero], want[~zero])
+    assert np.all((got[zero] & 0x7F) == 0)
+    # decode: torch's own table
+    codes = np.arange(256, dtype=np.uint8)
+    ref = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+    mine = fp8.decode(codes)
+    assert np.array_equal(np.isnan(ref), np.isnan(mine))
+    assert np.array_equal(ref[~np.isnan(ref)], mine[~np.isnan(mine)])
+
+
+def test_fp8_rounding_saturation_and_round_trip():
+    from oracle import fp8
+
+    vals = fp8.code_values()
+    finite_codes = np.array([c for c in range(256) if not np.isnan(vals[c]) and c != 0x80], dtype=np.uint8)
+    assert np.array_equal(fp8.encode(vals[finite_codes]), finite_codes)        # representable values are fixed points
+    pos = np.sort(vals[:0x7F])
+    mid = ((pos[:-1].astype(np.float64) + pos[1:].astype(np.float64)) / 2).astype(np.float32)   # exact in fp32
+    tie = fp8.encode(mid)
+    assert np.all(tie % 2 == 0)                                                # ties go to the even code
+    assert np.all((tie == np.arange(0x7E)) | (tie == np.arange(1, 0x7F)))
+    big = np.array([449.0, 1e4, 65504.0, -500.0, np.inf, -np.inf], dtype=np.float32)
+    assert fp8.encode(big).tolist() == [0x7E, 0x7E, 0x7E, 0xFE, 0x7E, 0xFE]
+    rng = np.random.default_rng(3)
+    x = rng.normal(scale=30.0, size=4096).astype(np.float32)
+    err = np.abs(fp8.decode(fp8.encode(x)) - np.clip(x, -448, 448))
+    assert np.all(err <= np.maximum(np.abs(x) * 2.0 ** -4, 2.0 ** -10))       # half a spacing of 2^-3 relative
+    assert np.all(np.diff(fp8.decode(fp8.encode(np.sort(x)))) >= 0)           # monotone
+
+
+def test_fp8_append_uses_the_head_scales():
+    from oracle import fp8
+
+    rng = np.random.default_rng(4)
+    k = rng.normal(size=(5, 2, 128)).astype(np.float16)
+    v = rng.normal(size=(5, 2, 128)).astype(np.float16)
+    scales = np.array([0.01, 0.02, 0.5, 0.004], dtype=np.float32)
+    pool = np.full((8, 4, 128), 0x55, dtype=np.uint8)
+    fp8.kv_append(k, v, np.array([3, 0, -1, 9, 7]), pool, scales)
+    assert np.all(pool[[1, 2, 4, 5, 6]] == 0x55)                               # untouched slots
+    back = fp8.dequantize_pool(pool, scales)
+    for t, slot in ((0, 3), (1, 0), (4, 7)):
+        for h in range(2):
+            want_k = np.clip(k[t, h].astype(np.float32), -448 * scales[h], 448 * scales[h])
+            assert np.all(np.abs(back[slot, h] - want_k) <= np.maximum(np.abs(want_k) * 2.0 ** -4, scales[h] * 2.0 ** -10))
+            want_v = np.clip(v[t, h].astype(np.float32), -448 * scales[2 + h], 448 * scales[2 + h])
+            assert np.all(np.abs(back[slot, 2 + h] - want_v) <= np.maximum(np.abs(want_v) * 2.0 ** -4,
+                                                                           scales[2 + h] * 2.0 ** -10))
+    assert np.all(np.abs(back[3, 3]) <= 448 * 0.004 + 1e-6)                    # a small scale saturates
