@@ -86,7 +86,8 @@ class DecodeLayerSet:
     A step = one plan launch (the cuts are shared by every layer of a decode step) + per layer one
     balanced decode call with the KV append fused in (decode kernel + merge kernel)."""
 
-    def __init__(self, case, layers: int, device: str, schedule: str = "balanced", shared_pages: int = 0):
+    def __init__(self, case, layers: int, device: str, schedule: str = "balanced", shared_pages: int = 0,
+                 kv_dtype: str = "f16"):
         import torch
         from llama_lite_npu_amd import _lib, ops
 
@@ -99,10 +100,19 @@ class DecodeLayerSet:
         c = case
         b, hq, hkv = c.batch, c.num_q_heads, c.num_kv_heads
         slots = c.num_pages * 16
-        pools = torch.empty((layers, slots, 2 * hkv, 128), dtype=torch.float16, device=device)
         gen = torch.Generator(device=device).manual_seed(4242)
-        for l in range(layers):
-            pools[l].normal_(generator=gen)
+        self.fp8 = kv_dtype == "fp8"
+        if self.fp8:
+            if schedule != "balanced" or shared_pages:
+                raise ValueError("fp8 pools are read by the balanced schedule without a shared prefix")
+            # E4M3 codes (no NaN codes) and one scale per head
+            pools = torch.randint(0, 0x7F, (layers, slots, 2 * hkv, 128), generator=gen, device=device,
+                                  dtype=torch.uint8)
+            self.scales = torch.full((2 * hkv,), 0.02, dtype=torch.float32, device=device)
+        else:
+            pools = torch.empty((layers, slots, 2 * hkv, 128), dtype=torch.float16, device=device)
+            for l in range(layers):
+                pools[l].normal_(generator=gen)
         self.pools = pools
         self.q = c.q
         self.out = torch.empty((layers, b, hq, 128), dtype=torch.float16, device=device)
@@ -139,7 +149,16 @@ class DecodeLayerSet:
                  c.num_pages, bts, self.chunks, shared_pages, c.softmax_scale, stream)
                 for l in range(layers)
             ]
-            self.plan_info = {"schedule": "balanced", "chunks": self.chunks, "shared_pages": shared_pages}
+            if self.fp8:
+                self.decode_args = [
+                    (self.q.data_ptr(), hq * 128, pools[l].data_ptr(), self.scales.data_ptr(),
+                     self.seq_lens.data_ptr(), self.plan.data_ptr(), self.plan_bytes, c.k_new.data_ptr(),
+                     c.v_new.data_ptr(), hkv * 128, hkv * 128, self.out[l].data_ptr(), self.ws.data_ptr(), ws_bytes,
+                     b, hq, hkv, 128, 16, c.num_pages, bts, self.chunks, c.softmax_scale, stream)
+                    for l in range(layers)
+                ]
+            self.plan_info = {"schedule": "balanced", "chunks": self.chunks, "shared_pages": shared_pages,
+                              "kv_dtype": kv_dtype}
         else:
             self.max_splits, self.min_pps = ops.decode_split_plan(b, hkv, self.table.shape[1], c.num_splits)
             self.ws = ops.decode_workspace(b, hq, self.max_splits, device)
@@ -169,7 +188,8 @@ class DecodeLayerSet:
             on = (lambda a: a) if stream is None else (lambda a: a[:-1] + (stream,))
             rc |= lib.litekv_decode_advance(*on(self.advance_args))
             rc |= lib.litekv_decode_plan_prefix(*on(self.plan_args))
-            dec, prof = lib.litekv_paged_decode_prefix, lib.litekv_profile_next_decode
+            dec = lib.litekv_paged_decode_balanced_fp8 if self.fp8 else lib.litekv_paged_decode_prefix
+            prof = lib.litekv_profile_next_decode
             for l in range(self.layers):
                 if events is not None:
                     prof(events[l][0], events[l][1])
@@ -201,10 +221,11 @@ class DecodeLayerSet:
 
 
 def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: str,
-               schedule: str = "balanced", shared_pages: int = 0, graph: bool = True) -> dict:
+               schedule: str = "balanced", shared_pages: int = 0, graph: bool = True,
+               kv_dtype: str = "f16") -> dict:
     import torch
 
-    ls = DecodeLayerSet(case, layers, device, schedule, shared_pages)
+    ls = DecodeLayerSet(case, layers, device, schedule, shared_pages, kv_dtype)
     for _ in range(max(1, warmup)):
         ls.step()
     torch.cuda.synchronize()
@@ -235,6 +256,11 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
     ms_per_step = wall * 1e3 / steps
     decode_bytes = case.decode_bytes()
     append_bytes = case.append_bytes()
+    if kv_dtype == "fp8":
+        # one byte per cached element: K/V traffic halves; the appended rows arrive as fp16
+        kv_read = int(case.seq_lens.sum()) * case.tok_bytes
+        decode_bytes -= kv_read // 2
+        append_bytes = case.batch * (case.tok_bytes + case.tok_bytes // 2 + 4)
     step_bytes = layers * (decode_bytes + append_bytes)
     replay = None
     if balanced and graph:
@@ -542,6 +568,8 @@ def main() -> int:
                     help="balanced schedule: pieces per kv head (default: one workgroup per compute unit)")
     ap.add_argument("--no-shared-prefix", action="store_true",
                     help="c4: read the shared prefix pages once per sequence like any other page")
+    ap.add_argument("--kv-dtype", default="f16", choices=["f16", "fp8"],
+                    help="storage of the KV pools (fp8: E4M3 codes with per-head scales; decode configs only)")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the leg that replays the decode step as one HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -590,10 +618,11 @@ def main() -> int:
         if name == "c5" and args.schedule == "balanced" and False:
             sched = "splits"
         shared = 0
-        if sched == "balanced" and not args.no_shared_prefix and not case.extra.get("private_prefix"):
+        if sched == "balanced" and not args.no_shared_prefix and not case.extra.get("private_prefix") \
+                and args.kv_dtype == "f16":
             shared = int(case.extra.get("n_shared", 0))
         return run_decode(case, layers, args.steps, args.warmup, device, case.name, sched, shared,
-                          graph=not args.no_graph), case
+                          graph=not args.no_graph, kv_dtype=args.kv_dtype), case
 
     if args.calibrate_copy:
         from llama_lite_npu_amd import ops
@@ -607,7 +636,7 @@ def main() -> int:
         torch.cuda.empty_cache()
 
     res, case = run(args.config)
-    traffic = MEASURED_TRAFFIC_BYTES.get((args.config, args.schedule))
+    traffic = MEASURED_TRAFFIC_BYTES.get((args.config, args.schedule)) if args.kv_dtype == "f16" else None
     if traffic is not None and args.config != "c3":
         res["roofline"]["traffic"] = traffic / (res["decode_kernel_us_mean"] * 1e-6) / 1e9
         res["roofline"]["traffic_bytes_per_launch"] = traffic
@@ -625,7 +654,8 @@ def main() -> int:
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": res["label"], "config": args.config, "launch": res.get("launch", "eager")},
+        "config": {"workload": res["label"], "config": args.config, "launch": res.get("launch", "eager"),
+                   "kv_dtype": args.kv_dtype},
         "roofline": res["roofline"],
         "detail": {k: v for k, v in res.items() if k not in ("roofline", "label", "value", "ms_per_step", "launch")},
     }

@@ -61,29 +61,26 @@ __host__ __device__ __forceinline__ int splits_for_pages(int pages, int max_spli
   return n < max_splits ? n : max_splits;
 }
 
-// One page as this lane requested it: Frag holds 8 elements, half8_t for an fp16 pool, a pair of
-// dwords (8 E4M3 codes) for an fp8 pool.
-template <typename Frag>
-struct RawPage {
-  Frag k[4];  // A-operand fragments of K: token n, d = 32*kk + 8*g .. +7
-  Frag v[4];  // V rows 4*i + g, 8-element column n
+// One page of an fp16 pool as this lane requested it.
+struct PageRegs {
+  half8_t k[4];  // A-operand fragments of K: token n, d = 32*kk + 8*g .. +7
+  half8_t v[4];  // V rows 4*i + g, 16-byte column n
 };
-typedef RawPage<half8_t> PageRegs;
 
-// Storage of the pool a kernel reads: element type and the 8-element fragment a lane loads.
+// One page of an fp8 pool: the same bytes per lane in half as many loads. The sum over d of a
+// dot product may run in any order as long as K and q agree, so a lane takes 16 consecutive
+// codes per load and MFMA step kk uses its lower or upper 8:
+//   k[j]: token n, d = 16*(g + 4*j) .. +15      step kk = 2*j + (0: lower, 1: upper 8 codes)
+//   v[i]: V row 8*i + 2*g + n/8, d = 16*(n%8) .. +15
+struct PageRegsFp8 {
+  uint4_t k[2];
+  uint4_t v[2];
+};
+
+// Storage of the pool a kernel reads.
 template <bool FP8> struct KvStore;
-template <> struct KvStore<false> { typedef half_t elem; typedef half8_t frag; };
-template <> struct KvStore<true> { typedef uint8_t elem; typedef uint2_t frag; };
-
-__device__ __forceinline__ PageRegs decoded(const RawPage<uint2_t> &r) {
-  PageRegs x;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    x.k[i] = fp8x8_to_half(r.k[i]);
-    x.v[i] = fp8x8_to_half(r.v[i]);
-  }
-  return x;
-}
+template <> struct KvStore<false> { typedef half_t elem; typedef PageRegs page; };
+template <> struct KvStore<true> { typedef uint8_t elem; typedef PageRegsFp8 page; };
 
 // Softmax state and output accumulator of the (up to 16) query heads of one kv head.
 // acc[j][i] is O^T[d = 16j + 4g + i][head n]; m is shared by the 4 lanes of a head, d is this
@@ -118,48 +115,70 @@ __device__ __forceinline__ void load_q(half8_t (&qf)[4], const half_t *q_row0, i
   }
 }
 
+// The same for an fp8 pool, in the d order of PageRegsFp8::k.
+__device__ __forceinline__ void load_q_fp8_order(half8_t (&qf)[4], const half_t *q_row0, int n, int g,
+                                                 int group) {
+  const half_t *qrow = q_row0 + (int64_t)n * kHeadDim + 16 * g;
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    qf[kk] = (n < group) ? *(const half8_t *)(qrow + 64 * (kk >> 1) + 8 * (kk & 1))
+                         : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  }
+}
+
 // Requests one page: k_lane / v_lane already point at this lane's row and column of page 0.
 // K/V bytes are used once per launch: the loads carry the streaming (non-temporal) hint, which
 // keeps the step metadata and q rows in L2 and measured 2 % (C2) to 7 % (C5) faster.
 // `dummy` (wavefront-uniform) marks a request past the end of the chunk, issued only to keep the
 // number of loads in flight constant: every lane then reads the same 16 bytes of the page
 // (streaming loads do not stay in L2, so re-reading the whole last page would cost HBM traffic).
-template <typename Elem, typename Frag>
-__device__ __forceinline__ void request_page(RawPage<Frag> &r, const Elem *k_lane,
-                                             const Elem *v_lane, int64_t page_off,
+__device__ __forceinline__ void request_page(PageRegs &r, const half_t *k_lane,
+                                             const half_t *v_lane, int64_t page_off,
                                              int64_t row_stride, bool dummy = false,
-                                             const Elem *pool = nullptr) {
-  const Elem *kr = dummy ? pool + page_off : k_lane + page_off;
+                                             const half_t *pool = nullptr) {
+  const half_t *kr = dummy ? pool + page_off : k_lane + page_off;
   const int64_t k_step = dummy ? 0 : 32;
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) r.k[kk] = __builtin_nontemporal_load((const Frag *)(kr + kk * k_step));
-  const Elem *vr = dummy ? pool + page_off : v_lane + page_off;
+  for (int kk = 0; kk < 4; ++kk) r.k[kk] = __builtin_nontemporal_load((const half8_t *)(kr + kk * k_step));
+  const half_t *vr = dummy ? pool + page_off : v_lane + page_off;
   const int64_t v_step = dummy ? 0 : 4 * row_stride;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) r.v[i] = __builtin_nontemporal_load((const Frag *)(vr + i * v_step));
+  for (int i = 0; i < 4; ++i) r.v[i] = __builtin_nontemporal_load((const half8_t *)(vr + i * v_step));
 }
 
-// Folds page `p` (tokens 16p .. 16p+15 of a sequence of `len` tokens) into the state.
-__device__ __forceinline__ void attend_page(HeadState &st, const PageRegs &r,
-                                            const half8_t (&qf)[4], half_t *vstage,
-                                            const half_t *vt_lane, int p, int len, int n, int g,
-                                            float scale_log2) {
+// fp8 pool: k_lane points at token n, code 16*g; v_lane at row 2*g + n/8, code 16*(n%8).
+__device__ __forceinline__ void request_page(PageRegsFp8 &r, const uint8_t *k_lane,
+                                             const uint8_t *v_lane, int64_t page_off,
+                                             int64_t row_stride, bool dummy = false,
+                                             const uint8_t *pool = nullptr) {
+  const uint8_t *kr = dummy ? pool + page_off : k_lane + page_off;
+  const int64_t k_step = dummy ? 0 : 64;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) r.k[j] = __builtin_nontemporal_load((const uint4_t *)(kr + j * k_step));
+  const uint8_t *vr = dummy ? pool + page_off : v_lane + page_off;
+  const int64_t v_step = dummy ? 0 : 8 * row_stride;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) r.v[i] = __builtin_nontemporal_load((const uint4_t *)(vr + i * v_step));
+}
+
+// Folds page `p` (tokens 16p .. 16p+15 of a sequence of `len` tokens) into the state. `kf` are
+// the page's K fragments, `stage_v(tail)` writes its V rows [16][128] into vstage (zeros for rows
+// past the sequence end when `tail`).
+template <typename StageV>
+__device__ __forceinline__ void attend_core(HeadState &st, const half8_t (&kf)[4],
+                                            const half8_t (&qf)[4], const half_t *vt_lane, int p,
+                                            int len, int n, int g, float scale_log2,
+                                            StageV stage_v) {
   const bool tail = (p + 1) * kPageSize > len;  // wavefront-uniform: last, partly filled page
   wave_lds_fence();
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    half8_t x = r.v[i];
-    // Slots past the sequence end hold arbitrary bits: keep them out of the MFMA.
-    if (tail && p * kPageSize + 4 * i + g >= len) x = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    *(half8_t *)(&vstage[(4 * i + g) * kVPitch + 8 * n]) = x;
-  }
+  stage_v(tail);
   wave_lds_fence();
 
   // two accumulators: the dependent MFMA chain is two deep instead of four
-  float4_t s = mfma_16x16x32(r.k[0], qf[0], float4_t{0.f, 0.f, 0.f, 0.f});
-  float4_t s1 = mfma_16x16x32(r.k[2], qf[2], float4_t{0.f, 0.f, 0.f, 0.f});
-  s = mfma_16x16x32(r.k[1], qf[1], s);
-  s1 = mfma_16x16x32(r.k[3], qf[3], s1);
+  float4_t s = mfma_16x16x32(kf[0], qf[0], float4_t{0.f, 0.f, 0.f, 0.f});
+  float4_t s1 = mfma_16x16x32(kf[2], qf[2], float4_t{0.f, 0.f, 0.f, 0.f});
+  s = mfma_16x16x32(kf[1], qf[1], s);
+  s1 = mfma_16x16x32(kf[3], qf[3], s1);
 
   float sv[4];
 #pragma unroll
@@ -201,6 +220,48 @@ __device__ __forceinline__ void attend_page(HeadState &st, const PageRegs &r,
                      (__attribute__((address_space(3))) short4_t *)(vt_lane + 16 * j)));
     st.acc[j] = mfma_16x16x16(vt, pt, st.acc[j]);
   }
+}
+
+
+__device__ __forceinline__ void attend_page(HeadState &st, const PageRegs &r,
+                                            const half8_t (&qf)[4], half_t *vstage,
+                                            const half_t *vt_lane, int p, int len, int n, int g,
+                                            float scale_log2) {
+  attend_core(st, r.k, qf, vt_lane, p, len, n, g, scale_log2, [&](bool tail) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      half8_t x = r.v[i];
+      // Slots past the sequence end hold arbitrary bits: keep them out of the MFMA.
+      if (tail && p * kPageSize + 4 * i + g >= len) x = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      *(half8_t *)(&vstage[(4 * i + g) * kVPitch + 8 * n]) = x;
+    }
+  });
+}
+
+// The fp8 page: codes become fp16 exactly (the head's scales are applied by the caller).
+__device__ __forceinline__ void attend_page(HeadState &st, const PageRegsFp8 &r,
+                                            const half8_t (&qf)[4], half_t *vstage,
+                                            const half_t *vt_lane, int p, int len, int n, int g,
+                                            float scale_log2) {
+  const half8_t kf[4] = {fp8x8_to_half(uint2_t{r.k[0][0], r.k[0][1]}),
+                         fp8x8_to_half(uint2_t{r.k[0][2], r.k[0][3]}),
+                         fp8x8_to_half(uint2_t{r.k[1][0], r.k[1][1]}),
+                         fp8x8_to_half(uint2_t{r.k[1][2], r.k[1][3]})};
+  attend_core(st, kf, qf, vt_lane, p, len, n, g, scale_log2, [&](bool tail) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row = 8 * i + 2 * g + (n >> 3);
+      half8_t lo = fp8x8_to_half(uint2_t{r.v[i][0], r.v[i][1]});
+      half8_t hi = fp8x8_to_half(uint2_t{r.v[i][2], r.v[i][3]});
+      if (tail && p * kPageSize + row >= len) {
+        lo = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        hi = lo;
+      }
+      half_t *dst = &vstage[row * kVPitch + 16 * (n & 7)];
+      *(half8_t *)dst = lo;
+      *(half8_t *)(dst + 8) = hi;
+    }
+  });
 }
 
 // Writes the normalised state either as the final fp16 row or as an fp32 partial + log-sum-exp.
@@ -629,7 +690,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   int len_after = (cur_b + 1 < batch) ? lens[cur_b + 1] : 0;  // read ahead for the crossing
 
   typedef typename KvStore<FP8>::elem Elem;
-  typedef typename KvStore<FP8>::frag Frag;
+  typedef typename KvStore<FP8>::page Page;
   // fp8 pool: the K scale joins the softmax scale, the V scale the final normalisation, and the
   // step's new rows are quantised with the reciprocals
   float k_inv = 1.0f, v_inv = 1.0f, v_scale = 1.0f;
@@ -643,26 +704,37 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
 
   const int hq0 = h * group;
   const int64_t row_stride = (int64_t)2 * num_kv_heads * kHeadDim;
-  Elem *k_lane = kv + (int64_t)h * kHeadDim + 8 * g + n * row_stride;
-  Elem *v_lane = kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
+  // this lane's row and column inside page 0 (see PageRegs / PageRegsFp8)
+  Elem *k_lane = kv + (int64_t)h * kHeadDim + (FP8 ? 16 : 8) * g + n * row_stride;
+  Elem *v_lane = FP8 ? kv + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7) +
+                           (2 * g + (n >> 3)) * row_stride
+                     : kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
   const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
+  half8_t qf[4];
+  auto fetch_q = [&](int b) {
+    const half_t *row0 = q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHeadDim;
+    if constexpr (FP8) {
+      load_q_fp8_order(qf, row0, n, g, group);
+    } else {
+      load_q(qf, row0, n, g, group);
+    }
+  };
 
   // Requests past the chunk still issue their loads (16 bytes of its last page) so the number of
   // vector loads in flight stays a compile-time constant and every wait names exactly the page
   // it needs.
   // Page ids travel through scalar loads, one request ahead of their use.
   int pid_next = 0;
-  auto request = [&](int i, RawPage<Frag> &r) {  // i = page index inside the chunk
+  auto request = [&](int i, Page &r) {  // i = page index inside the chunk
     const int64_t page_off = (int64_t)pid_next * kPageSize * row_stride;
     const int nx = i + 1 < f1 - f0 ? i + 1 : f1 - f0 - 1;
     pid_next = page_ids[nx];
-    request_page<Elem, Frag>(r, k_lane, v_lane, page_off, row_stride, i >= f1 - f0, kv);
+    request_page(r, k_lane, v_lane, page_off, row_stride, i >= f1 - f0, kv);
   };
 
   HeadState st;
   st.reset();
-  half8_t qf[4];
-  load_q(qf, q + (int64_t)cur_b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
+  fetch_q(cur_b);
 
   auto flush = [&]() {
     // the sequence lies inside this chunk and has no shared-prefix partials to merge with
@@ -673,7 +745,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
                 group, v_scale);
   };
 
-  RawPage<Frag> buf[DEPTH];
+  Page buf[DEPTH];
 #pragma unroll
   for (int dd = 0; dd < DEPTH; ++dd) {
     pid_next = first_ids[dd];
@@ -702,7 +774,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
             cu_lo = cu_hi;
             cu_hi += pg;
           } while (ff >= cu_hi);
-          load_q(qf, q + (int64_t)cur_b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
+          fetch_q(cur_b);
           st.reset();
           wait_vector_loads();
         }
@@ -716,37 +788,51 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
           const half_t *vn = v_new + (int64_t)cur_b * v_new_stride + (int64_t)h * kHeadDim;
           const int pid = page_ids[ff - f0];
           const int64_t slot_off = ((int64_t)pid * kPageSize + t_new) * row_stride;
-          auto stored = [&](half8_t x, float inv) {  // the row as the pool holds it
-            if constexpr (FP8) {
-              return half8_to_fp8(x, inv);
-            } else {
-              return x;
-            }
-          };
-          if (n == t_new) {
-            Elem *dst = kv + slot_off + (int64_t)h * kHeadDim + 8 * g;
+          if constexpr (FP8) {
+            // the rows are quantised as the append kernel would, stored, and attended as stored
+            if (n == t_new) {
+              uint8_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 16 * g;
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-              const Frag x = stored(*(const half8_t *)(kn + 32 * kk + 8 * g), k_inv);
-              buf[dd].k[kk] = x;
-              *(Frag *)(dst + 32 * kk) = x;
+              for (int j = 0; j < 2; ++j) {
+                const uint2_t lo = half8_to_fp8(*(const half8_t *)(kn + 64 * j + 16 * g), k_inv);
+                const uint2_t hi = half8_to_fp8(*(const half8_t *)(kn + 64 * j + 16 * g + 8), k_inv);
+                const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
+                buf[dd].k[j] = x;
+                *(uint4_t *)(dst + 64 * j) = x;
+              }
             }
-          }
-          if (g == (t_new & 3)) {
-            const Frag x = stored(*(const half8_t *)(vn + 8 * n), v_inv);
-            *(Frag *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n) = x;
+            if (2 * g + (n >> 3) == (t_new & 7)) {
+              const uint2_t lo = half8_to_fp8(*(const half8_t *)(vn + 16 * (n & 7)), v_inv);
+              const uint2_t hi = half8_to_fp8(*(const half8_t *)(vn + 16 * (n & 7) + 8), v_inv);
+              const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
+              *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7)) = x;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              if (i == (t_new >> 2)) buf[dd].v[i] = x;
+              for (int i = 0; i < 2; ++i) {
+                if (i == (t_new >> 3)) buf[dd].v[i] = x;
+              }
+            }
+          } else {
+            if (n == t_new) {
+              half_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 8 * g;
+#pragma unroll
+              for (int kk = 0; kk < 4; ++kk) {
+                const half8_t x = *(const half8_t *)(kn + 32 * kk + 8 * g);
+                buf[dd].k[kk] = x;
+                *(half8_t *)(dst + 32 * kk) = x;
+              }
+            }
+            if (g == (t_new & 3)) {
+              const half8_t x = *(const half8_t *)(vn + 8 * n);
+              *(half8_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n) = x;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                if (i == (t_new >> 2)) buf[dd].v[i] = x;
+              }
             }
           }
           wait_vector_loads();
         }
-        if constexpr (FP8) {
-          attend_page(st, decoded(buf[dd]), qf, vstage, vt_lane, p, len_b, n, g, scale_log2);
-        } else {
-          attend_page(st, buf[dd], qf, vstage, vt_lane, p, len_b, n, g, scale_log2);
-        }
+        attend_page(st, buf[dd], qf, vstage, vt_lane, p, len_b, n, g, scale_log2);
       }
       request(ff - f0 + DEPTH, buf[dd]);
     }

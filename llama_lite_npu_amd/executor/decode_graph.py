@@ -241,6 +241,7 @@ class _CapturedGraph:
     seq_lens_i32: Optional[torch.Tensor] = None
     block_table: Optional[torch.Tensor] = None
     device_decode: Optional[DeviceDecodeBatch] = None
+    static_info: Any = None     # keeps everything the graph reads or writes alive (the step's plan and workspace too)
 
 
 class DecodeGraphRunner:
@@ -354,7 +355,8 @@ class DecodeGraphRunner:
                 cur_select_index=static_info.cur_select_index, b_seq_len=static_info.b_seq_len,
                 b_req_idx=getattr(static_info, "b_req_idx", None),
                 seq_lens_i32=getattr(static_info, "seq_lens_i32", None),
-                block_table=getattr(static_info, "block_table", None), device_decode=device)
+                block_table=getattr(static_info, "block_table", None), device_decode=device,
+                static_info=static_info)
             self.capture_count += 1
             logger.info("Captured decode graph for model=%s batch=%d bucket=%d", self.model_type, key[0], key[1])
             return True
