@@ -9,7 +9,10 @@ arguments, driven by the same ``AttentionInfo``. Differences:
 * prefill reads K/V through the block table (context 0 for a fresh prompt, history for later
   chunks), so one kernel serves both branches of the reference;
 * ``qkv_epilogue`` folds the step before the append (QK RMSNorm, rotary embedding,
-  qwen3.py:124-129) into the append itself; the forward calls are then made with ``xk=None``.
+  qwen3.py:124-129) into the append itself; the forward calls are then made with ``xk=None``;
+* a layer whose pool holds fp8 codes (``atten_info.kv_scales[layer]`` set) quantises on append
+  and decodes straight from the codes; prefill over cached history first turns the batch's
+  pages into a scratch fp16 pool, fresh prompts attend to their own fp16 K/V.
 
 ``qk_scale`` follows the reference's convention (qwen3.py:295-298): the natural 1/sqrt(D) for
 decode, multiplied by log2(e) for prefill; it is un-folded here.
@@ -40,21 +43,53 @@ class Attention:
         positions, and k / v written into their slots. xq is updated in place and returned; call
         ``context_forward`` / ``token_forward`` afterwards with ``xk=None, xv=None``."""
         cos, sin = position_embeddings if position_embeddings is not None else (None, None)
-        return ops.qk_norm_rope_append(xq, xk, xv, atten_info.cur_select_index,
-                                       atten_info.kv_buffer[layer_index], q_norm_weight, k_norm_weight,
-                                       cos, sin, rms_eps)
+        pool = atten_info.kv_buffer[layer_index]
+        if not ops.is_fp8_pool(pool):
+            return ops.qk_norm_rope_append(xq, xk, xv, atten_info.cur_select_index, pool, q_norm_weight,
+                                           k_norm_weight, cos, sin, rms_eps)
+        # fp8 pool: the epilogue writes its rows into a scratch fp16 row per token, which is then quantised
+        t = xq.shape[0]
+        rows = torch.empty((t, 2 * self.num_kv_heads, self.head_dim), dtype=torch.float16, device=xq.device)
+        ops.qk_norm_rope_append(xq, xk, xv, torch.arange(t, dtype=torch.int32, device=xq.device), rows,
+                                q_norm_weight, k_norm_weight, cos, sin, rms_eps)
+        ops.kv_append_fp8(rows[:, :self.num_kv_heads], rows[:, self.num_kv_heads:], atten_info.cur_select_index,
+                          pool, atten_info.kv_scales[layer_index])
+        return xq
 
     def context_forward(self, xq, xk, xv, atten_info, layer_index: int, qk_scale=None) -> torch.Tensor:
         """Prefill: xq [T, Hq, D], xk / xv [T, Hkv, D] packed rows of the batch's prompts or chunks
         (None when ``qkv_epilogue`` already stored them)."""
         pool = atten_info.kv_buffer[layer_index]
+        scale = (1.0 / math.sqrt(self.head_dim)) if qk_scale is None else float(qk_scale) / LOG2E
+        if ops.is_fp8_pool(pool):
+            return self._context_forward_fp8(xq, xk, xv, atten_info, pool, atten_info.kv_scales[layer_index], scale)
         if xk is not None:
             ops.kv_append(xk, xv, atten_info.cur_select_index, pool)
-        scale = (1.0 / math.sqrt(self.head_dim)) if qk_scale is None else float(qk_scale) / LOG2E
         if getattr(atten_info, "is_paged_chunk_prefill", False):
             return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens,
                                      atten_info.context_lens_i32, int(atten_info.max_actual_q_seq_len), scale)
         return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens, None,
+                                 int(atten_info.max_actual_seq_len), scale)
+
+    def _context_forward_fp8(self, xq, xk, xv, atten_info, pool, scales, scale) -> torch.Tensor:
+        chunked = getattr(atten_info, "is_paged_chunk_prefill", False)
+        if xk is not None:
+            ops.kv_append_fp8(xk, xv, atten_info.cur_select_index, pool, scales)
+            if not chunked:
+                # a fresh prompt attends to its own K/V as computed, not as stored
+                return ops.varlen_prefill(xq, xk, xv, atten_info.b_start_loc, atten_info.seq_lens_i32,
+                                          int(atten_info.max_actual_seq_len), scale)
+        # history (or rows already stored by the epilogue): decode the batch's pages into a scratch pool
+        table = atten_info.block_table
+        b, width = table.shape
+        scratch = torch.empty((b * width * ops.PAGE_SIZE, 2 * self.num_kv_heads, self.head_dim),
+                              dtype=torch.float16, device=xq.device)
+        ops.page_dequant(pool, scratch, table.reshape(-1), None, scales)
+        local = torch.arange(b * width, dtype=torch.int32, device=xq.device).view(b, width)
+        if chunked:
+            return ops.paged_prefill(xq, scratch, local, atten_info.cu_q_lens, atten_info.context_lens_i32,
+                                     int(atten_info.max_actual_q_seq_len), scale)
+        return ops.paged_prefill(xq, scratch, local, atten_info.cu_q_lens, None,
                                  int(atten_info.max_actual_seq_len), scale)
 
     def token_forward(self, xq, xk, xv, atten_info, layer_index: int, qk_scale=None) -> torch.Tensor:
@@ -63,8 +98,12 @@ class Attention:
         pool = atten_info.kv_buffer[layer_index]
         scale = (1.0 / math.sqrt(self.head_dim)) if qk_scale is None else float(qk_scale)
         plan = getattr(atten_info, "decode_plan", None)
+        scales = atten_info.kv_scales[layer_index] if ops.is_fp8_pool(pool) else None
         if plan is not None:
-            return ops.decode_step(xq, pool, plan, xk, xv, scale)
+            return ops.decode_step(xq, pool, plan, xk, xv, scale, kv_scales=scales)
         if xk is not None:
-            ops.kv_append(xk, xv, atten_info.cur_select_index, pool)
-        return ops.paged_decode(xq, pool, atten_info.block_table, atten_info.seq_lens_i32, scale)
+            if scales is not None:
+                ops.kv_append_fp8(xk, xv, atten_info.cur_select_index, pool, scales)
+            else:
+                ops.kv_append(xk, xv, atten_info.cur_select_index, pool)
+        return ops.paged_decode(xq, pool, atten_info.block_table, atten_info.seq_lens_i32, scale, kv_scales=scales)

@@ -16,7 +16,8 @@ import torch
 
 @dataclass
 class AttentionInfo:
-    kv_buffer: list = field(default_factory=list)        # per layer [slots, 2*Hkv, D] fp16 pool
+    kv_buffer: list = field(default_factory=list)        # per layer [slots, 2*Hkv, D] pool (fp16, or E4M3 codes)
+    kv_scales: list = field(default_factory=list)        # per layer float32 [2*Hkv] scales of an fp8 pool, else None
     cur_select_index: Optional[torch.Tensor] = None      # slot mapping of the step's new tokens (int32)
     b_req_tokens_table: Any = None                       # per-token slot table, or None (built on demand)
     b_start_loc: Optional[torch.Tensor] = None           # packed-row start of each sequence (int32)

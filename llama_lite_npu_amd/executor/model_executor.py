@@ -51,6 +51,7 @@ class ModelExecutor:
                                                         self.kv_mem_manager, device=device)
         self.atten_info = AttentionInfo()
         self.atten_info.kv_buffer = self.kv_mem_manager.gpu_kv_buffer
+        self.atten_info.kv_scales = self.kv_mem_manager.kv_scales
         self.build_decode_plans = build_decode_plans and torch.device(device).type == "cuda"
         self.shared_prefix_min_pages = 4  # below that the two extra launches cost more than they save
         self._decode_plan = None
@@ -325,6 +326,8 @@ class ModelExecutor:
         """Leading pages the decode step attends once for the whole batch (prefix-cache hits map one
         page list into many requests, :547-620). 0 when the batch shares fewer than
         ``shared_prefix_min_pages`` pages."""
+        if self.kv_mem_manager.is_fp8:
+            return 0             # the shared-prefix kernel reads fp16 pools
         n = self.common_leading_pages(request_ids, upcoming_tokens)
         return n if n >= self.shared_prefix_min_pages else 0
 

@@ -36,7 +36,10 @@ class PagedKVCacheManager:
     """Fixed pool of ``num_pages`` KV pages of ``page_size`` tokens, reference counted.
 
     ``gpu_kv_buffer[l]`` is layer l's pool ``[num_pages * page_size, 2 * num_kv_heads,
-    head_dim]``: K heads first, then V heads (reference :54-62).
+    head_dim]``: K heads first, then V heads (reference :54-62). With ``dtype``
+    ``torch.float8_e4m3fn`` (or ``torch.uint8``) the pools hold E4M3 codes and
+    ``kv_scales[l]`` (float32 ``[2 * num_kv_heads]``, K heads then V heads, 1.0 until
+    ``set_kv_scales``) the per-head scales; for fp16 pools ``kv_scales[l]`` is None.
     """
 
     def __init__(self, num_layers: int, num_kv_heads: int, head_dim: int, num_pages: int,
@@ -54,6 +57,11 @@ class PagedKVCacheManager:
             torch.empty((self.max_tokens, 2 * self.num_kv_heads, self.head_dim), dtype=dtype, device=device)
             for _ in range(self.num_layers)
         ]
+        self.is_fp8 = dtype in (torch.uint8, torch.float8_e4m3fn)
+        self.kv_scales = [
+            torch.ones(2 * self.num_kv_heads, dtype=torch.float32, device=device) if self.is_fp8 else None
+            for _ in range(self.num_layers)
+        ]
         self._refcount = np.zeros(self.num_pages, dtype=np.int32)
         self._free_mask = np.ones(self.num_pages, dtype=np.bool_)
         # host views with the reference's attribute names (shared memory with the arrays above)
@@ -61,6 +69,16 @@ class PagedKVCacheManager:
         self.page_free = torch.from_numpy(self._free_mask)
         self._heap = list(range(self.num_pages))
         self.num_free_pages = self.num_pages
+
+    def set_kv_scales(self, layer: int, k_scales, v_scales) -> None:
+        """Per-head scales of an fp8 layer (value = code * scale); set them before anything is cached."""
+        if not self.is_fp8:
+            raise ValueError("fp16 pools have no scales")
+        both = torch.cat([torch.as_tensor(k_scales, dtype=torch.float32).reshape(-1),
+                          torch.as_tensor(v_scales, dtype=torch.float32).reshape(-1)])
+        if both.numel() != 2 * self.num_kv_heads or not bool((both > 0).all()):
+            raise ValueError("need one positive scale per K head and per V head")
+        self.kv_scales[layer].copy_(both)
 
     # ---- allocation ------------------------------------------------------------------------
     def pages_for(self, num_tokens: int) -> int:

@@ -197,3 +197,136 @@ def test_argument_checks():
         ops.paged_decode(q, pool, table, seq_lens, SCALE, kv_scales=scales, num_splits=2)
     with pytest.raises(ValueError, match="fp8"):
         ops.kv_append_fp8(q[:, :2], q[:, :2], seq_lens, pool.half(), scales)
+
+
+# ---- the executor and the attention layer on fp8 pools ------------------------------------------
+
+def _fp8_executor(layers=2, hq=16, hkv=8, num_pages=96):
+    from llama_lite_npu_amd.executor import ModelExecutor
+
+    ex = ModelExecutor(num_layers=layers, num_q_heads=hq, num_kv_heads=hkv, head_dim=D, num_pages=num_pages,
+                       max_seq_len=512, max_requests=8, device=DEV, dtype=torch.float8_e4m3fn)
+    for layer, pool in enumerate(ex.kv_mem_manager.gpu_kv_buffer):
+        pool.view(torch.uint8).fill_(0x55)
+        ex.kv_mem_manager.set_kv_scales(layer, [0.02 + 0.001 * h for h in range(hkv)],
+                                        [0.015 + 0.002 * h for h in range(hkv)])
+    return ex
+
+
+def _rows(tokens, heads, seed):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    return torch.randn((tokens, heads, D), generator=g, device=DEV, dtype=torch.float16)
+
+
+def _decoded_pool(ex, layer):
+    pool = ex.kv_mem_manager.gpu_kv_buffer[layer].view(torch.uint8).cpu().numpy()
+    return torch.from_numpy(fp8.dequantize_pool(pool, ex.kv_mem_manager.kv_scales[layer].cpu().numpy()))
+
+
+def test_executor_flow_on_fp8_pools():
+    print("fp8: executor prefill / chunked prefill / decode / compaction", flush=True)
+    from llama_lite_npu_amd.attention import Attention
+    from oracle import c_oracle
+    from tests.parity import to_np16
+
+    hq, hkv = 16, 8
+    ex = _fp8_executor(hq=hq, hkv=hkv)
+    assert ex.kv_mem_manager.is_fp8 and ex.atten_info.kv_scales[0] is not None
+    attn = Attention(hq, hkv, D)
+    log2e = 1.4426950408889634
+    lens = [37, 16, 90, 5]
+    ids = ex.reserve_paged_requests(lens)
+    ex.activate_paged_packed_prefill_batch(ids, lens)
+    info = ex.atten_info
+    for layer in range(2):
+        q, k, v = _rows(sum(lens), hq, 10 + layer), _rows(sum(lens), hkv, 20 + layer), _rows(sum(lens), hkv, 30 + layer)
+        out = attn.context_forward(q, k, v, info, layer, SCALE * log2e)
+        torch.cuda.synchronize()
+        # a fresh prompt attends to its own fp16 K/V ...
+        ref = c_oracle.varlen_prefill(to_np16(q), to_np16(k), to_np16(v), info.b_start_loc.cpu().numpy(),
+                                      np.asarray(lens, dtype=np.int32), SCALE)
+        assert_attention_close(out, ref, f"fp8 pool, fresh prefill, layer {layer}")
+        # ... and what went into the pages are the oracle's codes
+        scales = ex.kv_mem_manager.kv_scales[layer].cpu().numpy()
+        want = np.concatenate([fp8.quantize_rows(to_np16(k), scales[:hkv]), fp8.quantize_rows(to_np16(v), scales[hkv:])], axis=1)
+        got = ex.kv_mem_manager.gpu_kv_buffer[layer].view(torch.uint8)[info.cur_select_index.long()].cpu().numpy()
+        same = (got == want) | (((got & 0x7F) == 0) & ((want & 0x7F) == 0))
+        assert same.all()
+    # a later chunk of request 3 attends to cached (quantised) history through the scratch pool
+    ex.ensure_paged_request_capacity(ids[3], 5 + 40)
+    ex.activate_paged_chunk_prefill_batch((ids[3],), [5], [30])
+    info = ex.atten_info
+    q, k, v = _rows(30, hq, 41), _rows(30, hkv, 42), _rows(30, hkv, 43)
+    out = attn.context_forward(q, k, v, info, 0, SCALE * log2e)
+    torch.cuda.synchronize()
+    ref = cpu_ref.paged_prefill_ref(q.cpu(), _decoded_pool(ex, 0), info.block_table.cpu(), info.cu_q_lens.cpu(),
+                                    info.context_lens_i32.cpu(), SCALE).numpy()
+    assert_attention_close(out, ref, "fp8 pool, chunk over cached history")
+    # layer 1 has to see the chunk too before the requests decode together
+    attn.context_forward(_rows(30, hq, 44), _rows(30, hkv, 45), _rows(30, hkv, 46), info, 1, SCALE * log2e)
+    for step in range(18):
+        ex.extend_paged_requests(ids)
+        info = ex.atten_info
+        assert info.decode_plan is not None and info.decode_plan.shared_pages == 0
+        for layer in range(2):
+            q, k, v = _rows(4, hq, 100 + 2 * step + layer), _rows(4, hkv, 200 + 2 * step + layer), _rows(4, hkv, 300 + step)
+            out = attn.token_forward(q, k, v, info, layer, SCALE)
+            torch.cuda.synchronize()
+            ref = cpu_ref.paged_decode_ref(q.cpu(), _decoded_pool(ex, layer), info.block_table.cpu(),
+                                           info.seq_lens_i32.cpu(), SCALE).numpy()
+            assert_attention_close(out, ref, f"fp8 decode step {step} layer {layer}")
+    # pages of an fp8 pool move like any others: free a request, compact, same answers bit for bit
+    q = _rows(3, hq, 999)
+    ex.release_paged_request_ids((ids[1],))
+    keep = (ids[0], ids[2], ids[3])
+    ex.activate_paged_decode_batch(keep)
+    before = attn.token_forward(q, None, None, ex.atten_info, 0, SCALE).clone()
+    moves = ex.compact_kv_pool()
+    assert moves
+    ex.activate_paged_decode_batch(keep)
+    after = attn.token_forward(q, None, None, ex.atten_info, 0, SCALE)
+    torch.cuda.synchronize()
+    assert torch.equal(before, after)
+
+
+def test_fp8_decode_steps_replay_as_graphs():
+    print("fp8: device metadata + graph replay vs eager", flush=True)
+    from tests import test_gpu_decode_graph as dg
+
+    def build():
+        from llama_lite_npu_amd.executor import ModelExecutor
+
+        ex = ModelExecutor(num_layers=dg.LAYERS, num_q_heads=dg.HQ, num_kv_heads=dg.HKV, head_dim=D, num_pages=160,
+                           max_seq_len=256, max_requests=8, device=DEV, dtype=torch.float8_e4m3fn)
+        for layer, pool in enumerate(ex.kv_mem_manager.gpu_kv_buffer):
+            pool.view(torch.uint8).fill_(0x31)
+            ex.kv_mem_manager.set_kv_scales(layer, [0.03] * dg.HKV, [0.02] * dg.HKV)
+        return ex
+
+    def prefill(ex, lens, seed):
+        ids = ex.reserve_paged_requests(lens)
+        ex.activate_paged_packed_prefill_batch(ids, lens)
+        for layer in range(dg.LAYERS):
+            ops.kv_append_fp8(_rows(sum(lens), dg.HKV, seed + layer), _rows(sum(lens), dg.HKV, seed + 50 + layer),
+                              ex.atten_info.cur_select_index, ex.atten_info.kv_buffer[layer],
+                              ex.atten_info.kv_scales[layer])
+        return ids
+
+    host, dev = build(), build()
+    model_h, model_d = dg.TinyModel(), dg.TinyModel()
+    lens = [1, 17, 48, 100, 31]
+    ids_h, ids_d = prefill(host, lens, 7), prefill(dev, lens, 7)
+    dev.attach_model(model_d, "qwen3")
+    batch = dev.activate_device_decode_batch(ids_d, reserve_tokens=8)
+    tok_h = tok_d = torch.arange(len(lens), device=DEV).reshape(-1, 1) % dg.VOCAB
+    for step in range(20):
+        out_h = dg._host_step(host, model_h, ids_h, tok_h)
+        dev.extend_paged_requests(ids_d)
+        out_d = dev.forward(tok_d)
+        torch.cuda.synchronize()
+        assert torch.equal(out_h, out_d), f"step {step}"
+        tok_h, tok_d = dg._next_tokens(out_h), dg._next_tokens(out_d)
+    assert dev.graph_runner.replay_count == 19 and dev.graph_runner.fallback_count == 0
+    batch.check()
+    for a, b in zip(host.kv_mem_manager.gpu_kv_buffer, dev.kv_mem_manager.gpu_kv_buffer):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
