@@ -37,7 +37,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 # HBM bytes per launch of the decode kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by a 1 GiB
 # copy kernel); summary and commands in profiles/paged_decode_balanced_c2_pmc.txt. Only meaningful for
 # the workload it was measured on.
-MEASURED_TRAFFIC_BYTES = {("c2", "balanced"): 317.9e6}
+MEASURED_TRAFFIC_BYTES = {("c2", "balanced", "f16"): 317.9e6, ("c2", "balanced", "fp8"): 164.5e6}
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 
 
@@ -636,7 +636,7 @@ def main() -> int:
         torch.cuda.empty_cache()
 
     res, case = run(args.config)
-    traffic = MEASURED_TRAFFIC_BYTES.get((args.config, args.schedule)) if args.kv_dtype == "f16" else None
+    traffic = MEASURED_TRAFFIC_BYTES.get((args.config, args.schedule, args.kv_dtype))
     if traffic is not None and args.config != "c3":
         res["roofline"]["traffic"] = traffic / (res["decode_kernel_us_mean"] * 1e-6) / 1e9
         res["roofline"]["traffic_bytes_per_launch"] = traffic
