@@ -396,6 +396,38 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_
                                           const float *__restrict__ po2, int64_t po2_stride, int n2,
                                           half_t *out_row, int lane) {
   const int n_parts = TWO_RUNS ? n1 + n2 : n1;
+  if (!TWO_RUNS && n1 <= 16) {
+    // The usual case (a sequence spans a few chunks): every row and the log-sum-exps are
+    // requested at once, so the launch waits for one round trip to memory instead of one per
+    // group of rows. Same weights and the same order of additions as the general path below.
+    float2 r[16];
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      r[s] = float2{0.f, 0.f};
+      if (s < n1) r[s] = *(const float2 *)(po1 + (int64_t)s * po1_stride + 2 * lane);
+    }
+    const float l = lane < n1 ? lse1[(int64_t)lane * lse1_stride] : -INFINITY;
+    float mx = l;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, xor_lane(mx, off));
+    const float w = fast_exp2((l - mx) * kLog2e);
+    float den = w;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) den += xor_lane(den, off);
+    float num0 = 0.f, num1 = 0.f;
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      if (s < n1) {
+        const float ws = __shfl(w, s, kWave);
+        num0 += ws * r[s].x;
+        num1 += ws * r[s].y;
+      }
+    }
+    const float inv = 1.0f / den;
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    *(half2_t *)(out_row + 2 * lane) = half2_t{(half_t)(num0 * inv), (half_t)(num1 * inv)};
+    return;
+  }
   auto lse_of = [&](int s) {
     if (!TWO_RUNS || s < n1) return lse1[(int64_t)s * lse1_stride];
     return lse2[(int64_t)(s - n1) * lse2_stride];
