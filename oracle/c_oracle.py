@@ -7,7 +7,7 @@ boundary); attention results come back as unrounded float32.
 from __future__ import annotations
 
 import ctypes
-from ctypes import POINTER, c_float, c_int, c_int32, c_int64, c_uint16, c_void_p
+from ctypes import c_float, c_int, c_int64, c_uint16, c_void_p
 
 import numpy as np
 

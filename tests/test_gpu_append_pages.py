@@ -6,7 +6,7 @@ import torch
 
 from llama_lite_npu_amd import ops, workloads
 from oracle import c_oracle, cpu_ref
-from tests.parity import assert_bit_exact, to_np16
+from tests.parity import assert_bit_exact
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"

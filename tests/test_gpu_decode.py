@@ -1,6 +1,5 @@
 """GPU parity of paged flash-decoding against the CPU oracle, through the C ABI."""
 
-import numpy as np
 import pytest
 import torch
 

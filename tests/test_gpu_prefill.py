@@ -1,6 +1,5 @@
 """GPU parity of varlen causal prefill (paged and packed) against the CPU oracle."""
 
-import numpy as np
 import pytest
 import torch
 

@@ -3,7 +3,6 @@ reference's tests (tests/test_decode_p0.py:48-113, tests/test_paged_attention_re
 tests/test_continuous_batching.py:524-553) and its worked token-table example
 (lite_llama/executor/paged_attention.py:125-129), re-expressed against this package's classes."""
 
-import numpy as np
 import pytest
 import torch
 

@@ -6,7 +6,6 @@ at least one of these."""
 import math
 
 import numpy as np
-import pytest
 import torch
 
 from llama_lite_npu_amd import workloads
