@@ -638,14 +638,84 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
   }
 }
 
-// Balanced-schedule merge, one wavefront per (query head, sequence): combines the sequence's
+// Merge of many partial rows by a whole workgroup of kMergeWaves wavefronts (a single long
+// sequence spans every chunk of the step: one wavefront adding 256 rows one round trip after the
+// other took 23 us). Every wavefront merges a contiguous quarter of the pieces against the common
+// maximum, in index order and with 16 row loads in flight; wavefront 0 then adds the four partial
+// sums in wavefront order, so the result does not depend on timing.
+constexpr int kMergeWaves = 4;
+
+__device__ __forceinline__ void merge_row_wide(const float *__restrict__ lse, int64_t lse_stride,
+                                               const float *__restrict__ po, int64_t po_stride,
+                                               int n_parts, half_t *out_row, int tid, float *red) {
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  float mx = -INFINITY;
+  for (int s = tid; s < n_parts; s += kMergeWaves * kWave) mx = fmaxf(mx, lse[(int64_t)s * lse_stride]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, xor_lane(mx, off));
+  if (lane == 0) red[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+
+  const int per = (n_parts + kMergeWaves - 1) / kMergeWaves;
+  const int s_begin = wave * per;
+  const int s_end = s_begin + per < n_parts ? s_begin + per : n_parts;
+  float den = 0.f, num0 = 0.f, num1 = 0.f;
+  for (int base = s_begin; base < s_end; base += kWave) {
+    const float l = (base + lane < s_end) ? lse[(int64_t)(base + lane) * lse_stride] : -INFINITY;
+    const float w = fast_exp2((l - mx) * kLog2e);
+    den += w;
+    const int cnt = (s_end - base) < kWave ? (s_end - base) : kWave;
+    int s = 0;
+    for (; s + 16 <= cnt; s += 16) {
+      float2 r[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) r[u] = *(const float2 *)(po + (int64_t)(base + s + u) * po_stride + 2 * lane);
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const float wu = __shfl(w, s + u, kWave);
+        num0 += wu * r[u].x;
+        num1 += wu * r[u].y;
+      }
+    }
+    for (; s < cnt; ++s) {
+      const float2 r = *(const float2 *)(po + (int64_t)(base + s) * po_stride + 2 * lane);
+      const float wu = __shfl(w, s, kWave);
+      num0 += wu * r.x;
+      num1 += wu * r.y;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) den += xor_lane(den, off);
+  float *sums = red + 8;  // [kMergeWaves][kHeadDim], then the denominators
+  sums[wave * kHeadDim + 2 * lane] = num0;
+  sums[wave * kHeadDim + 2 * lane + 1] = num1;
+  if (lane == 0) sums[kMergeWaves * kHeadDim + wave] = den;
+  __syncthreads();
+  if (wave != 0) return;
+  float d = 0.f, o0 = 0.f, o1 = 0.f;
+#pragma unroll
+  for (int w2 = 0; w2 < kMergeWaves; ++w2) {
+    o0 += sums[w2 * kHeadDim + 2 * lane];
+    o1 += sums[w2 * kHeadDim + 2 * lane + 1];
+    d += sums[kMergeWaves * kHeadDim + w2];
+  }
+  const float inv = 1.0f / d;
+  typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+  *(half2_t *)(out_row + 2 * lane) = half2_t{(half_t)(o0 * inv), (half_t)(o1 * inv)};
+}
+
+// Balanced-schedule merge, one workgroup per (query head, sequence): combines the sequence's
 // pieces (partial slots c_first + b, c_first + b + 1, ...) if it spans several chunks, and the
-// `pre_splits` partials of the shared prefix if there is one.
-__global__ __launch_bounds__(kWave) void paged_decode_balanced_merge_kernel(
+// `pre_splits` partials of the shared prefix if there is one. Up to 16 pieces (and any number
+// with a shared prefix) are merged by the first wavefront alone.
+__global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merge_kernel(
     const int32_t *__restrict__ plan, const int32_t *__restrict__ seq_lens,
     half_t *__restrict__ out, const float *__restrict__ part_o,
     const float *__restrict__ part_lse, const float *__restrict__ pre_o,
     const float *__restrict__ pre_lse, int32_t pre_splits, int32_t batch, int32_t num_q_heads) {
+  __shared__ float red[8 + kMergeWaves * kHeadDim + kMergeWaves];
   const int hq = blockIdx.x;
   const int b = blockIdx.y;
   const int c_first = plan[plan_seq_info_offset() + 2 * b];
@@ -656,6 +726,12 @@ __global__ __launch_bounds__(kWave) void paged_decode_balanced_merge_kernel(
   const int64_t pre0 = (int64_t)b * num_q_heads + hq;
   const int64_t pre_step = (int64_t)batch * num_q_heads;
   half_t *out_row = out + ((int64_t)b * num_q_heads + hq) * kHeadDim;
+  if (pre_splits == 0 && n_parts > 16) {  // the same for every thread of the workgroup
+    merge_row_wide(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
+                   (int64_t)num_q_heads * kHeadDim, n_parts, out_row, threadIdx.x, red);
+    return;
+  }
+  if (threadIdx.x >= kWave) return;
   if (pre_splits == 0) {
     merge_row<false>(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
                      (int64_t)num_q_heads * kHeadDim, n_parts, nullptr, 0, nullptr, 0, 0, out_row,
@@ -1228,7 +1304,7 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   rc = check_launch(what);
   if (rc != LITEKV_OK) return rc;
   hipLaunchKernelGGL(paged_decode_balanced_merge_kernel,
-                     dim3((unsigned)num_q_heads, (unsigned)batch), dim3(kWave), 0,
+                     dim3((unsigned)num_q_heads, (unsigned)batch), dim3(kMergeWaves * kWave), 0,
                      static_cast<hipStream_t>(stream), static_cast<const int32_t *>(plan), seq_lens,
                      static_cast<half_t *>(out), part_o, part_lse, pre_o, pre_lse, pre_splits,
                      batch, num_q_heads);
