@@ -313,7 +313,7 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
         # come from HBM at least once; the logical rate (every reader counted) is kept beside it.
         res["roofline"].update(achieved=unique / (k_mean * 1e-3) / 1e9,
                                frac=unique / (k_mean * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                               logical_gbps=achieved, unique_bytes_per_launch=unique,
+                               logical_gbps=kernel_bytes / (k_mean * 1e-3) / 1e9, unique_bytes_per_launch=unique,
                                logical_bytes_per_launch=kernel_bytes)
     res.update(ls.plan_info)
     res["launch"] = "eager"
