@@ -318,6 +318,17 @@ int litekv_kv_append_fp8(const void *k, const void *v, int64_t k_token_stride,
                          int32_t num_kv_heads, int32_t head_dim, int64_t num_slots,
                          void *stream);
 
+/* litekv_qk_norm_rope_append into an fp8 pool: the rotated k row and the v row are quantised as
+ * by litekv_kv_append_fp8 (same codes for the same fp16 row); q as in the fp16 variant. */
+int litekv_qk_norm_rope_append_fp8(void *q, int64_t q_token_stride, const void *k,
+                                   int64_t k_token_stride, const void *v, int64_t v_token_stride,
+                                   const void *q_norm_weight, const void *k_norm_weight,
+                                   const void *cos_rows, const void *sin_rows,
+                                   int64_t cos_sin_token_stride, const int32_t *slot_mapping,
+                                   void *kv_pool_fp8, const float *scales, int32_t num_tokens,
+                                   int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                   int64_t num_slots, float rms_eps, void *stream);
+
 int litekv_page_dequant(const void *kv_pool_fp8, void *dst_pool, const int32_t *src_ids,
                         const int32_t *dst_ids, int32_t n, const float *scales,
                         int32_t num_kv_heads, int32_t head_dim, int32_t page_size,

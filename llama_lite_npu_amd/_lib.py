@@ -91,6 +91,11 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32,
          c_int64, c_void_p],
     ),
+    "litekv_qk_norm_rope_append_fp8": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int64, c_float, c_void_p],
+    ),
     "litekv_page_dequant": (
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_int32, c_int32, c_int32, c_int64,

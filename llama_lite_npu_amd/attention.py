@@ -44,17 +44,9 @@ class Attention:
         ``context_forward`` / ``token_forward`` afterwards with ``xk=None, xv=None``."""
         cos, sin = position_embeddings if position_embeddings is not None else (None, None)
         pool = atten_info.kv_buffer[layer_index]
-        if not ops.is_fp8_pool(pool):
-            return ops.qk_norm_rope_append(xq, xk, xv, atten_info.cur_select_index, pool, q_norm_weight,
-                                           k_norm_weight, cos, sin, rms_eps)
-        # fp8 pool: the epilogue writes its rows into a scratch fp16 row per token, which is then quantised
-        t = xq.shape[0]
-        rows = torch.empty((t, 2 * self.num_kv_heads, self.head_dim), dtype=torch.float16, device=xq.device)
-        ops.qk_norm_rope_append(xq, xk, xv, torch.arange(t, dtype=torch.int32, device=xq.device), rows,
-                                q_norm_weight, k_norm_weight, cos, sin, rms_eps)
-        ops.kv_append_fp8(rows[:, :self.num_kv_heads], rows[:, self.num_kv_heads:], atten_info.cur_select_index,
-                          pool, atten_info.kv_scales[layer_index])
-        return xq
+        scales = atten_info.kv_scales[layer_index] if ops.is_fp8_pool(pool) else None
+        return ops.qk_norm_rope_append(xq, xk, xv, atten_info.cur_select_index, pool, q_norm_weight,
+                                       k_norm_weight, cos, sin, rms_eps, kv_scales=scales)
 
     def context_forward(self, xq, xk, xv, atten_info, layer_index: int, qk_scale=None) -> torch.Tensor:
         """Prefill: xq [T, Hq, D], xk / xv [T, Hkv, D] packed rows of the batch's prompts or chunks

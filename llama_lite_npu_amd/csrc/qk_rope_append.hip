@@ -12,6 +12,7 @@
 // x1*cos - x2*sin, x2*cos + x1*sin (lite_llama/kernels/rope_emb.py:79-87) is evaluated in fp32
 // from fp16 inputs and rounded once.
 #include "common.h"
+#include "kv_fp8.h"
 
 namespace litekv {
 
@@ -25,13 +26,16 @@ __device__ __forceinline__ float row_sum(float v) {
   return v;
 }
 
+// FP8: the pool holds E4M3 codes; `scales` are its per-head scales (K heads, then V heads) and a
+// row is quantised on its way in, exactly as kv_append_fp8_kernel would quantise the fp16 row.
+template <bool FP8>
 __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
     half_t *__restrict__ q, int64_t q_stride, const half_t *__restrict__ k, int64_t k_stride,
     const half_t *__restrict__ v, int64_t v_stride, const half_t *__restrict__ q_weight,
     const half_t *__restrict__ k_weight, const half_t *__restrict__ cos_rows,
     const half_t *__restrict__ sin_rows, int64_t cs_stride, const int32_t *__restrict__ slot_mapping,
-    half_t *__restrict__ pool, int64_t total_rows, int32_t num_q_heads, int32_t num_kv_heads,
-    int64_t num_slots, float eps) {
+    void *__restrict__ pool_any, const float *__restrict__ scales, int64_t total_rows,
+    int32_t num_q_heads, int32_t num_kv_heads, int64_t num_slots, float eps) {
   const int l16 = threadIdx.x & 15;
   const int64_t row = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
   if (row >= total_rows) return;  // whole 16-lane groups leave together
@@ -40,13 +44,21 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
   const int r = (int)(row - token * rows_per_token);
   const int64_t slot = slot_mapping[token];
   const bool slot_ok = slot >= 0 && slot < num_slots;
-  half_t *slot_row = pool + slot * (int64_t)(2 * num_kv_heads * kHeadDim);
+  // stores 8 elements of head `kv_head` (K heads first, then V heads) of the token's slot
+  auto store_row = [&](int kv_head, half8_t x) {
+    const int64_t at = (slot * (int64_t)(2 * num_kv_heads) + kv_head) * kHeadDim + 8 * l16;
+    if constexpr (FP8) {
+      *(uint2_t *)(static_cast<uint8_t *>(pool_any) + at) = half8_to_fp8(x, 1.0f / scales[kv_head]);
+    } else {
+      *(half8_t *)(static_cast<half_t *>(pool_any) + at) = x;
+    }
+  };
 
   if (r >= num_q_heads + num_kv_heads) {  // a v row: plain copy into the slot
     const int head = r - num_q_heads - num_kv_heads;
     if (slot_ok) {
-      const half8_t x = *(const half8_t *)(v + token * v_stride + (int64_t)head * kHeadDim + 8 * l16);
-      *(half8_t *)(slot_row + (int64_t)(num_kv_heads + head) * kHeadDim + 8 * l16) = x;
+      store_row(num_kv_heads + head,
+                *(const half8_t *)(v + token * v_stride + (int64_t)head * kHeadDim + 8 * l16));
     }
     return;
   }
@@ -95,23 +107,21 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
   if (is_q) {
     *(half8_t *)(q + token * q_stride + (int64_t)head * kHeadDim + 8 * l16) = x;
   } else if (slot_ok) {
-    *(half8_t *)(slot_row + (int64_t)head * kHeadDim + 8 * l16) = x;
+    store_row(head, x);
   }
 }
 
 }  // namespace litekv
 
-extern "C" int litekv_qk_norm_rope_append(void *q, int64_t q_token_stride, const void *k,
-                                          int64_t k_token_stride, const void *v,
-                                          int64_t v_token_stride, const void *q_norm_weight,
-                                          const void *k_norm_weight, const void *cos_rows,
-                                          const void *sin_rows, int64_t cos_sin_token_stride,
-                                          const int32_t *slot_mapping, void *kv_pool,
-                                          int32_t num_tokens, int32_t num_q_heads,
-                                          int32_t num_kv_heads, int32_t head_dim, int64_t num_slots,
-                                          float rms_eps, void *stream) {
-  using namespace litekv;
-  const char *what = "qk_norm_rope_append";
+namespace litekv {
+static int launch_qk_epilogue(const char *what, void *q, int64_t q_token_stride, const void *k,
+                              int64_t k_token_stride, const void *v, int64_t v_token_stride,
+                              const void *q_norm_weight, const void *k_norm_weight,
+                              const void *cos_rows, const void *sin_rows,
+                              int64_t cos_sin_token_stride, const int32_t *slot_mapping,
+                              void *kv_pool, const float *fp8_scales, bool fp8, int32_t num_tokens,
+                              int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                              int64_t num_slots, float rms_eps, void *stream) {
   LITEKV_REQUIRE(num_tokens >= 0, "%s: num_tokens %d < 0", what, num_tokens);
   LITEKV_REQUIRE(head_dim == kHeadDim, "%s: head_dim %d unsupported (only %d)", what, head_dim,
                  kHeadDim);
@@ -122,6 +132,7 @@ extern "C" int litekv_qk_norm_rope_append(void *q, int64_t q_token_stride, const
     return LITEKV_OK;
   }
   LITEKV_REQUIRE(q && k && v && slot_mapping && kv_pool, "%s: null pointer", what);
+  LITEKV_REQUIRE(!fp8 || fp8_scales != nullptr, "%s: scales is null", what);
   LITEKV_REQUIRE((q_norm_weight == nullptr) == (k_norm_weight == nullptr),
                  "%s: q_norm_weight and k_norm_weight go together", what);
   LITEKV_REQUIRE((cos_rows == nullptr) == (sin_rows == nullptr), "%s: cos and sin go together", what);
@@ -144,13 +155,47 @@ extern "C" int litekv_qk_norm_rope_append(void *q, int64_t q_token_stride, const
   const int64_t total_rows = (int64_t)num_tokens * (num_q_heads + 2 * num_kv_heads);
   const int64_t blocks = (total_rows * kLanesPerRow + 255) / 256;
   LITEKV_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many tokens", what);
-  hipLaunchKernelGGL(qk_norm_rope_append_kernel, dim3((unsigned)blocks), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<half_t *>(q), q_token_stride,
-                     static_cast<const half_t *>(k), k_token_stride, static_cast<const half_t *>(v),
-                     v_token_stride, static_cast<const half_t *>(q_norm_weight),
+  auto kernel = fp8 ? qk_norm_rope_append_kernel<true> : qk_norm_rope_append_kernel<false>;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<half_t *>(q), q_token_stride, static_cast<const half_t *>(k),
+                     k_token_stride, static_cast<const half_t *>(v), v_token_stride,
+                     static_cast<const half_t *>(q_norm_weight),
                      static_cast<const half_t *>(k_norm_weight), static_cast<const half_t *>(cos_rows),
-                     static_cast<const half_t *>(sin_rows), cos_sin_token_stride, slot_mapping,
-                     static_cast<half_t *>(kv_pool), total_rows, num_q_heads, num_kv_heads, num_slots,
-                     rms_eps);
+                     static_cast<const half_t *>(sin_rows), cos_sin_token_stride, slot_mapping, kv_pool,
+                     fp8_scales, total_rows, num_q_heads, num_kv_heads, num_slots, rms_eps);
   return check_launch(what);
+}
+}  // namespace litekv
+
+extern "C" int litekv_qk_norm_rope_append(void *q, int64_t q_token_stride, const void *k,
+                                          int64_t k_token_stride, const void *v,
+                                          int64_t v_token_stride, const void *q_norm_weight,
+                                          const void *k_norm_weight, const void *cos_rows,
+                                          const void *sin_rows, int64_t cos_sin_token_stride,
+                                          const int32_t *slot_mapping, void *kv_pool,
+                                          int32_t num_tokens, int32_t num_q_heads,
+                                          int32_t num_kv_heads, int32_t head_dim, int64_t num_slots,
+                                          float rms_eps, void *stream) {
+  return litekv::launch_qk_epilogue("qk_norm_rope_append", q, q_token_stride, k, k_token_stride, v,
+                                    v_token_stride, q_norm_weight, k_norm_weight, cos_rows, sin_rows,
+                                    cos_sin_token_stride, slot_mapping, kv_pool, nullptr, false,
+                                    num_tokens, num_q_heads, num_kv_heads, head_dim, num_slots,
+                                    rms_eps, stream);
+}
+
+extern "C" int litekv_qk_norm_rope_append_fp8(void *q, int64_t q_token_stride, const void *k,
+                                              int64_t k_token_stride, const void *v,
+                                              int64_t v_token_stride, const void *q_norm_weight,
+                                              const void *k_norm_weight, const void *cos_rows,
+                                              const void *sin_rows, int64_t cos_sin_token_stride,
+                                              const int32_t *slot_mapping, void *kv_pool_fp8,
+                                              const float *scales, int32_t num_tokens,
+                                              int32_t num_q_heads, int32_t num_kv_heads,
+                                              int32_t head_dim, int64_t num_slots, float rms_eps,
+                                              void *stream) {
+  return litekv::launch_qk_epilogue("qk_norm_rope_append_fp8", q, q_token_stride, k, k_token_stride,
+                                    v, v_token_stride, q_norm_weight, k_norm_weight, cos_rows,
+                                    sin_rows, cos_sin_token_stride, slot_mapping, kv_pool_fp8, scales,
+                                    true, num_tokens, num_q_heads, num_kv_heads, head_dim, num_slots,
+                                    rms_eps, stream);
 }

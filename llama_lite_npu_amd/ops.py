@@ -129,13 +129,19 @@ def page_dequant(kv_pool: torch.Tensor, dst_pool: torch.Tensor, src_ids: torch.T
 def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor,
                         kv_pool: torch.Tensor, q_norm_weight: Optional[torch.Tensor] = None,
                         k_norm_weight: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
-                        sin: Optional[torch.Tensor] = None, rms_eps: float = 1e-6) -> torch.Tensor:
+                        sin: Optional[torch.Tensor] = None, rms_eps: float = 1e-6,
+                        kv_scales: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Per-head RMSNorm (optional) and rotary embedding (optional) of q [T, Hq, D] in place and of
     k [T, Hkv, D] on its way into the pool, plus the append of v: one launch for the reference's
     skip_rmsnorm x2 + rope_emb_forward + cat + update_kv_buffer. cos / sin are [T, >= D/2] rows of
-    each token's position. Returns q."""
-    _dev_half("q", q), _dev_half("k", k), _dev_half("v", v), _dev_half("kv_pool", kv_pool)
+    each token's position. An fp8 pool (with its ``kv_scales``) receives the quantised rows. Returns q."""
+    _dev_half("q", q), _dev_half("k", k), _dev_half("v", v)
     slots, hkv, d, _, _ = pool_geometry(kv_pool, 1)
+    fp8 = is_fp8_pool(kv_pool)
+    if fp8:
+        _dev_fp8_pool(kv_pool, kv_scales, hkv)
+    else:
+        _dev_half("kv_pool", kv_pool)
     t, hq = q.shape[0], q.shape[1]
     _need(q.dim() == 3 and q.shape[2] == d, "q must be [T, Hq, D]")
     _need(k.shape == (t, hkv, d) and v.shape == (t, hkv, d), "k / v must be [T, Hkv, D] matching the pool")
@@ -156,6 +162,12 @@ def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_
     slot_mapping = _dev_i32("slot_mapping", slot_mapping)
     _need(slot_mapping.numel() == t, "slot_mapping must hold one slot per token")
     lib = _lib.load()
+    if fp8:
+        _lib.check(lib.litekv_qk_norm_rope_append_fp8(
+            _ptr(q), _rows("q", q), _ptr(k), _rows("k", k), _ptr(v), _rows("v", v), _ptr(q_norm_weight),
+            _ptr(k_norm_weight), _ptr(cos), _ptr(sin), cs_stride, _ptr(slot_mapping), _ptr(kv_pool),
+            _ptr(kv_scales), t, hq, hkv, d, slots, float(rms_eps), _stream()))
+        return q
     _lib.check(lib.litekv_qk_norm_rope_append(
         _ptr(q), _rows("q", q), _ptr(k), _rows("k", k), _ptr(v), _rows("v", v), _ptr(q_norm_weight),
         _ptr(k_norm_weight), _ptr(cos), _ptr(sin), cs_stride, _ptr(slot_mapping), _ptr(kv_pool), t, hq, hkv, d,

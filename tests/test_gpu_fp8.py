@@ -330,3 +330,43 @@ def test_fp8_decode_steps_replay_as_graphs():
     batch.check()
     for a, b in zip(host.kv_mem_manager.gpu_kv_buffer, dev.kv_mem_manager.gpu_kv_buffer):
         assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+
+
+def test_fused_epilogue_into_an_fp8_pool_equals_epilogue_then_quantising_append():
+    print("fp8: fused QK-norm + RoPE + quantising append", flush=True)
+    t, hq, hkv = 77, 16, 4
+    g = torch.Generator(device=DEV).manual_seed(61)
+    qkv = torch.randn((t, hq + 2 * hkv, D), generator=g, device=DEV, dtype=torch.float16) * 1.5
+    q, k, v = qkv[:, :hq], qkv[:, hq:hq + hkv], qkv[:, hq + hkv:]
+    wq = (1.0 + 0.2 * torch.randn(D, generator=g, device=DEV)).half()
+    wk = (1.0 + 0.2 * torch.randn(D, generator=g, device=DEV)).half()
+    pos = torch.randint(0, 4096, (t,), generator=g, device=DEV).double()
+    inv = 10000.0 ** (-torch.arange(0, D, 2, device=DEV, dtype=torch.float64) / D)
+    emb = torch.cat([pos[:, None] * inv[None, :]] * 2, dim=1)
+    cos, sin = emb.cos().half(), emb.sin().half()
+    slots = torch.randperm(256, generator=torch.Generator().manual_seed(3))[:t].to(torch.int32).to(DEV)
+    slots[7] = -1
+    scales = torch.tensor([0.02, 0.03, 0.025, 0.04, 0.015, 0.02, 0.01, 0.03], device=DEV)
+    # two launches: epilogue into fp16 rows, then the quantising append
+    q_a = q.clone()
+    rows = torch.empty((t, 2 * hkv, D), dtype=torch.float16, device=DEV)
+    ops.qk_norm_rope_append(q_a, k, v, torch.arange(t, dtype=torch.int32, device=DEV), rows, wq, wk, cos, sin)
+    pool_a = torch.full((256, 2 * hkv, D), 0x55, dtype=torch.uint8, device=DEV)
+    ops.kv_append_fp8(rows[:, :hkv], rows[:, hkv:], slots, pool_a, scales)
+    # one launch
+    q_b = q.clone()
+    pool_b = torch.full((256, 2 * hkv, D), 0x55, dtype=torch.uint8, device=DEV)
+    ops.qk_norm_rope_append(q_b, k, v, slots, pool_b, wq, wk, cos, sin, kv_scales=scales)
+    torch.cuda.synchronize()
+    assert torch.equal(q_a, q_b)
+    assert torch.equal(pool_a, pool_b)
+    assert int((pool_b != 0x55).any(dim=(1, 2)).sum()) == t - 1          # the padded token stored nothing
+    # without norm and rotation it is the plain quantising append
+    pool_c = torch.full_like(pool_b, 0x55)
+    pool_d = torch.full_like(pool_b, 0x55)
+    ops.qk_norm_rope_append(q.clone(), k, v, slots, pool_c, kv_scales=scales)
+    ops.kv_append_fp8(k, v, slots, pool_d, scales)
+    torch.cuda.synchronize()
+    assert torch.equal(pool_c, pool_d)
+    with pytest.raises(ValueError, match="scales"):
+        ops.qk_norm_rope_append(q.clone(), k, v, slots, pool_c)
