@@ -338,18 +338,26 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
 
 
 def _time_us(fn, reps: int = 10, warm: int = 2) -> float:
+    """Mean device time of one `fn()` in microseconds: `reps` launches recorded back to back in one
+    HIP graph and replayed between two events (an event pair around a single short launch measures
+    mostly the events and the Python call, 10-15 us on this stack)."""
     import torch
 
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
-    for a, b in ev:
-        a.record()
-        fn()
-        b.record()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(reps):
+            fn()
+    graph.replay()
     torch.cuda.synchronize()
-    return sum(a.elapsed_time(b) for a, b in ev) / reps * 1e3
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    graph.replay()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps * 1e3
 
 
 def time_qk_epilogue(tokens: int, hq: int, hkv: int, slot_mapping, pool) -> dict:
@@ -444,19 +452,10 @@ def cpu_baseline_prefill(case, budget_s: float = 10.0) -> dict:
 
 
 def time_append(case_tokens_k, case_tokens_v, slot_mapping, pool, reps: int = 20) -> float:
-    """Mean microseconds of one KV-append launch (HIP events on the launch stream)."""
-    import torch
+    """Mean microseconds of one KV-append launch."""
     from llama_lite_npu_amd import ops
 
-    for _ in range(3):
-        ops.kv_append(case_tokens_k, case_tokens_v, slot_mapping, pool)
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
-    for a, b in ev:
-        a.record()
-        ops.kv_append(case_tokens_k, case_tokens_v, slot_mapping, pool)
-        b.record()
-    torch.cuda.synchronize()
-    return sum(a.elapsed_time(b) for a, b in ev) / reps * 1e3
+    return _time_us(lambda: ops.kv_append(case_tokens_k, case_tokens_v, slot_mapping, pool), reps=reps, warm=3)
 
 
 def run_prefill(case, steps: int, warmup: int, device: str, label: str) -> dict:
