@@ -396,17 +396,26 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_
                                           const float *__restrict__ po2, int64_t po2_stride, int n2,
                                           half_t *out_row, int lane) {
   const int n_parts = TWO_RUNS ? n1 + n2 : n1;
-  if (!TWO_RUNS && n1 <= 16) {
-    // The usual case (a sequence spans a few chunks): every row and the log-sum-exps are
-    // requested at once, so the launch waits for one round trip to memory instead of one per
-    // group of rows. Same weights and the same order of additions as the general path below.
+  auto lse_of = [&](int s) {
+    if (!TWO_RUNS || s < n1) return lse1[(int64_t)s * lse1_stride];
+    return lse2[(int64_t)(s - n1) * lse2_stride];
+  };
+  auto row_of = [&](int s) {
+    if (!TWO_RUNS || s < n1) return po1 + (int64_t)s * po1_stride;
+    return po2 + (int64_t)(s - n1) * po2_stride;
+  };
+  if (n_parts <= 16) {
+    // The usual case (a sequence spans a few chunks, with or without the slices of a shared
+    // prefix): every row and the log-sum-exps are requested at once, so the launch waits for one
+    // round trip to memory instead of one per group of rows. Same weights and the same order of
+    // additions as the general path below.
     float2 r[16];
 #pragma unroll
     for (int s = 0; s < 16; ++s) {
       r[s] = float2{0.f, 0.f};
-      if (s < n1) r[s] = *(const float2 *)(po1 + (int64_t)s * po1_stride + 2 * lane);
+      if (s < n_parts) r[s] = *(const float2 *)(row_of(s) + 2 * lane);
     }
-    const float l = lane < n1 ? lse1[(int64_t)lane * lse1_stride] : -INFINITY;
+    const float l = lane < n_parts ? lse_of(lane) : -INFINITY;
     float mx = l;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, xor_lane(mx, off));
@@ -417,7 +426,7 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_
     float num0 = 0.f, num1 = 0.f;
 #pragma unroll
     for (int s = 0; s < 16; ++s) {
-      if (s < n1) {
+      if (s < n_parts) {
         const float ws = __shfl(w, s, kWave);
         num0 += ws * r[s].x;
         num1 += ws * r[s].y;
@@ -428,14 +437,6 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_
     *(half2_t *)(out_row + 2 * lane) = half2_t{(half_t)(num0 * inv), (half_t)(num1 * inv)};
     return;
   }
-  auto lse_of = [&](int s) {
-    if (!TWO_RUNS || s < n1) return lse1[(int64_t)s * lse1_stride];
-    return lse2[(int64_t)(s - n1) * lse2_stride];
-  };
-  auto row_of = [&](int s) {
-    if (!TWO_RUNS || s < n1) return po1 + (int64_t)s * po1_stride;
-    return po2 + (int64_t)(s - n1) * po2_stride;
-  };
   float mx = -INFINITY;
   for (int s0 = 0; s0 < n_parts; s0 += kWave) {
     const float l = (s0 + lane < n_parts) ? lse_of(s0 + lane) : -INFINITY;
@@ -726,7 +727,7 @@ __global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merg
   const int64_t pre0 = (int64_t)b * num_q_heads + hq;
   const int64_t pre_step = (int64_t)batch * num_q_heads;
   half_t *out_row = out + ((int64_t)b * num_q_heads + hq) * kHeadDim;
-  if (pre_splits == 0 && n_parts > 16) {  // the same for every thread of the workgroup
+  if (pre_splits == 0 && n_parts > 16 && blockDim.x == kMergeWaves * kWave) {  // uniform in the workgroup
     merge_row_wide(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
                    (int64_t)num_q_heads * kHeadDim, n_parts, out_row, threadIdx.x, red);
     return;
@@ -1303,8 +1304,14 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   }
   rc = check_launch(what);
   if (rc != LITEKV_OK) return rc;
+  // A sequence has at most block_table_stride pages, so it spans at most that many chunks: the
+  // four-wavefront merge of long rows (more than 16 pieces, never with a shared prefix) is only
+  // launched where such a row can exist; the other wavefronts of a workgroup would leave at once
+  // and only cost their dispatch (C4: 9.9 -> 7 us).
+  const int max_pieces = chunks < block_table_stride ? chunks : block_table_stride;
+  const int merge_waves = (pre_splits == 0 && max_pieces > 16) ? kMergeWaves : 1;
   hipLaunchKernelGGL(paged_decode_balanced_merge_kernel,
-                     dim3((unsigned)num_q_heads, (unsigned)batch), dim3(kMergeWaves * kWave), 0,
+                     dim3((unsigned)num_q_heads, (unsigned)batch), dim3(merge_waves * kWave), 0,
                      static_cast<hipStream_t>(stream), static_cast<const int32_t *>(plan), seq_lens,
                      static_cast<half_t *>(out), part_o, part_lse, pre_o, pre_lse, pre_splits,
                      batch, num_q_heads);
