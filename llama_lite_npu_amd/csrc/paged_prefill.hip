@@ -210,11 +210,11 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                    :
                    : "s"(k_lds + dst + 1024u * i), "v"(ko), "s"(kbase)
-                   : "memory");
+                   : "memory", "m0");
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                    :
                    : "s"(v_lds + dst + 1024u * i), "v"(vo), "s"(vbase)
-                   : "memory");
+                   : "memory", "m0");
     };
     if (row0 + 15 <= last_key) {
 #pragma unroll
