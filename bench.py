@@ -34,10 +34,13 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
-# HBM bytes per launch of the decode kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by a 1 GiB
-# copy kernel); summary and commands in profiles/paged_decode_balanced_c2_pmc.txt. Only meaningful for
-# the workload it was measured on.
-MEASURED_TRAFFIC_BYTES = {("c2", "balanced", "f16"): 317.9e6, ("c2", "balanced", "fp8"): 164.5e6}
+# HBM bytes per launch of the roofline kernel(s) from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by a
+# 1 GiB copy kernel); summaries and commands in profiles/paged_decode_balanced_c2_pmc.txt,
+# profiles/paged_decode_balanced_fp8_c2.txt and profiles/hbm_traffic_c3_c4_c5_pmc.txt. Only
+# meaningful for the workload it was measured on. c4: prefix kernel + decode kernel + merge.
+MEASURED_TRAFFIC_BYTES = {("c2", "balanced", "f16"): 317.9e6, ("c2", "balanced", "fp8"): 164.5e6,
+                          ("c3", "balanced", "f16"): 387.7e6, ("c4", "balanced", "f16"): 150.6e6,
+                          ("c5", "balanced", "f16"): 5196.0e6}
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
 
 
@@ -636,10 +639,16 @@ def main() -> int:
 
     res, case = run(args.config)
     traffic = MEASURED_TRAFFIC_BYTES.get((args.config, args.schedule, args.kv_dtype))
-    if traffic is not None and args.config != "c3":
-        res["roofline"]["traffic"] = traffic / (res["decode_kernel_us_mean"] * 1e-6) / 1e9
+    if traffic is not None and (args.config != "c4" or not args.no_shared_prefix):
+        if args.config == "c3":
+            duration_us, algorithmic = res["prefill_us_mean"], case.min_bytes()
+        else:
+            duration_us = res["roofline"].get("duration_us", res["decode_kernel_us_mean"])
+            algorithmic = res["roofline"].get("unique_bytes_per_launch",
+                                              res["decode_bytes_per_layer"] + res["append_bytes_per_layer"])
+        res["roofline"]["traffic"] = traffic / (duration_us * 1e-6) / 1e9
         res["roofline"]["traffic_bytes_per_launch"] = traffic
-        res["roofline"]["algorithmic_bytes_per_launch"] = res["decode_bytes_per_layer"] + res["append_bytes_per_layer"]
+        res["roofline"]["algorithmic_bytes_per_launch"] = algorithmic
     line = {
         "metric": "paged decode attn HBM GB/s (% of 8 TB/s peak); KV-append GB/s; us/layer",
         "value": res.get("value", res.get("prefill_tflops")),
