@@ -297,6 +297,50 @@ __device__ __forceinline__ void store_state(const HeadState &st, bool final_row,
   }
 }
 
+// A finished state parked in LDS instead of being stored: stores count in the same hardware
+// counter as loads on this architecture, so a store issued in the middle of a chunk makes every
+// later counted wait of the page loop also wait for the store's acknowledgement (2.65 us per
+// sequence crossing on C2). The parked values are the ones store_state would have written
+// (normalised fp32 and the log-sum-exp); unpark_state writes them out at the end of the chunk,
+// each lane reading back what it wrote itself.
+constexpr int kParkHeads = 8;                                  // query heads per kv head that fit
+constexpr int kParkFloats = kParkHeads * kHeadDim + 16;        // rows, then one log-sum-exp per head
+
+__device__ __forceinline__ void park_state(const HeadState &st, float *park, int n, int g,
+                                           int group, float out_scale) {
+  float d_tot = st.d + xor_lane(st.d, 16);
+  d_tot += xor_lane(d_tot, 32);
+  const float inv = out_scale / d_tot;
+  if (n >= group) return;
+  float *row = park + n * kHeadDim + 4 * g;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    *(float4_t *)(row + 16 * j) = float4_t{st.acc[j][0] * inv, st.acc[j][1] * inv,
+                                           st.acc[j][2] * inv, st.acc[j][3] * inv};
+  }
+  if (g == 0) park[kParkHeads * kHeadDim + n] = (st.m + fast_log2(d_tot)) * kLn2;
+}
+
+__device__ __forceinline__ void unpark_state(const float *park, bool final_row, half_t *out_row,
+                                             float *part_row, float *part_lse_cell, int n, int g,
+                                             int group) {
+  if (n >= group) return;
+  const float *row = park + n * kHeadDim + 4 * g;
+  if (final_row) {
+    half_t *o = out_row + (int64_t)n * kHeadDim + 4 * g;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float4_t x = *(const float4_t *)(row + 16 * j);
+      *(half4_t *)(o + 16 * j) = half4_t{(half_t)x[0], (half_t)x[1], (half_t)x[2], (half_t)x[3]};
+    }
+  } else {
+    float *po = part_row + (int64_t)n * kHeadDim + 4 * g;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) *(float4_t *)(po + 16 * j) = *(const float4_t *)(row + 16 * j);
+    if (g == 0) part_lse_cell[n] = park[kParkHeads * kHeadDim + n];
+  }
+}
+
 // Waits for every vector memory load this wavefront has in flight (s_waitcnt vmcnt(0), other
 // counters untouched). Used at the end of rarely taken branches that load into registers the
 // main loop reads: without it the compiler must assume those loads are still pending after the
@@ -754,6 +798,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     float *__restrict__ part_lse, int32_t bt_stride, int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t group,
     int32_t heads_per_wg, int32_t replicas, int32_t chunks, int32_t skip, float scale_log2) {
   __shared__ __attribute__((aligned(16))) half_t vstage_all[kMaxWavesPerWg][kPageSize * kVPitch];
+  __shared__ __attribute__((aligned(16))) float park_all[kMaxWavesPerWg][kParkFloats];
 
   // readfirstlane tells the compiler the wavefront index is uniform (scalar branches and loads)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -820,12 +865,31 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
                      : kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
   const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
   half8_t qf[4];
-  auto fetch_q = [&](int b) {
+  auto fetch_q_into = [&](half8_t (&dst)[4], int b) {
     const half_t *row0 = q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHeadDim;
     if constexpr (FP8) {
-      load_q_fp8_order(qf, row0, n, g, group);
+      load_q_fp8_order(dst, row0, n, g, group);
     } else {
-      load_q(qf, row0, n, g, group);
+      load_q(dst, row0, n, g, group);
+    }
+  };
+  // This lane's parts of the step's new K and V rows of sequence b (see the fused append below).
+  auto fetch_new_rows = [&](uint4_t (&kr)[4], uint4_t (&vr)[2], int b) {
+    const half_t *kn = k_new + (int64_t)b * k_new_stride + (int64_t)h * kHeadDim;
+    const half_t *vn = v_new + (int64_t)b * v_new_stride + (int64_t)h * kHeadDim;
+    if constexpr (FP8) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        kr[2 * j] = *(const uint4_t *)(kn + 64 * j + 16 * g);
+        kr[2 * j + 1] = *(const uint4_t *)(kn + 64 * j + 16 * g + 8);
+      }
+      vr[0] = *(const uint4_t *)(vn + 16 * (n & 7));
+      vr[1] = *(const uint4_t *)(vn + 16 * (n & 7) + 8);
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) kr[kk] = *(const uint4_t *)(kn + 32 * kk + 8 * g);
+      vr[0] = *(const uint4_t *)(vn + 8 * n);
+      vr[1] = uint4_t{0, 0, 0, 0};  // fp8 only
     }
   };
 
@@ -843,7 +907,35 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
 
   HeadState st;
   st.reset();
-  fetch_q(cur_b);
+  fetch_q_into(qf, cur_b);
+  // What the first sequence crossing and the first fused append of the chunk need is requested
+  // here, unconditionally and before the pages (loads return in order: by the time a page has
+  // arrived these have too), so neither waits for a load it has just issued. Later crossings and
+  // appends of the same chunk (sequences shorter than a chunk) load and wait. The registers are
+  // written once, outside the loop: written in a rarely taken branch of it they become
+  // two-versioned at the loop's join and the compiler copies them on every page.
+  uint4_t q_ahead[4];  // raw dwords: as fp16 vectors the compiler splits them into halves up here
+  uint4_t k_ahead[4];
+  uint4_t v_ahead[2];
+  int ahead_b = cur_b + 1;  // the next sequence with pages, or batch
+  if (ahead_b < batch && pages_of(len_after) <= skip) {  // empty sequences in between: rare
+    ++ahead_b;
+    while (ahead_b < batch && pages_of(lens[ahead_b]) <= skip) ++ahead_b;
+  }
+  {
+    // Every lane loads, lanes past the group the group's last head: their columns are computed
+    // and never stored. A load under a lane condition is merged with its zero default through
+    // register copies that wait for it, here in front of the first page requests.
+    const int nn = n < group ? n : group - 1;
+    const half_t *row = q + (int64_t)(ahead_b < batch ? ahead_b : cur_b) * q_batch_stride +
+                        (int64_t)(hq0 + nn) * kHeadDim + (FP8 ? 16 : 8) * g;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {  // the d order of load_q / load_q_fp8_order
+      q_ahead[kk] = *(const uint4_t *)(row + (FP8 ? 64 * (kk >> 1) + 8 * (kk & 1) : 32 * kk));
+    }
+  }
+  const int rows_b = k_new != nullptr ? cur_b : -1;
+  if (k_new != nullptr) fetch_new_rows(k_ahead, v_ahead, cur_b);
 
   auto flush = [&]() {
     // the sequence lies inside this chunk and has no shared-prefix partials to merge with
@@ -852,6 +944,27 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     half_t *out_row = out + ((int64_t)cur_b * num_q_heads + hq0) * kHeadDim;
     store_state(st, whole, out_row, part_o + cell * kHeadDim, kHeadDim, part_lse + cell, 1, n, g,
                 group, v_scale);
+  };
+  // A sequence that ends inside the chunk is parked (see park_state) and written with the
+  // chunk's last one; a second one ending in the same chunk first sends the parked one off.
+  float *park = park_all[wave];
+  int parked_b = -1;
+  bool parked_whole = false;
+  auto unpark = [&]() {
+    const int64_t cell = (int64_t)(cidx + parked_b) * num_q_heads + hq0;
+    half_t *out_row = out + ((int64_t)parked_b * num_q_heads + hq0) * kHeadDim;
+    unpark_state(park, parked_whole, out_row, part_o + cell * kHeadDim, part_lse + cell, n, g, group);
+    parked_b = -1;
+  };
+  auto flush_at_crossing = [&]() {
+    if (group > kParkHeads) {
+      flush();
+      return;
+    }
+    if (parked_b >= 0) unpark();
+    park_state(st, park, n, g, group, v_scale);
+    parked_b = cur_b;
+    parked_whole = cu_lo >= f0 && cu_hi <= f1 && skip == 0;
   };
 
   Page buf[DEPTH];
@@ -872,7 +985,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
       const int ff = f + dd;
       if (ff < f1) {
         if (ff >= cu_hi) {  // the line enters the next non-empty sequence
-          flush();
+          flush_at_crossing();
           do {
             ++cur_b;
             len_b = len_after;
@@ -883,9 +996,14 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
             cu_lo = cu_hi;
             cu_hi += pg;
           } while (ff >= cu_hi);
-          fetch_q(cur_b);
           st.reset();
-          wait_vector_loads();
+          if (cur_b == ahead_b) {
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) qf[kk] = __builtin_bit_cast(half8_t, q_ahead[kk]);
+          } else {
+            fetch_q_into(qf, cur_b);
+            wait_vector_loads();
+          }
         }
         const int p = ff - cu_lo + skip;  // page index inside the sequence
         if (k_new != nullptr && (p + 1) * kPageSize >= len_b) {
@@ -893,8 +1011,17 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
           // appended here. Its K and V rows go to the pool and replace the stale values this
           // wavefront requested before the write.
           const int t_new = (len_b - 1) & (kPageSize - 1);
-          const half_t *kn = k_new + (int64_t)cur_b * k_new_stride + (int64_t)h * kHeadDim;
-          const half_t *vn = v_new + (int64_t)cur_b * v_new_stride + (int64_t)h * kHeadDim;
+          uint4_t k_row[4];
+          uint4_t v_row[2];
+          if (cur_b == rows_b) {
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) k_row[kk] = k_ahead[kk];
+            v_row[0] = v_ahead[0];
+            v_row[1] = v_ahead[1];
+          } else {
+            fetch_new_rows(k_row, v_row, cur_b);
+            wait_vector_loads();
+          }
           const int pid = page_ids[ff - f0];
           const int64_t slot_off = ((int64_t)pid * kPageSize + t_new) * row_stride;
           if constexpr (FP8) {
@@ -903,16 +1030,16 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
               uint8_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 16 * g;
 #pragma unroll
               for (int j = 0; j < 2; ++j) {
-                const uint2_t lo = half8_to_fp8(*(const half8_t *)(kn + 64 * j + 16 * g), k_inv);
-                const uint2_t hi = half8_to_fp8(*(const half8_t *)(kn + 64 * j + 16 * g + 8), k_inv);
+                const uint2_t lo = half8_to_fp8(__builtin_bit_cast(half8_t, k_row[2 * j]), k_inv);
+                const uint2_t hi = half8_to_fp8(__builtin_bit_cast(half8_t, k_row[2 * j + 1]), k_inv);
                 const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
                 buf[dd].k[j] = x;
                 *(uint4_t *)(dst + 64 * j) = x;
               }
             }
             if (2 * g + (n >> 3) == (t_new & 7)) {
-              const uint2_t lo = half8_to_fp8(*(const half8_t *)(vn + 16 * (n & 7)), v_inv);
-              const uint2_t hi = half8_to_fp8(*(const half8_t *)(vn + 16 * (n & 7) + 8), v_inv);
+              const uint2_t lo = half8_to_fp8(__builtin_bit_cast(half8_t, v_row[0]), v_inv);
+              const uint2_t hi = half8_to_fp8(__builtin_bit_cast(half8_t, v_row[1]), v_inv);
               const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
               *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7)) = x;
 #pragma unroll
@@ -925,13 +1052,13 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
               half_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 8 * g;
 #pragma unroll
               for (int kk = 0; kk < 4; ++kk) {
-                const half8_t x = *(const half8_t *)(kn + 32 * kk + 8 * g);
+                const half8_t x = __builtin_bit_cast(half8_t, k_row[kk]);
                 buf[dd].k[kk] = x;
                 *(half8_t *)(dst + 32 * kk) = x;
               }
             }
             if (g == (t_new & 3)) {
-              const half8_t x = *(const half8_t *)(vn + 8 * n);
+              const half8_t x = __builtin_bit_cast(half8_t, v_row[0]);
               *(half8_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n) = x;
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
@@ -939,7 +1066,6 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
               }
             }
           }
-          wait_vector_loads();
         }
         attend_page(st, buf[dd], qf, vstage, vt_lane, p, len_b, n, g, scale_log2);
       }
@@ -947,6 +1073,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     }
   }
   flush();
+  if (parked_b >= 0) unpark();
 }
 
 }  // namespace litekv
