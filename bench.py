@@ -38,7 +38,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 # 1 GiB copy kernel); summaries and commands in profiles/paged_decode_balanced_c2_pmc.txt,
 # profiles/paged_decode_balanced_fp8_c2.txt and profiles/hbm_traffic_c3_c4_c5_pmc.txt. Only
 # meaningful for the workload it was measured on. c4: prefix kernel + decode kernel + merge.
-MEASURED_TRAFFIC_BYTES = {("c2", "balanced", "f16"): 317.9e6, ("c2", "balanced", "fp8"): 164.5e6,
+MEASURED_TRAFFIC_BYTES = {("c2", "balanced", "f16"): 317.8e6, ("c2", "balanced", "fp8"): 164.5e6,
                           ("c3", "balanced", "f16"): 387.7e6, ("c4", "balanced", "f16"): 150.6e6,
                           ("c5", "balanced", "f16"): 5196.0e6}
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
