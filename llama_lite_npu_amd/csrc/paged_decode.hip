@@ -324,9 +324,9 @@ __device__ __forceinline__ void park_state(const HeadState &st, float *park, int
 __device__ __forceinline__ void unpark_state(const float *park, bool final_row, half_t *out_row,
                                              float *part_row, float *part_lse_cell, int n, int g,
                                              int group) {
-  if (n >= group) return;
-  const float *row = park + n * kHeadDim + 4 * g;
   if (final_row) {
+    if (n >= group) return;
+    const float *row = park + n * kHeadDim + 4 * g;
     half_t *o = out_row + (int64_t)n * kHeadDim + 4 * g;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -334,10 +334,16 @@ __device__ __forceinline__ void unpark_state(const float *park, bool final_row, 
       *(half4_t *)(o + 16 * j) = half4_t{(half_t)x[0], (half_t)x[1], (half_t)x[2], (half_t)x[3]};
     }
   } else {
-    float *po = part_row + (int64_t)n * kHeadDim + 4 * g;
+    // The partial rows of the group's heads are one contiguous run in the workspace and in the
+    // parking area alike: the whole wavefront copies it 1 KiB per instruction.
+    wave_lds_fence();
+    const int lane = 16 * g + n;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) *(float4_t *)(po + 16 * j) = *(const float4_t *)(row + 16 * j);
-    if (g == 0) part_lse_cell[n] = park[kParkHeads * kHeadDim + n];
+    for (int i = 0; i < kParkHeads / 2; ++i) {
+      const int at = 4 * (64 * i + lane);
+      if (at < group * kHeadDim) *(float4_t *)(part_row + at) = *(const float4_t *)(park + at);
+    }
+    if (lane < group) part_lse_cell[lane] = park[kParkHeads * kHeadDim + lane];
   }
 }
 
