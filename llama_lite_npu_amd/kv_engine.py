@@ -15,6 +15,14 @@ from dataclasses import dataclass
 from typing import Iterable, Sequence
 
 
+def _checked(name: str, value, low: int = 1) -> int:
+    """`value` as int; ValueError("<name> must be positive" / "... non-negative") below `low`."""
+    number = int(value)
+    if number < low:
+        raise ValueError(f"{name} must be {'positive' if low == 1 else 'non-negative'}")
+    return number
+
+
 @dataclass(frozen=True)
 class PrefixCacheMatch:
     """Longest cached block-aligned prefix: token count and the logical blocks holding it."""
@@ -84,9 +92,7 @@ class KVBlockRefCounter:
     """Reference counts of logical KV blocks; free blocks are handed out lowest id first."""
 
     def __init__(self, total_blocks: int) -> None:
-        total_blocks = int(total_blocks)
-        if total_blocks < 1:
-            raise ValueError("total_blocks must be positive")
+        total_blocks = _checked("total_blocks", total_blocks)
         self._counts = [0] * total_blocks
         self._free = list(range(total_blocks))  # already a valid min-heap
 
@@ -102,9 +108,7 @@ class KVBlockRefCounter:
         return self._counts[self._index(block_id)]
 
     def acquire(self, count: int) -> tuple[int, ...]:
-        count = int(count)
-        if count < 1:
-            raise ValueError("count must be positive")
+        count = _checked("count", count)
         if count > len(self._free):
             raise RuntimeError(f"insufficient KV blocks: need {count}, available {len(self._free)}")
         taken = tuple(heapq.heappop(self._free) for _ in range(count))
@@ -140,9 +144,7 @@ class PrefixCache:
     first block that is not cached and never covers a partial block."""
 
     def __init__(self, block_size: int) -> None:
-        block_size = int(block_size)
-        if block_size < 1:
-            raise ValueError("block_size must be positive")
+        block_size = _checked("block_size", block_size)
         self.block_size = block_size
         self._blocks: dict[tuple[int, ...], int] = {}
 
@@ -174,14 +176,10 @@ class ChunkedPrefillPlanner:
     """Cuts a prompt into consecutive chunks of at most ``chunk_size`` tokens."""
 
     def __init__(self, chunk_size: int) -> None:
-        chunk_size = int(chunk_size)
-        if chunk_size < 1:
-            raise ValueError("chunk_size must be positive")
+        chunk_size = _checked("chunk_size", chunk_size)
         self.chunk_size = chunk_size
 
     def plan(self, prompt_length: int) -> tuple[PrefillChunk, ...]:
-        prompt_length = int(prompt_length)
-        if prompt_length < 0:
-            raise ValueError("prompt_length must be non-negative")
+        prompt_length = _checked("prompt_length", prompt_length, low=0)
         starts = range(0, prompt_length, self.chunk_size)
         return tuple(PrefillChunk(s, min(s + self.chunk_size, prompt_length)) for s in starts)
