@@ -660,6 +660,7 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
       if (quot == 0 && c >= rem) {  // a chunk without pages
         entries[(int64_t)c * entry_stride + 0] = 0;
         entries[(int64_t)c * entry_stride + 1] = 0;
+        entries[(int64_t)c * entry_stride + 5] = -1;
       }
     }
   }
@@ -685,6 +686,11 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
       e[2] = b;
       e[3] = before;
       e[4] = before + my_pages;
+      // for a merge by chunk boundary: the sequence whose pieces start in the chunk before this
+      // one and continue here, and how many chunks it spans (-1: none starts there)
+      const bool continues = before < f && chunk_of(before) == c - 1;
+      e[5] = continues ? b : -1;
+      e[6] = continues ? chunk_of(before + my_pages - 1) - (c - 1) + 1 : 0;
     }
   }
 }
@@ -757,7 +763,9 @@ __device__ __forceinline__ void merge_row_wide(const float *__restrict__ lse, in
   *(half2_t *)(out_row + 2 * lane) = half2_t{(half_t)(o0 * inv), (half_t)(o1 * inv)};
 }
 
-// Balanced-schedule merge, one workgroup per (query head, sequence): combines the sequence's
+// Balanced-schedule merge, one workgroup per (query head, sequence) -- or, without a shared
+// prefix and with more sequences than chunk boundaries, per (query head, boundary): only a
+// sequence that crosses a boundary has pieces to merge -- : combines the sequence's
 // pieces (partial slots c_first + b, c_first + b + 1, ...) if it spans several chunks, and the
 // `pre_splits` partials of the shared prefix if there is one. Up to 16 pieces (and any number
 // with a shared prefix) are merged by the first wavefront alone.
@@ -765,12 +773,26 @@ __global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merg
     const int32_t *__restrict__ plan, const int32_t *__restrict__ seq_lens,
     half_t *__restrict__ out, const float *__restrict__ part_o,
     const float *__restrict__ part_lse, const float *__restrict__ pre_o,
-    const float *__restrict__ pre_lse, int32_t pre_splits, int32_t batch, int32_t num_q_heads) {
+    const float *__restrict__ pre_lse, int32_t pre_splits, int32_t batch, int32_t num_q_heads,
+    int32_t by_boundary, int32_t bt_stride, int32_t chunks, int32_t heads_per_wg) {
   __shared__ float red[8 + kMergeWaves * kHeadDim + kMergeWaves];
-  const int hq = blockIdx.x;
-  const int b = blockIdx.y;
-  const int c_first = plan[plan_seq_info_offset() + 2 * b];
-  const int n_parts = plan[plan_seq_info_offset() + 2 * b + 1];
+  // heads_per_wg 1: the workgroup has one row (query head); 4: each wavefront has its own
+  const int hq = blockIdx.x * heads_per_wg + (heads_per_wg > 1 ? (int)(threadIdx.x >> 6) : 0);
+  int b = blockIdx.y;
+  int c_first, n_parts;
+  if (by_boundary) {
+    // blockIdx.y names the boundary between chunks y and y + 1; the header of chunk y + 1 says
+    // which sequence, if any, has its first piece in chunk y and goes on (decode_plan_kernel).
+    const int32_t *e = plan + plan_entries_offset(batch) +
+                       (int64_t)(blockIdx.y + 1) * plan_entry_stride(batch, bt_stride, chunks);
+    b = e[5];
+    if (b < 0) return;
+    c_first = blockIdx.y;
+    n_parts = e[6];
+  } else {
+    c_first = plan[plan_seq_info_offset() + 2 * b];
+    n_parts = plan[plan_seq_info_offset() + 2 * b + 1];
+  }
   if (pre_splits == 0 && n_parts <= 1) return;  // empty, or written directly by the decode kernel
   if (pre_splits != 0 && seq_lens[b] <= 0) return;  // the decode kernel zeroed the row
   const int64_t cell0 = (int64_t)(c_first + b) * num_q_heads + hq;
@@ -778,19 +800,26 @@ __global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merg
   const int64_t pre_step = (int64_t)batch * num_q_heads;
   half_t *out_row = out + ((int64_t)b * num_q_heads + hq) * kHeadDim;
   if (pre_splits == 0 && n_parts > 16 && blockDim.x == kMergeWaves * kWave) {  // uniform in the workgroup
-    merge_row_wide(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
-                   (int64_t)num_q_heads * kHeadDim, n_parts, out_row, threadIdx.x, red);
+    // a long row takes the whole workgroup; with a row per wavefront the rows take turns
+    for (int r = 0; r < heads_per_wg; ++r) {
+      const int shift = heads_per_wg > 1 ? r - (int)(threadIdx.x >> 6) : 0;  // from this wavefront's row to row r
+      merge_row_wide(part_lse + cell0 + shift, num_q_heads, part_o + (cell0 + shift) * kHeadDim,
+                     (int64_t)num_q_heads * kHeadDim, n_parts, out_row + (int64_t)shift * kHeadDim,
+                     threadIdx.x, red);
+      __syncthreads();
+    }
     return;
   }
-  if (threadIdx.x >= kWave) return;
+  if (heads_per_wg == 1 && threadIdx.x >= kWave) return;
+  const int lane = threadIdx.x & (kWave - 1);
   if (pre_splits == 0) {
     merge_row<false>(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
                      (int64_t)num_q_heads * kHeadDim, n_parts, nullptr, 0, nullptr, 0, 0, out_row,
-                     threadIdx.x);
+                     lane);
   } else {
     merge_row<true>(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
                     (int64_t)num_q_heads * kHeadDim, n_parts, pre_lse + pre0, pre_step,
-                    pre_o + pre0 * kHeadDim, pre_step * kHeadDim, pre_splits, out_row, threadIdx.x);
+                    pre_o + pre0 * kHeadDim, pre_step * kHeadDim, pre_splits, out_row, lane);
   }
 }
 
@@ -1443,11 +1472,28 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   // and only cost their dispatch (C4: 9.9 -> 7 us).
   const int max_pieces = chunks < block_table_stride ? chunks : block_table_stride;
   const int merge_waves = (pre_splits == 0 && max_pieces > 16) ? kMergeWaves : 1;
+  // Sequences inside one chunk were written by the decode kernel; at most chunks - 1 sequences
+  // cross a chunk boundary. A batch of twice as many is merged by boundary (B 1024 of up to 40
+  // tokens: layer 58.7 -> 50.0 us; at B 256..300 one workgroup per sequence is still faster).
+  const bool by_boundary = pre_splits == 0 && batch >= 2 * chunks;
+  const int merge_rows = by_boundary ? chunks - 1 : batch;
+  if (merge_rows == 0) {
+    clear_error();
+    return LITEKV_OK;
+  }
+  // Many short rows are bound by the dispatch of their workgroups: four rows per workgroup then,
+  // one per wavefront (B 256 of up to 256 tokens: layer 53.5 -> 47.2 us).
+  const int merge_heads = (merge_waves == kMergeWaves && num_q_heads % kMergeWaves == 0 &&
+                           (int64_t)merge_rows * num_q_heads >= 8192)
+                              ? kMergeWaves
+                              : 1;
   hipLaunchKernelGGL(paged_decode_balanced_merge_kernel,
-                     dim3((unsigned)num_q_heads, (unsigned)batch), dim3(merge_waves * kWave), 0,
+                     dim3((unsigned)(num_q_heads / merge_heads), (unsigned)merge_rows),
+                     dim3(merge_waves * kWave), 0,
                      static_cast<hipStream_t>(stream), static_cast<const int32_t *>(plan), seq_lens,
                      static_cast<half_t *>(out), part_o, part_lse, pre_o, pre_lse, pre_splits,
-                     batch, num_q_heads);
+                     batch, num_q_heads, by_boundary ? 1 : 0, block_table_stride, chunks,
+                     merge_heads);
   return check_launch("paged_decode_balanced_merge");
 }
 }  // namespace litekv

@@ -126,3 +126,30 @@ def test_random_steps_behind_a_shared_prefix(seed):
         torch.cuda.synchronize()
         assert torch.equal(case.kv_pool.view(torch.int16), pool_ref.view(torch.int16))
         assert_attention_close(out, ref, f"random prefix step {seed}.{case_no}")
+
+
+@pytest.mark.parametrize("batch", [200, 600])
+def test_large_batches_take_the_packed_merge(batch):
+    """More than 8192 (sequence, head) rows: four rows per merge workgroup; more sequences than
+    twice the chunk boundaries (600 >= 512): merge by boundary. One long sequence among the short ones spans
+    more than 16 chunks, so the long-row merge runs inside the packed launch too."""
+    rng = random.Random(500 + batch)
+    lens = [rng.randint(0, 300 if batch < 400 else 90) for _ in range(batch)]
+    lens[batch // 3] = 6000
+    lens[5] = 0
+    print(f"large batch {batch}", flush=True)
+    case = workloads.make_decode_case("large", 9000 + batch, lens, 64, 8, device=DEV)
+    case.seq_lens[11] = 0                     # an empty row
+    pool_ref = case.kv_pool.clone()
+    ops.kv_append(case.k_new, case.v_new, case.slot_mapping, pool_ref)
+    ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool_ref), case.block_table.cpu().numpy(),
+                                case.seq_lens.cpu().numpy(), case.softmax_scale)
+    plan = ops.DecodePlan(case.block_table, case.seq_lens, 64, 8, case.num_pages)
+    assert plan.chunks == 256
+    out = ops.decode_step(case.q, case.kv_pool, plan, case.k_new, case.v_new, case.softmax_scale)
+    again = ops.decode_step(case.q, case.kv_pool, plan, None, None, case.softmax_scale)
+    torch.cuda.synchronize()
+    assert_attention_close(out, ref, f"large batch {batch}")
+    assert float(out[11].abs().max()) == 0.0
+    live = [i for i in range(batch) if i != 11]
+    assert torch.equal(again[live], out[live])
