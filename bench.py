@@ -10,7 +10,7 @@ KV append of the batch's new tokens fused into paged flash-decoding, and the
 merge of its partial results. All inputs are resident in HBM before the timed
 region. One JSON line is printed on
 stdout; `--all` adds one line per other configuration on stderr and in
-gpurun_out/bench_all.jsonl.
+`bench_all.jsonl` under `--out-dir`.
 
 `value` is algorithmic bytes of the whole step divided by its wall-clock time.
 `roofline` describes the dominant kernel (the decode kernel): algorithmic bytes
@@ -574,6 +574,8 @@ def main() -> int:
                     help="storage of the KV pools (fp8: E4M3 codes with per-head scales; decode configs only)")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the leg that replays the decode step as one HIP graph")
+    ap.add_argument("--out-dir", default="gpurun_out",
+                    help="where --all writes bench_all.jsonl (relative to the repository root)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one page_gather of exactly 1 GiB (read) + 1 GiB (write): a plain copy of "
                          "known size against which profiler byte counters can be scaled")
@@ -691,8 +693,8 @@ def main() -> int:
     print(json.dumps(line), flush=True)
 
     if args.all:
-        out_dir = ROOT / "gpurun_out"
-        out_dir.mkdir(exist_ok=True)
+        out_dir = ROOT / args.out_dir
+        out_dir.mkdir(parents=True, exist_ok=True)
         with open(out_dir / "bench_all.jsonl", "w") as f:
             f.write(json.dumps(line) + "\n")
             for name in ("c1", "c2", "c3", "c4", "c5"):
