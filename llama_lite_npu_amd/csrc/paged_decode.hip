@@ -846,13 +846,16 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   half_t *vstage = vstage_all[wave];
 
   // Empty sequences are on no chunk's line: chunk c zeroes the rows of sequences c, c + chunks, ...
-  for (int bz = cidx; bz < batch; bz += chunks) {
-    if (seq_lens[bz] <= 0 && n < group) {
-      half_t *o = out + ((int64_t)bz * num_q_heads + h * group + n) * kHeadDim + 4 * g;
+  // Like every store of this kernel it comes after the page loop (see park_state).
+  auto zero_empty_rows = [&]() {
+    for (int bz = cidx; bz < batch; bz += chunks) {
+      if (seq_lens[bz] <= 0 && n < group) {
+        half_t *o = out + ((int64_t)bz * num_q_heads + h * group + n) * kHeadDim + 4 * g;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) *(half4_t *)(o + 16 * j) = half4_t{0, 0, 0, 0};
+        for (int j = 0; j < 8; ++j) *(half4_t *)(o + 16 * j) = half4_t{0, 0, 0, 0};
+      }
     }
-  }
+  };
 
   const int entry_stride = plan_entry_stride(batch, bt_stride, chunks);
   const uniform_i32_ptr lens = as_uniform(seq_lens);
@@ -860,7 +863,10 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
       as_uniform(plan) + plan_entries_offset(batch) + (int64_t)cidx * entry_stride;
   const int f0 = entry[0];
   const int f1 = entry[1];
-  if (f1 <= f0) return;
+  if (f1 <= f0) {
+    zero_empty_rows();
+    return;
+  }
   int cur_b = entry[2];
   int cu_lo = entry[3];  // current sequence: [first, last) page on the line
   int cu_hi = entry[4];
@@ -1109,6 +1115,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   }
   flush();
   if (parked_b >= 0) unpark();
+  zero_empty_rows();
 }
 
 }  // namespace litekv
