@@ -418,6 +418,28 @@ int litekv_paged_prefill(const void *q, int64_t q_token_stride,
                          int32_t max_q_len, float softmax_scale, void *stream);
 
 /*
+ * The same over an fp8 (E4M3) pool with per-head scales (kv_scales: float32
+ * [2 * Hkv], K heads then V heads, value = code * scale), as written by
+ * litekv_kv_append_fp8: the chunk rows of a chunked prefill or of a
+ * prefix-cache hit attend to their history without the pages being
+ * dequantised first (the reference has no counterpart; its paged chunk kernel,
+ * lite_llama/kernels/paged_chunk_flashattention.py:225-327, reads fp16 only).
+ * The codes are converted exactly; the K scale is applied to the scores and
+ * the V scale to the normalised output in fp32.
+ */
+int litekv_paged_prefill_fp8(const void *q, int64_t q_token_stride,
+                             const void *kv_pool, const float *kv_scales,
+                             const int32_t *block_table,
+                             int32_t block_table_stride,
+                             const int32_t *cu_q_lens,
+                             const int32_t *context_lens, void *out,
+                             int64_t out_token_stride, int32_t batch,
+                             int32_t num_q_heads, int32_t num_kv_heads,
+                             int32_t head_dim, int32_t page_size,
+                             int64_t num_pages, int32_t max_q_len,
+                             float softmax_scale, void *stream);
+
+/*
  * Varlen causal prefill over packed contiguous K/V. Replaces
  * `flash_attention2_no_pad(q, k, v, sm_scale, b_start_loc, b_seq_len,
  * max_seq_len)` (lite_llama/kernels/flashattention2_nopad.py:169-221) for

@@ -118,6 +118,11 @@ SIGNATURES = {
         [c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
          c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_float, c_void_p],
     ),
+    "litekv_paged_prefill_fp8": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
+         c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_float, c_void_p],
+    ),
     "litekv_varlen_prefill": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p,

@@ -71,18 +71,13 @@ class Attention:
                 # a fresh prompt attends to its own K/V as computed, not as stored
                 return ops.varlen_prefill(xq, xk, xv, atten_info.b_start_loc, atten_info.seq_lens_i32,
                                           int(atten_info.max_actual_seq_len), scale)
-        # history (or rows already stored by the epilogue): decode the batch's pages into a scratch pool
-        table = atten_info.block_table
-        b, width = table.shape
-        scratch = torch.empty((b * width * ops.PAGE_SIZE, 2 * self.num_kv_heads, self.head_dim),
-                              dtype=torch.float16, device=xq.device)
-        ops.page_dequant(pool, scratch, table.reshape(-1), None, scales)
-        local = torch.arange(b * width, dtype=torch.int32, device=xq.device).view(b, width)
+        # history (or rows already stored by the epilogue): the kernel reads the codes themselves
         if chunked:
-            return ops.paged_prefill(xq, scratch, local, atten_info.cu_q_lens, atten_info.context_lens_i32,
-                                     int(atten_info.max_actual_q_seq_len), scale)
-        return ops.paged_prefill(xq, scratch, local, atten_info.cu_q_lens, None,
-                                 int(atten_info.max_actual_seq_len), scale)
+            return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens,
+                                     atten_info.context_lens_i32, int(atten_info.max_actual_q_seq_len), scale,
+                                     kv_scales=scales)
+        return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens, None,
+                                 int(atten_info.max_actual_seq_len), scale, kv_scales=scales)
 
     def token_forward(self, xq, xk, xv, atten_info, layer_index: int, qk_scale=None) -> torch.Tensor:
         """Decode: xq [B, Hq, D], xk / xv [B, Hkv, D], one new token per sequence (None when

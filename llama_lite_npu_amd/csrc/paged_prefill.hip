@@ -40,6 +40,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "kv_fp8.h"
 
 namespace litekv {
 
@@ -47,11 +48,12 @@ constexpr float kLog2eP = 1.4426950408889634f;
 
 // Where the keys of a sequence live.
 struct PagedSource {
-  const half_t *kv;             // pool [slots][2*Hkv][128]
+  const half_t *kv;             // pool [slots][2*Hkv][128], fp16 (or E4M3 codes, one byte each)
   const int32_t *block_table;   // [B][stride]
   int32_t bt_stride;
   int32_t num_kv_heads;
   int32_t num_pages;
+  const float *scales;          // fp8 pool: value = code * scale, K heads then V heads
 };
 // Shared-prefix decode (mode kSharedPrefix): the columns are (sequence, query head) pairs of one
 // decode step, the keys are a slice of the pages every sequence starts with, and the result is
@@ -103,7 +105,7 @@ __device__ __forceinline__ float max_across_groups(float x) {
   s = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
   return vmax2(__builtin_bit_cast(float, s[0]), __builtin_bit_cast(float, s[1]));
 }
-constexpr int kPagedPrefill = 0, kPackedPrefill = 1, kSharedPrefix = 2;
+constexpr int kPagedPrefill = 0, kPackedPrefill = 1, kSharedPrefix = 2, kPagedPrefillFp8 = 3;
 
 template <int MODE>
 __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_kernel(
@@ -113,6 +115,11 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     const int32_t *__restrict__ context_lens, int32_t group, int32_t head_splits,
     int32_t heads_per_wg, int32_t row_tiles, float scale_log2) {
   constexpr bool PAGED = MODE != kPackedPrefill;
+  // An fp8 pool cannot take the direct HBM -> LDS load: its codes go through registers, are
+  // converted to fp16 (exactly) and written to LDS in the same swizzled layout, so everything
+  // after the staging is shared. The K scale joins the softmax scale, the V scale the final
+  // normalisation, as in the decode kernel.
+  constexpr bool FP8 = MODE == kPagedPrefillFp8;
   // Two tiles of K and two of V: tile t sits in half t % 2.
   __shared__ __attribute__((aligned(1024))) half_t kbuf[2 * kTileHalfs];
   __shared__ __attribute__((aligned(1024))) half_t vbuf[2 * kTileHalfs];
@@ -128,6 +135,11 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   const int head0 = ((int)blockIdx.x - h * head_splits) * heads_per_wg;
   const int heads_here = (group - head0) < heads_per_wg ? (group - head0) : heads_per_wg;
   const int b = blockIdx.z;
+  float v_scale = 1.0f;
+  if constexpr (FP8) {
+    scale_log2 *= paged.scales[h];
+    v_scale = paged.scales[paged.num_kv_heads + h];
+  }
 
   // What the block works on: query rows m0.. of sequence b (prefill), or the column block
   // blockIdx.y of all (sequence, head) pairs against key slice blockIdx.z (shared prefix).
@@ -168,7 +180,8 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   // wavefront): lane l writes slot l % 16 of row 4i + l / 16.
   const int r_loc = lane >> 4;
   const int slot = lane & 15;
-  const uint32_t k_pitch = PAGED ? 2u * paged.num_kv_heads * kHeadDim * 2u : (uint32_t)packed.k_stride * 2u;
+  const uint32_t k_pitch = PAGED ? 2u * paged.num_kv_heads * kHeadDim * (FP8 ? 1u : 2u)
+                                 : (uint32_t)packed.k_stride * 2u;
   const uint32_t v_pitch = PAGED ? k_pitch : (uint32_t)packed.v_stride * 2u;
   uint32_t koff[4], voff[4];  // byte offsets from the wavefront's 16-row base
 #pragma unroll
@@ -187,8 +200,28 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   // Starts the loads of tile kt into its LDS half. The instruction is written as asm so that the
   // compiler does not make later LDS reads of the *other* half wait for it; the wait is the
   // explicit vmcnt(0) before the barrier that publishes the tile.
+  uint4_t raw_k[2], raw_v[2];  // fp8: this lane's 32 codes of K and of V of the tile requested last
   auto issue_tile = [&](int kt) {
     const int row0 = (tile0 + kt) * kKvTile + 16 * wave;  // first key of this wavefront's 16 rows
+    if constexpr (FP8) {
+      // lane l: row l / 4 of the wavefront's page, codes 32 * (l % 4) .. +31 of the head's row
+      int pidx = (tile0 + kt) * 4 + wave;
+      pidx = pidx < last_page ? pidx : last_page;
+      int pid = table[pidx];
+      pid = pid < 0 ? 0 : (pid >= paged.num_pages ? paged.num_pages - 1 : pid);
+      int tok = row0 + (lane >> 2);
+      tok = tok < last_key ? tok : last_key;  // rows past the last key re-read it
+      const int src_row = tok - pidx * kPageSize;
+      const uint8_t *base = (const uint8_t *)paged.kv +
+                            ((int64_t)pid * kPageSize + src_row) * (int64_t)k_pitch + 32 * (lane & 3);
+      const uint8_t *kp = base + h * kHeadDim;
+      const uint8_t *vp = base + (paged.num_kv_heads + h) * kHeadDim;
+      raw_k[0] = *(const uint4_t *)kp;
+      raw_k[1] = *(const uint4_t *)(kp + 16);
+      raw_v[0] = *(const uint4_t *)vp;
+      raw_v[1] = *(const uint4_t *)(vp + 16);
+      return;
+    }
     const char *kbase, *vbase;
     int src0;  // key index the bases point at
     if (PAGED) {
@@ -381,6 +414,21 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
 
   // Publishes tile kt (already requested) and requests tile kt + 1 into the other half.
   auto sync_and_prefetch = [&](int kt) {
+    if constexpr (FP8) {
+      // The codes of tile kt (requested a tile ago) become fp16 rows in its LDS half: 16-byte
+      // chunk c of row r goes where the direct load of the fp16 path would have put it.
+      const int r = lane >> 2;
+      const uint32_t row_at = (uint32_t)((kt & 1) * kTileHalfs + (16 * wave + r) * kHeadDim) * 2u;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int chunk = 4 * (lane & 3) + j;
+        const uint4_t ck = raw_k[j >> 1], cv = raw_v[j >> 1];
+        const half8_t kh = fp8x8_to_half((j & 1) ? uint2_t{ck[2], ck[3]} : uint2_t{ck[0], ck[1]});
+        const half8_t vh = fp8x8_to_half((j & 1) ? uint2_t{cv[2], cv[3]} : uint2_t{cv[0], cv[1]});
+        *(lds_half8_t *)(uintptr_t)(k_lds + row_at + 16u * (uint32_t)(chunk ^ r)) = kh;
+        *(lds_half8_t *)(uintptr_t)(v_lds + row_at + 16u * (uint32_t)(chunk ^ (2 * (r & 7)))) = vh;
+      }
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's part of tile kt is in LDS
     __syncthreads();                     // ... and everyone's; everyone is done with tile kt-1
     if (kt + 1 < n_tiles) issue_tile(kt + 1);
@@ -487,7 +535,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
 
 #pragma unroll
   for (int u = 0; u < kColTiles; ++u) {
-    const float inv = 1.0f / dsum[u][0];
+    const float inv = v_scale / dsum[u][0];
     if constexpr (MODE == kSharedPrefix) {
       if (out_row[u] >= 0) {
         const int64_t cell =
@@ -572,7 +620,7 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
   keys_per_split = (keys_per_split + kKvTile - 1) / kKvTile * kKvTile;
   splits = (prefix_keys + keys_per_split - 1) / keys_per_split;
   PagedSource paged{static_cast<const half_t *>(kv_pool), block_table, 0, num_kv_heads,
-                    (int32_t)num_pages};
+                    (int32_t)num_pages, nullptr};
   PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
   PrefixTask task{part_o, part_lse, q_batch_stride, batch, num_q_heads, prefix_keys, keys_per_split};
   hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kSharedPrefix>,
@@ -587,6 +635,56 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
 
 }  // namespace litekv
 
+namespace litekv {
+// Causal chunk attention over paged KV; `kv_scales` selects the fp8 pool.
+static int launch_paged_prefill(const char *what, const void *q, int64_t q_token_stride,
+                                const void *kv_pool, const float *kv_scales,
+                                const int32_t *block_table, int32_t block_table_stride,
+                                const int32_t *cu_q_lens, const int32_t *context_lens, void *out,
+                                int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
+                                int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                                int64_t num_pages, int32_t max_q_len, float softmax_scale,
+                                void *stream, bool fp8) {
+  int rc = validate_prefill(what, q, q_token_stride, out, out_token_stride, batch, num_q_heads,
+                            num_kv_heads, head_dim, max_q_len);
+  if (rc != LITEKV_OK) return rc;
+  LITEKV_REQUIRE(page_size == kPageSize, "%s: page_size %d unsupported (only %d)", what, page_size,
+                 kPageSize);
+  if (batch == 0 || max_q_len == 0) {
+    clear_error();
+    return LITEKV_OK;
+  }
+  LITEKV_REQUIRE(kv_pool && block_table && cu_q_lens, "%s: null pointer", what);
+  LITEKV_REQUIRE(!fp8 || kv_scales, "%s: null pointer (kv_scales)", what);
+  LITEKV_REQUIRE(aligned16(kv_pool), "%s: kv_pool must be 16-byte aligned", what);
+  LITEKV_REQUIRE(block_table_stride >= 1, "%s: block_table_stride %d < 1", what, block_table_stride);
+  LITEKV_REQUIRE(num_pages >= 1 && num_pages <= 0x7fffffffLL / kPageSize,
+                 "%s: num_pages %lld out of range", what, (long long)num_pages);
+  LITEKV_REQUIRE(num_kv_heads <= 1024, "%s: num_kv_heads %d > 1024", what, num_kv_heads);
+  PagedSource paged{static_cast<const half_t *>(kv_pool), block_table, block_table_stride,
+                    num_kv_heads, (int32_t)num_pages, kv_scales};
+  PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
+  const int group = num_q_heads / num_kv_heads;
+  const PrefillShape s = prefill_shape(group, max_q_len);
+  LITEKV_REQUIRE(s.row_blocks <= 65535u, "%s: max_q_len %d too large", what, max_q_len);
+  const dim3 grid((unsigned)(num_kv_heads * s.head_splits), s.row_blocks, (unsigned)batch);
+  if (fp8) {
+    hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kPagedPrefillFp8>, grid, dim3(kTiledWaves * kWave),
+                       0, static_cast<hipStream_t>(stream), static_cast<const half_t *>(q),
+                       q_token_stride, static_cast<half_t *>(out), out_token_stride, paged, packed,
+                       PrefixTask{}, cu_q_lens, (const int32_t *)nullptr, context_lens, group,
+                       s.head_splits, s.heads_per_wg, s.row_tiles, softmax_scale * kLog2eP);
+  } else {
+    hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kPagedPrefill>, grid, dim3(kTiledWaves * kWave), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const half_t *>(q),
+                       q_token_stride, static_cast<half_t *>(out), out_token_stride, paged, packed,
+                       PrefixTask{}, cu_q_lens, (const int32_t *)nullptr, context_lens, group,
+                       s.head_splits, s.heads_per_wg, s.row_tiles, softmax_scale * kLog2eP);
+  }
+  return check_launch(what);
+}
+}  // namespace litekv
+
 extern "C" int litekv_paged_prefill(const void *q, int64_t q_token_stride, const void *kv_pool,
                                     const int32_t *block_table, int32_t block_table_stride,
                                     const int32_t *cu_q_lens, const int32_t *context_lens,
@@ -594,37 +692,24 @@ extern "C" int litekv_paged_prefill(const void *q, int64_t q_token_stride, const
                                     int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                                     int32_t page_size, int64_t num_pages, int32_t max_q_len,
                                     float softmax_scale, void *stream) {
-  using namespace litekv;
-  int rc = validate_prefill("paged_prefill", q, q_token_stride, out, out_token_stride, batch,
-                            num_q_heads, num_kv_heads, head_dim, max_q_len);
-  if (rc != LITEKV_OK) return rc;
-  LITEKV_REQUIRE(page_size == kPageSize, "paged_prefill: page_size %d unsupported (only %d)",
-                 page_size, kPageSize);
-  if (batch == 0 || max_q_len == 0) {
-    clear_error();
-    return LITEKV_OK;
-  }
-  LITEKV_REQUIRE(kv_pool && block_table && cu_q_lens, "paged_prefill: null pointer");
-  LITEKV_REQUIRE(aligned16(kv_pool), "paged_prefill: kv_pool must be 16-byte aligned");
-  LITEKV_REQUIRE(block_table_stride >= 1, "paged_prefill: block_table_stride %d < 1",
-                 block_table_stride);
-  LITEKV_REQUIRE(num_pages >= 1 && num_pages <= 0x7fffffffLL / kPageSize,
-                 "paged_prefill: num_pages %lld out of range", (long long)num_pages);
-  LITEKV_REQUIRE(num_kv_heads <= 1024, "paged_prefill: num_kv_heads %d > 1024", num_kv_heads);
-  PagedSource paged{static_cast<const half_t *>(kv_pool), block_table, block_table_stride,
-                    num_kv_heads, (int32_t)num_pages};
-  PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
-  const int group = num_q_heads / num_kv_heads;
-  const PrefillShape s = prefill_shape(group, max_q_len);
-  LITEKV_REQUIRE(s.row_blocks <= 65535u, "paged_prefill: max_q_len %d too large", max_q_len);
-  hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kPagedPrefill>,
-                     dim3((unsigned)(num_kv_heads * s.head_splits), s.row_blocks, (unsigned)batch),
-                     dim3(kTiledWaves * kWave), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
-                     out_token_stride, paged, packed, PrefixTask{}, cu_q_lens, (const int32_t *)nullptr,
-                     context_lens, group, s.head_splits, s.heads_per_wg, s.row_tiles,
-                     softmax_scale * kLog2eP);
-  return check_launch("paged_prefill");
+  return litekv::launch_paged_prefill("paged_prefill", q, q_token_stride, kv_pool, nullptr, block_table,
+                                      block_table_stride, cu_q_lens, context_lens, out,
+                                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
+                                      page_size, num_pages, max_q_len, softmax_scale, stream, false);
+}
+
+extern "C" int litekv_paged_prefill_fp8(const void *q, int64_t q_token_stride, const void *kv_pool,
+                                        const float *kv_scales, const int32_t *block_table,
+                                        int32_t block_table_stride, const int32_t *cu_q_lens,
+                                        const int32_t *context_lens, void *out,
+                                        int64_t out_token_stride, int32_t batch,
+                                        int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                        int32_t page_size, int64_t num_pages, int32_t max_q_len,
+                                        float softmax_scale, void *stream) {
+  return litekv::launch_paged_prefill("paged_prefill_fp8", q, q_token_stride, kv_pool, kv_scales,
+                                      block_table, block_table_stride, cu_q_lens, context_lens, out,
+                                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
+                                      page_size, num_pages, max_q_len, softmax_scale, stream, true);
 }
 
 extern "C" int litekv_varlen_prefill(const void *q, int64_t q_token_stride, const void *k,
@@ -651,7 +736,7 @@ extern "C" int litekv_varlen_prefill(const void *q, int64_t q_token_stride, cons
   LITEKV_REQUIRE(k_token_stride < (1 << 25) && v_token_stride < (1 << 25),
                  "varlen_prefill: k/v token strides (%lld, %lld) too large",
                  (long long)k_token_stride, (long long)v_token_stride);
-  PagedSource paged{nullptr, nullptr, 0, num_kv_heads, 1};
+  PagedSource paged{nullptr, nullptr, 0, num_kv_heads, 1, nullptr};
   PackedSource packed{static_cast<const half_t *>(k), static_cast<const half_t *>(v),
                       k_token_stride, v_token_stride, seq_starts};
   const int group = num_q_heads / num_kv_heads;

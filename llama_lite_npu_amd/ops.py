@@ -460,12 +460,19 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
 def paged_prefill(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tensor,
                   cu_q_lens: torch.Tensor, context_lens: Optional[torch.Tensor], max_q_len: int,
                   softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
-                  page_size: int = PAGE_SIZE) -> torch.Tensor:
-    """Causal varlen attention of packed q [T, Hq, D] over paged KV (history + the chunk itself)."""
-    _dev_half("q", q), _dev_half("kv_pool", kv_pool)
+                  page_size: int = PAGE_SIZE, kv_scales: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal varlen attention of packed q [T, Hq, D] over paged KV (history + the chunk itself).
+    An fp8 pool (uint8 / float8_e4m3fn) comes with its per-head ``kv_scales``."""
+    _dev_half("q", q)
+    fp8 = is_fp8_pool(kv_pool)
+    if not fp8:
+        _dev_half("kv_pool", kv_pool)
+        _need(kv_scales is None, "kv_scales belong to an fp8 pool")
     q_stride = _rows("q", q)
     t, hq, d = q.shape
     _, hkv, dk, n_pages, _ = pool_geometry(kv_pool, page_size)
+    if fp8:
+        _dev_fp8_pool(kv_pool, kv_scales, hkv)
     _need(d == dk, "q and kv_pool differ in head_dim")
     cu_q_lens = _dev_i32("cu_q_lens", cu_q_lens)
     b = cu_q_lens.numel() - 1
@@ -479,6 +486,12 @@ def paged_prefill(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Ten
     if out is None:
         out = torch.empty((t, hq, d), dtype=torch.float16, device=q.device)
     lib = _lib.load()
+    if fp8:
+        _lib.check(lib.litekv_paged_prefill_fp8(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(block_table),
+                                                block_table.stride(0), _ptr(cu_q_lens), _ptr(context_lens),
+                                                _ptr(out), _rows("out", out), b, hq, hkv, d, page_size, n_pages,
+                                                int(max_q_len), float(softmax_scale), _stream()))
+        return out
     _lib.check(lib.litekv_paged_prefill(_ptr(q), q_stride, _ptr(kv_pool), _ptr(block_table),
                                         block_table.stride(0), _ptr(cu_q_lens), _ptr(context_lens),
                                         _ptr(out), _rows("out", out), b, hq, hkv, d, page_size, n_pages,

@@ -370,3 +370,44 @@ def test_fused_epilogue_into_an_fp8_pool_equals_epilogue_then_quantising_append(
     assert torch.equal(pool_c, pool_d)
     with pytest.raises(ValueError, match="scales"):
         ops.qk_norm_rope_append(q.clone(), k, v, slots, pool_c)
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_chunk_prefill_reads_an_fp8_pool_directly(seed):
+    """Chunk rows over an fp8 history (and their own rows, appended as codes): the oracle on the
+    decoded pool, within the attention tolerance; agrees with dequantising the pages first."""
+    import random
+    from llama_lite_npu_amd import workloads
+
+    rng = random.Random(600 + seed)
+    for case_no in range(6):
+        hq, hkv = rng.choice([(64, 8), (32, 4), (16, 8), (8, 8), (4, 2), (16, 1)])
+        b = rng.choice([1, 2, 4])
+        edges = [1, 15, 16, 17, 63, 64, 65, 128]
+        q_lens = [rng.choice([rng.choice(edges), rng.randint(1, 300)]) for _ in range(b)]
+        ctx = [rng.choice([0, rng.choice(edges), rng.randint(0, 900)]) for _ in range(b)]
+        print(f"fp8 chunk prefill {seed}.{case_no}: heads {hq}/{hkv} chunks {q_lens} histories {ctx}", flush=True)
+        case = workloads.make_prefill_case("fp8", 8000 + 100 * seed + case_no, q_lens, hq, hkv, context_lens=ctx,
+                                           device=DEV)
+        scales = torch.cat([0.02 * (1 + 0.1 * torch.arange(hkv)), 0.015 * (1 + 0.2 * torch.arange(hkv))]).float().to(DEV)
+        pool = torch.empty(case.kv_pool.shape, dtype=torch.uint8, device=DEV)
+        every_slot = torch.arange(pool.shape[0], dtype=torch.int32, device=DEV)
+        ops.kv_append_fp8(case.kv_pool[:, :hkv], case.kv_pool[:, hkv:], every_slot, pool, scales)   # the history
+        ops.kv_append_fp8(case.k, case.v, case.slot_mapping, pool, scales)                          # the chunk
+        out = ops.paged_prefill(case.q, pool, case.block_table, case.cu_q_lens, case.context_lens, case.max_q_len,
+                                SCALE, kv_scales=scales)
+        again = ops.paged_prefill(case.q, pool, case.block_table, case.cu_q_lens, case.context_lens, case.max_q_len,
+                                  SCALE, kv_scales=scales)
+        torch.cuda.synchronize()
+        values = torch.from_numpy(fp8.dequantize_pool(pool.cpu().numpy(), scales.cpu().numpy()))
+        ref = cpu_ref.paged_prefill_ref(case.q.cpu(), values, case.block_table.cpu(), case.cu_q_lens.cpu(),
+                                        case.context_lens.cpu(), SCALE).numpy()
+        assert_attention_close(out, ref, f"fp8 chunk prefill {seed}.{case_no}")
+        assert torch.equal(out, again)
+        # the two-pass way: pages to fp16 (rounding code * scale), then the fp16 kernel
+        scratch = torch.zeros(case.kv_pool.shape, dtype=torch.float16, device=DEV)
+        all_pages = torch.arange(case.num_pages, dtype=torch.int32, device=DEV)
+        ops.page_dequant(pool, scratch, all_pages, all_pages, scales)
+        two_pass = ops.paged_prefill(case.q, scratch, case.block_table, case.cu_q_lens, case.context_lens,
+                                     case.max_q_len, SCALE)
+        assert float((two_pass.float() - out.float()).abs().max()) <= 2e-3
