@@ -106,8 +106,8 @@ class DecodeLayerSet:
         gen = torch.Generator(device=device).manual_seed(4242)
         self.fp8 = kv_dtype == "fp8"
         if self.fp8:
-            if schedule != "balanced" or shared_pages:
-                raise ValueError("fp8 pools are read by the balanced schedule without a shared prefix")
+            if schedule != "balanced":
+                raise ValueError("fp8 pools are read by the balanced schedule")
             # E4M3 codes (no NaN codes) and one scale per head
             pools = torch.randint(0, 0x7F, (layers, slots, 2 * hkv, 128), generator=gen, device=device,
                                   dtype=torch.uint8)
@@ -155,9 +155,10 @@ class DecodeLayerSet:
             if self.fp8:
                 self.decode_args = [
                     (self.q.data_ptr(), hq * 128, pools[l].data_ptr(), self.scales.data_ptr(),
-                     self.seq_lens.data_ptr(), self.plan.data_ptr(), self.plan_bytes, c.k_new.data_ptr(),
-                     c.v_new.data_ptr(), hkv * 128, hkv * 128, self.out[l].data_ptr(), self.ws.data_ptr(), ws_bytes,
-                     b, hq, hkv, 128, 16, c.num_pages, bts, self.chunks, c.softmax_scale, stream)
+                     self.batch_table.data_ptr(), self.seq_lens.data_ptr(), self.plan.data_ptr(), self.plan_bytes,
+                     c.k_new.data_ptr(), c.v_new.data_ptr(), hkv * 128, hkv * 128, self.out[l].data_ptr(),
+                     self.ws.data_ptr(), ws_bytes, b, hq, hkv, 128, 16, c.num_pages, bts, self.chunks,
+                     shared_pages, c.softmax_scale, stream)
                     for l in range(layers)
                 ]
             self.plan_info = {"schedule": "balanced", "chunks": self.chunks, "shared_pages": shared_pages,
@@ -191,7 +192,7 @@ class DecodeLayerSet:
             on = (lambda a: a) if stream is None else (lambda a: a[:-1] + (stream,))
             rc |= lib.litekv_decode_advance(*on(self.advance_args))
             rc |= lib.litekv_decode_plan_prefix(*on(self.plan_args))
-            dec = lib.litekv_paged_decode_balanced_fp8 if self.fp8 else lib.litekv_paged_decode_prefix
+            dec = lib.litekv_paged_decode_prefix_fp8 if self.fp8 else lib.litekv_paged_decode_prefix
             prof = lib.litekv_profile_next_decode
             for l in range(self.layers):
                 if events is not None:
@@ -311,6 +312,8 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
         res["roofline"]["kernel"] = "shared prefix (varlen_prefill_tiled_kernel<2>) + paged_decode_balanced_kernel + merge"
         res["roofline"]["duration_us"] = k_mean * 1e3
     unique = case.unique_decode_bytes() + (append_bytes if balanced else 0)
+    if kv_dtype == "fp8":
+        unique -= (case.unique_decode_bytes() - (case.decode_bytes() - int(case.seq_lens.sum()) * case.tok_bytes)) // 2
     if unique < kernel_bytes:
         # Pages shared between block tables: the roofline fraction is taken on the bytes that must
         # come from HBM at least once; the logical rate (every reader counted) is kept beside it.
@@ -619,11 +622,8 @@ def main() -> int:
         if args.chunks:
             case.extra["chunks"] = args.chunks
         sched = args.schedule
-        if name == "c5" and args.schedule == "balanced" and False:
-            sched = "splits"
         shared = 0
-        if sched == "balanced" and not args.no_shared_prefix and not case.extra.get("private_prefix") \
-                and args.kv_dtype == "f16":
+        if sched == "balanced" and not args.no_shared_prefix and not case.extra.get("private_prefix"):
             shared = int(case.extra.get("n_shared", 0))
         return run_decode(case, layers, args.steps, args.warmup, device, case.name, sched, shared,
                           graph=not args.no_graph, kv_dtype=args.kv_dtype), case

@@ -345,6 +345,24 @@ int litekv_paged_decode_balanced_fp8(const void *q, int64_t q_batch_stride, void
                                      float softmax_scale, void *stream);
 
 /*
+ * litekv_paged_decode_prefix over an fp8 pool (plan from
+ * litekv_decode_plan_prefix, workspace from
+ * litekv_paged_decode_prefix_workspace_bytes): the shared pages of a cached
+ * prefix, which the reference maps into every request by reference
+ * (lite_llama/executor/model_executor.py:570-620), are attended once for the
+ * batch from their codes.
+ */
+int litekv_paged_decode_prefix_fp8(const void *q, int64_t q_batch_stride, void *kv_pool_fp8,
+                                   const float *scales, const int32_t *block_table,
+                                   const int32_t *seq_lens, void *plan, size_t plan_bytes,
+                                   const void *k_new, const void *v_new, int64_t k_new_stride,
+                                   int64_t v_new_stride, void *out, void *workspace,
+                                   size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+                                   int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                                   int64_t num_pages, int32_t block_table_stride, int32_t chunks,
+                                   int32_t shared_pages, float softmax_scale, void *stream);
+
+/*
  * Advances the metadata of a decode batch by one token on the device, so that
  * a captured graph of a decode step replays without host work. Replaces, per
  * step, PagedReqTokensManager.extend_req + batch_metadata

@@ -44,8 +44,10 @@ constexpr int kMaxPrefixSplits = 8;
 // Attention of every (sequence, query head) of a decode step over the first `shared_pages`
 // pages of block-table row 0 (which all sequences share), as normalised fp32 partial rows
 // part_o[split][batch][Hq][128] and log-sum-exps part_lse[split][batch][Hq]; *splits_out
-// receives the number of key slices written. Defined beside the prefill kernel it reuses.
+// receives the number of key slices written. `fp8_scales` (K heads, then V heads) marks an fp8 pool.
+// Defined beside the prefill kernel it reuses.
 int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_pool,
+                         const float *fp8_scales,
                          const int32_t *block_table, int32_t batch, int32_t num_q_heads,
                          int32_t num_kv_heads, int64_t num_pages, int32_t shared_pages,
                          float *part_o, float *part_lse, float softmax_scale, hipStream_t stream,

@@ -1440,7 +1440,7 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   int pre_splits = 0;
   if (shared_pages > 0) {
     LITEKV_REQUIRE(block_table != nullptr, "%s: block_table is null", what);
-    rc = launch_shared_prefix(q, q_batch_stride, kv_pool, block_table, batch, num_q_heads,
+    rc = launch_shared_prefix(q, q_batch_stride, kv_pool, fp8_scales, block_table, batch, num_q_heads,
                               num_kv_heads, num_pages, shared_pages, pre_o, pre_lse, softmax_scale,
                               static_cast<hipStream_t>(stream), &pre_splits);
     if (rc != LITEKV_OK) return rc;
@@ -1550,6 +1550,24 @@ extern "C" int litekv_paged_decode_prefix(
     float softmax_scale, void *stream) {
   return litekv::launch_balanced("paged_decode_prefix", q, q_batch_stride, kv_pool, nullptr, block_table,
                                  seq_lens, plan, plan_bytes, k_new, v_new, k_new_stride,
+                                 v_new_stride, out, workspace, workspace_bytes, batch, num_q_heads,
+                                 num_kv_heads, head_dim, page_size, num_pages, block_table_stride,
+                                 chunks, shared_pages, softmax_scale, stream);
+}
+
+extern "C" int litekv_paged_decode_prefix_fp8(
+    const void *q, int64_t q_batch_stride, void *kv_pool_fp8, const float *scales,
+    const int32_t *block_table, const int32_t *seq_lens, void *plan, size_t plan_bytes,
+    const void *k_new, const void *v_new, int64_t k_new_stride, int64_t v_new_stride, void *out,
+    void *workspace, size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+    int32_t num_kv_heads, int32_t head_dim, int32_t page_size, int64_t num_pages,
+    int32_t block_table_stride, int32_t chunks, int32_t shared_pages, float softmax_scale,
+    void *stream) {
+  if (scales == nullptr && batch > 0) {
+    return litekv::fail(LITEKV_ERR_INVALID_ARGUMENT, "paged_decode_prefix_fp8: scales is null");
+  }
+  return litekv::launch_balanced("paged_decode_prefix_fp8", q, q_batch_stride, kv_pool_fp8, scales,
+                                 block_table, seq_lens, plan, plan_bytes, k_new, v_new, k_new_stride,
                                  v_new_stride, out, workspace, workspace_bytes, batch, num_q_heads,
                                  num_kv_heads, head_dim, page_size, num_pages, block_table_stride,
                                  chunks, shared_pages, softmax_scale, stream);

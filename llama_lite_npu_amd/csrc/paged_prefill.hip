@@ -105,7 +105,8 @@ __device__ __forceinline__ float max_across_groups(float x) {
   s = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
   return vmax2(__builtin_bit_cast(float, s[0]), __builtin_bit_cast(float, s[1]));
 }
-constexpr int kPagedPrefill = 0, kPackedPrefill = 1, kSharedPrefix = 2, kPagedPrefillFp8 = 3;
+constexpr int kPagedPrefill = 0, kPackedPrefill = 1, kSharedPrefix = 2, kPagedPrefillFp8 = 3,
+              kSharedPrefixFp8 = 4;
 
 template <int MODE>
 __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_kernel(
@@ -119,7 +120,8 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   // converted to fp16 (exactly) and written to LDS in the same swizzled layout, so everything
   // after the staging is shared. The K scale joins the softmax scale, the V scale the final
   // normalisation, as in the decode kernel.
-  constexpr bool FP8 = MODE == kPagedPrefillFp8;
+  constexpr bool FP8 = MODE == kPagedPrefillFp8 || MODE == kSharedPrefixFp8;
+  constexpr bool SHARED = MODE == kSharedPrefix || MODE == kSharedPrefixFp8;
   // Two tiles of K and two of V: tile t sits in half t % 2.
   __shared__ __attribute__((aligned(1024))) half_t kbuf[2 * kTileHalfs];
   __shared__ __attribute__((aligned(1024))) half_t vbuf[2 * kTileHalfs];
@@ -147,7 +149,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   //   tile0   first key tile (tiles are counted from it)   last_key  last key that exists
   int q_start = 0, q_len = 0, m0 = 0, ctx = 0, kv_end, diag, last_key;
   int tile0 = 0;
-  if constexpr (MODE == kSharedPrefix) {
+  if constexpr (SHARED) {
     const int key_begin = (int)blockIdx.z * prefix.keys_per_split;
     if (key_begin >= prefix.prefix_keys) return;
     kv_end = key_begin + prefix.keys_per_split;
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
               (uint32_t)(((PAGED ? paged.num_kv_heads : 0) + h) * kHeadDim + 8 * cv) * 2u;
   }
   const int32_t *table =
-      PAGED ? paged.block_table + (MODE == kSharedPrefix ? 0 : (int64_t)b * paged.bt_stride) : nullptr;
+      PAGED ? paged.block_table + (SHARED ? 0 : (int64_t)b * paged.bt_stride) : nullptr;
   const int last_page = last_key >> 4;
 
   // Starts the loads of tile kt into its LDS half. The instruction is written as asm so that the
@@ -280,7 +282,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     bool ok;
     int hq;
     const half_t *qrow;
-    if constexpr (MODE == kSharedPrefix) {
+    if constexpr (SHARED) {
       const int col = (int)blockIdx.y * (16 * kWgColTiles) + 16 * t + n;  // (sequence, head) pair
       ok = col < prefix.batch * group;
       const int seq = ok ? col / group : 0;
@@ -536,7 +538,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
 #pragma unroll
   for (int u = 0; u < kColTiles; ++u) {
     const float inv = v_scale / dsum[u][0];
-    if constexpr (MODE == kSharedPrefix) {
+    if constexpr (SHARED) {
       if (out_row[u] >= 0) {
         const int64_t cell =
             ((int64_t)blockIdx.z * prefix.batch + out_row[u]) * prefix.num_q_heads + out_head[u];
@@ -598,7 +600,7 @@ static PrefillShape prefill_shape(int group, int max_q_len) {
 }
 
 int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_pool,
-                         const int32_t *block_table, int32_t batch, int32_t num_q_heads,
+                         const float *fp8_scales, const int32_t *block_table, int32_t batch, int32_t num_q_heads,
                          int32_t num_kv_heads, int64_t num_pages, int32_t shared_pages,
                          float *part_o, float *part_lse, float softmax_scale, hipStream_t stream,
                          int *splits_out) {
@@ -620,15 +622,23 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
   keys_per_split = (keys_per_split + kKvTile - 1) / kKvTile * kKvTile;
   splits = (prefix_keys + keys_per_split - 1) / keys_per_split;
   PagedSource paged{static_cast<const half_t *>(kv_pool), block_table, 0, num_kv_heads,
-                    (int32_t)num_pages, nullptr};
+                    (int32_t)num_pages, fp8_scales};
   PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
   PrefixTask task{part_o, part_lse, q_batch_stride, batch, num_q_heads, prefix_keys, keys_per_split};
-  hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kSharedPrefix>,
-                     dim3((unsigned)num_kv_heads, (unsigned)col_blocks, (unsigned)splits),
-                     dim3(kTiledWaves * kWave), 0, stream, static_cast<const half_t *>(q),
-                     (int64_t)0, (half_t *)nullptr, (int64_t)0, paged, packed, task,
-                     (const int32_t *)nullptr, (const int32_t *)nullptr, (const int32_t *)nullptr,
-                     group, 1, group, 1, softmax_scale * kLog2eP);
+  const dim3 grid((unsigned)num_kv_heads, (unsigned)col_blocks, (unsigned)splits);
+  if (fp8_scales != nullptr) {
+    hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kSharedPrefixFp8>, grid, dim3(kTiledWaves * kWave), 0,
+                       stream, static_cast<const half_t *>(q), (int64_t)0, (half_t *)nullptr,
+                       (int64_t)0, paged, packed, task, (const int32_t *)nullptr,
+                       (const int32_t *)nullptr, (const int32_t *)nullptr, group, 1, group, 1,
+                       softmax_scale * kLog2eP);
+  } else {
+    hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kSharedPrefix>, grid, dim3(kTiledWaves * kWave), 0,
+                       stream, static_cast<const half_t *>(q), (int64_t)0, (half_t *)nullptr,
+                       (int64_t)0, paged, packed, task, (const int32_t *)nullptr,
+                       (const int32_t *)nullptr, (const int32_t *)nullptr, group, 1, group, 1,
+                       softmax_scale * kLog2eP);
+  }
   *splits_out = splits;
   return check_launch(what);
 }

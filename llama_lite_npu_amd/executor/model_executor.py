@@ -326,8 +326,6 @@ class ModelExecutor:
         """Leading pages the decode step attends once for the whole batch (prefix-cache hits map one
         page list into many requests, :547-620). 0 when the batch shares fewer than
         ``shared_prefix_min_pages`` pages."""
-        if self.kv_mem_manager.is_fp8:
-            return 0             # the shared-prefix kernel reads fp16 pools
         n = self.common_leading_pages(request_ids, upcoming_tokens)
         return n if n >= self.shared_prefix_min_pages else 0
 

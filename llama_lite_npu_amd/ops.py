@@ -362,7 +362,13 @@ def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
     lib = _lib.load()
     if fp8:
         _dev_fp8_pool(kv_pool, kv_scales, hkv)
-        _need(plan.shared_pages == 0, "the shared-prefix decode reads fp16 pools only")
+        if plan.shared_pages > 0:
+            _lib.check(lib.litekv_paged_decode_prefix_fp8(
+                _ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(plan.block_table), _ptr(plan.seq_lens),
+                _ptr(plan.buffer), plan.plan_bytes, _ptr(k_new), _ptr(v_new), kn_stride, vn_stride, _ptr(out),
+                _ptr(plan.workspace), plan.workspace_bytes, b, hq, hkv, d, plan.page_size, n_pages, plan.bt_stride,
+                plan.chunks, plan.shared_pages, float(softmax_scale), _stream()))
+            return out
         _lib.check(lib.litekv_paged_decode_balanced_fp8(
             _ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(plan.seq_lens), _ptr(plan.buffer),
             plan.plan_bytes, _ptr(k_new), _ptr(v_new), kn_stride, vn_stride, _ptr(out), _ptr(plan.workspace),

@@ -122,10 +122,31 @@ def test_random_steps_behind_a_shared_prefix(seed):
         ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool_ref), case.block_table.cpu().numpy(),
                                     case.seq_lens.cpu().numpy(), case.softmax_scale)
         plan = ops.DecodePlan(case.block_table, case.seq_lens, hq, hkv, case.num_pages, chunks, shared_pages=declared)
+        pool0 = case.kv_pool.clone()
         out = ops.decode_step(case.q, case.kv_pool, plan, case.k_new, case.v_new, case.softmax_scale)
         torch.cuda.synchronize()
         assert torch.equal(case.kv_pool.view(torch.int16), pool_ref.view(torch.int16))
         assert_attention_close(out, ref, f"random prefix step {seed}.{case_no}")
+        # the same step over fp8 pools: codes as the quantising append writes them, attention
+        # within tolerance of the oracle on the decoded pool, equal to the step without the
+        # shared-prefix kernel up to the order of the sums
+        scales = torch.cat([0.02 * (1 + 0.1 * torch.arange(hkv)), 0.015 * (1 + 0.2 * torch.arange(hkv))]).float().to(DEV)
+        pool8 = torch.empty(pool0.shape, dtype=torch.uint8, device=DEV)
+        every_slot = torch.arange(pool8.shape[0], dtype=torch.int32, device=DEV)
+        ops.kv_append_fp8(pool0[:, :hkv], pool0[:, hkv:], every_slot, pool8, scales)
+        want8 = pool8.clone()
+        ops.kv_append_fp8(case.k_new, case.v_new, case.slot_mapping, want8, scales)
+        plain = ops.DecodePlan(case.block_table, case.seq_lens, hq, hkv, case.num_pages, chunks)
+        out_plain = ops.decode_step(case.q, want8.clone(), plain, None, None, case.softmax_scale, kv_scales=scales)
+        out8 = ops.decode_step(case.q, pool8, plan, case.k_new, case.v_new, case.softmax_scale, kv_scales=scales)
+        torch.cuda.synchronize()
+        got, exp = pool8.cpu().numpy(), want8.cpu().numpy()
+        assert int(((got != exp) & ~(((got & 0x7F) == 0) & ((exp & 0x7F) == 0))).sum()) == 0
+        values = torch.from_numpy(fp8.dequantize_pool(got, scales.cpu().numpy()))
+        ref8 = cpu_ref.paged_decode_ref(case.q.cpu(), values, case.block_table.cpu(), case.seq_lens.cpu(),
+                                        case.softmax_scale).numpy()
+        assert_attention_close(out8, ref8, f"random fp8 prefix step {seed}.{case_no}")
+        assert float((out8.float() - out_plain.float()).abs().max()) <= 1e-3
 
 
 @pytest.mark.parametrize("batch", [200, 600])

@@ -411,3 +411,40 @@ def test_chunk_prefill_reads_an_fp8_pool_directly(seed):
         two_pass = ops.paged_prefill(case.q, scratch, case.block_table, case.cu_q_lens, case.context_lens,
                                      case.max_q_len, SCALE)
         assert float((two_pass.float() - out.float()).abs().max()) <= 2e-3
+
+
+def test_cached_system_prompt_over_fp8_pools_is_attended_once_for_the_batch():
+    """Three requests share a 96-token prefix through the block cache of an fp8 executor: the
+    decode step gets a shared-prefix plan and the codes of the shared pages are read once."""
+    print("fp8: executor, shared prefix decode", flush=True)
+    from llama_lite_npu_amd.attention import Attention
+
+    hq, hkv = 16, 8
+    ex = _fp8_executor(layers=1, hq=hq, hkv=hkv, num_pages=128)
+    attn = Attention(hq, hkv, D)
+    log2e = 1.4426950408889634
+    system = tuple(range(2000, 2096))               # 6 full pages
+    (a,) = ex.reserve_paged_requests([96])
+    ex.activate_paged_packed_prefill_batch((a,), [96])
+    attn.context_forward(_rows(96, hq, 61), _rows(96, hkv, 62), _rows(96, hkv, 63), ex.atten_info, 0, SCALE * log2e)
+    ex.store_paged_request_prefix(system, a, first_token_id=5)
+    others = []
+    for i, extra in enumerate((20, 3)):
+        prompt = system + tuple(range(3000 + 100 * i, 3000 + 100 * i + extra))
+        req, matched, first = ex.share_paged_prefix_from_cache(prompt)
+        assert matched == 96 and first is None
+        ex.ensure_paged_request_capacity(req, 96 + extra + 8)
+        ex.activate_paged_chunk_prefill_batch((req,), [96], [extra])
+        attn.context_forward(_rows(extra, hq, 70 + i), _rows(extra, hkv, 80 + i), _rows(extra, hkv, 90 + i),
+                             ex.atten_info, 0, SCALE * log2e)
+        others.append(req)
+    batch = (a, *others)
+    ex.extend_paged_requests(batch)
+    assert ex.atten_info.decode_plan.shared_pages == 6
+    qd, kd, vd = _rows(3, hq, 95), _rows(3, hkv, 96), _rows(3, hkv, 97)
+    out = attn.token_forward(qd, kd, vd, ex.atten_info, 0, SCALE)
+    torch.cuda.synchronize()
+    info = ex.atten_info
+    ref = cpu_ref.paged_decode_ref(qd.cpu(), _decoded_pool(ex, 0), info.block_table.cpu(), info.seq_lens_i32.cpu(),
+                                   SCALE).numpy()
+    assert_attention_close(out, ref, "fp8 decode over a shared system prompt")
