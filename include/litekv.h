@@ -345,6 +345,18 @@ int litekv_paged_decode_balanced_fp8(const void *q, int64_t q_batch_stride, void
                                      float softmax_scale, void *stream);
 
 /*
+ * litekv_paged_decode (per-sequence splits, both stages) over an fp8 pool; the
+ * merge stage is litekv_paged_decode_merge, which never touches the pool.
+ */
+int litekv_paged_decode_fp8(const void *q, int64_t q_batch_stride, const void *kv_pool_fp8,
+                            const float *scales, const int32_t *block_table,
+                            int32_t block_table_stride, const int32_t *seq_lens, void *out,
+                            void *workspace, size_t workspace_bytes, int32_t batch,
+                            int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                            int32_t page_size, int64_t num_pages, int32_t max_splits,
+                            int32_t min_pages_per_split, float softmax_scale, void *stream);
+
+/*
  * litekv_paged_decode_prefix over an fp8 pool (plan from
  * litekv_decode_plan_prefix, workspace from
  * litekv_paged_decode_prefix_workspace_bytes): the shared pages of a cached

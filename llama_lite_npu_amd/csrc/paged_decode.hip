@@ -361,9 +361,10 @@ __device__ __forceinline__ int clamp_page(int pid, int num_pages) {
 // Schedule "splits": one wavefront per (kv head, split, sequence).
 // Partials: part_o[b][hq][split][D], part_lse[b][hq][split].
 // ---------------------------------------------------------------------------------------------
-template <int DEPTH>
+template <int DEPTH, bool FP8>
 __global__ __launch_bounds__(64) void paged_decode_split_kernel(
-    const half_t *__restrict__ q, int64_t q_batch_stride, const half_t *__restrict__ kv,
+    const half_t *__restrict__ q, int64_t q_batch_stride,
+    const typename KvStore<FP8>::elem *__restrict__ kv, const float *__restrict__ scales,
     const int32_t *__restrict__ block_table, int32_t bt_stride,
     const int32_t *__restrict__ seq_lens, half_t *__restrict__ out, float *__restrict__ part_o,
     float *__restrict__ part_lse, int32_t num_q_heads, int32_t num_kv_heads, int32_t group,
@@ -394,18 +395,30 @@ __global__ __launch_bounds__(64) void paged_decode_split_kernel(
   const int p0 = (int)(((int64_t)split * pages) / n_splits);
   const int p1 = (int)(((int64_t)(split + 1) * pages) / n_splits);
 
+  typedef typename KvStore<FP8>::elem Elem;
+  typedef typename KvStore<FP8>::page Page;
   half8_t qf[4];
-  load_q(qf, q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
+  float v_scale = 1.0f;
+  if constexpr (FP8) {  // the K scale joins the softmax scale, the V scale the normalisation
+    load_q_fp8_order(qf, q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
+    scale_log2 *= scales[h];
+    v_scale = scales[num_kv_heads + h];
+  } else {
+    load_q(qf, q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
+  }
 
   const int64_t row_stride = (int64_t)2 * num_kv_heads * kHeadDim;  // elements per slot
-  const half_t *k_lane = kv + (int64_t)h * kHeadDim + 8 * g + n * row_stride;
-  const half_t *v_lane = kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
+  // this lane's row and column inside page 0 (see PageRegs / PageRegsFp8)
+  const Elem *k_lane = kv + (int64_t)h * kHeadDim + (FP8 ? 16 : 8) * g + n * row_stride;
+  const Elem *v_lane = FP8 ? kv + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7) +
+                                 (2 * g + (n >> 3)) * row_stride
+                           : kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
   const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
   const int32_t *table = block_table + (int64_t)b * bt_stride;
 
   HeadState st;
   st.reset();
-  PageRegs buf[DEPTH];
+  Page buf[DEPTH];
 
   // Page ids are wavefront-uniform: they travel through scalar loads one step ahead of their
   // use. Requests past the range still issue their loads (16 bytes of its last page), which keeps
@@ -413,7 +426,7 @@ __global__ __launch_bounds__(64) void paged_decode_split_kernel(
   // page it needs and never drains the younger prefetches.
   auto page_id = [&](int p) { return clamp_page(table[p < p1 ? p : p1 - 1], num_pages); };
   int pid_next = page_id(p0);
-  auto request = [&](int p, PageRegs &r) {
+  auto request = [&](int p, Page &r) {
     const int64_t page_off = (int64_t)pid_next * kPageSize * row_stride;
     pid_next = page_id(p + 1);
     request_page(r, k_lane, v_lane, page_off, row_stride, p >= p1, kv);
@@ -431,7 +444,7 @@ __global__ __launch_bounds__(64) void paged_decode_split_kernel(
 
   const int64_t cell = ((int64_t)b * num_q_heads + hq0) * max_splits + split;
   store_state(st, n_splits == 1, out_row, part_o + cell * kHeadDim, (int64_t)max_splits * kHeadDim,
-              part_lse + cell, max_splits, n, g, group);
+              part_lse + cell, max_splits, n, g, group, v_scale);
 }
 
 // Merges partial rows of one query head into its final fp16 row; run by one whole wavefront.
@@ -1196,8 +1209,9 @@ static int check_split_plan(const char *what, int32_t max_splits, int32_t min_pa
   return LITEKV_OK;
 }
 
-static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split) {
-  const char *what = "paged_decode_split";
+static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split,
+                        const float *fp8_scales = nullptr) {
+  const char *what = fp8_scales ? "paged_decode_split_fp8" : "paged_decode_split";
   int rc = check_split_plan(what, max_splits, min_pages_per_split);
   if (rc != LITEKV_OK) return rc;
   rc = validate_decode(what, a,
@@ -1212,14 +1226,22 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   float *part_o = max_splits > 1 ? static_cast<float *>(a.workspace) : nullptr;
   float *part_lse =
       max_splits > 1 ? part_o + (size_t)a.batch * a.num_q_heads * max_splits * a.head_dim : nullptr;
-  hipLaunchKernelGGL(paged_decode_split_kernel<LITEKV_DECODE_DEPTH>,
-                     dim3((unsigned)a.num_kv_heads, (unsigned)max_splits, (unsigned)a.batch),
-                     dim3(kWave), 0, static_cast<hipStream_t>(a.stream),
-                     static_cast<const half_t *>(a.q), a.q_batch_stride,
-                     static_cast<const half_t *>(a.kv_pool), a.block_table, a.block_table_stride,
-                     a.seq_lens, static_cast<half_t *>(a.out), part_o, part_lse, a.num_q_heads,
-                     a.num_kv_heads, group, max_splits, min_pages_per_split, (int32_t)a.num_pages,
-                     a.softmax_scale * kLog2e);
+  const dim3 grid((unsigned)a.num_kv_heads, (unsigned)max_splits, (unsigned)a.batch);
+  if (fp8_scales != nullptr) {
+    hipLaunchKernelGGL((paged_decode_split_kernel<LITEKV_DECODE_DEPTH, true>), grid, dim3(kWave), 0,
+                       static_cast<hipStream_t>(a.stream), static_cast<const half_t *>(a.q),
+                       a.q_batch_stride, static_cast<const uint8_t *>(a.kv_pool), fp8_scales,
+                       a.block_table, a.block_table_stride, a.seq_lens, static_cast<half_t *>(a.out),
+                       part_o, part_lse, a.num_q_heads, a.num_kv_heads, group, max_splits,
+                       min_pages_per_split, (int32_t)a.num_pages, a.softmax_scale * kLog2e);
+  } else {
+    hipLaunchKernelGGL((paged_decode_split_kernel<LITEKV_DECODE_DEPTH, false>), grid, dim3(kWave), 0,
+                       static_cast<hipStream_t>(a.stream), static_cast<const half_t *>(a.q),
+                       a.q_batch_stride, static_cast<const half_t *>(a.kv_pool), fp8_scales,
+                       a.block_table, a.block_table_stride, a.seq_lens, static_cast<half_t *>(a.out),
+                       part_o, part_lse, a.num_q_heads, a.num_kv_heads, group, max_splits,
+                       min_pages_per_split, (int32_t)a.num_pages, a.softmax_scale * kLog2e);
+  }
   return check_launch(what);
 }
 
@@ -1600,6 +1622,26 @@ extern "C" int litekv_paged_decode_merge(const int32_t *seq_lens, void *out, con
   litekv::DecodeArgs a{nullptr, 0, nullptr, nullptr, 1, seq_lens, out,
                        const_cast<void *>(workspace), workspace_bytes, batch, num_q_heads, 1,
                        head_dim, page_size, 1, 0.f, stream};
+  return litekv::launch_merge(a, max_splits, min_pages_per_split);
+}
+
+extern "C" int litekv_paged_decode_fp8(const void *q, int64_t q_batch_stride,
+                                       const void *kv_pool_fp8, const float *scales,
+                                       const int32_t *block_table, int32_t block_table_stride,
+                                       const int32_t *seq_lens, void *out, void *workspace,
+                                       size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+                                       int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                                       int64_t num_pages, int32_t max_splits,
+                                       int32_t min_pages_per_split, float softmax_scale,
+                                       void *stream) {
+  if (scales == nullptr && batch > 0) {
+    return litekv::fail(LITEKV_ERR_INVALID_ARGUMENT, "paged_decode_fp8: scales is null");
+  }
+  litekv::DecodeArgs a{q, q_batch_stride, kv_pool_fp8, block_table, block_table_stride, seq_lens, out,
+                       workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim,
+                       page_size, num_pages, softmax_scale, stream};
+  int rc = litekv::launch_split(a, max_splits, min_pages_per_split, batch > 0 ? scales : nullptr);
+  if (rc != LITEKV_OK) return rc;
   return litekv::launch_merge(a, max_splits, min_pages_per_split);
 }
 

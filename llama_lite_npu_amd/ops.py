@@ -409,7 +409,7 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
     kv head (default: one workgroup per CU); a DecodePlan is built for the call unless one is
     passed. schedule "splits" (chosen when num_splits, max_splits or min_pages_per_split is
     given): every sequence is cut into its own splits; two launches (`stage` selects one).
-    An fp8 pool (with its ``kv_scales``) is read by the balanced schedule only.
+    An fp8 pool comes with its ``kv_scales``; either schedule reads it.
     """
     _dev_half("q", q)
     if not is_fp8_pool(kv_pool):
@@ -430,7 +430,10 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
             plan = DecodePlan(block_table, seq_lens, hq, hkv, n_pages, chunks, page_size, shared_pages)
         return decode_step(q, kv_pool, plan, None, None, softmax_scale, out, kv_scales)
 
-    _need(not is_fp8_pool(kv_pool), "fp8 pools are read by the balanced schedule only")
+    fp8 = is_fp8_pool(kv_pool)
+    if fp8:
+        _dev_fp8_pool(kv_pool, kv_scales, hkv)
+        _need(stage == "both", "an fp8 pool is read by both stages in one call")
     _need(block_table.dim() == 2 and block_table.shape[0] == b, "block_table must be [B, max_blocks]")
     block_table = _dev_i32("block_table", block_table)
     seq_lens = _dev_i32("seq_lens", seq_lens)
@@ -451,7 +454,12 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
     if workspace is None:
         workspace = decode_workspace(b, hq, max_splits, q.device)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    if stage in ("both", "split"):
+    if fp8:
+        _lib.check(lib.litekv_paged_decode_fp8(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(block_table),
+                                               block_table.stride(0), _ptr(seq_lens), _ptr(out), _ptr(workspace),
+                                               ws_bytes, b, hq, hkv, d, page_size, n_pages, max_splits,
+                                               min_pages_per_split, float(softmax_scale), _stream()))
+    elif stage in ("both", "split"):
         fn = lib.litekv_paged_decode if stage == "both" else lib.litekv_paged_decode_split
         _lib.check(fn(_ptr(q), q_stride, _ptr(kv_pool), _ptr(block_table), block_table.stride(0),
                       _ptr(seq_lens), _ptr(out), _ptr(workspace), ws_bytes, b, hq, hkv, d, page_size,

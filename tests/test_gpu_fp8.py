@@ -126,6 +126,17 @@ def test_decode_over_an_fp8_pool_matches_the_oracle_on_the_decoded_values(hq, hk
     assert_attention_close(other, _oracle(q, pool, scales, table, seq_lens), "fp8 decode, 37 chunks")
 
 
+def test_per_sequence_splits_read_an_fp8_pool_too():
+    print("fp8 decode, per-sequence splits", flush=True)
+    q, pool, scales, table, seq_lens = _fp8_case(57, [0, 1, 16, 17, 300, 1000, 64], 32, 4)
+    ref = _oracle(q, pool, scales, table, seq_lens)
+    for kw in ({"num_splits": 1}, {"num_splits": 4}, {"max_splits": 16, "min_pages_per_split": 2}):
+        out = ops.paged_decode(q, pool, table, seq_lens, SCALE, kv_scales=scales, **kw)
+        torch.cuda.synchronize()
+        assert_attention_close(out, ref, f"fp8 splits {kw}")
+        assert float(out[0].abs().max()) == 0.0
+
+
 def test_quantisation_error_is_the_only_difference_from_fp16():
     """The same K/V in an fp16 pool: outputs differ by what E4M3's 3 mantissa bits allow, not more."""
     print("fp8 vs fp16 decode", flush=True)
@@ -193,8 +204,8 @@ def test_argument_checks():
         ops.paged_decode(q, pool, table, seq_lens, SCALE)
     with pytest.raises(ValueError, match="scales"):
         ops.paged_decode(q, pool, table, seq_lens, SCALE, kv_scales=scales[:3])
-    with pytest.raises(ValueError, match="balanced"):
-        ops.paged_decode(q, pool, table, seq_lens, SCALE, kv_scales=scales, num_splits=2)
+    with pytest.raises(ValueError, match="both stages"):
+        ops.paged_decode(q, pool, table, seq_lens, SCALE, kv_scales=scales, num_splits=2, stage="split")
     with pytest.raises(ValueError, match="fp8"):
         ops.kv_append_fp8(q[:, :2], q[:, :2], seq_lens, pool.half(), scales)
 
