@@ -427,13 +427,34 @@ def compaction_step(case) -> dict:
             "decode_repeat_same_bits": bool(torch.equal(after, again))}
 
 
+def _host_threads() -> int:
+    """Threads for the CPU baseline: what the environment grants (OMP_NUM_THREADS), else the
+    visible cores, never more than 16 (one GPU's share of a host)."""
+    try:
+        granted = int(os.environ.get("OMP_NUM_THREADS", "0"))
+    except ValueError:
+        granted = 0
+    return max(1, min(granted if granted > 0 else (os.cpu_count() or 1), 16))
+
+
+def _cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline_prefill(case, budget_s: float = 10.0) -> dict:
     """Per-sequence causal attention of the whole C3 workload in torch on the host cores
     (restates flashattention2_nopad.py:250-274), min over repetitions for about `budget_s` s."""
     import torch
     from oracle import cpu_ref
 
-    cores = os.cpu_count() or 1
+    cores = _host_threads()
     torch.set_num_threads(cores)
     c = case.to("cpu")
     starts = c.cu_q_lens[:-1]
@@ -453,6 +474,7 @@ def cpu_baseline_prefill(case, budget_s: float = 10.0) -> dict:
         used += dt
     best = min(times) if times else first
     return {"value": case.flops() / best / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "cpu_model": _cpu_model(),
             "sample": f"the whole workload ({case.flops() / 1e12:.3f} TFLOP causal), torch CPU restatement, "
                       f"min of {max(1, len(times))} reps after 1 warm-up, {best:.3f} s"}
 
@@ -524,7 +546,7 @@ def cpu_baseline_decode(case, budget_s: float = 10.0) -> dict:
     import torch
     from oracle import cpu_ref
 
-    cores = os.cpu_count() or 1
+    cores = _host_threads()
     torch.set_num_threads(cores)
     c = case.to("cpu")
     kv = torch.cat([c.k_new, c.v_new], dim=1)
@@ -552,6 +574,7 @@ def cpu_baseline_decode(case, budget_s: float = 10.0) -> dict:
         "unit": "GB/s",
         "cores": cores,
         "kind": "port",
+        "cpu_model": _cpu_model(),
         "sample": f"1 of the layers of the same workload (append + decode, {nbytes / 1e6:.1f} MB algorithmic), "
                   f"torch CPU restatement, min of {max(1, len(times))} reps after 1 warm-up, {best:.3f} s",
         "seconds_per_layer": best,
