@@ -360,23 +360,31 @@ __device__ __forceinline__ int clamp_page(int pid, int num_pages) {
 // ---------------------------------------------------------------------------------------------
 // Schedule "splits": one wavefront per (kv head, split, sequence).
 // Partials: part_o[b][hq][split][D], part_lse[b][hq][split].
+// The wavefronts are independent (no barrier). A workgroup holds 1, 2 or 4 of them (blockDim.x /
+// 64; neighbouring kv heads of one sequence), chosen by the host: few wavefronts want
+// one per workgroup so that they spread over all compute units, many short ones want four,
+// because the dispatcher places workgroups at a fixed rate whatever their size (512 sequences of
+// 32 tokens, 8 kv heads: 30.5 us as 4096 workgroups). Not eight: at three wavefronts per SIMD a
+// compute unit would hold one such workgroup and leave a third of its slots empty.
 // ---------------------------------------------------------------------------------------------
+constexpr int kSplitWaves = 4;
+extern __shared__ __attribute__((aligned(16))) half_t split_vstage[];  // [waves][kPageSize * kVPitch]
 template <int DEPTH, bool FP8>
-__global__ __launch_bounds__(64) void paged_decode_split_kernel(
+__global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
     const half_t *__restrict__ q, int64_t q_batch_stride,
     const typename KvStore<FP8>::elem *__restrict__ kv, const float *__restrict__ scales,
     const int32_t *__restrict__ block_table, int32_t bt_stride,
     const int32_t *__restrict__ seq_lens, half_t *__restrict__ out, float *__restrict__ part_o,
     float *__restrict__ part_lse, int32_t num_q_heads, int32_t num_kv_heads, int32_t group,
     int32_t max_splits, int32_t min_pages_per_split, int32_t num_pages, float scale_log2) {
-  __shared__ __attribute__((aligned(16))) half_t vstage[kPageSize * kVPitch];
-
-  const int lane = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
   const int n = lane & 15;   // query head inside the group (column of S^T)
   const int g = lane >> 4;   // lane group: owns tokens 4g..4g+3 of a page
-  const int h = blockIdx.x;  // kv head
+  const int h = blockIdx.x * (blockDim.x >> 6) + wave;  // kv head
   const int split = blockIdx.y;
   const int b = blockIdx.z;
+  half_t *vstage = split_vstage + wave * (kPageSize * kVPitch);
 
   const int len = seq_lens[b];
   const int hq0 = h * group;
@@ -1226,16 +1234,24 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   float *part_o = max_splits > 1 ? static_cast<float *>(a.workspace) : nullptr;
   float *part_lse =
       max_splits > 1 ? part_o + (size_t)a.batch * a.num_q_heads * max_splits * a.head_dim : nullptr;
-  const dim3 grid((unsigned)a.num_kv_heads, (unsigned)max_splits, (unsigned)a.batch);
+  // Wavefronts per workgroup: one where sequences are split (long chains: a workgroup would
+  // hold its slots until its longest wavefront is done), else as many heads of a sequence as
+  // leave at least two workgroups per compute unit.
+  const int64_t units = (int64_t)a.batch * a.num_kv_heads;
+  int waves = max_splits == 1 ? kSplitWaves : 1;
+  while (waves > 1 && (units / waves < 512 || a.num_kv_heads % waves != 0)) waves >>= 1;
+  const dim3 grid((unsigned)(a.num_kv_heads / waves), (unsigned)max_splits, (unsigned)a.batch);
+  const dim3 block((unsigned)(waves * kWave));
+  const size_t lds = (size_t)waves * kPageSize * kVPitch * sizeof(half_t);
   if (fp8_scales != nullptr) {
-    hipLaunchKernelGGL((paged_decode_split_kernel<LITEKV_DECODE_DEPTH, true>), grid, dim3(kWave), 0,
+    hipLaunchKernelGGL((paged_decode_split_kernel<LITEKV_DECODE_DEPTH, true>), grid, block, lds,
                        static_cast<hipStream_t>(a.stream), static_cast<const half_t *>(a.q),
                        a.q_batch_stride, static_cast<const uint8_t *>(a.kv_pool), fp8_scales,
                        a.block_table, a.block_table_stride, a.seq_lens, static_cast<half_t *>(a.out),
                        part_o, part_lse, a.num_q_heads, a.num_kv_heads, group, max_splits,
                        min_pages_per_split, (int32_t)a.num_pages, a.softmax_scale * kLog2e);
   } else {
-    hipLaunchKernelGGL((paged_decode_split_kernel<LITEKV_DECODE_DEPTH, false>), grid, dim3(kWave), 0,
+    hipLaunchKernelGGL((paged_decode_split_kernel<LITEKV_DECODE_DEPTH, false>), grid, block, lds,
                        static_cast<hipStream_t>(a.stream), static_cast<const half_t *>(a.q),
                        a.q_batch_stride, static_cast<const half_t *>(a.kv_pool), fp8_scales,
                        a.block_table, a.block_table_stride, a.seq_lens, static_cast<half_t *>(a.out),

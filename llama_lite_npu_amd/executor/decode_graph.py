@@ -85,7 +85,9 @@ class DeviceDecodeBatch:
         self.shared_pages = int(shared_pages)
         self.decode_plan = ops.DecodePlan(self.block_table, self.seq_lens_i32, executor.local_q_heads,
                                           executor.local_kv_heads, executor.kv_mem_manager.num_pages,
-                                          page_size=executor.page_size, shared_pages=self.shared_pages)
+                                          page_size=executor.page_size, shared_pages=self.shared_pages,
+                                          slot_mapping=self.cur_select_index,
+                                          token_bytes=getattr(executor, "kv_token_bytes", None))
         self.load(request_ids, reserve_tokens, host_ahead)
 
     # ---- host side -------------------------------------------------------------------------
@@ -125,6 +127,7 @@ class DeviceDecodeBatch:
         self.reserve(reserve_tokens)
         self.overflow.zero_()
         self.pending = bool(host_ahead)
+        self._choose_schedule()
         self._launch_advance(0)
 
     def reserve(self, tokens_ahead: int) -> None:
@@ -158,6 +161,16 @@ class DeviceDecodeBatch:
             self._upload_capacity()
         self.pending = True
         self.steps += 1
+        if self.steps % 16 == 0:       # lengths drift slowly: a look every few steps is enough
+            self._choose_schedule()
+
+    def _choose_schedule(self) -> None:
+        """Balanced or per-sequence decode for the coming steps, from the host's lengths. The
+        schedule in use keeps a 10 % advantage so that a batch near the boundary does not flip
+        (a graph runner holds one graph per schedule)."""
+        plan = self.decode_plan
+        counts = self.executor.req_tokens_manager.req_token_count
+        plan.choose_schedule([counts[r] for r in self.request_ids], margin=0.95 if plan.per_sequence else 1.15)
 
     @property
     def max_actual_seq_len(self) -> int:
@@ -288,12 +301,15 @@ class DecodeGraphRunner:
     def _key(self, input_ids, atten_info) -> tuple:
         key = self.graph_key(input_ids, atten_info.max_actual_seq_len)
         device = getattr(atten_info, "device_decode", None)
+        plan = getattr(atten_info, "decode_plan", None)
+        # a graph holds the kernels of the decode schedule it was captured with
+        per_sequence = bool(plan is not None and plan.per_sequence)
         if device is not None:
-            return key + (id(device),)   # the graph is tied to that batch's tensors
+            return key + (id(device), per_sequence)   # the graph is tied to that batch's tensors
         table = getattr(atten_info, "block_table", None)
         if self.PARTITION_SIZE is None and self.max_blocks is None and table is not None:
-            return key + (int(table.shape[1]),)   # a trimmed table: its width sizes the plan
-        return key
+            return key + (int(table.shape[1]), per_sequence)   # a trimmed table: its width sizes the plan
+        return key + (per_sequence,) if per_sequence else key
 
     # ---- capture ---------------------------------------------------------------------------
     def _static_info(self, atten_info):
@@ -313,7 +329,9 @@ class DecodeGraphRunner:
 
             info.decode_plan = ops.DecodePlan(info.block_table, info.seq_lens_i32, plan.num_q_heads,
                                               plan.num_kv_heads, plan.num_pages, plan.chunks, plan.page_size,
-                                              plan.shared_pages)
+                                              plan.shared_pages, slot_mapping=info.cur_select_index,
+                                              token_bytes=plan.token_bytes)
+            info.decode_plan.per_sequence = bool(plan.per_sequence and info.cur_select_index is not None)
         return info
 
     def capture(self, input_ids: torch.Tensor, position_ids: torch.Tensor, atten_info) -> bool:

@@ -53,6 +53,8 @@ class ModelExecutor:
         self.atten_info.kv_buffer = self.kv_mem_manager.gpu_kv_buffer
         self.atten_info.kv_scales = self.kv_mem_manager.kv_scales
         self.build_decode_plans = build_decode_plans and torch.device(device).type == "cuda"
+        # K + V bytes of one token in a layer's pool (what a decode step reads per token attended)
+        self.kv_token_bytes = 2 * self.local_kv_heads * head_dim * torch.empty((), dtype=dtype).element_size()
         self.shared_prefix_min_pages = 4  # below that the two extra launches cost more than they save
         self._decode_plan = None
         self._paged_request_ids: tuple[int, ...] = ()
@@ -302,7 +304,10 @@ class ModelExecutor:
             info.decode_plan = ops.DecodePlan(info.block_table, info.seq_lens_i32, self.local_q_heads,
                                               self.local_kv_heads, self.kv_mem_manager.num_pages,
                                               page_size=self.page_size,
-                                              shared_pages=self.shared_prefix_pages(ids))
+                                              shared_pages=self.shared_prefix_pages(ids),
+                                              slot_mapping=info.cur_select_index,
+                                              host_seq_lens=[mgr.req_token_count[r] for r in ids],
+                                              token_bytes=self.kv_token_bytes)
 
     def common_leading_pages(self, request_ids: Sequence[int], upcoming_tokens: int = 0) -> int:
         """How many leading pages are the same physical pages, and full, in every request of the

@@ -8,7 +8,7 @@ enqueue work on ``torch.cuda.current_stream()``.
 from __future__ import annotations
 
 import math
-from typing import Optional
+from typing import Optional, Sequence
 
 import torch
 
@@ -234,21 +234,53 @@ def balanced_chunks(num_kv_heads: int) -> int:
     return int(_lib.load().litekv_paged_decode_balanced_chunks(int(num_kv_heads)))
 
 
-class DecodePlan:
-    """Per-step cut of the batch's pages into equal chunks (one launch, reused by every layer).
+def per_sequence_decode_is_faster(batch: int, num_kv_heads: int, max_pages: int, total_pages: int,
+                                  token_bytes: int, page_size: int = PAGE_SIZE, margin: float = 1.05) -> bool:
+    """Which of the two decode schedules a step should take, from what the host knows about it.
 
-    Built from the block table and lengths of the step; holds the device plan buffer (chunk
-    entries) and the partial-result workspace of the balanced schedule. Launches that share a
+    One wavefront per (sequence, kv head) (``num_splits=1`` of the splits schedule: append launch +
+    one kernel, no merge) costs a dependent chain of page steps as long as the longest sequence,
+    the bytes at the rate such unbalanced streams reach, or the placement of its wavefronts,
+    whichever is largest. The balanced schedule (fused step + merge) costs two launches whose
+    fixed part is larger, the bytes at a higher rate, and a little per sequence. Constants (us, bytes
+    per us) are fits to 230 measured shapes on an MI355X (8 to 2048 sequences, 32 to 4096 tokens, uniform
+    and ragged, 8 and 4 kv heads): choosing by this rule is within 0.5 % of always choosing the faster
+    schedule on average (worst case 15 %), always balanced is 19 % slower on average. ``margin``: how
+    much faster the per-sequence estimate must be to be chosen."""
+    if batch <= 0 or total_pages <= 0:
+        return False
+    nbytes = float(total_pages) * page_size * token_bytes
+    per_sequence = max(6.0 + 0.57 * max_pages, 4.0 + nbytes / 4.5e6, 4.0 + 5.5e-3 * batch * num_kv_heads)
+    balanced = 12.0 + nbytes / 5.6e6 + 0.03 * batch
+    return per_sequence * margin < balanced
+
+
+class DecodePlan:
+    """Per-step decision how the batch's pages are attended, shared by every layer of the step.
+
+    Balanced schedule (default): the cut of the batch's pages into equal chunks (one launch), the
+    device plan buffer (chunk entries) and the partial-result workspace. Launches that share a
     plan share its workspace and must run one after the other (same stream).
+    Per-sequence schedule (``per_sequence`` True, see ``choose_schedule``): nothing to build;
+    ``decode_step`` then appends through ``slot_mapping`` and runs one wavefront per (sequence, kv head).
     """
 
     def __init__(self, block_table: torch.Tensor, seq_lens: torch.Tensor, num_q_heads: int,
                  num_kv_heads: int, num_pages: int, chunks: Optional[int] = None,
-                 page_size: int = PAGE_SIZE, shared_pages: int = 0):
+                 page_size: int = PAGE_SIZE, shared_pages: int = 0,
+                 slot_mapping: Optional[torch.Tensor] = None, host_seq_lens: Optional[Sequence[int]] = None,
+                 token_bytes: Optional[int] = None):
         """``shared_pages``: leading block-table entries that are the same physical pages in every
-        row (a shared cached prefix); they are then attended once for the whole batch."""
+        row (a shared cached prefix); they are then attended once for the whole batch.
+        ``slot_mapping`` [B] int32: the slots of the step's new tokens (what a separate append
+        takes); with it and ``host_seq_lens`` (the lengths as the host knows them) the plan picks
+        the per-sequence schedule where ``per_sequence_decode_is_faster`` says so. ``token_bytes``:
+        K + V bytes of one token in the pool (default: fp16)."""
         lib = _lib.load()
         self.shared_pages = int(shared_pages)
+        self.per_sequence = False
+        self.slot_mapping = None if slot_mapping is None else _dev_i32("slot_mapping", slot_mapping)
+        self.token_bytes = int(token_bytes) if token_bytes is not None else 2 * int(num_kv_heads) * HEAD_DIM * 2
         _need(0 <= self.shared_pages <= block_table.shape[1], "shared_pages out of range")
         _need(block_table.dim() == 2, "block_table must be [B, max_blocks]")
         self.block_table = _dev_i32("block_table", block_table)
@@ -268,10 +300,24 @@ class DecodePlan:
         ws_bytes = int(ws_fn(self.batch, self.num_q_heads, HEAD_DIM, self.chunks))
         self.workspace = torch.empty(max(4, ws_bytes // 4), dtype=torch.float32, device=dev)
         self.workspace_bytes = ws_bytes
+        if host_seq_lens is not None:
+            self.choose_schedule(host_seq_lens)
         self.refresh()
 
+    def choose_schedule(self, host_seq_lens: Sequence[int], margin: float = 1.05) -> bool:
+        """Sets ``per_sequence`` from the lengths as the host knows them (no device read). Needs
+        ``slot_mapping``; a plan with a shared prefix stays balanced. Returns the choice."""
+        if self.slot_mapping is None or self.shared_pages > 0:
+            self.per_sequence = False
+            return False
+        pages = [(int(n) + self.page_size - 1) // self.page_size for n in host_seq_lens if n > 0]
+        self.per_sequence = bool(pages) and per_sequence_decode_is_faster(
+            self.batch, self.num_kv_heads, max(pages), sum(pages), self.token_bytes, self.page_size, margin)
+        return self.per_sequence
+
     def refresh(self, block_table: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None) -> None:
-        """Recomputes the cuts after the tables or lengths changed (same shapes)."""
+        """Recomputes the cuts after the tables or lengths changed (same shapes). Nothing to do
+        while the plan is on the per-sequence schedule."""
         if block_table is not None:
             bt = _dev_i32("block_table", block_table)
             _need(bt.shape == self.block_table.shape and bt.stride(0) == self.bt_stride, "block_table shape changed")
@@ -280,6 +326,8 @@ class DecodePlan:
             sl = _dev_i32("seq_lens", seq_lens)
             _need(sl.numel() == self.batch, "seq_lens shape changed")
             self.seq_lens = sl
+        if self.per_sequence:
+            return
         lib = _lib.load()
         _lib.check(lib.litekv_decode_plan_prefix(_ptr(self.block_table), self.bt_stride, _ptr(self.seq_lens),
                                                  self.batch, self.num_kv_heads, self.page_size, self.num_pages,
@@ -331,10 +379,20 @@ def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
                 k_new: Optional[torch.Tensor] = None, v_new: Optional[torch.Tensor] = None,
                 softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
                 kv_scales: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The balanced schedule for one layer: optional append of k_new / v_new ([B, Hkv, D]) at logical
-    position seq_lens[b] - 1 fused into the attention of q [B, Hq, D] over the planned pages, then the
-    merge of the sequences that span several chunks. An fp8 pool (uint8 / float8_e4m3fn) comes with
-    its per-head ``kv_scales``."""
+    """One layer of a decode step under ``plan``. Balanced schedule: optional append of k_new / v_new
+    ([B, Hkv, D]) at logical position seq_lens[b] - 1 fused into the attention of q [B, Hq, D] over
+    the planned pages, then the merge of the sequences that span several chunks. Per-sequence
+    schedule (``plan.per_sequence``): the append through ``plan.slot_mapping``, then one wavefront
+    per (sequence, kv head). An fp8 pool (uint8 / float8_e4m3fn) comes with its per-head ``kv_scales``."""
+    if plan.per_sequence:
+        _need((k_new is None) == (v_new is None), "k_new and v_new go together")
+        if k_new is not None:
+            if is_fp8_pool(kv_pool):
+                kv_append_fp8(k_new, v_new, plan.slot_mapping, kv_pool, kv_scales)
+            else:
+                kv_append(k_new, v_new, plan.slot_mapping, kv_pool)
+        return paged_decode(q, kv_pool, plan.block_table, plan.seq_lens, softmax_scale, num_splits=1, out=out,
+                            page_size=plan.page_size, schedule="splits", kv_scales=kv_scales)
     _dev_half("q", q)
     fp8 = is_fp8_pool(kv_pool)
     if not fp8:

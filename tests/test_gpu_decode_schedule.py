@@ -1,0 +1,116 @@
+"""GPU: the per-sequence decode schedule chosen by a plan from host-known lengths gives the same
+result as the balanced one (attention tolerance against the oracle, pool bit for bit), for fp16
+and fp8 pools, through the executor, and across a change of schedule under graph replay."""
+
+import math
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from llama_lite_npu_amd import ops, workloads
+from oracle import c_oracle, cpu_ref, fp8
+from tests.parity import assert_attention_close, to_np16
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _plans(case, hq, hkv, lens, token_bytes=None):
+    routed = ops.DecodePlan(case.block_table, case.seq_lens, hq, hkv, case.num_pages, slot_mapping=case.slot_mapping,
+                            host_seq_lens=[n + 1 for n in lens], token_bytes=token_bytes)
+    balanced = ops.DecodePlan(case.block_table, case.seq_lens, hq, hkv, case.num_pages)
+    return routed, balanced
+
+
+@pytest.mark.parametrize("hq,hkv", [(64, 8), (32, 4), (16, 2), (40, 8), (8, 1)])
+def test_short_batches_take_the_per_sequence_schedule_with_the_same_result(hq, hkv):
+    rng = random.Random(hq + hkv)
+    lens = [rng.choice([0, rng.randint(1, 40), rng.randint(1, 120)]) for _ in range(48)]
+    print(f"per-sequence schedule: heads {hq}/{hkv} lens {lens[:10]}...", flush=True)
+    case = workloads.make_decode_case("sched", 31, lens, hq, hkv, device=DEV)
+    routed, balanced = _plans(case, hq, hkv, lens)
+    assert routed.per_sequence and not balanced.per_sequence
+    pool_a, pool_b = case.kv_pool.clone(), case.kv_pool.clone()
+    out_a = ops.decode_step(case.q, pool_a, routed, case.k_new, case.v_new, case.softmax_scale)
+    out_b = ops.decode_step(case.q, pool_b, balanced, case.k_new, case.v_new, case.softmax_scale)
+    torch.cuda.synchronize()
+    assert torch.equal(pool_a.view(torch.int16), pool_b.view(torch.int16))
+    ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool_a), case.block_table.cpu().numpy(),
+                                case.seq_lens.cpu().numpy(), case.softmax_scale)
+    assert_attention_close(out_a, ref, "per-sequence")
+    assert_attention_close(out_b, ref, "balanced")
+    # rows already stored (the fused epilogue did it): no append, same attention
+    again = ops.decode_step(case.q, pool_a, routed, None, None, case.softmax_scale)
+    assert torch.equal(again, out_a)
+
+
+def test_long_sequences_and_shared_prefixes_stay_balanced():
+    print("per-sequence schedule: cases that must not take it", flush=True)
+    lens = [37, 128, 511, 3000]
+    case = workloads.make_decode_case("sched", 32, lens, 16, 8, device=DEV)
+    routed, _ = _plans(case, 16, 8, lens)
+    assert not routed.per_sequence
+    short = [40] * 32
+    case = workloads.make_decode_case("sched", 33, short, 16, 8, device=DEV)
+    no_slots = ops.DecodePlan(case.block_table, case.seq_lens, 16, 8, case.num_pages, host_seq_lens=[41] * 32)
+    assert not no_slots.per_sequence                       # nothing to append through
+    shared = workloads.config_c4(DEV, batch=8, prefix=256, lo=8, hi=40)
+    plan = ops.DecodePlan(shared.block_table, shared.seq_lens, 64, 8, shared.num_pages, shared_pages=16,
+                          slot_mapping=shared.slot_mapping, host_seq_lens=shared.seq_lens.tolist())
+    assert not plan.per_sequence
+
+
+def test_fp8_pools_take_it_too():
+    hq, hkv = 32, 8
+    rng = random.Random(9)
+    lens = [rng.randint(1, 120) for _ in range(64)]
+    print("per-sequence schedule over an fp8 pool", flush=True)
+    case = workloads.make_decode_case("sched", 34, lens, hq, hkv, device=DEV)
+    scales = torch.cat([0.02 * (1 + 0.1 * torch.arange(hkv)), 0.015 * (1 + 0.2 * torch.arange(hkv))]).float().to(DEV)
+    pool = torch.empty(case.kv_pool.shape, dtype=torch.uint8, device=DEV)
+    every = torch.arange(pool.shape[0], dtype=torch.int32, device=DEV)
+    ops.kv_append_fp8(case.kv_pool[:, :hkv], case.kv_pool[:, hkv:], every, pool, scales)
+    routed, balanced = _plans(case, hq, hkv, lens, token_bytes=2 * hkv * 128)
+    assert routed.per_sequence
+    pool_a, pool_b = pool.clone(), pool.clone()
+    out_a = ops.decode_step(case.q, pool_a, routed, case.k_new, case.v_new, case.softmax_scale, kv_scales=scales)
+    out_b = ops.decode_step(case.q, pool_b, balanced, case.k_new, case.v_new, case.softmax_scale, kv_scales=scales)
+    torch.cuda.synchronize()
+    a, b = pool_a.cpu().numpy(), pool_b.cpu().numpy()
+    assert int(((a != b) & ~(((a & 0x7F) == 0) & ((b & 0x7F) == 0))).sum()) == 0
+    values = torch.from_numpy(fp8.dequantize_pool(a, scales.cpu().numpy()))
+    ref = cpu_ref.paged_decode_ref(case.q.cpu(), values, case.block_table.cpu(), case.seq_lens.cpu(),
+                                   case.softmax_scale).numpy()
+    assert_attention_close(out_a, ref, "fp8 per-sequence")
+    assert_attention_close(out_b, ref, "fp8 balanced")
+
+
+def test_graph_replay_follows_a_change_of_schedule():
+    """A small batch starts on the per-sequence schedule and outgrows it: the device batch moves
+    to the balanced one, the runner captures a second graph, and every step still matches an
+    executor that builds its metadata on the host."""
+    from tests.test_gpu_decode_graph import TinyModel, _executor, _host_step, _next_tokens, _prefill
+
+    print("graph replay across a change of decode schedule", flush=True)
+    host, graphed = _executor(num_pages=400, max_seq_len=512), _executor(num_pages=400, max_seq_len=512)
+    model_h, model_g = TinyModel(), TinyModel()
+    lens = [100, 20, 90, 5]
+    ids_h, ids_g = _prefill(host, lens, 4), _prefill(graphed, lens, 4)
+    graphed.attach_model(model_g, "qwen3")
+    batch = graphed.activate_device_decode_batch(ids_g, reserve_tokens=32)
+    assert batch.decode_plan.per_sequence
+    tok_h = tok_g = torch.tensor([[7], [8], [9], [10]], device=DEV)
+    seen = set()
+    for step in range(120):
+        out_h = _host_step(host, model_h, ids_h, tok_h)
+        graphed.extend_paged_requests(ids_g)
+        out_g = graphed.forward(tok_g)
+        torch.cuda.synchronize()
+        seen.add(batch.decode_plan.per_sequence)
+        assert float((out_h - out_g).abs().max()) <= 3 * 2e-3, f"step {step}"     # three layers summed
+        tok_h = tok_g = _next_tokens(out_h)
+    assert seen == {True, False} and not batch.decode_plan.per_sequence
+    assert graphed.graph_runner.capture_count == 2
+    batch.check()
