@@ -5,14 +5,16 @@ Mirror of ``Attention.context_forward / token_forward`` in the reference's model
 arguments, driven by the same ``AttentionInfo``. Differences:
 
 * no ``torch.cat([xk, xv])``: K and V rows go to the pool straight from their own tensors;
-* decode is one fused launch (append + attention) when the step carries a ``DecodePlan``;
+* decode follows the step's ``DecodePlan``: one fused launch (append + attention) and a merge
+  on the balanced schedule, or an append and one wavefront per (sequence, kv head) where the
+  plan found the step small enough for that to be faster;
 * prefill reads K/V through the block table (context 0 for a fresh prompt, history for later
   chunks), so one kernel serves both branches of the reference;
 * ``qkv_epilogue`` folds the step before the append (QK RMSNorm, rotary embedding,
   qwen3.py:124-129) into the append itself; the forward calls are then made with ``xk=None``;
 * a layer whose pool holds fp8 codes (``atten_info.kv_scales[layer]`` set) quantises on append
-  and decodes straight from the codes; prefill over cached history first turns the batch's
-  pages into a scratch fp16 pool, fresh prompts attend to their own fp16 K/V.
+  and attends straight from the codes, in decode and in chunks over cached history; fresh
+  prompts attend to their own fp16 K/V.
 
 ``qk_scale`` follows the reference's convention (qwen3.py:295-298): the natural 1/sqrt(D) for
 decode, multiplied by log2(e) for prefill; it is un-folded here.
