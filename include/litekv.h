@@ -357,6 +357,37 @@ int litekv_paged_decode_fp8(const void *q, int64_t q_batch_stride, const void *k
                             int32_t min_pages_per_split, float softmax_scale, void *stream);
 
 /*
+ * litekv_paged_decode with the step's append fused in: the wavefront that
+ * attends a sequence's last page first writes the step's token (rows k_new[b],
+ * v_new[b] of [batch][num_kv_heads][128] fp16, element strides per sequence)
+ * at logical position seq_lens[b] - 1 of the pages the block table names, as
+ * litekv_kv_append would through that token's slot, and attends it. Replaces,
+ * in one launch for max_splits == 1, the reference's per-layer pair
+ * update_kv_buffer + flash_decoding (models/qwen3.py:62-74;
+ * kernels/update_kv_buffer.py:46-81, kernels/flashdecoding.py:294-342) for
+ * steps small enough that one wavefront per (sequence, kv head) beats the
+ * balanced cut. The _fp8 variant quantises the rows with the pool's scales
+ * exactly as litekv_kv_append_fp8 does.
+ */
+int litekv_paged_decode_append(const void *q, int64_t q_batch_stride, void *kv_pool,
+                               const int32_t *block_table, int32_t block_table_stride,
+                               const int32_t *seq_lens, const void *k_new, const void *v_new,
+                               int64_t k_new_stride, int64_t v_new_stride, void *out,
+                               void *workspace, size_t workspace_bytes, int32_t batch,
+                               int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                               int32_t page_size, int64_t num_pages, int32_t max_splits,
+                               int32_t min_pages_per_split, float softmax_scale, void *stream);
+int litekv_paged_decode_append_fp8(const void *q, int64_t q_batch_stride, void *kv_pool_fp8,
+                                   const float *scales, const int32_t *block_table,
+                                   int32_t block_table_stride, const int32_t *seq_lens,
+                                   const void *k_new, const void *v_new, int64_t k_new_stride,
+                                   int64_t v_new_stride, void *out, void *workspace,
+                                   size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+                                   int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                                   int64_t num_pages, int32_t max_splits,
+                                   int32_t min_pages_per_split, float softmax_scale, void *stream);
+
+/*
  * litekv_paged_decode_prefix over an fp8 pool (plan from
  * litekv_decode_plan_prefix, workspace from
  * litekv_paged_decode_prefix_workspace_bytes): the shared pages of a cached

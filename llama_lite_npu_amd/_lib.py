@@ -55,6 +55,18 @@ SIGNATURES = {
          c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32, c_float,
          c_void_p],
     ),
+    "litekv_paged_decode_append": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+         c_void_p, c_void_p, c_size_t, c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32,
+         c_int32, c_float, c_void_p],
+    ),
+    "litekv_paged_decode_append_fp8": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
+         c_int64, c_void_p, c_void_p, c_size_t, c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,
+         c_int32, c_int32, c_float, c_void_p],
+    ),
     "litekv_paged_decode_split": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_size_t,

@@ -357,6 +357,27 @@ __device__ __forceinline__ int clamp_page(int pid, int num_pages) {
   return pid < 0 ? 0 : (pid >= num_pages ? num_pages - 1 : pid);
 }
 
+// This lane's parts of the step's new K and V rows (fp16, head h of one sequence): the pieces
+// that sit where the lane's page registers hold the token's row (see PageRegs / PageRegsFp8).
+template <bool FP8>
+__device__ __forceinline__ void load_new_rows(uint4_t (&kr)[4], uint4_t (&vr)[2], const half_t *kn,
+                                              const half_t *vn, int n, int g) {
+  if constexpr (FP8) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      kr[2 * j] = *(const uint4_t *)(kn + 64 * j + 16 * g);
+      kr[2 * j + 1] = *(const uint4_t *)(kn + 64 * j + 16 * g + 8);
+    }
+    vr[0] = *(const uint4_t *)(vn + 16 * (n & 7));
+    vr[1] = *(const uint4_t *)(vn + 16 * (n & 7) + 8);
+  } else {
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) kr[kk] = *(const uint4_t *)(kn + 32 * kk + 8 * g);
+    vr[0] = *(const uint4_t *)(vn + 8 * n);
+    vr[1] = uint4_t{0, 0, 0, 0};  // fp8 only
+  }
+}
+
 // ---------------------------------------------------------------------------------------------
 // Schedule "splits": one wavefront per (kv head, split, sequence).
 // Partials: part_o[b][hq][split][D], part_lse[b][hq][split].
@@ -369,14 +390,16 @@ __device__ __forceinline__ int clamp_page(int pid, int num_pages) {
 // ---------------------------------------------------------------------------------------------
 constexpr int kSplitWaves = 4;
 extern __shared__ __attribute__((aligned(16))) half_t split_vstage[];  // [waves][kPageSize * kVPitch]
-template <int DEPTH, bool FP8>
+template <int DEPTH, bool FP8, bool APPEND>
 __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
     const half_t *__restrict__ q, int64_t q_batch_stride,
-    const typename KvStore<FP8>::elem *__restrict__ kv, const float *__restrict__ scales,
+    typename KvStore<FP8>::elem *__restrict__ kv, const float *__restrict__ scales,
     const int32_t *__restrict__ block_table, int32_t bt_stride,
-    const int32_t *__restrict__ seq_lens, half_t *__restrict__ out, float *__restrict__ part_o,
-    float *__restrict__ part_lse, int32_t num_q_heads, int32_t num_kv_heads, int32_t group,
-    int32_t max_splits, int32_t min_pages_per_split, int32_t num_pages, float scale_log2) {
+    const int32_t *__restrict__ seq_lens, const half_t *__restrict__ k_new,
+    const half_t *__restrict__ v_new, int64_t k_new_stride, int64_t v_new_stride,
+    half_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_lse,
+    int32_t num_q_heads, int32_t num_kv_heads, int32_t group, int32_t max_splits,
+    int32_t min_pages_per_split, int32_t num_pages, float scale_log2) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int n = lane & 15;   // query head inside the group (column of S^T)
@@ -406,21 +429,31 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
   typedef typename KvStore<FP8>::elem Elem;
   typedef typename KvStore<FP8>::page Page;
   half8_t qf[4];
-  float v_scale = 1.0f;
+  float v_scale = 1.0f, k_inv = 1.0f, v_inv = 1.0f;
   if constexpr (FP8) {  // the K scale joins the softmax scale, the V scale the normalisation
     load_q_fp8_order(qf, q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
-    scale_log2 *= scales[h];
+    const float ks = scales[h];
+    scale_log2 *= ks;
     v_scale = scales[num_kv_heads + h];
+    k_inv = 1.0f / ks;  // the step's new rows are quantised with the reciprocals
+    v_inv = 1.0f / v_scale;
   } else {
     load_q(qf, q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
+  }
+  // Fused append: the wavefront that attends the sequence's last page writes the step's token
+  // into it. Its rows are requested here, before the pages.
+  uint4_t k_row[4] = {}, v_row[2] = {};
+  if constexpr (APPEND) {
+    load_new_rows<FP8>(k_row, v_row, k_new + (int64_t)b * k_new_stride + (int64_t)h * kHeadDim,
+                       v_new + (int64_t)b * v_new_stride + (int64_t)h * kHeadDim, n, g);
   }
 
   const int64_t row_stride = (int64_t)2 * num_kv_heads * kHeadDim;  // elements per slot
   // this lane's row and column inside page 0 (see PageRegs / PageRegsFp8)
-  const Elem *k_lane = kv + (int64_t)h * kHeadDim + (FP8 ? 16 : 8) * g + n * row_stride;
-  const Elem *v_lane = FP8 ? kv + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7) +
-                                 (2 * g + (n >> 3)) * row_stride
-                           : kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
+  Elem *k_lane = kv + (int64_t)h * kHeadDim + (FP8 ? 16 : 8) * g + n * row_stride;
+  Elem *v_lane = FP8 ? kv + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7) +
+                           (2 * g + (n >> 3)) * row_stride
+                     : kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
   const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
   const int32_t *table = block_table + (int64_t)b * bt_stride;
 
@@ -445,7 +478,60 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
   for (int p = p0; p < p1; p += DEPTH) {
 #pragma unroll
     for (int dd = 0; dd < DEPTH; ++dd) {
-      if (p + dd < p1) attend_page(st, buf[dd], qf, vstage, vt_lane, p + dd, len, n, g, scale_log2);
+      if (p + dd < p1) {
+        if (APPEND && (p + dd + 1) * kPageSize >= len) {
+          // The sequence's last page: the step's new token (logical position len - 1) goes to
+          // the pool and replaces the stale values this wavefront loaded before the write; an
+          // fp8 pool gets the codes the append kernel would store and is attended as stored.
+          // (Written out here: behind a function taking the page by reference the page
+          // registers of both pages in flight end up in scratch memory.)
+          const int t_new = (len - 1) & (kPageSize - 1);
+          const int64_t slot_off = ((int64_t)page_id(p + dd) * kPageSize + t_new) * row_stride;
+          Page &r = buf[dd];
+          if constexpr (FP8) {
+            if (n == t_new) {
+              uint8_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 16 * g;
+#pragma unroll
+              for (int j = 0; j < 2; ++j) {
+                const uint2_t lo = half8_to_fp8(__builtin_bit_cast(half8_t, k_row[2 * j]), k_inv);
+                const uint2_t hi = half8_to_fp8(__builtin_bit_cast(half8_t, k_row[2 * j + 1]), k_inv);
+                const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
+                r.k[j] = x;
+                *(uint4_t *)(dst + 64 * j) = x;
+              }
+            }
+            if (2 * g + (n >> 3) == (t_new & 7)) {
+              const uint2_t lo = half8_to_fp8(__builtin_bit_cast(half8_t, v_row[0]), v_inv);
+              const uint2_t hi = half8_to_fp8(__builtin_bit_cast(half8_t, v_row[1]), v_inv);
+              const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
+              *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7)) = x;
+#pragma unroll
+              for (int i = 0; i < 2; ++i) {
+                if (i == (t_new >> 3)) r.v[i] = x;
+              }
+            }
+          } else {
+            if (n == t_new) {
+              half_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 8 * g;
+#pragma unroll
+              for (int kk = 0; kk < 4; ++kk) {
+                const half8_t x = __builtin_bit_cast(half8_t, k_row[kk]);
+                r.k[kk] = x;
+                *(half8_t *)(dst + 32 * kk) = x;
+              }
+            }
+            if (g == (t_new & 3)) {
+              const half8_t x = __builtin_bit_cast(half8_t, v_row[0]);
+              *(half8_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n) = x;
+#pragma unroll
+              for (int i = 0; i < 4; ++i) {
+                if (i == (t_new >> 2)) r.v[i] = x;
+              }
+            }
+          }
+        }
+        attend_page(st, buf[dd], qf, vstage, vt_lane, p + dd, len, n, g, scale_log2);
+      }
       request(p + dd + DEPTH, buf[dd]);
     }
   }
@@ -1160,6 +1246,10 @@ struct DecodeArgs {
   int64_t num_pages;
   float softmax_scale;
   void *stream;
+  // the step's new rows [B][Hkv][D] for the append fused into the splits schedule (or null)
+  const void *k_new = nullptr;
+  const void *v_new = nullptr;
+  int64_t k_new_stride = 0, v_new_stride = 0;
 };
 
 // Checks shared by every decode entry point; `need_inputs` is false for the merge-only calls.
@@ -1243,20 +1333,37 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   const dim3 grid((unsigned)(a.num_kv_heads / waves), (unsigned)max_splits, (unsigned)a.batch);
   const dim3 block((unsigned)(waves * kWave));
   const size_t lds = (size_t)waves * kPageSize * kVPitch * sizeof(half_t);
+  LITEKV_REQUIRE((a.k_new == nullptr) == (a.v_new == nullptr), "%s: k_new and v_new go together", what);
+  if (a.k_new != nullptr) {
+    const int64_t row = (int64_t)a.num_kv_heads * a.head_dim;
+    LITEKV_REQUIRE(aligned16(a.k_new) && aligned16(a.v_new), "%s: k_new, v_new must be 16-byte aligned",
+                   what);
+    LITEKV_REQUIRE(a.k_new_stride >= row && a.v_new_stride >= row && a.k_new_stride % 8 == 0 &&
+                       a.v_new_stride % 8 == 0,
+                   "%s: k_new/v_new strides (%lld, %lld) invalid", what, (long long)a.k_new_stride,
+                   (long long)a.v_new_stride);
+  }
+  // The pool is written only by the instantiations with the fused append.
+  void *pool = const_cast<void *>(a.kv_pool);
+  auto launch = [&](auto kernel, auto *kv) {
+    hipLaunchKernelGGL(kernel, grid, block, lds, static_cast<hipStream_t>(a.stream),
+                       static_cast<const half_t *>(a.q), a.q_batch_stride, kv, fp8_scales,
+                       a.block_table, a.block_table_stride, a.seq_lens,
+                       static_cast<const half_t *>(a.k_new), static_cast<const half_t *>(a.v_new),
+                       a.k_new_stride, a.v_new_stride, static_cast<half_t *>(a.out), part_o, part_lse,
+                       a.num_q_heads, a.num_kv_heads, group, max_splits, min_pages_per_split,
+                       (int32_t)a.num_pages, a.softmax_scale * kLog2e);
+  };
   if (fp8_scales != nullptr) {
-    hipLaunchKernelGGL((paged_decode_split_kernel<LITEKV_DECODE_DEPTH, true>), grid, block, lds,
-                       static_cast<hipStream_t>(a.stream), static_cast<const half_t *>(a.q),
-                       a.q_batch_stride, static_cast<const uint8_t *>(a.kv_pool), fp8_scales,
-                       a.block_table, a.block_table_stride, a.seq_lens, static_cast<half_t *>(a.out),
-                       part_o, part_lse, a.num_q_heads, a.num_kv_heads, group, max_splits,
-                       min_pages_per_split, (int32_t)a.num_pages, a.softmax_scale * kLog2e);
+    if (a.k_new != nullptr) {
+      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, true, true>, static_cast<uint8_t *>(pool));
+    } else {
+      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, true, false>, static_cast<uint8_t *>(pool));
+    }
+  } else if (a.k_new != nullptr) {
+    launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, false, true>, static_cast<half_t *>(pool));
   } else {
-    hipLaunchKernelGGL((paged_decode_split_kernel<LITEKV_DECODE_DEPTH, false>), grid, block, lds,
-                       static_cast<hipStream_t>(a.stream), static_cast<const half_t *>(a.q),
-                       a.q_batch_stride, static_cast<const half_t *>(a.kv_pool), fp8_scales,
-                       a.block_table, a.block_table_stride, a.seq_lens, static_cast<half_t *>(a.out),
-                       part_o, part_lse, a.num_q_heads, a.num_kv_heads, group, max_splits,
-                       min_pages_per_split, (int32_t)a.num_pages, a.softmax_scale * kLog2e);
+    launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, false, false>, static_cast<half_t *>(pool));
   }
   return check_launch(what);
 }
@@ -1672,6 +1779,48 @@ extern "C" int litekv_paged_decode(const void *q, int64_t q_batch_stride, const 
                        workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim,
                        page_size, num_pages, softmax_scale, stream};
   int rc = litekv::launch_split(a, max_splits, min_pages_per_split);
+  if (rc != LITEKV_OK) return rc;
+  return litekv::launch_merge(a, max_splits, min_pages_per_split);
+}
+
+extern "C" int litekv_paged_decode_append(const void *q, int64_t q_batch_stride, void *kv_pool,
+                                          const int32_t *block_table, int32_t block_table_stride,
+                                          const int32_t *seq_lens, const void *k_new,
+                                          const void *v_new, int64_t k_new_stride,
+                                          int64_t v_new_stride, void *out, void *workspace,
+                                          size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+                                          int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                                          int64_t num_pages, int32_t max_splits,
+                                          int32_t min_pages_per_split, float softmax_scale,
+                                          void *stream) {
+  if ((k_new == nullptr || v_new == nullptr) && batch > 0) {
+    return litekv::fail(LITEKV_ERR_INVALID_ARGUMENT, "paged_decode_append: k_new / v_new is null");
+  }
+  litekv::DecodeArgs a{q, q_batch_stride, kv_pool, block_table, block_table_stride, seq_lens, out,
+                       workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim,
+                       page_size, num_pages, softmax_scale, stream, k_new, v_new, k_new_stride,
+                       v_new_stride};
+  int rc = litekv::launch_split(a, max_splits, min_pages_per_split);
+  if (rc != LITEKV_OK) return rc;
+  return litekv::launch_merge(a, max_splits, min_pages_per_split);
+}
+
+extern "C" int litekv_paged_decode_append_fp8(
+    const void *q, int64_t q_batch_stride, void *kv_pool_fp8, const float *scales,
+    const int32_t *block_table, int32_t block_table_stride, const int32_t *seq_lens,
+    const void *k_new, const void *v_new, int64_t k_new_stride, int64_t v_new_stride, void *out,
+    void *workspace, size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+    int32_t num_kv_heads, int32_t head_dim, int32_t page_size, int64_t num_pages,
+    int32_t max_splits, int32_t min_pages_per_split, float softmax_scale, void *stream) {
+  if ((scales == nullptr || k_new == nullptr || v_new == nullptr) && batch > 0) {
+    return litekv::fail(LITEKV_ERR_INVALID_ARGUMENT,
+                        "paged_decode_append_fp8: scales / k_new / v_new is null");
+  }
+  litekv::DecodeArgs a{q, q_batch_stride, kv_pool_fp8, block_table, block_table_stride, seq_lens, out,
+                       workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim,
+                       page_size, num_pages, softmax_scale, stream, k_new, v_new, k_new_stride,
+                       v_new_stride};
+  int rc = litekv::launch_split(a, max_splits, min_pages_per_split, batch > 0 ? scales : nullptr);
   if (rc != LITEKV_OK) return rc;
   return litekv::launch_merge(a, max_splits, min_pages_per_split);
 }

@@ -86,7 +86,6 @@ class DeviceDecodeBatch:
         self.decode_plan = ops.DecodePlan(self.block_table, self.seq_lens_i32, executor.local_q_heads,
                                           executor.local_kv_heads, executor.kv_mem_manager.num_pages,
                                           page_size=executor.page_size, shared_pages=self.shared_pages,
-                                          slot_mapping=self.cur_select_index,
                                           token_bytes=getattr(executor, "kv_token_bytes", None))
         self.load(request_ids, reserve_tokens, host_ahead)
 
@@ -329,9 +328,8 @@ class DecodeGraphRunner:
 
             info.decode_plan = ops.DecodePlan(info.block_table, info.seq_lens_i32, plan.num_q_heads,
                                               plan.num_kv_heads, plan.num_pages, plan.chunks, plan.page_size,
-                                              plan.shared_pages, slot_mapping=info.cur_select_index,
-                                              token_bytes=plan.token_bytes)
-            info.decode_plan.per_sequence = bool(plan.per_sequence and info.cur_select_index is not None)
+                                              plan.shared_pages, token_bytes=plan.token_bytes)
+            info.decode_plan.per_sequence = bool(plan.per_sequence)
         return info
 
     def capture(self, input_ids: torch.Tensor, position_ids: torch.Tensor, atten_info) -> bool:

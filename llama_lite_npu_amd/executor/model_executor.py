@@ -305,7 +305,6 @@ class ModelExecutor:
                                               self.local_kv_heads, self.kv_mem_manager.num_pages,
                                               page_size=self.page_size,
                                               shared_pages=self.shared_prefix_pages(ids),
-                                              slot_mapping=info.cur_select_index,
                                               host_seq_lens=[mgr.req_token_count[r] for r in ids],
                                               token_bytes=self.kv_token_bytes)
 

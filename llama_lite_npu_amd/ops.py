@@ -262,24 +262,21 @@ class DecodePlan:
     device plan buffer (chunk entries) and the partial-result workspace. Launches that share a
     plan share its workspace and must run one after the other (same stream).
     Per-sequence schedule (``per_sequence`` True, see ``choose_schedule``): nothing to build;
-    ``decode_step`` then appends through ``slot_mapping`` and runs one wavefront per (sequence, kv head).
+    ``decode_step`` then runs one wavefront per (sequence, kv head), the append fused in.
     """
 
     def __init__(self, block_table: torch.Tensor, seq_lens: torch.Tensor, num_q_heads: int,
                  num_kv_heads: int, num_pages: int, chunks: Optional[int] = None,
                  page_size: int = PAGE_SIZE, shared_pages: int = 0,
-                 slot_mapping: Optional[torch.Tensor] = None, host_seq_lens: Optional[Sequence[int]] = None,
-                 token_bytes: Optional[int] = None):
+                 host_seq_lens: Optional[Sequence[int]] = None, token_bytes: Optional[int] = None):
         """``shared_pages``: leading block-table entries that are the same physical pages in every
         row (a shared cached prefix); they are then attended once for the whole batch.
-        ``slot_mapping`` [B] int32: the slots of the step's new tokens (what a separate append
-        takes); with it and ``host_seq_lens`` (the lengths as the host knows them) the plan picks
-        the per-sequence schedule where ``per_sequence_decode_is_faster`` says so. ``token_bytes``:
+        ``host_seq_lens``: the lengths as the host knows them; with them the plan picks the
+        per-sequence schedule where ``per_sequence_decode_is_faster`` says so. ``token_bytes``:
         K + V bytes of one token in the pool (default: fp16)."""
         lib = _lib.load()
         self.shared_pages = int(shared_pages)
         self.per_sequence = False
-        self.slot_mapping = None if slot_mapping is None else _dev_i32("slot_mapping", slot_mapping)
         self.token_bytes = int(token_bytes) if token_bytes is not None else 2 * int(num_kv_heads) * HEAD_DIM * 2
         _need(0 <= self.shared_pages <= block_table.shape[1], "shared_pages out of range")
         _need(block_table.dim() == 2, "block_table must be [B, max_blocks]")
@@ -305,9 +302,9 @@ class DecodePlan:
         self.refresh()
 
     def choose_schedule(self, host_seq_lens: Sequence[int], margin: float = 1.05) -> bool:
-        """Sets ``per_sequence`` from the lengths as the host knows them (no device read). Needs
-        ``slot_mapping``; a plan with a shared prefix stays balanced. Returns the choice."""
-        if self.slot_mapping is None or self.shared_pages > 0:
+        """Sets ``per_sequence`` from the lengths as the host knows them (no device read). A plan
+        with a shared prefix stays balanced. Returns the choice."""
+        if self.shared_pages > 0:
             self.per_sequence = False
             return False
         pages = [(int(n) + self.page_size - 1) // self.page_size for n in host_seq_lens if n > 0]
@@ -382,17 +379,12 @@ def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
     """One layer of a decode step under ``plan``. Balanced schedule: optional append of k_new / v_new
     ([B, Hkv, D]) at logical position seq_lens[b] - 1 fused into the attention of q [B, Hq, D] over
     the planned pages, then the merge of the sequences that span several chunks. Per-sequence
-    schedule (``plan.per_sequence``): the append through ``plan.slot_mapping``, then one wavefront
-    per (sequence, kv head). An fp8 pool (uint8 / float8_e4m3fn) comes with its per-head ``kv_scales``."""
+    schedule (``plan.per_sequence``): the same in one launch of one wavefront per (sequence, kv
+    head), no merge. An fp8 pool (uint8 / float8_e4m3fn) comes with its per-head ``kv_scales``."""
     if plan.per_sequence:
-        _need((k_new is None) == (v_new is None), "k_new and v_new go together")
-        if k_new is not None:
-            if is_fp8_pool(kv_pool):
-                kv_append_fp8(k_new, v_new, plan.slot_mapping, kv_pool, kv_scales)
-            else:
-                kv_append(k_new, v_new, plan.slot_mapping, kv_pool)
         return paged_decode(q, kv_pool, plan.block_table, plan.seq_lens, softmax_scale, num_splits=1, out=out,
-                            page_size=plan.page_size, schedule="splits", kv_scales=kv_scales)
+                            page_size=plan.page_size, schedule="splits", kv_scales=kv_scales,
+                            k_new=k_new, v_new=v_new)
     _dev_half("q", q)
     fp8 = is_fp8_pool(kv_pool)
     if not fp8:
@@ -457,7 +449,8 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
                  workspace: Optional[torch.Tensor] = None, page_size: int = PAGE_SIZE,
                  stage: str = "both", schedule: Optional[str] = None,
                  chunks: Optional[int] = None, plan: Optional[DecodePlan] = None,
-                 shared_pages: int = 0, kv_scales: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 shared_pages: int = 0, kv_scales: Optional[torch.Tensor] = None,
+                 k_new: Optional[torch.Tensor] = None, v_new: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Decode attention of q [B, Hq, D] over the pages named by block_table [B, max_blocks].
 
     ``shared_pages`` (balanced schedule): the first that many entries of every block-table row are
@@ -468,6 +461,8 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
     passed. schedule "splits" (chosen when num_splits, max_splits or min_pages_per_split is
     given): every sequence is cut into its own splits; two launches (`stage` selects one).
     An fp8 pool comes with its ``kv_scales``; either schedule reads it.
+    ``k_new`` / ``v_new`` [B, Hkv, D] (splits schedule, both stages): the step's new token of every
+    sequence is written at logical position seq_lens[b] - 1 by the same launch and attended.
     """
     _dev_half("q", q)
     if not is_fp8_pool(kv_pool):
@@ -482,8 +477,10 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
         schedule = "splits" if any(x is not None for x in split_args) or stage != "both" else "balanced"
     _need(schedule in ("balanced", "splits"), f"unknown schedule {schedule!r}")
 
+    _need((k_new is None) == (v_new is None), "k_new and v_new go together")
     if schedule == "balanced":
         _need(stage == "both", "the balanced schedule is a single launch")
+        _need(k_new is None, "the balanced schedule appends through decode_step")
         if plan is None:
             plan = DecodePlan(block_table, seq_lens, hq, hkv, n_pages, chunks, page_size, shared_pages)
         return decode_step(q, kv_pool, plan, None, None, softmax_scale, out, kv_scales)
@@ -512,7 +509,21 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
     if workspace is None:
         workspace = decode_workspace(b, hq, max_splits, q.device)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    if fp8:
+    if k_new is not None:
+        _need(stage == "both", "the fused append belongs to the call that runs both stages")
+        _dev_half("k_new", k_new), _dev_half("v_new", v_new)
+        _need(k_new.shape == (b, hkv, d) and v_new.shape == (b, hkv, d), "k_new / v_new must be [B, Hkv, D]")
+        rows = (_ptr(k_new), _ptr(v_new), _rows("k_new", k_new), _rows("v_new", v_new))
+        tail = (_ptr(out), _ptr(workspace), ws_bytes, b, hq, hkv, d, page_size, n_pages, max_splits,
+                min_pages_per_split, float(softmax_scale), _stream())
+        if fp8:
+            _lib.check(lib.litekv_paged_decode_append_fp8(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales),
+                                                          _ptr(block_table), block_table.stride(0), _ptr(seq_lens),
+                                                          *rows, *tail))
+        else:
+            _lib.check(lib.litekv_paged_decode_append(_ptr(q), q_stride, _ptr(kv_pool), _ptr(block_table),
+                                                      block_table.stride(0), _ptr(seq_lens), *rows, *tail))
+    elif fp8:
         _lib.check(lib.litekv_paged_decode_fp8(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(block_table),
                                                block_table.stride(0), _ptr(seq_lens), _ptr(out), _ptr(workspace),
                                                ws_bytes, b, hq, hkv, d, page_size, n_pages, max_splits,

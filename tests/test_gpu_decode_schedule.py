@@ -1,6 +1,7 @@
-"""GPU: the per-sequence decode schedule chosen by a plan from host-known lengths gives the same
-result as the balanced one (attention tolerance against the oracle, pool bit for bit), for fp16
-and fp8 pools, through the executor, and across a change of schedule under graph replay."""
+"""GPU: the per-sequence decode schedule chosen by a plan from host-known lengths (append fused
+into one wavefront per sequence and kv head) gives the same result as the balanced one (attention
+tolerance against the oracle, pool bit for bit), for fp16 and fp8 pools, and across a change of
+schedule under graph replay; the fused append of the splits schedule with several splits."""
 
 import math
 import random
@@ -18,7 +19,7 @@ DEV = "cuda:0"
 
 
 def _plans(case, hq, hkv, lens, token_bytes=None):
-    routed = ops.DecodePlan(case.block_table, case.seq_lens, hq, hkv, case.num_pages, slot_mapping=case.slot_mapping,
+    routed = ops.DecodePlan(case.block_table, case.seq_lens, hq, hkv, case.num_pages,
                             host_seq_lens=[n + 1 for n in lens], token_bytes=token_bytes)
     balanced = ops.DecodePlan(case.block_table, case.seq_lens, hq, hkv, case.num_pages)
     return routed, balanced
@@ -52,13 +53,9 @@ def test_long_sequences_and_shared_prefixes_stay_balanced():
     case = workloads.make_decode_case("sched", 32, lens, 16, 8, device=DEV)
     routed, _ = _plans(case, 16, 8, lens)
     assert not routed.per_sequence
-    short = [40] * 32
-    case = workloads.make_decode_case("sched", 33, short, 16, 8, device=DEV)
-    no_slots = ops.DecodePlan(case.block_table, case.seq_lens, 16, 8, case.num_pages, host_seq_lens=[41] * 32)
-    assert not no_slots.per_sequence                       # nothing to append through
     shared = workloads.config_c4(DEV, batch=8, prefix=256, lo=8, hi=40)
     plan = ops.DecodePlan(shared.block_table, shared.seq_lens, 64, 8, shared.num_pages, shared_pages=16,
-                          slot_mapping=shared.slot_mapping, host_seq_lens=shared.seq_lens.tolist())
+                          host_seq_lens=shared.seq_lens.tolist())
     assert not plan.per_sequence
 
 
@@ -114,3 +111,56 @@ def test_graph_replay_follows_a_change_of_schedule():
     assert seen == {True, False} and not batch.decode_plan.per_sequence
     assert graphed.graph_runner.capture_count == 2
     batch.check()
+
+
+@pytest.mark.parametrize("splits", [1, 2, 5, 16])
+def test_append_fused_into_the_splits_schedule(splits):
+    """litekv_paged_decode_append[_fp8]: pool = separate append bit for bit, attention = the oracle
+    on that pool, whatever the number of splits (the last split's wavefront writes the token)."""
+    rng = random.Random(40 + splits)
+    for hq, hkv in ((64, 8), (16, 2), (12, 4)):
+        lens = [rng.choice([0, 15, 16, 17, rng.randint(0, 70), rng.randint(100, 1500)]) for _ in range(9)]
+        print(f"fused append, {splits} splits, heads {hq}/{hkv}, lens {lens}", flush=True)
+        case = workloads.make_decode_case("fa", 50 + splits, lens, hq, hkv, device=DEV)
+        want = case.kv_pool.clone()
+        ops.kv_append(case.k_new, case.v_new, case.slot_mapping, want)
+        pool = case.kv_pool.clone()
+        out = ops.paged_decode(case.q, pool, case.block_table, case.seq_lens, case.softmax_scale, schedule="splits",
+                               num_splits=splits, k_new=case.k_new, v_new=case.v_new)
+        torch.cuda.synchronize()
+        assert torch.equal(pool.view(torch.int16), want.view(torch.int16))
+        ref = c_oracle.paged_decode(to_np16(case.q), to_np16(want), case.block_table.cpu().numpy(),
+                                    case.seq_lens.cpu().numpy(), case.softmax_scale)
+        assert_attention_close(out, ref, f"fused append {splits}")
+        # fp8 pool: the codes of a separate quantising append, attention over the decoded codes
+        scales = torch.cat([0.02 * (1 + 0.1 * torch.arange(hkv)), 0.015 * (1 + 0.2 * torch.arange(hkv))]).float().to(DEV)
+        codes = torch.empty(case.kv_pool.shape, dtype=torch.uint8, device=DEV)
+        every = torch.arange(codes.shape[0], dtype=torch.int32, device=DEV)
+        ops.kv_append_fp8(case.kv_pool[:, :hkv], case.kv_pool[:, hkv:], every, codes, scales)
+        want8 = codes.clone()
+        ops.kv_append_fp8(case.k_new, case.v_new, case.slot_mapping, want8, scales)
+        out8 = ops.paged_decode(case.q, codes, case.block_table, case.seq_lens, case.softmax_scale, schedule="splits",
+                                num_splits=splits, kv_scales=scales, k_new=case.k_new, v_new=case.v_new)
+        torch.cuda.synchronize()
+        a, b = codes.cpu().numpy(), want8.cpu().numpy()
+        assert int(((a != b) & ~(((a & 0x7F) == 0) & ((b & 0x7F) == 0))).sum()) == 0
+        values = torch.from_numpy(fp8.dequantize_pool(a, scales.cpu().numpy()))
+        ref8 = cpu_ref.paged_decode_ref(case.q.cpu(), values, case.block_table.cpu(), case.seq_lens.cpu(),
+                                        case.softmax_scale).numpy()
+        assert_attention_close(out8, ref8, f"fused append fp8 {splits}")
+
+
+def test_fused_append_argument_checks():
+    case = workloads.make_decode_case("fa", 60, [20, 30], 16, 8, device=DEV)
+    with pytest.raises(ValueError, match="k_new and v_new go together"):
+        ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, schedule="splits", num_splits=1,
+                         k_new=case.k_new)
+    with pytest.raises(ValueError, match="both stages"):
+        ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, schedule="splits", num_splits=2,
+                         stage="split", k_new=case.k_new, v_new=case.v_new)
+    with pytest.raises(ValueError, match="decode_step"):
+        ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, schedule="balanced",
+                         k_new=case.k_new, v_new=case.v_new)
+    with pytest.raises(ValueError, match=r"\[B, Hkv, D\]"):
+        ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, schedule="splits", num_splits=1,
+                         k_new=case.k_new[:1], v_new=case.v_new[:1])
