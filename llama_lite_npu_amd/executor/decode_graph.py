@@ -169,7 +169,7 @@ class DeviceDecodeBatch:
         (a graph runner holds one graph per schedule)."""
         plan = self.decode_plan
         counts = self.executor.req_tokens_manager.req_token_count
-        plan.choose_schedule([counts[r] for r in self.request_ids], margin=0.95 if plan.per_sequence else 1.15)
+        plan.choose_schedule([counts[r] for r in self.request_ids], margin=1.0 if plan.per_sequence else 1.2)
 
     @property
     def max_actual_seq_len(self) -> int:

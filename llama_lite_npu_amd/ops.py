@@ -235,23 +235,24 @@ def balanced_chunks(num_kv_heads: int) -> int:
 
 
 def per_sequence_decode_is_faster(batch: int, num_kv_heads: int, max_pages: int, total_pages: int,
-                                  token_bytes: int, page_size: int = PAGE_SIZE, margin: float = 1.05) -> bool:
+                                  token_bytes: int, page_size: int = PAGE_SIZE, margin: float = 1.1) -> bool:
     """Which of the two decode schedules a step should take, from what the host knows about it.
 
-    One wavefront per (sequence, kv head) (``num_splits=1`` of the splits schedule: append launch +
-    one kernel, no merge) costs a dependent chain of page steps as long as the longest sequence,
-    the bytes at the rate such unbalanced streams reach, or the placement of its wavefronts,
-    whichever is largest. The balanced schedule (fused step + merge) costs two launches whose
-    fixed part is larger, the bytes at a higher rate, and a little per sequence. Constants (us, bytes
-    per us) are fits to 230 measured shapes on an MI355X (8 to 2048 sequences, 32 to 4096 tokens, uniform
-    and ragged, 8 and 4 kv heads): choosing by this rule is within 0.5 % of always choosing the faster
-    schedule on average (worst case 15 %), always balanced is 19 % slower on average. ``margin``: how
-    much faster the per-sequence estimate must be to be chosen."""
+    One wavefront per (sequence, kv head) (``num_splits=1`` of the splits schedule with the append
+    fused in: one launch, no merge) costs a dependent chain of page steps as long as the longest
+    sequence, the bytes at the rate such unbalanced streams reach, or the placement of its
+    wavefronts, whichever is largest. The balanced schedule (fused step + merge) costs two launches
+    whose fixed part is larger, the bytes at a higher rate, and a little per sequence. Constants
+    (us, bytes per us) are fits to 248 measured shapes on an MI355X (8 to 2048 sequences, 32 to 4096
+    tokens, uniform and ragged, 64/8 and 32/4 heads, each schedule replayed from a graph): choosing
+    by this rule is within 0.4 % of always choosing the faster schedule on average (worst case 14 %),
+    always balanced is 29 % slower on average. ``margin``: how much faster the per-sequence estimate
+    must be to be chosen."""
     if batch <= 0 or total_pages <= 0:
         return False
     nbytes = float(total_pages) * page_size * token_bytes
-    per_sequence = max(6.0 + 0.57 * max_pages, 4.0 + nbytes / 4.5e6, 4.0 + 5.5e-3 * batch * num_kv_heads)
-    balanced = 12.0 + nbytes / 5.6e6 + 0.03 * batch
+    per_sequence = max(5.0 + 0.57 * max_pages, 3.0 + nbytes / 5.0e6, 3.0 + 5.5e-3 * batch * num_kv_heads)
+    balanced = 13.0 + nbytes / 5.6e6 + 0.03 * batch
     return per_sequence * margin < balanced
 
 
@@ -301,7 +302,7 @@ class DecodePlan:
             self.choose_schedule(host_seq_lens)
         self.refresh()
 
-    def choose_schedule(self, host_seq_lens: Sequence[int], margin: float = 1.05) -> bool:
+    def choose_schedule(self, host_seq_lens: Sequence[int], margin: float = 1.1) -> bool:
         """Sets ``per_sequence`` from the lengths as the host knows them (no device read). A plan
         with a shared prefix stays balanced. Returns the choice."""
         if self.shared_pages > 0:

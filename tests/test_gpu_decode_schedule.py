@@ -100,7 +100,7 @@ def test_graph_replay_follows_a_change_of_schedule():
     assert batch.decode_plan.per_sequence
     tok_h = tok_g = torch.tensor([[7], [8], [9], [10]], device=DEV)
     seen = set()
-    for step in range(120):
+    for step in range(160):
         out_h = _host_step(host, model_h, ids_h, tok_h)
         graphed.extend_paged_requests(ids_g)
         out_g = graphed.forward(tok_g)
