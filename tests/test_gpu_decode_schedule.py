@@ -164,3 +164,28 @@ def test_fused_append_argument_checks():
     with pytest.raises(ValueError, match=r"\[B, Hkv, D\]"):
         ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, schedule="splits", num_splits=1,
                          k_new=case.k_new[:1], v_new=case.v_new[:1])
+
+
+@pytest.mark.parametrize("lens", [[30, 100, 64, 7], [40, 2500, 900, 16]], ids=["short", "long"])
+def test_drop_in_flash_decoding_on_either_schedule(lens):
+    """The reference-signature wrapper picks the schedule from the batch size and the longest
+    sequence it is told; both choices give the oracle's attention."""
+    from llama_lite_npu_amd import kernels as compat
+
+    hq, hkv = 16, 8
+    print(f"flash_decoding wrapper, lens {lens}", flush=True)
+    case = workloads.make_decode_case("compat", 70, lens, hq, hkv, device=DEV)
+    pool = case.kv_pool
+    ops.kv_append(case.k_new, case.v_new, case.slot_mapping, pool)
+    # the reference's per-token table: slot of every logical position
+    token_table = (case.block_table.long()[:, :, None] * 16 + torch.arange(16, device=DEV)).reshape(len(lens), -1)
+    max_len = max(lens) + 1
+    picks_per_sequence = ops.per_sequence_decode_is_faster(len(lens), hkv, (max_len + 15) // 16,
+                                                           len(lens) * ((max_len + 15) // 16), 2 * hkv * 128 * 2)
+    assert picks_per_sequence == (max(lens) < 200)
+    out = compat.flash_decoding(case.q, pool[:, :hkv], pool[:, hkv:], case.softmax_scale,
+                                token_table.to(torch.int32), case.seq_lens.long(), max_len)
+    torch.cuda.synchronize()
+    ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool), case.block_table.cpu().numpy(),
+                                case.seq_lens.cpu().numpy(), case.softmax_scale)
+    assert_attention_close(out, ref, "flash_decoding wrapper")
