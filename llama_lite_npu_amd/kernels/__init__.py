@@ -61,7 +61,8 @@ def flash_decoding(q, k_cache, v_cache, qk_scale, b_req_tokens_table, b_seq_len,
     # sequence taken to be that long) one wavefront per sequence and kv head is the faster schedule.
     hkv, d = k_cache.shape[1], k_cache.shape[2]
     max_pages = cols // PAGE_SIZE
-    if ops.per_sequence_decode_is_faster(b, hkv, max_pages, b * max_pages, 2 * hkv * d * q.element_size()):
+    if ops.per_sequence_decode_is_faster(b, hkv, max_pages, b * max_pages, 2 * hkv * d * q.element_size(),
+                                         heads_per_kv_head=q.shape[1] // hkv):
         return ops.paged_decode(q, pool, table, b_seq_len, float(qk_scale), num_splits=1, schedule="splits")
     return ops.paged_decode(q, pool, table, b_seq_len, float(qk_scale))
 

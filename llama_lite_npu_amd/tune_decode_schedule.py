@@ -72,7 +72,8 @@ def main() -> int:
                                                               case.softmax_scale, schedule="splits", num_splits=1,
                                                               out=out, k_new=case.k_new, v_new=case.v_new))
                 pages = [(n + 1 + 15) // 16 for n in lens]
-                pick_seq = ops.per_sequence_decode_is_faster(b, hkv, max(pages), sum(pages), token_bytes)
+                pick_seq = ops.per_sequence_decode_is_faster(b, hkv, max(pages), sum(pages), token_bytes,
+                                                             heads_per_kv_head=hq // hkv)
                 picked, best = (t_seq if pick_seq else t_bal), min(t_seq, t_bal)
                 ratio_rule += picked / best
                 ratio_balanced += t_bal / best

@@ -46,3 +46,15 @@ def test_degenerate_inputs():
     for mp in range(1, 200):
         if per_sequence(32, 8, mp, 32 * mp, TOK, margin=1.2):
             assert per_sequence(32, 8, mp, 32 * mp, TOK, margin=1.0)
+
+
+def test_wide_head_groups_lean_towards_one_wavefront_per_sequence():
+    # 16 query heads per kv head slow the balanced schedule only: some steps change sides, none the other way
+    moved = 0
+    for batch in (8, 16, 64, 128):
+        for mp in range(1, 80):
+            narrow = per_sequence(batch, 8, mp, batch * mp, TOK)
+            wide = per_sequence(batch, 8, mp, batch * mp, TOK, heads_per_kv_head=16)
+            assert wide or not narrow
+            moved += wide and not narrow
+    assert moved > 0
