@@ -600,7 +600,7 @@ def main() -> int:
                     help="storage of the KV pools (fp8: E4M3 codes with per-head scales; decode configs only)")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the leg that replays the decode step as one HIP graph")
-    ap.add_argument("--out-dir", default="gpurun_out",
+    ap.add_argument("--out-dir", default="bench_out",
                     help="where --all writes bench_all.jsonl (relative to the repository root)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one page_gather of exactly 1 GiB (read) + 1 GiB (write): a plain copy of "
