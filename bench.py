@@ -217,9 +217,11 @@ class DecodeLayerSet:
 
     def capture(self):
         """The whole step (metadata, plan, every layer) recorded once as a HIP graph."""
+        from llama_lite_npu_amd.executor.decode_graph import quiet_capture
+
         torch = self.torch
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with quiet_capture(graph):
             self.step(stream=torch.cuda.current_stream().cuda_stream)
         return graph
 
@@ -348,12 +350,13 @@ def _time_us(fn, reps: int = 10, warm: int = 2) -> float:
     HIP graph and replayed between two events (an event pair around a single short launch measures
     mostly the events and the Python call, 10-15 us on this stack)."""
     import torch
+    from llama_lite_npu_amd.executor.decode_graph import quiet_capture
 
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    with quiet_capture(graph):
         for _ in range(reps):
             fn()
     graph.replay()

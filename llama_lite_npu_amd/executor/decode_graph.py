@@ -20,7 +20,9 @@ again. Two things differ:
 
 from __future__ import annotations
 
+import contextlib
 import copy
+import gc
 import logging
 from dataclasses import dataclass
 from typing import Any, Callable, Optional, Sequence
@@ -221,6 +223,23 @@ class DeviceDecodeBatch:
             raise RuntimeError(f"device sequence lengths {got} differ from the host's {want}")
 
 
+@contextlib.contextmanager
+def quiet_capture(graph, **kwargs):
+    """``torch.cuda.graph`` with Python's cyclic collector held off. A collection that starts
+    while the stream is capturing can destroy an older graph or return pool memory to the
+    driver; HIP refuses both during a capture and the process aborts. Dead cycles are collected
+    before the capture begins instead (PyTorch no longer does that on its own)."""
+    gc.collect()
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph, **kwargs):
+            yield
+    finally:
+        if was_enabled:
+            gc.enable()
+
+
 class _TorchHipGraphs:
     """The graph calls the runner needs, as PyTorch-ROCm exposes hipGraph."""
 
@@ -232,7 +251,7 @@ class _TorchHipGraphs:
         return torch.cuda.CUDAGraph()
 
     def graph(self, graph, pool=None):
-        return torch.cuda.graph(graph, pool=pool)
+        return quiet_capture(graph, pool=pool)
 
     def synchronize(self) -> None:
         torch.cuda.synchronize()

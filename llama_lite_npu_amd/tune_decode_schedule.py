@@ -17,6 +17,7 @@ import argparse
 import torch
 
 from . import ops, workloads
+from .executor.decode_graph import quiet_capture
 
 DEV = "cuda:0"
 
@@ -29,7 +30,7 @@ def _replayed_us(fn, inner: int = 16, reps: int = 5) -> float:
     with torch.cuda.stream(side):
         fn()
         torch.cuda.synchronize()
-        with torch.cuda.graph(graph, stream=side):
+        with quiet_capture(graph, stream=side):
             for _ in range(inner):
                 fn()
     torch.cuda.synchronize()
