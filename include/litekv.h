@@ -185,6 +185,37 @@ int litekv_paged_decode_merge(const int32_t *seq_lens, void *out,
                               void *stream);
 
 /*
+ * litekv_paged_decode for callers that cannot allocate device memory. It has
+ * no counterpart in the reference (whose flash_decoding allocates mid_o /
+ * mid_o_logexpsum with torch.empty on every call, flashdecoding.py:310-321);
+ * it is for code under HIP graph capture, serving loops that must not reach an
+ * allocator and harnesses that forbid hipMalloc. Same arguments, result and
+ * two launches as litekv_paged_decode, minus the workspace: the fp32 partial
+ * rows and log-sum-exps live in a device array built into the library,
+ * LITEKV_STATIC_SCRATCH_BYTES long, which every GPU the library runs on holds
+ * until the process ends. The call itself allocates and frees nothing.
+ *   limit   litekv_paged_decode_workspace_bytes(batch, num_q_heads, head_dim,
+ *           max_splits) must not exceed LITEKV_STATIC_SCRATCH_BYTES, else
+ *           LITEKV_ERR_INVALID_ARGUMENT (32 MiB: e.g. batch 32 x 64 query
+ *           heads x 31 splits, or batch 128 x 32 heads x 15 splits)
+ *   sharing every call on a GPU uses that GPU's one array: calls that overlap
+ *           in time on one GPU (two streams, two threads) race; calls on one
+ *           stream are ordered. Nothing in it has to start at zero: the merge
+ *           reads only the cells the split launch of the same call wrote.
+ *   set-up  the array's address on a device is looked up on the first call
+ *           made with that device current (no allocation, but make that first
+ *           call outside a graph capture).
+ */
+#define LITEKV_STATIC_SCRATCH_BYTES (32u << 20)
+
+int litekv_paged_decode_static(const void *q, int64_t q_batch_stride, const void *kv_pool,
+                               const int32_t *block_table, int32_t block_table_stride,
+                               const int32_t *seq_lens, void *out, int32_t batch,
+                               int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                               int32_t page_size, int64_t num_pages, int32_t max_splits,
+                               int32_t min_pages_per_split, float softmax_scale, void *stream);
+
+/*
  * Paged flash-decoding, balanced schedule. Same
  * result contract as litekv_paged_decode (it replaces the same reference
  * function, lite_llama/kernels/flashdecoding.py:294-342), other work

@@ -49,6 +49,12 @@ SIGNATURES = {
          c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32, c_float,
          c_void_p],
     ),
+    "litekv_paged_decode_static": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p,
+         c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32, c_float,
+         c_void_p],
+    ),
     "litekv_paged_decode_fp8": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_size_t,

@@ -30,6 +30,8 @@
 // In both schedules the cuts are a pure function of seq_lens and of host
 // scalars, and the merge adds the fp32 partials in index order: results do not
 // depend on timing.
+#include <atomic>
+
 #include "common.h"
 #include "kv_fp8.h"
 
@@ -1821,6 +1823,79 @@ extern "C" int litekv_paged_decode_append_fp8(
                        page_size, num_pages, softmax_scale, stream, k_new, v_new, k_new_stride,
                        v_new_stride};
   int rc = litekv::launch_split(a, max_splits, min_pages_per_split, batch > 0 ? scales : nullptr);
+  if (rc != LITEKV_OK) return rc;
+  return litekv::launch_merge(a, max_splits, min_pages_per_split);
+}
+
+// ---------------------------------------------------------------------------------------------
+// litekv_paged_decode_static: litekv_paged_decode for callers that cannot allocate. The partial
+// rows and log-sum-exps of the split kernel live in a file-scope device array instead of a
+// caller's workspace. Every device the library runs on holds its own copy of the array until
+// the process ends; its address on a device is looked up once, with that device current.
+// ---------------------------------------------------------------------------------------------
+namespace litekv {
+
+static __device__ __align__(256) unsigned char scratch[LITEKV_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxStaticDevices = 64;
+// Device address of `scratch` per device ordinal (null until looked up). Written once per
+// device; a race between two first calls stores the same address twice.
+static std::atomic<void *> g_scratch_ptr[kMaxStaticDevices];
+
+static int static_scratch(const char *what, void **ptr_out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) {
+    return fail(LITEKV_ERR_LAUNCH, "%s: hipGetDevice failed: %s", what, hipGetErrorString(err));
+  }
+  LITEKV_REQUIRE(dev >= 0 && dev < kMaxStaticDevices, "%s: device ordinal %d out of [0, %d)", what,
+                 dev, kMaxStaticDevices);
+  void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || ptr == nullptr) {
+      return fail(LITEKV_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) failed on device %d: %s", what,
+                  dev, hipGetErrorString(err));
+    }
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *ptr_out = ptr;
+  return LITEKV_OK;
+}
+
+}  // namespace litekv
+
+extern "C" int litekv_paged_decode_static(const void *q, int64_t q_batch_stride, const void *kv_pool,
+                                          const int32_t *block_table, int32_t block_table_stride,
+                                          const int32_t *seq_lens, void *out, int32_t batch,
+                                          int32_t num_q_heads, int32_t num_kv_heads,
+                                          int32_t head_dim, int32_t page_size, int64_t num_pages,
+                                          int32_t max_splits, int32_t min_pages_per_split,
+                                          float softmax_scale, void *stream) {
+  const char *what = "paged_decode_static";
+  LITEKV_REQUIRE(batch >= 0 && num_q_heads > 0 && head_dim > 0 && max_splits >= 1 &&
+                     max_splits <= 65535,
+                 "%s: batch %d, num_q_heads %d, head_dim %d or max_splits %d out of range", what,
+                 batch, num_q_heads, head_dim, max_splits);
+  // the product is formed in 64 bits from values below 2^16 (batch, heads, splits are checked
+  // again by the shared validation) or small (head_dim)
+  LITEKV_REQUIRE(batch <= 65535 && num_q_heads <= 65535 && head_dim <= 1024,
+                 "%s: batch %d, num_q_heads %d or head_dim %d out of range", what, batch,
+                 num_q_heads, head_dim);
+  const size_t need = litekv::splits_workspace_bytes(batch, num_q_heads, head_dim, max_splits);
+  LITEKV_REQUIRE(need <= (size_t)LITEKV_STATIC_SCRATCH_BYTES,
+                 "%s: batch %d x %d query heads x %d splits needs %zu bytes of partial results, the "
+                 "built-in scratch holds %zu; use litekv_paged_decode with a workspace",
+                 what, batch, num_q_heads, max_splits, need, (size_t)LITEKV_STATIC_SCRATCH_BYTES);
+  void *ws = nullptr;
+  if (need > 0) {
+    int rc = litekv::static_scratch(what, &ws);
+    if (rc != LITEKV_OK) return rc;
+  }
+  litekv::DecodeArgs a{q, q_batch_stride, kv_pool, block_table, block_table_stride, seq_lens, out,
+                       ws, need, batch, num_q_heads, num_kv_heads, head_dim,
+                       page_size, num_pages, softmax_scale, stream};
+  int rc = litekv::launch_split(a, max_splits, min_pages_per_split);
   if (rc != LITEKV_OK) return rc;
   return litekv::launch_merge(a, max_splits, min_pages_per_split);
 }

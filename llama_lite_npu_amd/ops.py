@@ -547,6 +547,35 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
     return out
 
 
+def paged_decode_static(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tensor,
+                        seq_lens: torch.Tensor, out: torch.Tensor, max_splits: int,
+                        min_pages_per_split: int, softmax_scale: Optional[float] = None,
+                        page_size: int = PAGE_SIZE) -> torch.Tensor:
+    """``paged_decode`` on the splits schedule without any allocation: ``out`` comes from the
+    caller, index tensors must already be int32 on the device, and the partial results live in
+    the scratch array built into the library (at most STATIC_SCRATCH_BYTES of them, else
+    LiteKVError). Calls that overlap in time on one GPU share that array and race."""
+    _dev_half("q", q), _dev_half("kv_pool", kv_pool), _dev_half("out", out)
+    _need(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2], "q must be [B, Hq, D] with contiguous heads")
+    b, hq, d = q.shape
+    _, hkv, dk, n_pages, _ = pool_geometry(kv_pool, page_size)
+    _need(d == dk, "q and kv_pool differ in head_dim")
+    _need(out.shape == (b, hq, d) and out.is_contiguous(), "out must be contiguous [B, Hq, D]")
+    for name, t in (("block_table", block_table), ("seq_lens", seq_lens)):
+        _need(t.is_cuda and t.dtype == torch.int32, f"{name} must be an int32 device tensor")
+    _need(block_table.dim() == 2 and block_table.shape[0] == b and block_table.stride(1) == 1,
+          "block_table must be [B, max_blocks]")
+    _need(seq_lens.numel() == b and seq_lens.is_contiguous(), "seq_lens must be contiguous [B]")
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    q_stride = q.stride(0) if b > 1 else max(q.stride(0), hq * d)
+    _lib.check(_lib.load().litekv_paged_decode_static(
+        _ptr(q), q_stride, _ptr(kv_pool), _ptr(block_table), block_table.stride(0), _ptr(seq_lens),
+        _ptr(out), b, hq, hkv, d, page_size, n_pages, int(max_splits), int(min_pages_per_split),
+        float(softmax_scale), _stream()))
+    return out
+
+
 def paged_prefill(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tensor,
                   cu_q_lens: torch.Tensor, context_lens: Optional[torch.Tensor], max_q_len: int,
                   softmax_scale: Optional[float] = None, out: Optional[torch.Tensor] = None,

@@ -54,6 +54,10 @@ def test_loader_checks_abi_version_and_reports_errors_without_a_gpu():
     assert lib.litekv_decode_plan_bytes(32, 257, 8, 256) > 0
     rc = lib.litekv_page_copy(None, None, None, 0, 65536, 10, None)
     assert rc == 0   # empty move list is a no-op
+    # the entry point with built-in scratch refuses steps beyond its 32 MiB before touching a device
+    rc = lib.litekv_paged_decode_static(None, 0, None, None, 1, None, None, 128, 32, 4, 128, 16, 1000, 16, 1,
+                                        0.1, None)
+    assert rc == 1 and b"built-in scratch holds 33554432" in lib.litekv_last_error()
 
 
 def test_product_package_never_imports_the_oracle():
