@@ -456,13 +456,18 @@ int litekv_paged_decode_prefix_fp8(const void *q, int64_t q_batch_stride, void *
  *                  for the lengths as they are, 1 is a decode step)
  *   seq_lens_i64   [B] int64 or NULL: copy of seq_lens (b_seq_len)
  *   slot_mapping   [B] int32 out: slot of logical token seq_lens[b] - 1
- *                  (cur_select_index); -1 when the row is empty or invalid
- *   position_ids   [B] int64 or NULL: seq_lens[b] - 1
+ *                  (cur_select_index); -1 when the row is empty or refused
+ *   position_ids   [B] int64 or NULL: seq_lens[b] - 1 (0 for an empty or
+ *                  refused row)
  *   block_table    [B][block_table_stride] int32 out: first `width` entries
  *                  of each row's page list, in batch order
  *   overflow       int32[1] or NULL: set to 1 (never cleared here) when a row
- *                  could not advance (bad request id, capacity reached); that
- *                  row keeps its length
+ *                  was refused (bad request id, negative length, capacity
+ *                  reached). A refused row gets length -1 and slot -1 and
+ *                  stays refused on later steps: the decode and append
+ *                  kernels treat it as empty (zero output, nothing stored),
+ *                  so no cached token is overwritten; the caller reads the
+ *                  flag at its next synchronisation and rebuilds the batch
  */
 int litekv_decode_advance(const int32_t *request_tables, int64_t request_table_stride,
                           int32_t max_requests, const int32_t *request_ids,

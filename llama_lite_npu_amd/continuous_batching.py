@@ -556,7 +556,15 @@ class ContinuousBatchModelBackend:
         for req_idx in ids:
             self._positions[req_idx] += 1
         ex.extend_paged_requests(ids)
-        return [int(t) for t in sampled.detach().cpu().tolist()] if self.return_host_tokens else []
+        if not self.return_host_tokens:
+            return []
+        tokens = [int(t) for t in sampled.detach().cpu().tolist()]
+        # the readback above has waited for the step: the device batch's refusal flag is current
+        batch = getattr(ex, "_device_batch", None) if self.device_decode else None
+        if batch is not None and int(batch.overflow.item()) != 0:
+            raise RuntimeError("Paged KV allocation failed during decode: a step on the device ran past a "
+                               "request's reserved pages")
+        return tokens
 
     # ---- release -------------------------------------------------------------------------------
     def release(self, requests: Sequence[BatchRequest]) -> None:

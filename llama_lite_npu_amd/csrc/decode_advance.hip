@@ -38,9 +38,13 @@ __global__ __launch_bounds__(256) void decode_advance_kernel(
   cap = cap < room ? cap : room;
   const int64_t want = (int64_t)len + increment;
   const bool ok = r_ok && len >= 0 && want <= cap;
-  const int32_t next = ok ? (int32_t)want : (len >= 0 && len <= cap ? len : 0);
+  // A refused row becomes empty for good: length -1 (every kernel of the path treats a length
+  // <= 0 as "no tokens": zero output, nothing appended), slot -1 (the append kernels skip it),
+  // and it stays refused on later steps. Keeping its old length would let the step's append,
+  // which writes at logical position length - 1, overwrite the last cached token.
+  const int32_t next = ok ? (int32_t)want : -1;
   int32_t slot = -1;  // the append kernels skip a negative slot
-  if (r_ok && next >= 1) {
+  if (ok && next >= 1) {
     const int32_t page = row[(next - 1) / page_size];
     if (page >= 0 && page < num_pages) slot = page * page_size + (next - 1) % page_size;
   }

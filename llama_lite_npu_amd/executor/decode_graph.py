@@ -324,10 +324,16 @@ class DecodeGraphRunner:
         per_sequence = bool(plan is not None and plan.per_sequence)
         if device is not None:
             return key + (id(device), per_sequence)   # the graph is tied to that batch's tensors
+        # Host-metadata steps replay through a static plan built at capture: the graph holds that
+        # plan's launches, so a batch that shares another number of leading pages (a cached
+        # prefix attended once for the batch) needs a graph of its own. A graph captured with a
+        # shared prefix would otherwise make every later batch of that size attend row 0's pages.
+        shared = int(getattr(plan, "shared_pages", 0) or 0) if plan is not None else 0
+        extra = (("shared", shared),) if shared > 0 else ()
         table = getattr(atten_info, "block_table", None)
         if self.PARTITION_SIZE is None and self.max_blocks is None and table is not None:
-            return key + (int(table.shape[1]), per_sequence)   # a trimmed table: its width sizes the plan
-        return key + (per_sequence,) if per_sequence else key
+            return key + (int(table.shape[1]), per_sequence) + extra   # a trimmed table: its width sizes the plan
+        return key + ((per_sequence,) if per_sequence else ()) + extra
 
     # ---- capture ---------------------------------------------------------------------------
     def _static_info(self, atten_info):

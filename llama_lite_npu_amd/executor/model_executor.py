@@ -59,6 +59,7 @@ class ModelExecutor:
         self._decode_plan = None
         self._paged_request_ids: tuple[int, ...] = ()
         self._device_batch = None            # DeviceDecodeBatch in charge of the running decode batch
+        self._decode_meta_sig = None         # what the decode metadata in atten_info was last built from
         self._device_batches: dict = {}      # (batch size, shared pages) -> DeviceDecodeBatch
         self.model = None
         self.graph_runner = None
@@ -180,6 +181,7 @@ class ModelExecutor:
         info.decode_plan = None
         info.device_decode = None
         self._device_batch = None
+        self._decode_meta_sig = None
 
     def _i32(self, values) -> torch.Tensor:
         return torch.as_tensor(np.asarray(values, dtype=np.int32), device=self.device)
@@ -285,9 +287,15 @@ class ModelExecutor:
     def activate_paged_decode_batch(self, request_ids: tuple[int, ...]) -> None:
         """Metadata of one decode step: each sequence's length already counts the token whose K/V
         this step appends, and ``cur_select_index`` is that token's slot."""
-        self._reset_paged_chunk_prefill_metadata()
         mgr = self.req_tokens_manager
         ids = tuple(int(r) for r in request_ids)
+        # The backend activates the batch before a step and extend_paged_requests does after it:
+        # the second of two calls with nothing changed in between (same requests, lengths and page
+        # lists, no other batch activated) finds the metadata and the step plan already in place.
+        sig = (ids, mgr.table_epoch, tuple(mgr.req_token_count.get(r) for r in ids))
+        if sig == self._decode_meta_sig:
+            return
+        self._reset_paged_chunk_prefill_metadata()
         req_ids, seq_lens, last = mgr.batch_metadata(list(ids))
         info = self.atten_info
         self._paged_request_ids = ids
@@ -307,6 +315,7 @@ class ModelExecutor:
                                               shared_pages=self.shared_prefix_pages(ids),
                                               host_seq_lens=[mgr.req_token_count[r] for r in ids],
                                               token_bytes=self.kv_token_bytes)
+        self._decode_meta_sig = sig
 
     def common_leading_pages(self, request_ids: Sequence[int], upcoming_tokens: int = 0) -> int:
         """How many leading pages are the same physical pages, and full, in every request of the

@@ -174,6 +174,7 @@ class PagedReqTokensManager:
         self.req_token_count: dict[int, int] = {}
         self.req_active = torch.zeros(self.max_requests, dtype=torch.bool, device="cpu")
         self.free_req_indices = list(range(self.max_requests))
+        self.table_epoch = 0    # grows whenever a request's page list changes or a request is freed
 
     # ---- device tables ---------------------------------------------------------------------
     def _publish_pages(self, req_idx: int, first: int = 0) -> None:
@@ -181,6 +182,7 @@ class PagedReqTokensManager:
         pages = self.req_page_table[req_idx].numpy().astype(np.int32)
         if first >= pages.size:
             return
+        self.table_epoch += 1
         self._table_host[req_idx, first:pages.size] = pages[first:]
         self.block_table[req_idx, first:pages.size] = torch.from_numpy(pages[first:]).to(self.device)
 
@@ -290,6 +292,7 @@ class PagedReqTokensManager:
 
     def free_req(self, req_idx: int) -> None:
         if req_idx in self.req_page_table:
+            self.table_epoch += 1
             self.page_mgr.free(self.req_page_table.pop(req_idx))
             del self.req_token_count[req_idx]
             del self.req_page_count[req_idx]
@@ -331,19 +334,26 @@ class PagedReqTokensManager:
 
     # ---- page moves ------------------------------------------------------------------------
     def copy_on_write(self, req_indices: Iterable[int]) -> list[tuple[int, int]]:
-        """Gives every listed request a private copy of its last page if that page is shared
-        (refcount > 1): a fresh page is allocated, the bytes are copied in every layer, the table
+        """Gives every listed request a private copy of the partly filled page its next token goes
+        into if that page is shared (refcount > 1, counting the holders this call has not already
+        moved away): a fresh page is allocated, the bytes are copied in every layer, the table
         entry is swapped and the old reference dropped. Returns the (src, dst) moves made.
         Needed before appending into a page another holder can still read; the reference shares
         such pages without copying (model_executor.py:672-678)."""
         moves: list[tuple[int, int]] = []
         touched: list[tuple[int, int]] = []
+        dropping: dict[int, int] = {}      # references this call has already decided to drop, per page
+        ps = self.page_mgr.page_size
         for req_idx in req_indices:
             pages = self.req_page_table[req_idx]
-            last = len(pages) - 1
+            count = self.req_token_count[req_idx]
+            if count % ps == 0:
+                continue                   # the next token opens a page of its own: nothing to protect
+            last = (count - 1) // ps       # the page the next token goes into (reserved pages may follow it)
             old = int(pages[last])
-            if self.page_mgr.refcount(old) <= 1:
-                continue
+            if self.page_mgr.refcount(old) - dropping.get(old, 0) <= 1:
+                continue                   # the last holder left keeps the page
+            dropping[old] = dropping.get(old, 0) + 1
             fresh = self.page_mgr.alloc(1)
             if fresh is None:
                 raise RuntimeError("Paged KV allocation failed during copy-on-write")

@@ -356,7 +356,8 @@ def decode_advance(request_tables: torch.Tensor, request_ids: torch.Tensor, seq_
     slot of logical token seq_lens[b] - 1 in request request_ids[b]'s page list (a row of
     request_tables [max_requests, max_pages]), position_ids[b] = seq_lens[b] - 1, and block_table
     [B, width] = the batch's page lists. Rows that cannot advance (capacity reached, bad request id)
-    keep their length and raise the overflow flag."""
+    raise the overflow flag and end empty for good (length -1, slot -1): every kernel of the path
+    treats them as holding no tokens, so the step's append never lands on a cached token."""
     _need(request_tables.dim() == 2 and request_tables.stride(1) == 1, "request_tables must be [max_requests, max_pages]")
     _fixed("request_tables", request_tables, torch.int32)
     b = request_ids.numel()

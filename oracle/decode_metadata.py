@@ -15,7 +15,9 @@ Pinned in tests/test_oracle.py by: the worked example in the reference's docstri
 10 tokens, pages [3, 7, 12] -> slots [12, 13, 14, 15, 28, 29, 30, 31, 48, 49], paged_attention.py:125-129);
 brute force over every token of random page lists against an explicit per-token table; the
 invariant that N single steps from length L give the slots token_slots lists at L .. L+N-1; and
-the refusal cases (capacity reached, request id out of range) leaving the length untouched.
+the refusal cases (capacity reached, request id out of range): such a row ends empty (length -1,
+slot -1) and stays refused, so nothing is appended over a cached token (the reference raises on
+the host at this point, paged_attention.py:333-337, before anything is written).
 """
 
 from __future__ import annotations
@@ -57,10 +59,12 @@ def decode_advance(request_tables: np.ndarray, request_ids: np.ndarray, seq_lens
         if ok:
             nxt = length + increment
         else:
+            # a refused row becomes empty for good (length -1, no slot): the step's append writes at
+            # position length - 1, so a row that kept its length would lose its last cached token
             overflow = 1
-            nxt = length if 0 <= length <= cap else 0
+            nxt = -1
         new_lens[i] = nxt
-        if known and nxt >= 1:
+        if ok and nxt >= 1:
             page = int(request_tables[r, (nxt - 1) // page_size])
             if 0 <= page < num_pages:
                 slots[i] = page * page_size + (nxt - 1) % page_size

@@ -163,6 +163,47 @@ def test_decode_advance_refusals_match_the_oracle():
         ops.decode_advance(t, torch.from_numpy(ids).to(DEV), seq.long(), slot, rows, num_pages)
 
 
+def test_refused_row_appends_nothing_and_attends_nothing():
+    """A row whose reserved pages are used up is refused by the device advance; the step's append
+    (fused into either decode schedule, or through the slot mapping) must leave its cached tokens
+    alone, its output is zero, and the other rows are attended as if it were not there."""
+    print("decode step with a refused row", flush=True)
+    from llama_lite_npu_amd import workloads
+
+    case = workloads.make_decode_case("refused", 31, [30, 15, 47], HQ, HKV, device=DEV)
+    capacity = torch.tensor([32, 15, 48], dtype=torch.int32, device=DEV)     # row 1: 15 cached, no room
+    ids = torch.arange(3, dtype=torch.int32, device=DEV)
+    for per_sequence in (False, True):
+        pool = case.kv_pool.clone()
+        seq = case.context_lens.to(DEV).to(torch.int32).clone()
+        slot = torch.zeros(3, dtype=torch.int32, device=DEV)
+        rows = torch.zeros_like(case.block_table)
+        flag = torch.zeros(1, dtype=torch.int32, device=DEV)
+        ops.decode_advance(case.block_table, ids, seq, slot, rows, case.num_pages, capacity=capacity, overflow=flag)
+        torch.cuda.synchronize()
+        assert seq.tolist() == [31, -1, 48] and int(flag.item()) == 1 and int(slot[1]) == -1
+        plan = ops.DecodePlan(rows, seq, HQ, HKV, case.num_pages, chunks=5)
+        plan.per_sequence = per_sequence
+        out = ops.decode_step(case.q, pool, plan, case.k_new, case.v_new, SCALE)
+        torch.cuda.synchronize()
+        want_pool = case.kv_pool.clone()                 # index assignment of the two live rows only
+        for b in (0, 2):
+            want_pool[int(slot[b]), :HKV], want_pool[int(slot[b]), HKV:] = case.k_new[b], case.v_new[b]
+        assert torch.equal(pool, want_pool), "the refused row's pages (or any other slot) were written"
+        separate = case.kv_pool.clone()
+        ops.kv_append(case.k_new, case.v_new, slot, separate)
+        assert torch.equal(separate, want_pool)
+        assert float(out[1].abs().max()) == 0.0
+        live = torch.tensor([31, 0, 48], dtype=torch.int32)
+        ref = c_oracle.paged_decode(to_np16(case.q), to_np16(want_pool), case.block_table.cpu().numpy(),
+                                    live.numpy(), SCALE)
+        assert_attention_close(out, ref, f"refused row, per_sequence={per_sequence}")
+        # the next step refuses the row again instead of restarting it at token 0
+        ops.decode_advance(case.block_table, ids, seq, slot, rows, case.num_pages, capacity=capacity, overflow=flag)
+        torch.cuda.synchronize()
+        assert seq.tolist() == [32, -1, -1] and slot.tolist()[1:] == [-1, -1]
+
+
 def test_replayed_steps_equal_eager_steps_bit_for_bit():
     print("graph replay (device metadata) vs eager host metadata", flush=True)
     host, dev = _executor(), _executor()
@@ -238,36 +279,68 @@ def test_host_metadata_steps_replay_through_static_copies():
     assert _pools_equal(host, graphed)
 
 
+def _shared_prefix_batch(ex, model):
+    """Three requests whose first 6 pages are one cached system prompt; returns their ids."""
+    attn = model.attn
+    system = tuple(range(2000, 2096))           # 6 full pages
+    g = torch.Generator(device=DEV).manual_seed(77)
+
+    def rows(n, heads):
+        return torch.randn((n, heads, D), generator=g, device=DEV, dtype=torch.float16)
+
+    (a,) = ex.reserve_paged_requests([96])
+    ex.activate_paged_packed_prefill_batch((a,), [96])
+    for layer in range(LAYERS):
+        attn.context_forward(rows(96, HQ), rows(96, HKV), rows(96, HKV), ex.atten_info, layer, SCALE * LOG2E)
+    ex.store_paged_request_prefix(system, a, first_token_id=5)
+    batch_ids = [a]
+    for i, extra in enumerate((20, 3)):
+        prompt = system + tuple(range(3000 + 100 * i, 3000 + 100 * i + extra))
+        req, matched, _ = ex.share_paged_prefix_from_cache(prompt)
+        assert matched == 96
+        ex.ensure_paged_request_capacity(req, 96 + extra + 8)
+        ex.activate_paged_chunk_prefill_batch((req,), [96], [extra])
+        for layer in range(LAYERS):
+            attn.context_forward(rows(extra, HQ), rows(extra, HKV), rows(extra, HKV), ex.atten_info, layer,
+                                 SCALE * LOG2E)
+        batch_ids.append(req)
+    return tuple(batch_ids)
+
+
+def test_graph_of_a_shared_prefix_batch_is_not_replayed_for_a_batch_sharing_nothing():
+    """Host-metadata steps replay through a static plan made at capture. A batch that shares a
+    cached prefix and a batch of the same size that shares nothing need different plans: each
+    must get its own graph, every replay equal to the eager step bit for bit."""
+    print("graph replay: shared-prefix batch, then a same-size batch without one", flush=True)
+    host, graphed = _executor(num_pages=200, max_requests=8), _executor(num_pages=200, max_requests=8)
+    model_h, model_g = TinyModel(), TinyModel()
+    shared_h, shared_g = _shared_prefix_batch(host, model_h), _shared_prefix_batch(graphed, model_g)
+    private_h, private_g = _prefill(host, [40, 7, 70], 9), _prefill(graphed, [40, 7, 70], 9)
+    assert shared_h == shared_g and private_h == private_g
+    graphed.attach_model(model_g, "qwen3")
+    tok_h = tok_g = torch.tensor([[1], [2], [3]], device=DEV)
+    for phase, (ids_h, ids_g, shared) in enumerate(((shared_h, shared_g, 6), (private_h, private_g, 0),
+                                                    (shared_h, shared_g, 6), (private_h, private_g, 0))):
+        for step in range(3):
+            out_h = _host_step(host, model_h, ids_h, tok_h)
+            assert host.atten_info.decode_plan.shared_pages == shared
+            graphed.extend_paged_requests(ids_g)
+            out_g = graphed.forward(tok_g, graphed.atten_info.b_seq_len - 1)
+            torch.cuda.synchronize()
+            assert torch.equal(out_h, out_g), f"phase {phase} step {step}"
+            tok_h, tok_g = _next_tokens(out_h), _next_tokens(out_g)
+    runner = graphed.graph_runner
+    assert runner.capture_count == 2 and runner.replay_count == 12 and runner.fallback_count == 0
+    assert _pools_equal(host, graphed)
+
+
 def test_shared_prefix_batch_steps_on_the_device():
     print("graph replay over a shared cached prefix", flush=True)
     outs = []
     for use_device in (False, True):
         ex = _executor(num_pages=160)
         model = TinyModel()
-        attn = model.attn
-        system = tuple(range(2000, 2096))           # 6 full pages
-        g = torch.Generator(device=DEV).manual_seed(77)
-
-        def rows(n, heads):
-            return torch.randn((n, heads, D), generator=g, device=DEV, dtype=torch.float16)
-
-        (a,) = ex.reserve_paged_requests([96])
-        ex.activate_paged_packed_prefill_batch((a,), [96])
-        for layer in range(LAYERS):
-            attn.context_forward(rows(96, HQ), rows(96, HKV), rows(96, HKV), ex.atten_info, layer, SCALE * LOG2E)
-        ex.store_paged_request_prefix(system, a, first_token_id=5)
-        batch_ids = [a]
-        for i, extra in enumerate((20, 3)):
-            prompt = system + tuple(range(3000 + 100 * i, 3000 + 100 * i + extra))
-            req, matched, _ = ex.share_paged_prefix_from_cache(prompt)
-            assert matched == 96
-            ex.ensure_paged_request_capacity(req, 96 + extra + 8)
-            ex.activate_paged_chunk_prefill_batch((req,), [96], [extra])
-            for layer in range(LAYERS):
-                attn.context_forward(rows(extra, HQ), rows(extra, HKV), rows(extra, HKV), ex.atten_info, layer,
-                                     SCALE * LOG2E)
-            batch_ids.append(req)
-        ids = tuple(batch_ids)
+        ids = _shared_prefix_batch(ex, model)
         tok = torch.tensor([[1], [2], [3]], device=DEV)
         steps = []
         if use_device:

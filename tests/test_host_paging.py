@@ -235,6 +235,36 @@ def test_compaction_plan_moves_high_pages_into_holes(monkeypatch):
     assert ex.req_tokens_manager.block_table[ids[3], :3].tolist() == [3, 0, 2]
 
 
+def test_copy_on_write_leaves_the_page_to_its_last_holder(monkeypatch):
+    """Two requests share a partly filled page that nobody else holds: one of them moves to a
+    private copy, the other keeps the page (one allocation, one copy). A full last page and
+    reserved pages behind the logical end are left alone."""
+    page_mgr, req_mgr = _managers(num_pages=6, max_requests=4, max_seq_len=16)
+    copies = []
+    monkeypatch.setattr(page_mgr, "copy_pages", lambda s, d: copies.append((list(s), list(d))))
+    assert req_mgr.alloc_req(0, 6)                                   # pages 0, 1; page 1 holds 2 of 4 tokens
+    pages = req_mgr.req_page_table[0]
+    assert req_mgr.share_req_from_pages(1, pages, 6)
+    moves = req_mgr.copy_on_write((0, 1))
+    assert moves == [(1, 2)] and copies == [([1], [2])]
+    assert req_mgr.request_pages(0) == (0, 2) and req_mgr.request_pages(1) == (0, 1)
+    assert int(page_mgr.page_refcount[1]) == 1 and int(page_mgr.page_refcount[2]) == 1
+    assert int(page_mgr.page_refcount[0]) == 2
+    assert req_mgr.copy_on_write((0, 1)) == []                       # now private: nothing left to do
+    # a full last page: the next token opens a new page, the shared one is never written
+    assert req_mgr.alloc_req(2, 4)                                   # page 3, full
+    assert req_mgr.share_req_from_pages(3, req_mgr.req_page_table[2], 4)
+    assert req_mgr.copy_on_write((2, 3)) == [] and len(copies) == 1
+    # reserved pages behind the logical end are not the page the next token goes into
+    req_mgr.free_req(3)
+    req_mgr.free_req(2)
+    assert req_mgr.alloc_req(2, 2, 8)                                # 2 tokens, two pages reserved
+    first = req_mgr.req_page_table[2][:1]
+    assert req_mgr.share_req_from_pages(3, first, 2)
+    (move,) = req_mgr.copy_on_write((3,))
+    assert move[0] == int(first[0])
+
+
 def test_shared_prefix_pages_counts_full_common_pages():
     """Requests that map the same cached pages (block prefix cache) share them in a decode step;
     the page receiving a request's next token never counts."""

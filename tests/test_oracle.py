@@ -366,7 +366,7 @@ def test_decode_advance_walks_the_per_token_table():
     assert slots0.tolist() == [per_token[r, n - 1] for r, n in zip(ids, lens)]
 
 
-def test_decode_advance_refusals_leave_the_length():
+def test_decode_advance_refused_rows_end_empty_and_stay_refused():
     from oracle import decode_metadata
 
     ps, width, num_pages = 4, 3, 16
@@ -376,10 +376,18 @@ def test_decode_advance_refusals_leave_the_length():
     cap = np.array([12, 8, 12, 12], dtype=np.int32)         # row 1 has reached its reserved pages
     new_lens, slots, pos, rows, overflow = decode_metadata.decode_advance(tables, ids, lens, cap, width, ps, num_pages)
     assert overflow == 1
-    assert new_lens.tolist() == [12, 8, 3, 1]
-    assert slots.tolist() == [3 * 4 + 3, 5 * 4 + 3, -1, 4 * 4 + 0]
-    assert pos.tolist() == [11, 7, 2, 0]
+    assert new_lens.tolist() == [-1, -1, -1, 1]             # refused rows: no tokens, no slot
+    assert slots.tolist() == [-1, -1, -1, 4 * 4 + 0]
+    assert pos.tolist() == [0, 0, 0, 0]
     assert rows[2].tolist() == [0, 0, 0]
+    # a refused row stays refused (a fresh start at length 0 would write over its first page)
+    again, slots2, _, _, overflow2 = decode_metadata.decode_advance(tables, ids, new_lens, cap, width, ps, num_pages)
+    assert overflow2 == 1 and again.tolist() == [-1, -1, -1, 2] and slots2.tolist() == [-1, -1, -1, 4 * 4 + 1]
+    # recomputing for the lengths as they are (increment 0) refuses nothing that fits
+    same, slots0, pos0, _, overflow0 = decode_metadata.decode_advance(tables, ids[:2], lens[:2], cap[:2], width, ps,
+                                                                      num_pages, increment=0)
+    assert overflow0 == 0 and same.tolist() == [12, 8] and slots0.tolist() == [3 * 4 + 3, 5 * 4 + 3]
+    assert pos0.tolist() == [11, 7]
 
 
 # ---- fp8 (E4M3FN) storage ----------------------------------------------------------------------
