@@ -63,17 +63,21 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 __device__ __forceinline__ float xor_lane(float v, int mask) { return __shfl_xor(v, mask, kWave); }
 
 // Maximum over the four lanes l, l^16, l^32, l^48 (the lane groups that share a column of an
-// MFMA accumulator). The swaps exchange 16- and 32-lane halves between their two operands, so
-// max(first, second) of the swapped pair is the pairwise maximum: two vector ALU instructions
-// per step instead of a round trip through the LDS crossbar.
+// MFMA accumulator). v_permlane16_swap exchanges the odd 16-lane rows of its first operand with
+// the even rows of its second, v_permlane32_swap the upper half of the first with the lower half
+// of the second; fed the same value twice, the two results hold each lane's own value and its
+// partner's, so their maximum is the pairwise maximum: two vector ALU instructions per step
+// instead of a round trip through the LDS crossbar. Written as asm: the compiler's builtin for
+// these instructions hands back the first result in both elements of its return value, which
+// turns the maximum into a broadcast of lane group 0. The s_nop covers the wait states between a
+// vector ALU write and a permlane read of the same register, which nobody inserts around asm.
 __device__ __forceinline__ float max_over_lane_groups(float x) {
-  typedef unsigned uint2_t __attribute__((ext_vector_type(2)));
-  unsigned bits = __builtin_bit_cast(unsigned, x);
-  uint2_t s = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
-  const float y = fmaxf(__builtin_bit_cast(float, s[0]), __builtin_bit_cast(float, s[1]));
-  bits = __builtin_bit_cast(unsigned, y);
-  s = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
-  return fmaxf(__builtin_bit_cast(float, s[0]), __builtin_bit_cast(float, s[1]));
+  float a = x, b = x;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  a = __builtin_fmaxf(a, b);
+  b = a;
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return __builtin_fmaxf(a, b);
 }
 
 // D(16x16) += A(16x32) * B(32x16), fp16 inputs, fp32 accumulate.

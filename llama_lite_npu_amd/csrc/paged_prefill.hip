@@ -27,12 +27,23 @@
 // back as 16-byte rows by 16 lanes of different rows) and V (read back transposed, 8 rows x
 // 32 bytes at a time); both reads are then free of bank conflicts.
 //
+// The softmax scale (times log2 e) is folded into q when it is loaded, and in the fast tiles the
+// score accumulators start from -m (the running maximum of their column) instead of zero, so the
+// MFMA result is already the exponent: a probability costs one v_exp_f32 and half a packed
+// conversion. Whether the running maximum still holds is checked on the packed fp16
+// probabilities (any above 2^8, or not finite, sends the sub-tile to general_tile), not by a
+// column maximum over the fp32 scores.
+//
 // The accumulators are only ever rescaled in straight-line code (general_tile): a conditional
 // rescale inside the key loop makes the compiler copy all 72 accumulator registers at the join
-// on every tile. Tiles below the diagonal run in a loop that leaves as soon as a column maximum
-// grows by more than 8 and otherwise touches the accumulators with MFMAs only.
+// on every tile. Tiles below the diagonal run in a loop of three straight-line blocks, each laid
+// out as a pipeline with scheduling fences and group barriers: the eight K fragments of a
+// half-tile are requested at once and each register is refilled with the other half's fragment as
+// soon as its MFMA pair has issued; V fragments are requested a block ahead of their use; the
+// exponentials of one half run beside the MFMAs of the other; the next tile's HBM -> LDS loads
+// leave a quarter at a time between MFMA pairs instead of in one burst behind the barrier.
 //
-// About 216 registers per lane leave two wavefronts per SIMD: two workgroups share a compute
+// About 235 registers per lane leave two wavefronts per SIMD: two workgroups share a compute
 // unit and drift apart, so one's softmax (vector ALU) overlaps the other's MFMAs and a
 // finishing block's prologue/epilogue hides behind its neighbour. Grid: x = kv head (times the
 // head split), y = row block (long blocks first), z = sequence; with 8 kv heads a head's blocks
@@ -93,18 +104,6 @@ __device__ __forceinline__ float vmax3(float a, float b, float c) {
   return __builtin_fmaxf(__builtin_fmaxf(a, b), c);
 }
 __device__ __forceinline__ float vmax2(float a, float b) { return __builtin_fmaxf(a, b); }
-// Maximum over the four lanes that hold one column (lanes l, l^16, l^32, l^48). The swaps
-// exchange 16- and 32-lane halves between their two operands, so max(first, second) of the
-// swapped pair is the pairwise maximum, without a trip through LDS.
-__device__ __forceinline__ float max_across_groups(float x) {
-  typedef unsigned uint2_t __attribute__((ext_vector_type(2)));
-  unsigned bits = __builtin_bit_cast(unsigned, x);
-  uint2_t s = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
-  float y = vmax2(__builtin_bit_cast(float, s[0]), __builtin_bit_cast(float, s[1]));
-  bits = __builtin_bit_cast(unsigned, y);
-  s = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
-  return vmax2(__builtin_bit_cast(float, s[0]), __builtin_bit_cast(float, s[1]));
-}
 constexpr int kPagedPrefill = 0, kPackedPrefill = 1, kSharedPrefix = 2, kPagedPrefillFp8 = 3,
               kSharedPrefixFp8 = 4;
 
@@ -137,11 +136,15 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   const int head0 = ((int)blockIdx.x - h * head_splits) * heads_per_wg;
   const int heads_here = (group - head0) < heads_per_wg ? (group - head0) : heads_per_wg;
   const int b = blockIdx.z;
-  float v_scale = 1.0f;
+  // The softmax scale (times log2 e) is folded into q when it is loaded, so a score leaves the
+  // MFMA in the exponent's unit. An fp8 pool's K scale stays a multiplier of the scores
+  // (k_mul): folded into fp16 q it could push small elements into the subnormal range.
+  float v_scale = 1.0f, k_mul = 1.0f;
   if constexpr (FP8) {
-    scale_log2 *= paged.scales[h];
+    k_mul = paged.scales[h];
     v_scale = paged.scales[paged.num_kv_heads + h];
   }
+  const float k_mul_inv = 1.0f / k_mul;
 
   // What the block works on: query rows m0.. of sequence b (prefill), or the column block
   // blockIdx.y of all (sequence, head) pairs against key slice blockIdx.z (shared prefix).
@@ -303,16 +306,22 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     out_head[u] = hq;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      qf[u][kk] = ok ? *(const half8_t *)(qrow + 32 * kk) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      const half8_t raw = ok ? *(const half8_t *)(qrow + 32 * kk) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      typedef float float8_t __attribute__((ext_vector_type(8)));
+      qf[u][kk] = __builtin_convertvector(__builtin_convertvector(raw, float8_t) * scale_log2, half8_t);
     }
   }
 
   float4_t acc[8][kColTiles];
   float4_t dsum[kColTiles];
   float m_run[kColTiles];
+  // Seed of the score accumulators in the fast tiles: -m_run (divided by k_mul), in all four
+  // elements, so that the MFMA result is already the exponent.
+  float4_t seed[kColTiles];
 #pragma unroll
   for (int u = 0; u < kColTiles; ++u) {
     m_run[u] = -INFINITY;
+    seed[u] = float4_t{0.f, 0.f, 0.f, 0.f};
     dsum[u] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j][u] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -347,11 +356,12 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   half8_t pk[kColTiles];
 
   // S^T of 32 keys (rows 32 s2 .. +31 of the staged K tile) against this wavefront's columns.
-  auto scores_into = [&](float4_t (&st)[2][kColTiles], int s2) {
+  auto scores_into = [&](float4_t (&st)[2][kColTiles], int s2, auto seeded_tag) {
+    constexpr bool SEEDED = decltype(seeded_tag)::value;
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
 #pragma unroll
-      for (int u = 0; u < kColTiles; ++u) st[m][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+      for (int u = 0; u < kColTiles; ++u) st[m][u] = SEEDED ? seed[u] : float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
         const half8_t a =
@@ -378,18 +388,64 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     mx = vmax3(mx, st[0][u][3], st[1][u][0]);
     mx = vmax3(mx, st[1][u][1], st[1][u][2]);
     mx = vmax2(mx, st[1][u][3]);
-    return max_across_groups(mx) * scale_log2;  // scale > 0: max and scaling commute
+    return max_over_lane_groups(mx) * k_mul;  // k_mul > 0: max and scaling commute
   };
   // p = 2^(s * scale - m), cast to fp16, in B-operand order.
+  typedef float float2_t __attribute__((ext_vector_type(2)));
+  typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+  // General path: p = 2^(s * k_mul - m) from unseeded scores.
   auto exponentials_of = [&](const float4_t (&st)[2][kColTiles], half8_t (&pk)[kColTiles], int u) {
     const float neg_m = -m_run[u];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float p0 = fast_exp2(__builtin_fmaf(st[0][u][i], scale_log2, neg_m));
-      const float p1 = fast_exp2(__builtin_fmaf(st[1][u][i], scale_log2, neg_m));
-      pk[u][i] = (half_t)p0;
-      pk[u][4 + i] = (half_t)p1;
+    for (int m = 0; m < 2; ++m) {
+#pragma unroll
+      for (int i = 0; i < 4; i += 2) {
+        float2_t p;
+        if constexpr (FP8) {
+          p = float2_t{fast_exp2(__builtin_fmaf(st[m][u][i], k_mul, neg_m)),
+                       fast_exp2(__builtin_fmaf(st[m][u][i + 1], k_mul, neg_m))};
+        } else {
+          p = float2_t{fast_exp2(st[m][u][i] + neg_m), fast_exp2(st[m][u][i + 1] + neg_m)};
+        }
+        const half2_t ph = __builtin_convertvector(p, half2_t);
+        pk[u][4 * m + i] = ph[0];
+        pk[u][4 * m + i + 1] = ph[1];
+      }
     }
+  };
+  // Fast path: the scores were seeded with -m, so they are the exponents themselves.
+  auto exponentials_seeded = [&](const float4_t (&st)[2][kColTiles], half8_t (&pk)[kColTiles], int u) {
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+#pragma unroll
+      for (int i = 0; i < 4; i += 2) {
+        float2_t p;
+        if constexpr (FP8) {
+          p = float2_t{fast_exp2(st[m][u][i] * k_mul), fast_exp2(st[m][u][i + 1] * k_mul)};
+        } else {
+          p = float2_t{fast_exp2(st[m][u][i]), fast_exp2(st[m][u][i + 1])};
+        }
+        const half2_t ph = __builtin_convertvector(p, half2_t);
+        pk[u][4 * m + i] = ph[0];
+        pk[u][4 * m + i + 1] = ph[1];
+      }
+    }
+  };
+  // True if any probability of the sub-tile exceeds 2^8 (or is not finite): the running maximum
+  // is then too low for these keys and the sub-tile has to be redone with a rescale. Probabilities
+  // are non-negative, so their fp16 bit patterns order like their values.
+  auto overflowed = [&](const half8_t (&pk)[kColTiles]) -> bool {
+    typedef _Float16 half8v __attribute__((ext_vector_type(8)));
+    const half8v mx8 = __builtin_elementwise_max(pk[0], pk[1]);
+    typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+    const half4v lo4 = __builtin_shufflevector(mx8, mx8, 0, 1, 2, 3);
+    const half4v hi4 = __builtin_shufflevector(mx8, mx8, 4, 5, 6, 7);
+    const half4v mx4 = __builtin_elementwise_max(lo4, hi4);
+    const half2_t mx2 = __builtin_elementwise_max(__builtin_shufflevector(mx4, mx4, 0, 1),
+                                                  __builtin_shufflevector(mx4, mx4, 2, 3));
+    const uint32_t bits = __builtin_bit_cast(uint32_t, mx2);
+    const uint32_t top = (bits & 0xffffu) > (bits >> 16) ? (bits & 0xffffu) : (bits >> 16);
+    return __builtin_amdgcn_ballot_w64(top > 0x5C00u) != 0;  // 0x5C00 = 256.0
   };
   // O^T += V^T . P^T,  l += 1^T . P^T for keys 32 s2 .. +31 of the staged V tile.
   auto accumulate_with = [&](const half8_t (&pk)[kColTiles], int s2) {
@@ -407,7 +463,16 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       for (int u = 0; u < kColTiles; ++u) acc[j][u] = mfma_16x16x32(a, pk[u], acc[j][u]);
     }
   };
-  auto scores_sub = [&](int s2) { scores_into(st, s2); };
+  // V^T fragment j (A operand: d rows 16j.., keys 32 s2 + {4g..4g+3, 16+4g..}) of the staged tile.
+  auto load_vfrag = [&](int j, int s2) -> half8_t {
+    const uint32_t at = v_addr[j] + 2u * 32 * s2 * kHeadDim;
+    const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t *)(uintptr_t)at);
+    const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (lds_short4_t *)(uintptr_t)(at + 2u * 16 * kHeadDim));
+    const short8_t both = short8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(half8_t, both);
+  };
+  auto scores_sub = [&](int s2) { scores_into(st, s2, std::false_type{}); };
   auto column_max = [&](int u) { return column_max_of(st, u); };
   auto exponentials = [&](int u) { exponentials_of(st, pk, u); };
   auto accumulate_sub = [&](int s2) { accumulate_with(pk, s2); };
@@ -415,7 +480,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   half8_t pk1[kColTiles];
 
   // Publishes tile kt (already requested) and requests tile kt + 1 into the other half.
-  auto sync_and_prefetch = [&](int kt) {
+  auto sync_and_prefetch = [&](int kt, bool issue_next = true) {
     if constexpr (FP8) {
       // The codes of tile kt (requested a tile ago) become fp16 rows in its LDS half: 16-byte
       // chunk c of row r goes where the direct load of the fp16 path would have put it.
@@ -433,7 +498,35 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's part of tile kt is in LDS
     __syncthreads();                     // ... and everyone's; everyone is done with tile kt-1
-    if (kt + 1 < n_tiles) issue_tile(kt + 1);
+    if (issue_next && kt + 1 < n_tiles) issue_tile(kt + 1);
+  };
+  // The same loads for a tile that lies wholly inside the sequence's keys, split in two steps so
+  // that they can ride between MFMAs instead of leaving in one burst behind the barrier:
+  // tile_bases() reads the page id (scalar), issue_rows(i) requests row group i of K and of V.
+  const char *next_kbase = nullptr, *next_vbase = nullptr;
+  uint32_t next_dst = 0;
+  auto tile_bases = [&](int kt) {
+    const int row0 = (tile0 + kt) * kKvTile + 16 * wave;
+    if (PAGED) {
+      int pid = table[(tile0 + kt) * 4 + wave];
+      pid = pid < 0 ? 0 : (pid >= paged.num_pages ? paged.num_pages - 1 : pid);
+      next_kbase = (const char *)paged.kv + (int64_t)pid * ((int64_t)kPageSize * k_pitch);
+      next_vbase = next_kbase;
+    } else {
+      next_kbase = (const char *)packed.k + (int64_t)(q_start + row0) * k_pitch;
+      next_vbase = (const char *)packed.v + (int64_t)(q_start + row0) * v_pitch;
+    }
+    next_dst = (uint32_t)((kt & 1) * kTileHalfs + 16 * wave * kHeadDim) * 2u;
+  };
+  auto issue_rows = [&](int i) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(k_lds + next_dst + 1024u * i), "v"(koff[i]), "s"(next_kbase)
+                 : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(v_lds + next_dst + 1024u * i), "v"(voff[i]), "s"(next_vbase)
+                 : "memory", "m0");
   };
 
   // General sub-tiles of tile kt from `first` on: causal mask, and the accumulators are rescaled
@@ -453,6 +546,8 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
         const float m_new = vmax2(m_run[u], column_max(u));
         const float alpha = fast_exp2(m_run[u] - m_new);
         m_run[u] = m_new;
+        const float sd = -m_new * k_mul_inv;
+        seed[u] = float4_t{sd, sd, sd, sd};
         dsum[u] *= alpha;
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[j][u] *= alpha;
@@ -476,17 +571,14 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       for (int s2 = 0; s2 < 2; ++s2) {
         const int key0 = (tile0 + kt) * kKvTile + 32 * s2;
         if (MASKED && key0 >= kv_end) break;
-        scores_sub(s2);
+        scores_into(st, s2, std::true_type{});
         if (MASKED) {
           mask_sub(0, key0);
           mask_sub(1, key0);
         }
-        const float mx0 = column_max(0), mx1 = column_max(1);
-        if (__builtin_amdgcn_ballot_w64(mx0 > m_run[0] + 8.0f || mx1 > m_run[1] + 8.0f) != 0) {
-          return 1 + s2;
-        }
-        exponentials(0);
-        exponentials(1);
+        exponentials_seeded(st, pk, 0);
+        exponentials_seeded(st, pk, 1);
+        if (overflowed(pk)) return 1 + s2;
         accumulate_sub(s2);
       }
     }
@@ -499,22 +591,94 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   // from its first half).
   auto fast_plain_tiles = [&](int kt_end) -> int {
     for (; kt < kt_end; ++kt) {
-      sync_and_prefetch(kt);
+      sync_and_prefetch(kt, FP8);
       flip_halves();
-      scores_into(st, 0);
-      scores_into(st1, 1);
-      const float a0 = column_max_of(st, 0), a1 = column_max_of(st, 1);
-      const float b0 = column_max_of(st1, 0), b1 = column_max_of(st1, 1);
-      const float lim0 = m_run[0] + 8.0f, lim1 = m_run[1] + 8.0f;
-      if (__builtin_amdgcn_ballot_w64(a0 > lim0 || a1 > lim1 || b0 > lim0 || b1 > lim1) != 0) {
-        return 1;
+      if constexpr (!FP8) tile_bases(kt + 1);
+      // Block 1: scores of both halves, the first half's exponentials beside the second half's
+      // MFMAs, and the first half's V fragments requested before the block ends.
+      // Region 1: all eight K fragments of the first half are requested at once.
+      auto load_kfrag = [&](int s2, int i) -> half8_t {   // fragment i = (kk = i / 2, m = i % 2)
+        return *(const lds_half8_t *)(uintptr_t)(k_addr[i >> 1] + 2u * (32 * s2 + 16 * (i & 1)) * kHeadDim);
+      };
+      half8_t kf[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) kf[i] = load_kfrag(0, i);
+#pragma unroll
+      for (int m = 0; m < 2; ++m) {
+#pragma unroll
+        for (int u = 0; u < kColTiles; ++u) st[m][u] = st1[m][u] = seed[u];
       }
-      exponentials_of(st, pk, 0);
-      exponentials_of(st, pk, 1);
-      accumulate_with(pk, 0);
-      exponentials_of(st1, pk1, 0);
-      exponentials_of(st1, pk1, 1);
-      accumulate_with(pk1, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      // Region 2: the first half's MFMAs; each fragment register takes the second half's
+      // fragment once its pair is issued. Four accumulators in rotation: no MFMA waits for
+      // the one before it.
+      half8_t kf1[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int u = 0; u < kColTiles; ++u) st[i & 1][u] = mfma_16x16x32(kf[i], qf[u][i >> 1], st[i & 1][u]);
+        kf1[i] = load_kfrag(1, i);
+        if constexpr (!FP8) {
+          if (i & 1) issue_rows(i >> 1);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (!FP8 && (i & 1)) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      // Region 3: the second half's MFMAs beside the first half's exponentials; the first
+      // half's V fragments are requested on the way.
+      half8_t vf[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int u = 0; u < kColTiles; ++u) st1[i & 1][u] = mfma_16x16x32(kf1[i], qf[u][i >> 1], st1[i & 1][u]);
+        vf[i] = load_vfrag(i, 0);
+      }
+      exponentials_seeded(st, pk, 0);
+      exponentials_seeded(st, pk, 1);
+      const bool over_a = overflowed(pk);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+      }
+      if (over_a) return 1;
+      // Block 2: second product of the first half beside the second half's exponentials; each
+      // fragment register takes the second half's fragment as soon as its MFMAs are issued.
+      half8_t vf2[8];
+#pragma unroll
+      for (int u = 0; u < kColTiles; ++u) dsum[u] = mfma_16x16x32(ones, pk[u], dsum[u]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+#pragma unroll
+        for (int u = 0; u < kColTiles; ++u) acc[j][u] = mfma_16x16x32(vf[j], pk[u], acc[j][u]);
+        vf2[j] = load_vfrag(j, 1);
+      }
+      exponentials_seeded(st1, pk1, 0);
+      exponentials_seeded(st1, pk1, 1);
+      const bool over_b = overflowed(pk1);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+      if (over_b) return 2;
+      // Block 3: second product of the second half.
+#pragma unroll
+      for (int u = 0; u < kColTiles; ++u) dsum[u] = mfma_16x16x32(ones, pk1[u], dsum[u]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+#pragma unroll
+        for (int u = 0; u < kColTiles; ++u) acc[j][u] = mfma_16x16x32(vf2[j], pk1[u], acc[j][u]);
+      }
     }
     return 0;
   };
@@ -526,7 +690,10 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     sync_and_prefetch(0);
     general_tile(0, 0);
     while (kt < n_tiles) {
-      int grew = fast_plain_tiles(n_plain);
+      int n_spread = (last_key + 1) / kKvTile - 1 - tile0;   // tiles kt < n_spread: tile kt + 1 is full
+      n_spread = n_spread < n_tiles - 1 ? n_spread : n_tiles - 1;
+      n_spread = n_spread < n_plain ? n_spread : n_plain;
+      int grew = fast_plain_tiles(n_spread);
       if (grew == 0) grew = fast_tiles(n_tiles, std::true_type{});
       if (grew != 0) {
         general_tile(kt, grew - 1);

@@ -119,6 +119,61 @@ def test_zero_length_sequence_gives_zeros():
         assert float(out[1].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("chunks", [2, 4, 9])
+def test_balanced_many_short_rows_with_empty_ones_between(chunks):
+    """Twice as many sequences as chunks and more: the merge then runs over the chunk boundaries
+    (only a sequence that crosses one has pieces). Empty rows sit at the start, at the end, next
+    to each other and right where chunks are cut."""
+    print(f"decode balanced, short rows with empty ones, chunks={chunks}", flush=True)
+    lens = [5, 33, 0, 18, 70, 0, 0, 2, 47, 16, 0, 90, 31, 1, 0, 64, 15, 17, 0, 40, 8, 0, 29, 12]
+    case = workloads.make_decode_case("short-empty", 83 + chunks, lens, 16, 4, device=DEV)
+    empty = [i for i, n in enumerate(lens) if n == 0] + [0, len(lens) - 1]
+    for i in empty:
+        case.seq_lens[i] = 0
+    assert len(lens) >= 2 * chunks
+    ref = _oracle(case)
+    out = _run(case, schedule="balanced", chunks=chunks)
+    assert_attention_close(out, ref, f"short rows with empty ones, chunks={chunks}")
+    for i in empty:
+        assert float(out[i].abs().max()) == 0.0
+    assert torch.equal(out, _run(case, schedule="balanced", chunks=chunks))
+    # the same step with the append fused in
+    plan = ops.DecodePlan(case.block_table, case.seq_lens, 16, 4, case.num_pages, chunks=chunks)
+    pool = case.kv_pool.clone()
+    fused = ops.decode_step(case.q, pool, plan, case.k_new, case.v_new, case.softmax_scale)
+    torch.cuda.synchronize()
+    want_pool = case.kv_pool.clone()
+    live = [i for i in range(len(lens)) if i not in empty]
+    for b in live:
+        want_pool[int(case.slot_mapping[b]), :4], want_pool[int(case.slot_mapping[b]), 4:] = case.k_new[b], case.v_new[b]
+    assert torch.equal(pool, want_pool)
+    ref2 = c_oracle.paged_decode(to_np16(case.q), to_np16(want_pool), case.block_table.cpu().numpy(),
+                                 case.seq_lens.cpu().numpy(), case.softmax_scale)
+    assert_attention_close(fused, ref2, f"fused append, short rows with empty ones, chunks={chunks}")
+
+
+@pytest.mark.parametrize("spike_at", [5, 70, 301, 590])
+def test_score_spike_far_above_the_running_maximum(spike_at):
+    """One key scores about 2^40 times higher than all the keys before it, so its probability
+    against the running maximum would overflow fp16: the maximum has to follow it, in whichever
+    lane group of its page the key sits and under every schedule."""
+    print(f"decode score spike at key {spike_at}", flush=True)
+    case = workloads.make_decode_case("spike", 90 + spike_at, [599, 130, 40], 16, 2, device=DEV)
+    gen = torch.Generator().manual_seed(91)
+    direction = torch.randn(workloads.HEAD_DIM, generator=gen)
+    direction = direction / direction.norm()
+    case.q.copy_((6.0 * direction + 0.3 * torch.randn(case.q.shape, generator=gen)).half())
+    pool = 0.3 * torch.randn(case.kv_pool.shape, generator=gen)
+    table = case.block_table.cpu()
+    for b, at in ((0, spike_at), (1, min(spike_at, 100)), (2, 17)):
+        slot = int(table[b, at // 16]) * 16 + at % 16
+        pool[slot, :2] += 52.0 * direction          # K heads: 6 * 52 / sqrt(128) * log2(e), about +40
+    case.kv_pool.copy_(pool.half())
+    ref = _oracle(case)
+    for kw in ({}, {"schedule": "balanced", "chunks": 7}, {"num_splits": 1}, {"num_splits": 5}):
+        assert_attention_close(_run(case, **kw), ref, f"spike at {spike_at} {kw}")
+
+
 def test_split_count_and_page_permutation_invariance():
     """Same logical KV under another physical page assignment and any split count."""
     print("decode invariance", flush=True)

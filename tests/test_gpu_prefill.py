@@ -104,6 +104,32 @@ def test_prefill_running_maximum_keeps_growing():
     assert_attention_close(out, _oracle_paged(case), "growing maximum")
 
 
+@pytest.mark.parametrize("spike_at", [70, 300, 321, 1000])
+def test_prefill_score_spike_far_above_the_running_maximum(spike_at):
+    """One key scores about 2^40 times higher than everything before it (its probability would
+    overflow fp16 against the running maximum): the tile has to be redone with a rescale, whether
+    the key sits in the first or second half of its tile, below the diagonal or on it."""
+    print(f"prefill score spike at key {spike_at}", flush=True)
+    case = workloads.make_prefill_case("spike", 430 + spike_at, [1100, 400], 16, 2, device=DEV)
+    gen = torch.Generator().manual_seed(431)
+    direction = torch.randn(workloads.HEAD_DIM, generator=gen)
+    direction = direction / direction.norm()
+    case.q.copy_((6.0 * direction + 0.3 * torch.randn(case.q.shape, generator=gen)).half())
+    k = 0.3 * torch.randn(case.k.shape, generator=gen)
+    k[spike_at] += 52.0 * direction              # 6 * 52 / sqrt(128) * log2(e): about +40 in log2 units
+    k[1100 + 200] += 52.0 * direction            # second sequence: a spike of its own
+    case.k.copy_(k.half())
+    _append(case)
+    out = ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, None, case.max_q_len,
+                            case.softmax_scale)
+    torch.cuda.synchronize()
+    assert_attention_close(out, _oracle_paged(case), f"spike at {spike_at}")
+    packed = ops.varlen_prefill(case.q, case.k, case.v, case.cu_q_lens[:-1], case.seq_lens, case.max_q_len,
+                                case.softmax_scale)
+    torch.cuda.synchronize()
+    assert_attention_close(packed, _oracle_paged(case), f"spike at {spike_at}, packed K/V")
+
+
 def test_prefill_never_reads_values_past_the_sequence_end():
     """Slots after the last token of a page (and unowned pages) hold NaN: they must not leak."""
     print("prefill NaN in unused slots", flush=True)
