@@ -34,14 +34,37 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
-# HBM bytes per launch of the roofline kernel(s) from rocprofv3 FETCH_SIZE + WRITE_SIZE (scaled by a
-# 1 GiB copy kernel); summaries and commands in profiles/paged_decode_balanced_c2_pmc.txt,
-# profiles/paged_decode_balanced_fp8_c2.txt and profiles/hbm_traffic_c3_c4_c5_pmc.txt. Only
-# meaningful for the workload it was measured on. c4: prefix kernel + decode kernel + merge.
-MEASURED_TRAFFIC_BYTES = {("c2", "balanced", "f16"): 317.8e6, ("c2", "balanced", "fp8"): 164.5e6,
-                          ("c3", "balanced", "f16"): 387.7e6, ("c4", "balanced", "f16"): 150.6e6,
-                          ("c5", "balanced", "f16"): 5196.0e6}
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, published
+
+
+METRIC = "paged decode attn HBM GB/s (% of 8 TB/s peak); KV-append GB/s; us/layer"
+TRAFFIC_FILE = ROOT / "profiles" / "traffic.json"
+
+
+def measured_traffic(config: str, schedule: str, kv_dtype: str):
+    """HBM bytes per launch of a configuration's roofline kernel(s) as rocprofv3 counted them
+    (FETCH_SIZE + WRITE_SIZE scaled by a copy of known size; profiles/traffic.json names the
+    summary each figure comes from). A figure only describes the kernel source it was taken on:
+    the file's SHA-256 at that time is stored with it, and a source that has changed since gives
+    None. Returns (bytes or None, the stamp that is printed with the result)."""
+    import hashlib
+
+    try:
+        entries = json.loads(TRAFFIC_FILE.read_text())["entries"]
+    except (OSError, ValueError, KeyError):
+        return None, None
+    for e in entries:
+        if (e["config"], e["schedule"], e["kv_dtype"]) != (config, schedule, kv_dtype):
+            continue
+        current = True
+        for rel, digest in e["kernel_sources"].items():
+            try:
+                current &= hashlib.sha256((ROOT / rel).read_bytes()).hexdigest() == digest
+            except OSError:
+                current = False
+        stamp = {"profile": e["profile"], "taken_at_commit": e["commit"], "kernel_sources_unchanged": current}
+        return (float(e["bytes_per_launch"]) if current else None), stamp
+    return None, None
 
 
 def _median(xs):
@@ -543,15 +566,22 @@ def run_prefill(case, steps: int, warmup: int, device: str, label: str) -> dict:
     }
 
 
-def cpu_baseline_decode(case, budget_s: float = 10.0) -> dict:
+def cpu_baseline_decode(case, budget_s: float = 10.0, max_sequences=None) -> dict:
     """The reference's torch CPU path (append + gathered fp32 attention) for ONE layer of `case`,
-    on the host cores: 1 warm-up, then repetitions for about `budget_s` seconds, min taken."""
+    on the host cores: 1 warm-up, then repetitions for about `budget_s` seconds, min taken.
+    `max_sequences`: time only the first that many sequences and scale the rate as measured (the
+    result is then flagged as extrapolated; the pool stays on the GPU side, only those sequences'
+    pages are brought to the host)."""
     import torch
     from oracle import cpu_ref
 
     cores = _host_threads()
     torch.set_num_threads(cores)
-    c = case.to("cpu")
+    extrapolated = max_sequences is not None and max_sequences < case.batch
+    if extrapolated:
+        c = _first_sequences(case, int(max_sequences))
+    else:
+        c = case.to("cpu")
     kv = torch.cat([c.k_new, c.v_new], dim=1)
     pool = c.kv_pool
 
@@ -578,10 +608,119 @@ def cpu_baseline_decode(case, budget_s: float = 10.0) -> dict:
         "cores": cores,
         "kind": "port",
         "cpu_model": _cpu_model(),
-        "sample": f"1 of the layers of the same workload (append + decode, {nbytes / 1e6:.1f} MB algorithmic), "
-                  f"torch CPU restatement, min of {max(1, len(times))} reps after 1 warm-up, {best:.3f} s",
-        "seconds_per_layer": best,
+        "sample": (f"the first {c.batch} of {case.batch} sequences of one layer (rate extrapolated to the "
+                   f"whole layer), " if extrapolated else "1 of the layers of the same workload, ")
+                  + f"append + decode, {nbytes / 1e6:.1f} MB algorithmic, torch CPU restatement, "
+                    f"min of {max(1, len(times))} reps after 1 warm-up, {best:.3f} s",
+        "extrapolated": extrapolated,
+        "seconds_per_layer": best * (case.decode_bytes() + case.append_bytes()) / nbytes,
     }
+
+
+def _first_sequences(case, n: int):
+    """The first n sequences of a decode case as a case of their own on the CPU: their pages are
+    pulled out of the pool into a dense one (same bytes, new page ids)."""
+    import torch
+    from llama_lite_npu_amd import workloads
+
+    lens = case.seq_lens[:n].cpu().to(torch.int64)
+    n_pages = ((lens + 15) // 16).tolist()
+    table = case.block_table[:n].cpu()
+    live = torch.cat([table[b, :p] for b, p in enumerate(n_pages)]).to(torch.long)
+    pool = case.kv_pool.view(case.num_pages, 16, *case.kv_pool.shape[1:])[live.to(case.kv_pool.device)].cpu()
+    new_table = torch.zeros((n, max(n_pages)), dtype=torch.int32)
+    cur = 0
+    for b, p in enumerate(n_pages):
+        new_table[b, :p] = torch.arange(cur, cur + p, dtype=torch.int32)
+        cur += p
+    ctx = case.context_lens[:n].cpu()
+    slots = torch.tensor([int(new_table[b, int(ctx[b]) // 16]) * 16 + int(ctx[b]) % 16 for b in range(n)],
+                         dtype=torch.int32)
+    return workloads.DecodeCase(
+        name=case.name, num_q_heads=case.num_q_heads, num_kv_heads=case.num_kv_heads, context_lens=ctx,
+        seq_lens=case.seq_lens[:n].cpu(), block_table=new_table, slot_mapping=slots, num_pages=cur,
+        q=case.q[:n].cpu(), k_new=case.k_new[:n].cpu(), v_new=case.v_new[:n].cpu(),
+        kv_pool=pool.reshape(cur * 16, *case.kv_pool.shape[1:]), num_splits=case.num_splits)
+
+
+CONFIGS = ("c1", "c2", "c3", "c4", "c5")
+
+
+def measure(name: str, args, device: str, cpu_budget_s: float, schedule=None) -> dict:
+    """One configuration measured in full: the step (value, ms_per_step), the roofline of its
+    dominant kernel(s), the launches beside it, and the CPU baseline, in the schema of the
+    headline line."""
+    import torch
+    from llama_lite_npu_amd import workloads
+
+    schedule = schedule or args.schedule
+    steps = args.steps if args.steps is not None else (30 if name == "c3" else 10)
+    warmup = args.warmup if args.warmup is not None else (10 if name == "c3" else 3)
+    if name == "c3":
+        case = workloads.config_c3(device)
+        res = run_prefill(case, steps, warmup, device, case.name)
+        kv_dtype = "f16"
+    else:
+        layers = args.layers or {"c1": 64, "c2": 64, "c4": 16, "c5": 1}[name]
+        case = {"c1": workloads.config_c1, "c2": workloads.config_c2, "c4": workloads.config_c4,
+                "c5": workloads.config_c5}[name](device)
+        if args.chunks:
+            case.extra["chunks"] = args.chunks
+        shared = 0
+        if schedule == "balanced" and not args.no_shared_prefix and not case.extra.get("private_prefix"):
+            shared = int(case.extra.get("n_shared", 0))
+        kv_dtype = args.kv_dtype if schedule == "balanced" else "f16"
+        res = run_decode(case, layers, steps, warmup, device, case.name, schedule, shared,
+                         graph=not args.no_graph, kv_dtype=kv_dtype)
+    traffic, stamp = measured_traffic(name, schedule, kv_dtype)
+    res["roofline"]["traffic_source"] = stamp
+    if traffic is not None and (name != "c4" or not args.no_shared_prefix):
+        if name == "c3":
+            duration_us, algorithmic = res["prefill_us_mean"], case.min_bytes()
+        else:
+            duration_us = res["roofline"].get("duration_us", res["decode_kernel_us_mean"])
+            algorithmic = res["roofline"].get("unique_bytes_per_launch",
+                                              res["decode_bytes_per_layer"] + res["append_bytes_per_layer"])
+        res["roofline"]["traffic"] = traffic / (duration_us * 1e-6) / 1e9
+        res["roofline"]["traffic_bytes_per_launch"] = traffic
+        res["roofline"]["algorithmic_bytes_per_launch"] = algorithmic
+    row = {
+        "value": res.get("value", res.get("prefill_tflops")),
+        "unit": "GB/s" if "value" in res else "TFLOP/s",
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": res["ms_per_step"],
+        "dtype": "f16",
+        "config": {"workload": res["label"], "config": name, "launch": res.get("launch", "eager"),
+                   "kv_dtype": kv_dtype, "schedule": schedule if name != "c3" else None},
+        "roofline": res["roofline"],
+        "detail": {k: v for k, v in res.items() if k not in ("roofline", "label", "value", "ms_per_step", "launch")},
+    }
+    if name != "c3":
+        row["config"].update(batch=case.batch, num_q_heads=case.num_q_heads, num_kv_heads=case.num_kv_heads,
+                             head_dim=128, page_size=16, layers=res["layers"],
+                             tokens_attended=int(case.seq_lens.sum()))
+        row["pct_of_hbm_peak"] = 100.0 * res["roofline"]["frac"]
+        ap_us = time_append(case.k_new, case.v_new, case.slot_mapping, case.kv_pool)
+        row["detail"]["append_us"] = ap_us
+        row["detail"]["append_gbps"] = case.append_bytes() / (ap_us * 1e-6) / 1e9
+        row["detail"].update(time_qk_epilogue(case.batch, case.num_q_heads, case.num_kv_heads,
+                                              case.slot_mapping, case.kv_pool))
+        if name == "c4":
+            row["detail"].update(cow_step(case))
+        if name == "c5" and schedule == "balanced":
+            row["detail"].update(compaction_step(case))
+        if not args.no_cpu_baseline:
+            row["cpu_baseline"] = cpu_baseline_decode(case, cpu_budget_s, max_sequences=8 if name == "c5" else None)
+    else:
+        row["pct_of_mfma_peak"] = 100.0 * res["roofline"]["frac"]
+        row["detail"].update(time_qk_epilogue(int(case.seq_lens.sum()), case.num_q_heads, case.num_kv_heads,
+                                              case.slot_mapping, case.kv_pool))
+        if not args.no_cpu_baseline:
+            row["cpu_baseline"] = cpu_baseline_prefill(case, cpu_budget_s)
+    del case
+    torch.cuda.empty_cache()
+    return row
 
 
 def main() -> int:
@@ -589,9 +728,12 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None, help="timed steps (default 10; 30 for c3)")
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps first (default 3; 10 for c3)")
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--config", default="c2", choices=list(CONFIGS))
     ap.add_argument("--layers", type=int, default=None, help="independent KV pools per step (c2 default 64)")
-    ap.add_argument("--all", action="store_true", help="also report the other configurations (stderr)")
+    ap.add_argument("--only", action="store_true",
+                    help="measure --config alone (default: the other configurations follow in detail.configs)")
+    ap.add_argument("--all", action="store_true",
+                    help="also write one line per configuration, same schema, to bench_all.jsonl under --out-dir")
     ap.add_argument("--schedule", default="balanced", choices=["balanced", "splits"],
                     help="decode work decomposition (splits: separate append, split and merge launches)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -609,18 +751,13 @@ def main() -> int:
                     help="also launch one page_gather of exactly 1 GiB (read) + 1 GiB (write): a plain copy of "
                          "known size against which profiler byte counters can be scaled")
     args = ap.parse_args()
-    # A prefill step is ~0.4 ms: the part needs more of them to settle at its sustained clock.
-    if args.steps is None:
-        args.steps = 30 if args.config == "c3" else 10
-    if args.warmup is None:
-        args.warmup = 10 if args.config == "c3" else 3
     if args.gpus != 1:
         print("bench.py: this build measures the path on ONE GPU (one process, one device); "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
         return 2
 
     import torch
-    from llama_lite_npu_amd import _lib, workloads
+    from llama_lite_npu_amd import _lib
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the path has no CPU implementation", file=sys.stderr)
@@ -628,31 +765,6 @@ def main() -> int:
     _lib.load()
     device = "cuda:0"
     torch.cuda.set_device(0)
-
-    def decode_cfg(name):
-        if name == "c1":
-            return workloads.config_c1(device), (args.layers or 64)
-        if name == "c2":
-            return workloads.config_c2(device), (args.layers or 64)
-        if name == "c4":
-            return workloads.config_c4(device), (args.layers or 16)
-        if name == "c5":
-            return workloads.config_c5(device), (args.layers or 1)
-        raise ValueError(name)
-
-    def run(name):
-        if name == "c3":
-            case = workloads.config_c3(device)
-            return run_prefill(case, args.steps, args.warmup, device, case.name), case
-        case, layers = decode_cfg(name)
-        if args.chunks:
-            case.extra["chunks"] = args.chunks
-        sched = args.schedule
-        shared = 0
-        if sched == "balanced" and not args.no_shared_prefix and not case.extra.get("private_prefix"):
-            shared = int(case.extra.get("n_shared", 0))
-        return run_decode(case, layers, args.steps, args.warmup, device, case.name, sched, shared,
-                          graph=not args.no_graph, kv_dtype=args.kv_dtype), case
 
     if args.calibrate_copy:
         from llama_lite_npu_amd import ops
@@ -665,73 +777,52 @@ def main() -> int:
         del src, dst
         torch.cuda.empty_cache()
 
-    res, case = run(args.config)
-    traffic = MEASURED_TRAFFIC_BYTES.get((args.config, args.schedule, args.kv_dtype))
-    if traffic is not None and (args.config != "c4" or not args.no_shared_prefix):
-        if args.config == "c3":
-            duration_us, algorithmic = res["prefill_us_mean"], case.min_bytes()
-        else:
-            duration_us = res["roofline"].get("duration_us", res["decode_kernel_us_mean"])
-            algorithmic = res["roofline"].get("unique_bytes_per_launch",
-                                              res["decode_bytes_per_layer"] + res["append_bytes_per_layer"])
-        res["roofline"]["traffic"] = traffic / (duration_us * 1e-6) / 1e9
-        res["roofline"]["traffic_bytes_per_launch"] = traffic
-        res["roofline"]["algorithmic_bytes_per_launch"] = algorithmic
+    head = measure(args.config, args, device, cpu_budget_s=10.0)
     line = {
-        "metric": "paged decode attn HBM GB/s (% of 8 TB/s peak); KV-append GB/s; us/layer",
-        "value": res.get("value", res.get("prefill_tflops")),
-        "unit": "GB/s" if "value" in res else "TFLOP/s",
+        "metric": METRIC,
+        "value": head["value"],
+        "unit": head["unit"],
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": res["ms_per_step"],
+        "steps": head["steps"],
+        "warmup": head["warmup"],
+        "ms_per_step": head["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": res["label"], "config": args.config, "launch": res.get("launch", "eager"),
-                   "kv_dtype": args.kv_dtype},
-        "roofline": res["roofline"],
-        "detail": {k: v for k, v in res.items() if k not in ("roofline", "label", "value", "ms_per_step", "launch")},
+        "config": head["config"],
+        "roofline": head["roofline"],
+        "detail": head["detail"],
     }
-    if args.config != "c3":
-        line["config"].update(batch=case.batch, num_q_heads=case.num_q_heads, num_kv_heads=case.num_kv_heads,
-                              head_dim=128, page_size=16, layers=res["layers"],
-                              tokens_attended=int(case.seq_lens.sum()))
-        line["pct_of_hbm_peak"] = 100.0 * res["roofline"]["frac"]
-        ap_us = time_append(case.k_new, case.v_new, case.slot_mapping, case.kv_pool)
-        line["detail"]["append_us"] = ap_us
-        line["detail"]["append_gbps"] = case.append_bytes() / (ap_us * 1e-6) / 1e9
-        line["detail"].update(time_qk_epilogue(case.batch, case.num_q_heads, case.num_kv_heads,
-                                               case.slot_mapping, case.kv_pool))
-        if args.config == "c4":
-            line["detail"].update(cow_step(case))
-        if args.config == "c5":
-            line["detail"].update(compaction_step(case))
-        if not args.no_cpu_baseline:
-            line["cpu_baseline"] = cpu_baseline_decode(case)
-    else:
-        line["detail"].update(time_qk_epilogue(int(case.seq_lens.sum()), case.num_q_heads, case.num_kv_heads,
-                                               case.slot_mapping, case.kv_pool))
-        if not args.no_cpu_baseline:
-            line["cpu_baseline"] = cpu_baseline_prefill(case)
+    for key in ("pct_of_hbm_peak", "pct_of_mfma_peak", "cpu_baseline"):
+        if key in head:
+            line[key] = head[key]
+    rows = {args.config: head}
+    if not args.only:
+        # Every other configuration, each with its own roofline and CPU baseline (a few seconds of
+        # host time each). C5 is reported on both schedules: the balanced cut (the default) and the
+        # 16 per-sequence splits its description names.
+        others = {}
+        for name in CONFIGS:
+            if name == args.config:
+                continue
+            others[name] = measure(name, args, device, cpu_budget_s=3.0)
+            if name == "c5":
+                others["c5_16_splits"] = measure("c5", args, device, cpu_budget_s=0.0, schedule="splits")
+                others["c5_16_splits"].pop("cpu_baseline", None)   # the same CPU work as c5
+        rows.update(others)
+        line["detail"]["configs"] = others
     print(json.dumps(line), flush=True)
 
     if args.all:
         out_dir = ROOT / args.out_dir
         out_dir.mkdir(parents=True, exist_ok=True)
         with open(out_dir / "bench_all.jsonl", "w") as f:
-            f.write(json.dumps(line) + "\n")
-            for name in ("c1", "c2", "c3", "c4", "c5"):
-                if name == args.config:
-                    continue
-                del res, case
-                torch.cuda.empty_cache()
-                res, case = run(name)
-                f.write(json.dumps(res) + "\n")
-                f.flush()
-                print(json.dumps(res), file=sys.stderr, flush=True)
+            for name, row in rows.items():
+                full = {"metric": METRIC, "n_gpus": 1, "higher_is_better": True, "scaling": "weak",
+                        "vs_baseline": None, "data": "synthetic", **row}
+                f.write(json.dumps(full) + "\n")
     return 0
 
 
