@@ -478,15 +478,6 @@ int litekv_decode_advance(const int32_t *request_tables, int64_t request_table_s
                           int32_t increment, void *stream);
 
 /*
- * Profiling aid (no counterpart in the reference): the next
- * litekv_paged_decode_balanced launch made by this thread carries the two
- * hipEvent_t handles as its start and stop events, so its device-side
- * duration can be read with hipEventElapsedTime without extra packets in the
- * stream. Pass NULLs to cancel.
- */
-int litekv_profile_next_decode(void *start_event, void *stop_event);
-
-/*
  * Varlen causal prefill over paged KV. Replaces
  * `paged_chunk_flash_attention(q, k_cache, v_cache, sm_scale, req_token_table,
  * req_ids, q_start_loc, context_lens, q_seq_lens, max_q_len)`

@@ -62,7 +62,7 @@ def _hipcc() -> str:
 
 
 def _headers() -> list[Path]:
-    return sorted(CSRC.glob("*.h")) + [CSRC.parents[1] / "include" / "litekv.h"]
+    return sorted(CSRC.glob("*.h")) + sorted((CSRC.parents[1] / "include").glob("*.h"))
 
 
 def is_stale() -> bool:

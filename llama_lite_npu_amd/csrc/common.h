@@ -8,6 +8,7 @@
 #include <stdio.h>
 
 #include "../../include/litekv.h"
+#include "../../include/litekv_profile.h"
 
 namespace litekv {
 

@@ -9,11 +9,21 @@ import pytest
 
 ROOT = Path(__file__).resolve().parents[1]
 HEADER = ROOT / "include" / "litekv.h"
+PROFILE_HEADER = ROOT / "include" / "litekv_profile.h"     # measurement aid, outside the product ABI
+
+
+def _declared_in(path):
+    text = re.sub(r"/\*.*?\*/", "", path.read_text(), flags=re.S)
+    return set(re.findall(r"\b(litekv_[a-z0-9_]+)\s*\(", text))
 
 
 def declared_symbols():
-    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
-    return sorted(set(re.findall(r"\b(litekv_[a-z0-9_]+)\s*\(", text)))
+    return sorted(_declared_in(HEADER) | _declared_in(PROFILE_HEADER))
+
+
+def test_product_header_holds_no_stateful_entry_point():
+    assert _declared_in(PROFILE_HEADER) == {"litekv_profile_next_decode"}
+    assert "litekv_profile_next_decode" not in _declared_in(HEADER)
 
 
 def test_header_declares_the_path():
