@@ -387,6 +387,49 @@ class ModelExecutor:
                     f"max_seq_len={mgr.max_seq_len}, free_pages={mgr.page_mgr.num_free_pages}")
         self.activate_paged_decode_batch(tuple(request_ids))
 
+    def prefill_alloc_kv_cache(self, max_prompt_len: int, actual_prompt_lens, b_req_idx,
+                               image_batch_size=None, debug_mode: bool = False):
+        """Static-batch prefill (:411-494, the entry ``generate_stream.py:155-174`` calls before
+        ``decode_alloc_kv_cache``): prompts padded to ``max_prompt_len`` rows each. Request
+        ``b_req_idx[i]`` gets pages for ``max_prompt_len`` tokens and the logical length
+        ``actual_prompt_lens[i]``; ``cur_select_index`` lists the slots of all ``max_prompt_len`` rows
+        of every request (the padding rows are stored too, as the reference does), ``b_start_loc`` is
+        ``i * max_prompt_len``. The first decode step then writes its token at position
+        ``actual_prompt_lens[i]``, over the first padding row, and attends ``actual + 1`` tokens,
+        which is what the reference's own worked example shows (:419-429: select index
+        ``start + len``). Its paged branch instead counts ``max_prompt_len`` tokens per request
+        (:450-455), so that a shorter prompt's first decode step appends behind the padding and
+        attends a padding row; that is not reproduced. Returns ``(cur_select_index, None)``."""
+        if image_batch_size is not None:
+            raise RuntimeError("image prompts are outside the paged attention path")
+        self._reset_paged_chunk_prefill_metadata()
+        max_prompt_len = int(max_prompt_len)
+        ids = tuple(int(r) for r in (b_req_idx.detach().cpu().tolist() if torch.is_tensor(b_req_idx) else b_req_idx))
+        lens = [int(n) for n in (actual_prompt_lens.detach().cpu().reshape(-1).tolist()
+                                 if torch.is_tensor(actual_prompt_lens) else actual_prompt_lens)]
+        if len(lens) != len(ids) or not ids:
+            raise ValueError("actual_prompt_lens and b_req_idx must name the same, non-empty batch")
+        if any(n < 1 or n > max_prompt_len for n in lens):
+            raise ValueError("prompt lengths must lie in [1, max_prompt_len]")
+        mgr = self.req_tokens_manager
+        made: list[int] = []
+        for req_idx, n in zip(ids, lens):
+            if not mgr.alloc_req(req_idx, n, max_prompt_len):
+                for done in made:
+                    mgr.free_req(done)
+                raise RuntimeError("Paged KV allocation failed during prefill")
+            made.append(req_idx)
+        padded = [max_prompt_len] * len(ids)
+        self._set_batch(ids, padded, padded, [mgr.slots(r, 0, max_prompt_len) for r in ids])
+        info = self.atten_info
+        info.b_seq_len = self._i64(lens)          # the prompts' own lengths, as the reference keeps them
+        info.max_actual_seq_len = max_prompt_len
+        if debug_mode:
+            print(f"context_num_tokens: {max_prompt_len * len(ids)}, max_prompt_len: {max_prompt_len},\n"
+                  f" cur_select_index: {info.cur_select_index},\n b_seq_len: {info.b_seq_len},\n"
+                  f" b_start_loc: {info.b_start_loc}")
+        return info.cur_select_index, None
+
     def decode_alloc_kv_cache(self, batch_size: int) -> torch.Tensor:
         """Static-batch decode step over the request ids cached at prefill time."""
         if len(self._paged_request_ids) != batch_size:

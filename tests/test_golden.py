@@ -93,3 +93,35 @@ def test_chunked_prefill_examples():
     assert [t is not None for t in tokens] == later["completed"]
     assert ex.seen["chunked"] and ex.seen["context"] == later["context_lengths"]
     assert ex.seen["chunk"] == later["chunk_lengths"]
+
+
+def test_static_batch_prefill_then_decode_select_indices():
+    """The worked example in the docstring of the reference's prefill_alloc_kv_cache: four padded
+    prompts, then two decode steps whose tokens land right behind each prompt's own length."""
+    ex = GOLDEN["static_batch_prefill"]
+    stride = ex["slots_per_request"]                 # one page per request reproduces the example's slot ranges
+    executor = ModelExecutor(num_layers=1, num_q_heads=2, num_kv_heads=1, head_dim=8, num_pages=4,
+                             max_seq_len=stride, max_requests=4, page_size=stride, device="cpu")
+    select, patches = executor.prefill_alloc_kv_cache(ex["max_prompt_len"], torch.tensor(ex["b_seq_len"]),
+                                                      torch.arange(4, dtype=torch.int32))
+    assert patches is None
+    info = executor.atten_info
+    assert select.tolist() == sum(ex["prefill_select_index"], [])
+    assert info.b_start_loc.tolist() == [i * ex["max_prompt_len"] for i in range(4)]
+    assert info.b_seq_len.tolist() == ex["b_seq_len"] and info.max_actual_seq_len == ex["max_prompt_len"]
+    assert info.b_req_idx.tolist() == [0, 1, 2, 3]
+    assert [p[0] * stride for p in map(executor.req_tokens_manager.request_pages, range(4))] == ex["start_index"]
+    for step in ex["decode_steps"]:
+        assert executor.decode_alloc_kv_cache(4).tolist() == step["cur_select_index"]
+        assert info.b_seq_len.tolist() == step["cur_b_seq_len"]
+    # a batch that does not fit gives the reference's error and leaves nothing allocated behind
+    executor.release_paged_requests()
+    small = ModelExecutor(num_layers=1, num_q_heads=2, num_kv_heads=1, head_dim=8, num_pages=2,
+                          max_seq_len=8, max_requests=4, page_size=4, device="cpu")
+    try:
+        small.prefill_alloc_kv_cache(8, [8, 3], [0, 1])
+    except RuntimeError as exc:
+        assert "Paged KV allocation failed during prefill" in str(exc)
+    else:
+        raise AssertionError("allocation beyond the pool did not fail")
+    assert small.kv_mem_manager.num_free_pages == 2

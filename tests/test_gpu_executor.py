@@ -296,3 +296,48 @@ def test_qkv_epilogue_then_attention_equals_separate_steps():
     out = attn.token_forward(qd, None, None, ex.atten_info, 0, SCALE)
     torch.cuda.synchronize()
     assert_attention_close(out, _oracle_decode(ex, qd, 0), "decode after fused epilogue")
+
+
+def test_static_batch_prefill_then_decode_equals_the_packed_flow():
+    """prefill_alloc_kv_cache (prompts padded to the longest) followed by decode_alloc_kv_cache
+    steps gives, on the prompts' own rows and on every decode step, what the packed no-pad flow
+    gives for the same prompts."""
+    print("executor: static batch (padded) vs packed flow", flush=True)
+    lens = [20, 7, 33]
+    longest = max(lens)
+    attn = Attention(HQ, HKV, D)
+    q, k, v = _qkv(sum(lens), 71)                        # the prompts' rows, packed
+    starts = np.concatenate([[0], np.cumsum(lens)[:-1]])
+    # --- packed flow
+    packed = _executor(layers=1)
+    ids_p = packed.reserve_paged_requests(lens, [n + 8 for n in lens])
+    packed.activate_paged_packed_prefill_batch(ids_p, lens)
+    out_p = attn.context_forward(q, k, v, packed.atten_info, 0, qk_scale=SCALE * LOG2E)
+    # --- static batch: the same rows at the head of each padded block, noise behind them
+    static = _executor(layers=1)
+    qs, ks, vs = _qkv(len(lens) * longest, 72)
+    for i, (s, n) in enumerate(zip(starts, lens)):
+        qs[i * longest:i * longest + n] = q[s:s + n]
+        ks[i * longest:i * longest + n] = k[s:s + n]
+        vs[i * longest:i * longest + n] = v[s:s + n]
+    select, _ = static.prefill_alloc_kv_cache(longest, torch.tensor(lens), torch.arange(len(lens), dtype=torch.int32))
+    assert select.numel() == len(lens) * longest
+    out_s = attn.context_forward(qs, ks, vs, static.atten_info, 0, qk_scale=SCALE * LOG2E)
+    torch.cuda.synchronize()
+    for i, (s, n) in enumerate(zip(starts, lens)):
+        diff = (out_s[i * longest:i * longest + n].float() - out_p[s:s + n].float()).abs().max()
+        assert float(diff) <= 1e-3, f"prompt {i}: {float(diff)}"
+    ref = c_oracle.varlen_prefill(to_np16(q), to_np16(k), to_np16(v), starts.astype(np.int32),
+                                  np.array(lens, dtype=np.int32), SCALE)
+    assert_attention_close(out_p, ref, "packed prefill")
+    # --- decode steps: the token goes behind each prompt's own length, over the padding row
+    for step in range(3):
+        qd, kd, vd = _qkv(len(lens), 80 + step)
+        packed.extend_paged_requests(ids_p)
+        o_p = attn.token_forward(qd, kd, vd, packed.atten_info, 0, SCALE)
+        static.decode_alloc_kv_cache(len(lens))
+        assert static.atten_info.b_seq_len.tolist() == [n + step + 1 for n in lens]
+        o_s = attn.token_forward(qd, kd, vd, static.atten_info, 0, SCALE)
+        torch.cuda.synchronize()
+        assert float((o_s.float() - o_p.float()).abs().max()) <= 1e-3, f"decode step {step}"
+        assert_attention_close(o_s, _oracle_decode(static, qd, 0), f"static batch decode step {step}")
