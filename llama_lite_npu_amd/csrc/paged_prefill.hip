@@ -712,10 +712,15 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
         float *po = prefix.part_o + cell * kHeadDim + 4 * g;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          *(float4_t *)(po + 16 * j) = float4_t{acc[j][u][0] * inv, acc[j][u][1] * inv,
-                                                acc[j][u][2] * inv, acc[j][u][3] * inv};
+          // read once, by the merge launch: streaming stores (see store_state in paged_decode.hip)
+          __builtin_nontemporal_store(float4_t{acc[j][u][0] * inv, acc[j][u][1] * inv,
+                                               acc[j][u][2] * inv, acc[j][u][3] * inv},
+                                      (float4_t *)(po + 16 * j));
         }
-        if (g == 0) prefix.part_lse[cell] = (m_run[u] + fast_log2(dsum[u][0])) * 0.6931471805599453f;
+        if (g == 0) {
+          __builtin_nontemporal_store((m_run[u] + fast_log2(dsum[u][0])) * 0.6931471805599453f,
+                                      prefix.part_lse + cell);
+        }
       }
       continue;
     }
@@ -780,8 +785,10 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
   const int prefix_keys = shared_pages * kPageSize;
   const int col_blocks = (batch * group + 16 * kWgColTiles - 1) / (16 * kWgColTiles);
   LITEKV_REQUIRE(col_blocks <= 65535, "%s: batch %d too large", what, batch);
-  // Enough key slices for about one workgroup per compute unit, at least 128 keys each.
-  int splits = 256 / (num_kv_heads * col_blocks);
+  // Enough key slices for a workgroup on every other compute unit, at least 128 keys each: every
+  // slice is one more partial row per (sequence, head) to write here and to read in the merge
+  // (C4, per layer: 8 slices 47.1 us, 4 slices 44.3 us, 2 slices 49.3 us).
+  int splits = 128 / (num_kv_heads * col_blocks);
   splits = splits < 1 ? 1 : (splits > kMaxPrefixSplits ? kMaxPrefixSplits : splits);
   const int max_by_keys = (prefix_keys + 127) / 128;
   splits = splits < max_by_keys ? splits : max_by_keys;
