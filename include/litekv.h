@@ -257,6 +257,11 @@ size_t litekv_paged_decode_balanced_workspace_bytes(int32_t batch, int32_t num_q
 
 size_t litekv_decode_plan_bytes(int32_t batch, int32_t block_table_stride,
                                 int32_t num_kv_heads, int32_t chunks);
+/* The same for a pool whose pages hold page_size (16, 32 or 64) tokens: the plan
+ * lists 16-token pages, page_size / 16 per block-table entry.
+ * litekv_decode_plan_bytes is the page_size 16 case. 0 for another page_size. */
+size_t litekv_decode_plan_bytes_paged(int32_t batch, int32_t block_table_stride,
+                                      int32_t num_kv_heads, int32_t chunks, int32_t page_size);
 
 int litekv_decode_plan(const int32_t *block_table, int32_t block_table_stride,
                        const int32_t *seq_lens, int32_t batch, int32_t num_kv_heads,

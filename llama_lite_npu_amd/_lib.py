@@ -87,6 +87,7 @@ SIGNATURES = {
     "litekv_paged_decode_balanced_chunks": (c_int32, [c_int32]),
     "litekv_paged_decode_balanced_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "litekv_decode_plan_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
+    "litekv_decode_plan_bytes_paged": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32]),
     "litekv_decode_plan": (
         c_int32,
         [c_void_p, c_int32, c_void_p, c_int32, c_int32, c_int32, c_int64, c_int32, c_void_p, c_size_t,

@@ -365,6 +365,13 @@ __device__ __forceinline__ int clamp_page(int pid, int num_pages) {
   return pid < 0 ? 0 : (pid >= num_pages ? num_pages - 1 : pid);
 }
 
+// Pools whose pages hold 16 << shift tokens: the kernels keep working on 16-token pages, and the
+// 16-token page j of a sequence is part j % (1 << shift) of the sequence's page j >> shift, whose
+// tokens are contiguous in the pool. `entry` is the block-table entry of that page.
+__device__ __forceinline__ int sub_page_id(int entry, int j, int shift, int num_pages) {
+  return (clamp_page(entry, num_pages) << shift) + (j & ((1 << shift) - 1));
+}
+
 // This lane's parts of the step's new K and V rows (fp16, head h of one sequence): the pieces
 // that sit where the lane's page registers hold the token's row (see PageRegs / PageRegsFp8).
 template <bool FP8>
@@ -407,7 +414,7 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
     const half_t *__restrict__ v_new, int64_t k_new_stride, int64_t v_new_stride,
     half_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_lse,
     int32_t num_q_heads, int32_t num_kv_heads, int32_t group, int32_t max_splits,
-    int32_t min_pages_per_split, int32_t num_pages, float scale_log2) {
+    int32_t min_pages_per_split, int32_t num_pages, int32_t page_shift, float scale_log2) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int n = lane & 15;   // query head inside the group (column of S^T)
@@ -473,7 +480,10 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
   // use. Requests past the range still issue their loads (16 bytes of its last page), which keeps
   // the number of vector loads in flight a compile-time constant, so each wait names exactly the
   // page it needs and never drains the younger prefetches.
-  auto page_id = [&](int p) { return clamp_page(table[p < p1 ? p : p1 - 1], num_pages); };
+  auto page_id = [&](int p) {
+    const int pp = p < p1 ? p : p1 - 1;
+    return sub_page_id(table[pp >> page_shift], pp, page_shift, num_pages);
+  };
   int pid_next = page_id(p0);
   auto request = [&](int p, Page &r) {
     const int64_t page_off = (int64_t)pid_next * kPageSize * row_stride;
@@ -723,9 +733,12 @@ __host__ __device__ __forceinline__ int plan_entries_offset(int batch) {
 // into and records which chunks the sequence spans; block 0 also writes the meta words and
 // marks the chunks past the end of the line as empty.
 __global__ __launch_bounds__(256) void decode_plan_kernel(
-    const int32_t *__restrict__ block_table, int32_t bt_stride,
+    const int32_t *__restrict__ block_table, int32_t table_stride, int32_t bt_stride,
     const int32_t *__restrict__ seq_lens, int32_t batch, int32_t num_kv_heads, int32_t chunks,
-    int32_t entry_stride, int32_t num_pages, int32_t skip, int32_t *__restrict__ plan) {
+    int32_t entry_stride, int32_t num_pages, int32_t page_shift, int32_t skip,
+    int32_t *__restrict__ plan) {
+  // table_stride: entries per block-table row; bt_stride, skip: the same row and the shared
+  // prefix counted in 16-token pages (entries << page_shift)
   __shared__ int red[4][3];
   const int b = blockIdx.x;
   const int tid = threadIdx.x;
@@ -796,13 +809,14 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
     plan[plan_seq_info_offset() + 2 * b + 1] =
         my_pages > 0 ? chunk_of(before + my_pages - 1) - c_first + 1 : 0;
   }
-  const int32_t *row = block_table + (int64_t)b * bt_stride + skip;
+  const int32_t *row = block_table + (int64_t)b * table_stride;
   for (int p = tid; p < my_pages; p += 256) {
     const int f = before + p;
     const int c = chunk_of(f);
     const int first = chunk_start(c);
     int32_t *e = entries + (int64_t)c * entry_stride;
-    e[kEntryHeader + (f - first)] = clamp_page(row[p], num_pages);
+    e[kEntryHeader + (f - first)] =
+        sub_page_id(row[(p + skip) >> page_shift], p + skip, page_shift, num_pages);
     if (f == first) {
       e[0] = f;
       e[1] = chunk_start(c + 1);
@@ -1269,14 +1283,19 @@ struct DecodeArgs {
   int64_t k_new_stride = 0, v_new_stride = 0;
 };
 
+// log2(page_size / 16) for the page sizes the kernels take (16, 32, 64 tokens), or -1.
+static int page_shift_of(int32_t page_size) {
+  return page_size == 16 ? 0 : page_size == 32 ? 1 : page_size == 64 ? 2 : -1;
+}
+
 // Checks shared by every decode entry point; `need_inputs` is false for the merge-only calls.
 static int validate_decode(const char *what, const DecodeArgs &a, size_t workspace_needed,
                            bool need_inputs) {
   LITEKV_REQUIRE(a.batch >= 0 && a.batch <= 65535, "%s: batch %d out of [0, 65535]", what, a.batch);
   LITEKV_REQUIRE(a.head_dim == kHeadDim, "%s: head_dim %d unsupported (only %d)", what, a.head_dim,
                  kHeadDim);
-  LITEKV_REQUIRE(a.page_size == kPageSize, "%s: page_size %d unsupported (only %d)", what,
-                 a.page_size, kPageSize);
+  LITEKV_REQUIRE(page_shift_of(a.page_size) >= 0, "%s: page_size %d unsupported (16, 32 or 64)",
+                 what, a.page_size);
   LITEKV_REQUIRE(a.num_q_heads > 0 && a.num_q_heads <= 65535, "%s: num_q_heads %d out of range",
                  what, a.num_q_heads);
   if (a.batch == 0) return LITEKV_OK;
@@ -1303,8 +1322,10 @@ static int validate_decode(const char *what, const DecodeArgs &a, size_t workspa
                    "%s: q and kv_pool must be 16-byte aligned", what);
     LITEKV_REQUIRE(a.block_table_stride >= 1, "%s: block_table_stride %d < 1", what,
                    a.block_table_stride);
-    LITEKV_REQUIRE(a.num_pages >= 1 && a.num_pages <= 0x7fffffffLL / kPageSize,
+    LITEKV_REQUIRE(a.num_pages >= 1 && a.num_pages <= 0x7fffffffLL / a.page_size,
                    "%s: num_pages %lld out of range", what, (long long)a.num_pages);
+    LITEKV_REQUIRE((int64_t)a.block_table_stride * (a.page_size / kPageSize) <= 0x7fffffffLL / 4,
+                   "%s: block_table_stride %d too large", what, a.block_table_stride);
   }
   return LITEKV_OK;
 }
@@ -1314,6 +1335,13 @@ static int validate_decode(const char *what, const DecodeArgs &a, size_t workspa
 static size_t splits_workspace_bytes(int64_t batch, int64_t hq, int64_t d, int64_t s) {
   if (batch <= 0 || hq <= 0 || d <= 0 || s <= 1) return 0;
   return (size_t)(batch * hq * s * (d + 1)) * sizeof(float);
+}
+
+// The kernels count in 16-token pages: the caller's lower bound on a split, given in pages of the
+// pool, in those (saturating).
+static int32_t min_16_token_pages(int32_t min_pages_per_split, int32_t page_size) {
+  const int64_t m = (int64_t)min_pages_per_split * (page_size / kPageSize);
+  return (int32_t)(m < 0x7fffffffLL ? m : 0x7fffffffLL);
 }
 
 static int check_split_plan(const char *what, int32_t max_splits, int32_t min_pages_per_split) {
@@ -1368,8 +1396,9 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
                        a.block_table, a.block_table_stride, a.seq_lens,
                        static_cast<const half_t *>(a.k_new), static_cast<const half_t *>(a.v_new),
                        a.k_new_stride, a.v_new_stride, static_cast<half_t *>(a.out), part_o, part_lse,
-                       a.num_q_heads, a.num_kv_heads, group, max_splits, min_pages_per_split,
-                       (int32_t)a.num_pages, a.softmax_scale * kLog2e);
+                       a.num_q_heads, a.num_kv_heads, group, max_splits,
+                       min_16_token_pages(min_pages_per_split, a.page_size), (int32_t)a.num_pages,
+                       page_shift_of(a.page_size), a.softmax_scale * kLog2e);
   };
   if (fp8_scales != nullptr) {
     if (a.k_new != nullptr) {
@@ -1402,7 +1431,7 @@ static int launch_merge(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   hipLaunchKernelGGL(paged_decode_merge_kernel, dim3((unsigned)a.num_q_heads, (unsigned)a.batch),
                      dim3(kWave), 0, static_cast<hipStream_t>(a.stream), a.seq_lens,
                      static_cast<half_t *>(a.out), part_o, part_lse, a.num_q_heads, max_splits,
-                     min_pages_per_split);
+                     min_16_token_pages(min_pages_per_split, a.page_size));
   return check_launch(what);
 }
 
@@ -1434,6 +1463,7 @@ static size_t prefix_workspace_bytes(int64_t batch, int64_t hq, int64_t d, int64
          (size_t)(kMaxPrefixSplits * batch * hq * (d + 1)) * sizeof(float);
 }
 
+// bt_stride: block-table entries per row times page_size / 16
 static size_t plan_bytes_for(int64_t batch, int64_t bt_stride, int64_t hkv, int64_t chunks) {
   if (batch <= 0 || bt_stride <= 0 || hkv <= 0 || chunks <= 0) return 0;
   const int64_t words = plan_entries_offset((int)batch) +
@@ -1491,15 +1521,26 @@ extern "C" size_t litekv_decode_plan_bytes(int32_t batch, int32_t block_table_st
   return litekv::plan_bytes_for(batch, block_table_stride, num_kv_heads, chunks);
 }
 
+extern "C" size_t litekv_decode_plan_bytes_paged(int32_t batch, int32_t block_table_stride,
+                                                 int32_t num_kv_heads, int32_t chunks,
+                                                 int32_t page_size) {
+  const int shift = litekv::page_shift_of(page_size);
+  if (shift < 0) return 0;
+  return litekv::plan_bytes_for(batch, (int64_t)block_table_stride << shift, num_kv_heads, chunks);
+}
+
 namespace litekv {
 static int launch_plan(const char *what, const int32_t *block_table, int32_t block_table_stride,
                        const int32_t *seq_lens, int32_t batch, int32_t num_kv_heads,
                        int32_t page_size, int64_t num_pages, int32_t chunks, int32_t shared_pages,
                        void *plan, size_t plan_bytes, void *stream) {
   LITEKV_REQUIRE(batch >= 0 && batch <= 65535, "%s: batch %d out of [0, 65535]", what, batch);
-  LITEKV_REQUIRE(page_size == kPageSize, "%s: page_size %d unsupported (only %d)", what, page_size,
-                 kPageSize);
-  int rc = check_chunks(what, batch, block_table_stride, num_kv_heads, chunks);
+  const int shift = page_shift_of(page_size);
+  LITEKV_REQUIRE(shift >= 0, "%s: page_size %d unsupported (16, 32 or 64)", what, page_size);
+  LITEKV_REQUIRE(block_table_stride >= 1 && block_table_stride <= (0x7fffffff >> 4),
+                 "%s: block_table_stride %d out of range", what, block_table_stride);
+  const int32_t sub_stride = block_table_stride << shift;  // a row in 16-token pages
+  int rc = check_chunks(what, batch, sub_stride, num_kv_heads, chunks);
   if (rc != LITEKV_OK) return rc;
   LITEKV_REQUIRE(shared_pages >= 0 && shared_pages <= block_table_stride,
                  "%s: shared_pages %d out of [0, block_table_stride %d]", what, shared_pages,
@@ -1510,16 +1551,16 @@ static int launch_plan(const char *what, const int32_t *block_table, int32_t blo
   }
   LITEKV_REQUIRE(block_table && seq_lens && plan, "%s: null pointer", what);
   LITEKV_REQUIRE(aligned16(plan), "%s: plan must be 16-byte aligned", what);
-  LITEKV_REQUIRE(num_pages >= 1 && num_pages <= 0x7fffffffLL / kPageSize,
+  LITEKV_REQUIRE(num_pages >= 1 && num_pages <= 0x7fffffffLL / page_size,
                  "%s: num_pages %lld out of range", what, (long long)num_pages);
-  const size_t need = plan_bytes_for(batch, block_table_stride, num_kv_heads, chunks);
+  const size_t need = plan_bytes_for(batch, sub_stride, num_kv_heads, chunks);
   LITEKV_REQUIRE(plan_bytes >= need, "%s: plan buffer of %zu bytes needed, got %zu", what, need,
                  plan_bytes);
   hipLaunchKernelGGL(decode_plan_kernel, dim3((unsigned)batch), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), block_table, block_table_stride, seq_lens,
-                     batch, num_kv_heads, chunks,
-                     plan_entry_stride(batch, block_table_stride, chunks), (int32_t)num_pages,
-                     shared_pages, static_cast<int32_t *>(plan));
+                     static_cast<hipStream_t>(stream), block_table, block_table_stride, sub_stride,
+                     seq_lens, batch, num_kv_heads, chunks,
+                     plan_entry_stride(batch, sub_stride, chunks), (int32_t)num_pages, shift,
+                     shared_pages << shift, static_cast<int32_t *>(plan));
   return check_launch(what);
 }
 }  // namespace litekv
@@ -1560,7 +1601,12 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
                            int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
                            int64_t num_pages, int32_t block_table_stride, int32_t chunks,
                            int32_t shared_pages, float softmax_scale, void *stream) {
-  int rc = check_chunks(what, batch, block_table_stride, num_kv_heads, chunks);
+  const int shift = page_shift_of(page_size);
+  LITEKV_REQUIRE(shift >= 0, "%s: page_size %d unsupported (16, 32 or 64)", what, page_size);
+  LITEKV_REQUIRE(block_table_stride >= 1 && block_table_stride <= (0x7fffffff >> 4),
+                 "%s: block_table_stride %d out of range", what, block_table_stride);
+  const int32_t sub_stride = block_table_stride << shift;  // a block-table row in 16-token pages
+  int rc = check_chunks(what, batch, sub_stride, num_kv_heads, chunks);
   if (rc != LITEKV_OK) return rc;
   static const int32_t dummy_table = 0;  // the decode kernel reads page ids from the plan
   DecodeArgs a{q, q_batch_stride, kv_pool, block_table ? block_table : &dummy_table,
@@ -1580,7 +1626,7 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   }
   LITEKV_REQUIRE(plan != nullptr && aligned16(plan), "%s: plan must be a 16-byte aligned buffer",
                  what);
-  const size_t need = plan_bytes_for(batch, block_table_stride, num_kv_heads, chunks);
+  const size_t need = plan_bytes_for(batch, sub_stride, num_kv_heads, chunks);
   LITEKV_REQUIRE(plan_bytes >= need, "%s: plan buffer of %zu bytes needed, got %zu", what, need,
                  plan_bytes);
   LITEKV_REQUIRE((k_new == nullptr) == (v_new == nullptr), "%s: k_new and v_new go together", what);
@@ -1603,8 +1649,8 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   if (shared_pages > 0) {
     LITEKV_REQUIRE(block_table != nullptr, "%s: block_table is null", what);
     rc = launch_shared_prefix(q, q_batch_stride, kv_pool, fp8_scales, block_table, batch, num_q_heads,
-                              num_kv_heads, num_pages, shared_pages, pre_o, pre_lse, softmax_scale,
-                              static_cast<hipStream_t>(stream), &pre_splits);
+                              num_kv_heads, num_pages, shared_pages, shift, pre_o, pre_lse,
+                              softmax_scale, static_cast<hipStream_t>(stream), &pre_splits);
     if (rc != LITEKV_OK) return rc;
   }
   const unsigned wgs = (unsigned)((chunks + s.replicas - 1) / s.replicas);
@@ -1619,9 +1665,9 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
                           static_cast<uint8_t *>(kv_pool), fp8_scales, seq_lens,
                           static_cast<const int32_t *>(plan), static_cast<const half_t *>(k_new),
                           static_cast<const half_t *>(v_new), k_new_stride, v_new_stride,
-                          static_cast<half_t *>(out), part_o, part_lse, block_table_stride, batch,
+                          static_cast<half_t *>(out), part_o, part_lse, sub_stride, batch,
                           num_q_heads, num_kv_heads, num_q_heads / num_kv_heads, s.heads_per_wg,
-                          s.replicas, chunks, shared_pages, softmax_scale * kLog2e);
+                          s.replicas, chunks, shared_pages << shift, softmax_scale * kLog2e);
   } else {
     hipExtLaunchKernelGGL((paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, false>), grid, block, 0,
                           static_cast<hipStream_t>(stream), ev0, ev1, 0,
@@ -1629,9 +1675,9 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
                           static_cast<half_t *>(kv_pool), fp8_scales, seq_lens,
                           static_cast<const int32_t *>(plan), static_cast<const half_t *>(k_new),
                           static_cast<const half_t *>(v_new), k_new_stride, v_new_stride,
-                          static_cast<half_t *>(out), part_o, part_lse, block_table_stride, batch,
+                          static_cast<half_t *>(out), part_o, part_lse, sub_stride, batch,
                           num_q_heads, num_kv_heads, num_q_heads / num_kv_heads, s.heads_per_wg,
-                          s.replicas, chunks, shared_pages, softmax_scale * kLog2e);
+                          s.replicas, chunks, shared_pages << shift, softmax_scale * kLog2e);
   }
   rc = check_launch(what);
   if (rc != LITEKV_OK) return rc;
@@ -1639,7 +1685,7 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   // four-wavefront merge of long rows (more than 16 pieces, never with a shared prefix) is only
   // launched where such a row can exist; the other wavefronts of a workgroup would leave at once
   // and only cost their dispatch (C4: 9.9 -> 7 us).
-  const int max_pieces = chunks < block_table_stride ? chunks : block_table_stride;
+  const int max_pieces = chunks < sub_stride ? chunks : sub_stride;
   const int merge_waves = (pre_splits == 0 && max_pieces > 16) ? kMergeWaves : 1;
   // Sequences inside one chunk were written by the decode kernel; at most chunks - 1 sequences
   // cross a chunk boundary. A batch of twice as many is merged by boundary (B 1024 of up to 40
@@ -1661,8 +1707,7 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
                      dim3(merge_waves * kWave), 0,
                      static_cast<hipStream_t>(stream), static_cast<const int32_t *>(plan), seq_lens,
                      static_cast<half_t *>(out), part_o, part_lse, pre_o, pre_lse, pre_splits,
-                     batch, num_q_heads, by_boundary ? 1 : 0, block_table_stride, chunks,
-                     merge_heads);
+                     batch, num_q_heads, by_boundary ? 1 : 0, sub_stride, chunks, merge_heads);
   return check_launch("paged_decode_balanced_merge");
 }
 }  // namespace litekv

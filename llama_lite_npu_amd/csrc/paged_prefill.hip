@@ -65,6 +65,7 @@ struct PagedSource {
   int32_t num_kv_heads;
   int32_t num_pages;
   const float *scales;          // fp8 pool: value = code * scale, K heads then V heads
+  int32_t page_shift;           // pages of 16 << page_shift tokens
 };
 // Shared-prefix decode (mode kSharedPrefix): the columns are (sequence, query head) pairs of one
 // decode step, the keys are a slice of the pages every sequence starts with, and the result is
@@ -201,6 +202,13 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   const int32_t *table =
       PAGED ? paged.block_table + (SHARED ? 0 : (int64_t)b * paged.bt_stride) : nullptr;
   const int last_page = last_key >> 4;
+  // The kernel works on 16-token pages: page j of them is part j % (1 << page_shift) of the
+  // sequence's page j >> page_shift, whose tokens are contiguous in the pool.
+  auto page_of = [&](int pidx) {
+    int pid = table[pidx >> paged.page_shift];
+    pid = pid < 0 ? 0 : (pid >= paged.num_pages ? paged.num_pages - 1 : pid);
+    return (pid << paged.page_shift) + (pidx & ((1 << paged.page_shift) - 1));
+  };
 
   // Starts the loads of tile kt into its LDS half. The instruction is written as asm so that the
   // compiler does not make later LDS reads of the *other* half wait for it; the wait is the
@@ -212,8 +220,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       // lane l: row l / 4 of the wavefront's page, codes 32 * (l % 4) .. +31 of the head's row
       int pidx = (tile0 + kt) * 4 + wave;
       pidx = pidx < last_page ? pidx : last_page;
-      int pid = table[pidx];
-      pid = pid < 0 ? 0 : (pid >= paged.num_pages ? paged.num_pages - 1 : pid);
+      const int pid = page_of(pidx);
       int tok = row0 + (lane >> 2);
       tok = tok < last_key ? tok : last_key;  // rows past the last key re-read it
       const int src_row = tok - pidx * kPageSize;
@@ -232,8 +239,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     if (PAGED) {
       int pidx = (tile0 + kt) * 4 + wave;
       pidx = pidx < last_page ? pidx : last_page;
-      int pid = table[pidx];
-      pid = pid < 0 ? 0 : (pid >= paged.num_pages ? paged.num_pages - 1 : pid);
+      const int pid = page_of(pidx);
       kbase = (const char *)paged.kv + (int64_t)pid * ((int64_t)kPageSize * k_pitch);
       vbase = kbase;
       src0 = pidx * kPageSize;
@@ -508,8 +514,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   auto tile_bases = [&](int kt) {
     const int row0 = (tile0 + kt) * kKvTile + 16 * wave;
     if (PAGED) {
-      int pid = table[(tile0 + kt) * 4 + wave];
-      pid = pid < 0 ? 0 : (pid >= paged.num_pages ? paged.num_pages - 1 : pid);
+      const int pid = page_of((tile0 + kt) * 4 + wave);
       next_kbase = (const char *)paged.kv + (int64_t)pid * ((int64_t)kPageSize * k_pitch);
       next_vbase = next_kbase;
     } else {
@@ -774,15 +779,15 @@ static PrefillShape prefill_shape(int group, int max_q_len) {
 int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_pool,
                          const float *fp8_scales, const int32_t *block_table, int32_t batch, int32_t num_q_heads,
                          int32_t num_kv_heads, int64_t num_pages, int32_t shared_pages,
-                         float *part_o, float *part_lse, float softmax_scale, hipStream_t stream,
-                         int *splits_out) {
+                         int32_t page_shift, float *part_o, float *part_lse, float softmax_scale,
+                         hipStream_t stream, int *splits_out) {
   const char *what = "shared_prefix";
   const int group = num_q_heads / num_kv_heads;
   LITEKV_REQUIRE(group >= 1 && group <= 16, "%s: %d query heads per kv head unsupported", what, group);
   LITEKV_REQUIRE(num_kv_heads <= 1024, "%s: num_kv_heads %d > 1024", what, num_kv_heads);
   LITEKV_REQUIRE(shared_pages >= 1 && shared_pages <= (1 << 24), "%s: shared_pages %d out of range",
                  what, shared_pages);
-  const int prefix_keys = shared_pages * kPageSize;
+  const int prefix_keys = (shared_pages << page_shift) * kPageSize;
   const int col_blocks = (batch * group + 16 * kWgColTiles - 1) / (16 * kWgColTiles);
   LITEKV_REQUIRE(col_blocks <= 65535, "%s: batch %d too large", what, batch);
   // Enough key slices for a workgroup on every other compute unit, at least 128 keys each: every
@@ -796,7 +801,7 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
   keys_per_split = (keys_per_split + kKvTile - 1) / kKvTile * kKvTile;
   splits = (prefix_keys + keys_per_split - 1) / keys_per_split;
   PagedSource paged{static_cast<const half_t *>(kv_pool), block_table, 0, num_kv_heads,
-                    (int32_t)num_pages, fp8_scales};
+                    (int32_t)num_pages, fp8_scales, page_shift};
   PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
   PrefixTask task{part_o, part_lse, q_batch_stride, batch, num_q_heads, prefix_keys, keys_per_split};
   const dim3 grid((unsigned)num_kv_heads, (unsigned)col_blocks, (unsigned)splits);
@@ -832,8 +837,8 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
   int rc = validate_prefill(what, q, q_token_stride, out, out_token_stride, batch, num_q_heads,
                             num_kv_heads, head_dim, max_q_len);
   if (rc != LITEKV_OK) return rc;
-  LITEKV_REQUIRE(page_size == kPageSize, "%s: page_size %d unsupported (only %d)", what, page_size,
-                 kPageSize);
+  const int page_shift = page_size == 16 ? 0 : page_size == 32 ? 1 : page_size == 64 ? 2 : -1;
+  LITEKV_REQUIRE(page_shift >= 0, "%s: page_size %d unsupported (16, 32 or 64)", what, page_size);
   if (batch == 0 || max_q_len == 0) {
     clear_error();
     return LITEKV_OK;
@@ -842,11 +847,11 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
   LITEKV_REQUIRE(!fp8 || kv_scales, "%s: null pointer (kv_scales)", what);
   LITEKV_REQUIRE(aligned16(kv_pool), "%s: kv_pool must be 16-byte aligned", what);
   LITEKV_REQUIRE(block_table_stride >= 1, "%s: block_table_stride %d < 1", what, block_table_stride);
-  LITEKV_REQUIRE(num_pages >= 1 && num_pages <= 0x7fffffffLL / kPageSize,
+  LITEKV_REQUIRE(num_pages >= 1 && num_pages <= 0x7fffffffLL / page_size,
                  "%s: num_pages %lld out of range", what, (long long)num_pages);
   LITEKV_REQUIRE(num_kv_heads <= 1024, "%s: num_kv_heads %d > 1024", what, num_kv_heads);
   PagedSource paged{static_cast<const half_t *>(kv_pool), block_table, block_table_stride,
-                    num_kv_heads, (int32_t)num_pages, kv_scales};
+                    num_kv_heads, (int32_t)num_pages, kv_scales, page_shift};
   PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
   const int group = num_q_heads / num_kv_heads;
   const PrefillShape s = prefill_shape(group, max_q_len);

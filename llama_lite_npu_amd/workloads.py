@@ -47,10 +47,12 @@ class DecodeCase:
     q: torch.Tensor                     # [B, Hq, D] fp16
     k_new: torch.Tensor                 # [B, Hkv, D] fp16
     v_new: torch.Tensor
-    kv_pool: torch.Tensor               # [num_pages*16, 2*Hkv, D] fp16
+    kv_pool: torch.Tensor               # [num_pages*page_size, 2*Hkv, D] fp16
     softmax_scale: float = 1.0 / math.sqrt(HEAD_DIM)
     num_splits: Optional[int] = None
     extra: dict = field(default_factory=dict)
+    page_size: int = PAGE_SIZE
+    head_dim: int = HEAD_DIM
 
     @property
     def batch(self) -> int:
@@ -58,14 +60,14 @@ class DecodeCase:
 
     @property
     def tok_bytes(self) -> int:
-        return 2 * self.num_kv_heads * HEAD_DIM * 2
+        return 2 * self.num_kv_heads * self.head_dim * 2
 
     def decode_bytes(self) -> int:
         """Algorithmic bytes of one decode-attention launch: K/V of every attended token,
         q and out rows, the block-table entries and the lengths."""
         toks = int(self.seq_lens.sum())
-        pages = int(((self.seq_lens + PAGE_SIZE - 1) // PAGE_SIZE).sum())
-        return (toks * self.tok_bytes + 2 * self.batch * self.num_q_heads * HEAD_DIM * 2
+        pages = int(((self.seq_lens + self.page_size - 1) // self.page_size).sum())
+        return (toks * self.tok_bytes + 2 * self.batch * self.num_q_heads * self.head_dim * 2
                 + pages * 4 + self.batch * 4)
 
     def append_bytes(self) -> int:
@@ -79,15 +81,15 @@ class DecodeCase:
         fill = {}
         pages = 0
         for b, n in enumerate(lens):
-            n_pages = (n + PAGE_SIZE - 1) // PAGE_SIZE
+            n_pages = (n + self.page_size - 1) // self.page_size
             pages += n_pages
             ids = table[b, :n_pages].tolist()
             for j, pid in enumerate(ids):
-                used = min(PAGE_SIZE, n - j * PAGE_SIZE)
+                used = min(self.page_size, n - j * self.page_size)
                 if used > fill.get(pid, 0):
                     fill[pid] = used
         toks = sum(fill.values())
-        return (toks * self.tok_bytes + 2 * self.batch * self.num_q_heads * HEAD_DIM * 2
+        return (toks * self.tok_bytes + 2 * self.batch * self.num_q_heads * self.head_dim * 2
                 + pages * 4 + self.batch * 4)
 
     def to(self, device) -> "DecodeCase":
@@ -119,10 +121,10 @@ def table_from_lists(page_lists, max_blocks: Optional[int] = None) -> torch.Tens
 def make_decode_case(name: str, seed: int, context_lens: Sequence[int], num_q_heads: int,
                      num_kv_heads: int, num_pages: Optional[int] = None, slack: float = 0.10,
                      device="cpu", num_splits: Optional[int] = None,
-                     page_lists=None) -> DecodeCase:
+                     page_lists=None, page_size: int = PAGE_SIZE, head_dim: int = HEAD_DIM) -> DecodeCase:
     ctx = torch.tensor(list(context_lens), dtype=torch.int32)
     seq = ctx + 1
-    pages = ((seq + PAGE_SIZE - 1) // PAGE_SIZE).tolist()
+    pages = ((seq + page_size - 1) // page_size).tolist()
     if page_lists is None:
         if num_pages is None:
             num_pages = int(math.ceil(sum(pages) * (1.0 + slack)))
@@ -131,16 +133,16 @@ def make_decode_case(name: str, seed: int, context_lens: Sequence[int], num_q_he
     table = table_from_lists(page_lists)
     b = len(pages)
     slot = torch.tensor(
-        [int(page_lists[i][int(ctx[i]) // PAGE_SIZE]) * PAGE_SIZE + int(ctx[i]) % PAGE_SIZE for i in range(b)],
+        [int(page_lists[i][int(ctx[i]) // page_size]) * page_size + int(ctx[i]) % page_size for i in range(b)],
         dtype=torch.int32)
     return DecodeCase(
         name=name, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads, context_lens=ctx, seq_lens=seq,
         block_table=table, slot_mapping=slot, num_pages=num_pages,
-        q=_randn_half((b, num_q_heads, HEAD_DIM), seed + 2, device),
-        k_new=_randn_half((b, num_kv_heads, HEAD_DIM), seed + 3, device),
-        v_new=_randn_half((b, num_kv_heads, HEAD_DIM), seed + 4, device),
-        kv_pool=_randn_half((num_pages * PAGE_SIZE, 2 * num_kv_heads, HEAD_DIM), seed + 5, device),
-        num_splits=num_splits,
+        q=_randn_half((b, num_q_heads, head_dim), seed + 2, device),
+        k_new=_randn_half((b, num_kv_heads, head_dim), seed + 3, device),
+        v_new=_randn_half((b, num_kv_heads, head_dim), seed + 4, device),
+        kv_pool=_randn_half((num_pages * page_size, 2 * num_kv_heads, head_dim), seed + 5, device),
+        softmax_scale=1.0 / math.sqrt(head_dim), num_splits=num_splits, page_size=page_size, head_dim=head_dim,
     ).to(device)
 
 
@@ -227,6 +229,8 @@ class PrefillCase:
     v: torch.Tensor
     kv_pool: torch.Tensor
     softmax_scale: float = 1.0 / math.sqrt(HEAD_DIM)
+    page_size: int = PAGE_SIZE
+    head_dim: int = HEAD_DIM
 
     @property
     def batch(self) -> int:
@@ -241,12 +245,12 @@ class PrefillCase:
         4 * Hq * D * ctx * q for the rectangular history part."""
         l = self.seq_lens.to(torch.int64)
         c = self.context_lens.to(torch.int64)
-        return int((2 * self.num_q_heads * HEAD_DIM * (l * (l + 1) + 2 * c * l)).sum())
+        return int((2 * self.num_q_heads * self.head_dim * (l * (l + 1) + 2 * c * l)).sum())
 
     def min_bytes(self) -> int:
         t = int(self.seq_lens.sum()) + int(self.context_lens.sum())
         tq = int(self.seq_lens.sum())
-        return 2 * tq * self.num_q_heads * HEAD_DIM * 2 + t * 2 * self.num_kv_heads * HEAD_DIM * 2
+        return 2 * tq * self.num_q_heads * self.head_dim * 2 + t * 2 * self.num_kv_heads * self.head_dim * 2
 
     def to(self, device) -> "PrefillCase":
         kw = dict(self.__dict__)
@@ -258,11 +262,11 @@ class PrefillCase:
 
 def make_prefill_case(name: str, seed: int, seq_lens: Sequence[int], num_q_heads: int, num_kv_heads: int,
                       context_lens: Optional[Sequence[int]] = None, device="cpu",
-                      slack: float = 0.10) -> PrefillCase:
+                      slack: float = 0.10, page_size: int = PAGE_SIZE, head_dim: int = HEAD_DIM) -> PrefillCase:
     ql = torch.tensor(list(seq_lens), dtype=torch.int32)
     ctx = torch.zeros_like(ql) if context_lens is None else torch.tensor(list(context_lens), dtype=torch.int32)
     total = ql + ctx
-    pages = ((total + PAGE_SIZE - 1) // PAGE_SIZE).tolist()
+    pages = ((total + page_size - 1) // page_size).tolist()
     num_pages = int(math.ceil(sum(pages) * (1.0 + slack))) + 1
     lists = assign_pages(pages, num_pages, seed + 1)
     table = table_from_lists(lists)
@@ -271,16 +275,17 @@ def make_prefill_case(name: str, seed: int, seq_lens: Sequence[int], num_q_heads
     slots = []
     for i in range(len(pages)):
         t = torch.arange(int(ctx[i]), int(total[i]))
-        slots.append(lists[i].to(torch.long)[t // PAGE_SIZE] * PAGE_SIZE + t % PAGE_SIZE)
+        slots.append(lists[i].to(torch.long)[t // page_size] * page_size + t % page_size)
     slot_mapping = torch.cat(slots).to(torch.int32)
     t_total = int(ql.sum())
     return PrefillCase(
         name=name, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads, seq_lens=ql, context_lens=ctx,
         cu_q_lens=cu, block_table=table, slot_mapping=slot_mapping, num_pages=num_pages,
-        q=_randn_half((t_total, num_q_heads, HEAD_DIM), seed + 2, device),
-        k=_randn_half((t_total, num_kv_heads, HEAD_DIM), seed + 3, device),
-        v=_randn_half((t_total, num_kv_heads, HEAD_DIM), seed + 4, device),
-        kv_pool=_randn_half((num_pages * PAGE_SIZE, 2 * num_kv_heads, HEAD_DIM), seed + 5, device),
+        q=_randn_half((t_total, num_q_heads, head_dim), seed + 2, device),
+        k=_randn_half((t_total, num_kv_heads, head_dim), seed + 3, device),
+        v=_randn_half((t_total, num_kv_heads, head_dim), seed + 4, device),
+        kv_pool=_randn_half((num_pages * page_size, 2 * num_kv_heads, head_dim), seed + 5, device),
+        softmax_scale=1.0 / math.sqrt(head_dim), page_size=page_size, head_dim=head_dim,
     ).to(device)
 
 

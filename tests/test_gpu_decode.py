@@ -14,11 +14,12 @@ DEV = "cuda:0"
 def _oracle(case, seq_lens=None):
     sl = case.seq_lens if seq_lens is None else seq_lens
     return c_oracle.paged_decode(to_np16(case.q), to_np16(case.kv_pool), case.block_table.cpu().numpy(),
-                                 sl.cpu().numpy(), case.softmax_scale)
+                                 sl.cpu().numpy(), case.softmax_scale, page_size=case.page_size)
 
 
 def _run(case, **kw):
-    out = ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, case.softmax_scale, **kw)
+    out = ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, case.softmax_scale,
+                           page_size=case.page_size, **kw)
     torch.cuda.synchronize()
     return out
 
@@ -261,10 +262,10 @@ def test_invalid_arguments_raise():
                          min_pages_per_split=1, workspace=torch.empty(4, device=DEV))
 
 
-def _shared_prefix_case(seed, hq, hkv, shared_pages, suffix_ctx):
+def _shared_prefix_case(seed, hq, hkv, shared_pages, suffix_ctx, page_size=16):
     """Every block-table row starts with the same `shared_pages` pages; context = prefix + suffix."""
-    ctx = [shared_pages * 16 + s for s in suffix_ctx]
-    priv = [(c + 1 + 15) // 16 - shared_pages for c in ctx]
+    ctx = [shared_pages * page_size + s for s in suffix_ctx]
+    priv = [(c + 1 + page_size - 1) // page_size - shared_pages for c in ctx]
     num_pages = shared_pages + sum(priv) + 7
     perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(seed)).to(torch.int32)
     shared, cur, lists = perm[:shared_pages], shared_pages, []
@@ -272,7 +273,7 @@ def _shared_prefix_case(seed, hq, hkv, shared_pages, suffix_ctx):
         lists.append(torch.cat([shared, perm[cur:cur + n]]))
         cur += n
     return workloads.make_decode_case("shared", seed, ctx, hq, hkv, num_pages=num_pages, device=DEV,
-                                      page_lists=lists)
+                                      page_lists=lists, page_size=page_size)
 
 
 @pytest.mark.parametrize("hq,hkv,shared_pages,suffix", [
@@ -313,3 +314,83 @@ def test_shared_prefix_fused_append_and_empty_rows():
                                 lens.cpu().numpy(), case.softmax_scale)
     assert_attention_close(out, ref, "shared prefix + fused append")
     assert float(out[2].abs().max()) == 0.0
+
+
+# ---- pools with pages of 32 and 64 tokens (the reference's --page_size, server.py:1038-1161) ----
+
+PAGE_SIZES = [32, 64]
+EDGE_CONTEXTS = [0, 1, 15, 16, 17, 31, 32, 33, 47, 48, 63, 64, 65, 127, 128, 255, 700, 1200]
+
+
+@pytest.mark.parametrize("page_size", PAGE_SIZES)
+@pytest.mark.parametrize("hq,hkv", [(64, 8), (16, 4), (8, 1)])
+def test_page_sizes_every_schedule(page_size, hq, hkv):
+    """Both schedules on a pool of larger pages: lengths that end on, before and after every
+    16-token boundary inside a page and on the page boundary itself."""
+    print(f"decode page_size {page_size} heads {hq}/{hkv}", flush=True)
+    case = workloads.make_decode_case("pages", 300 + page_size + hq, EDGE_CONTEXTS, hq, hkv, device=DEV,
+                                      page_size=page_size)
+    ops.kv_append(case.k_new, case.v_new, case.slot_mapping, case.kv_pool)
+    ref = _oracle(case)
+    for kw in ({"num_splits": 1}, {"num_splits": 3}, {"max_splits": 16, "min_pages_per_split": 2},
+               {"schedule": "balanced"}, {"schedule": "balanced", "chunks": 7},
+               {"schedule": "balanced", "chunks": 1000}):
+        print("  ", kw, flush=True)
+        assert_attention_close(_run(case, **kw), ref, f"page_size {page_size} {hq}/{hkv} {kw}")
+
+
+@pytest.mark.parametrize("page_size", PAGE_SIZES)
+def test_page_sizes_fused_append_step(page_size):
+    """The fused append on larger pages: pool bit exact with the append kernel, output as the oracle's;
+    empty rows in between."""
+    print(f"decode fused step, page_size {page_size}", flush=True)
+    case = workloads.make_decode_case("pages-fused", 340 + page_size, EDGE_CONTEXTS, 32, 4, device=DEV,
+                                      page_size=page_size)
+    lens = case.seq_lens.clone()
+    lens[3] = 0
+    lens[9] = 0
+    pool_ref = case.kv_pool.clone()
+    ops.kv_append(case.k_new, case.v_new, case.slot_mapping, pool_ref)
+    ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool_ref), case.block_table.cpu().numpy(),
+                                lens.cpu().numpy(), case.softmax_scale, page_size=page_size)
+    keep = torch.ones(case.kv_pool.shape[0], dtype=torch.bool, device=DEV)
+    keep[case.slot_mapping[[3, 9]].long()] = False      # empty sequences append nothing
+    for chunks in (None, 5):
+        pool = case.kv_pool.clone()
+        plan = ops.DecodePlan(case.block_table, lens, 32, 4, case.num_pages, chunks, page_size=page_size)
+        out = ops.decode_step(case.q, pool, plan, case.k_new, case.v_new, case.softmax_scale)
+        torch.cuda.synchronize()
+        assert torch.equal(pool[keep].view(torch.int16), pool_ref[keep].view(torch.int16)), "append not bit exact"
+        assert_attention_close(out, ref, f"fused step page_size {page_size} chunks {chunks}")
+        assert float(out[3].abs().max()) == 0.0 and float(out[9].abs().max()) == 0.0
+    # the per-sequence schedule with its fused append
+    pool = case.kv_pool.clone()
+    out = ops.paged_decode(case.q, pool, case.block_table, lens, case.softmax_scale, num_splits=1,
+                           page_size=page_size, k_new=case.k_new, v_new=case.v_new)
+    torch.cuda.synchronize()
+    assert torch.equal(pool[keep].view(torch.int16), pool_ref[keep].view(torch.int16))
+    assert_attention_close(out, ref, f"per-sequence fused step page_size {page_size}")
+
+
+@pytest.mark.parametrize("page_size", PAGE_SIZES)
+@pytest.mark.parametrize("hq,hkv,shared_pages,suffix", [
+    (64, 8, 5, [0, 5, 15, 16, 40, 300]),
+    (16, 8, 1, [3, 0, 90]),
+    (32, 4, 11, list(range(0, 170, 10))),
+])
+def test_page_sizes_shared_prefix(page_size, hq, hkv, shared_pages, suffix):
+    print(f"decode shared prefix page_size {page_size} {hq}/{hkv} pages={shared_pages}", flush=True)
+    case = _shared_prefix_case(800 + hq + shared_pages + page_size, hq, hkv, shared_pages, suffix, page_size)
+    ref = _oracle(case)
+    for chunks in (None, 5):
+        out = _run(case, schedule="balanced", chunks=chunks, shared_pages=shared_pages)
+        assert_attention_close(out, ref, f"shared prefix page_size {page_size} chunks={chunks}")
+
+
+def test_unsupported_page_size_is_refused():
+    from llama_lite_npu_amd._lib import LiteKVError
+    case = workloads.make_decode_case("p48", 391, [40, 3, 90], 16, 8, device=DEV, page_size=48)
+    with pytest.raises(LiteKVError, match="page_size"):
+        ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, page_size=48, num_splits=1)
+    with pytest.raises((LiteKVError, ValueError), match="page_size"):
+        ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, page_size=48, schedule="balanced")

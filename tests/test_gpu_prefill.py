@@ -18,7 +18,7 @@ def _append(case):
 def _oracle_paged(case):
     return c_oracle.paged_prefill(to_np16(case.q), to_np16(case.kv_pool), case.block_table.cpu().numpy(),
                                   case.cu_q_lens.cpu().numpy(), case.context_lens.cpu().numpy(),
-                                  case.softmax_scale)
+                                  case.softmax_scale, page_size=case.page_size)
 
 
 @pytest.mark.parametrize("hq,hkv,lens", [
@@ -155,3 +155,24 @@ def test_prefill_repeats_bit_for_bit():
     torch.cuda.synchronize()
     for o in outs[1:]:
         assert torch.equal(outs[0], o)
+
+
+@pytest.mark.parametrize("page_size", [32, 64])
+@pytest.mark.parametrize("hq,hkv,lens,ctx", [
+    (16, 8, [1, 2, 15, 16, 17, 33, 47, 48, 63, 64, 65], None),
+    (64, 8, [128, 77, 200], None),
+    (32, 4, [300, 5, 96], [100, 31, 64]),       # chunks over cached history
+    (16, 1, [130, 40], [17, 700]),
+])
+def test_paged_prefill_page_sizes(page_size, hq, hkv, lens, ctx):
+    """Pools with pages of 32 and 64 tokens (the reference's --page_size): prompts and chunks over
+    history whose ends fall on every kind of boundary inside and between pages."""
+    print(f"prefill page_size {page_size} {hq}/{hkv} {lens} ctx {ctx}", flush=True)
+    case = workloads.make_prefill_case("pp", 900 + page_size + hq, lens, hq, hkv, context_lens=ctx, device=DEV,
+                                       page_size=page_size)
+    _append(case)
+    out = ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens,
+                            case.context_lens if ctx is not None else None, case.max_q_len, case.softmax_scale,
+                            page_size=page_size)
+    torch.cuda.synchronize()
+    assert_attention_close(out, _oracle_paged(case), f"paged prefill page_size {page_size}")
