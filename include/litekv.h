@@ -549,6 +549,91 @@ int litekv_varlen_prefill(const void *q, int64_t q_token_stride,
                           int32_t head_dim, int32_t max_seq_len,
                           int64_t num_tokens, float softmax_scale, void *stream);
 
+
+/*
+ * int8 KV pools. The same pools, scales, call shapes and result contracts as
+ * the fp8 entry points above, with signed 8-bit codes instead of E4M3:
+ *     code  = clamp(round_to_nearest_even(x * (1 / scale)), -127, 127)
+ *     value = code * scale
+ * (the reference's int8 cache, lite_llama/kernels/others/
+ * context_flashattention_nopad.py:374-553, is read there without scales; the
+ * per-head scales are the fp8 pools'). Every code is an fp16 number, so
+ * attention over an int8 pool is fp16 attention over the codes with the K
+ * scale joining the softmax scale and the V scale the final normalisation.
+ * Each function below is its _fp8 namesake (litekv_page_dequant_int8:
+ * litekv_page_dequant) for an int8 pool; litekv_page_copy / litekv_page_gather
+ * move int8 pages as they are.
+ */
+int litekv_kv_append_int8(const void *k, const void *v, int64_t k_token_stride,
+                         int64_t v_token_stride, const int32_t *slot_mapping,
+                         void *kv_pool_int8, const float *scales, int32_t num_tokens,
+                         int32_t num_kv_heads, int32_t head_dim, int64_t num_slots,
+                         void *stream);
+
+int litekv_qk_norm_rope_append_int8(void *q, int64_t q_token_stride, const void *k,
+                                   int64_t k_token_stride, const void *v, int64_t v_token_stride,
+                                   const void *q_norm_weight, const void *k_norm_weight,
+                                   const void *cos_rows, const void *sin_rows,
+                                   int64_t cos_sin_token_stride, const int32_t *slot_mapping,
+                                   void *kv_pool_int8, const float *scales, int32_t num_tokens,
+                                   int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                   int64_t num_slots, float rms_eps, void *stream);
+
+int litekv_page_dequant_int8(const void *kv_pool_int8, void *dst_pool, const int32_t *src_ids,
+                        const int32_t *dst_ids, int32_t n, const float *scales,
+                        int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                        int64_t num_src_pages, int64_t num_dst_pages, void *stream);
+
+int litekv_paged_decode_balanced_int8(const void *q, int64_t q_batch_stride, void *kv_pool_int8,
+                                     const float *scales, const int32_t *seq_lens, void *plan,
+                                     size_t plan_bytes, const void *k_new, const void *v_new,
+                                     int64_t k_new_stride, int64_t v_new_stride, void *out,
+                                     void *workspace, size_t workspace_bytes, int32_t batch,
+                                     int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                     int32_t page_size, int64_t num_pages,
+                                     int32_t block_table_stride, int32_t chunks,
+                                     float softmax_scale, void *stream);
+
+int litekv_paged_decode_int8(const void *q, int64_t q_batch_stride, const void *kv_pool_int8,
+                            const float *scales, const int32_t *block_table,
+                            int32_t block_table_stride, const int32_t *seq_lens, void *out,
+                            void *workspace, size_t workspace_bytes, int32_t batch,
+                            int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                            int32_t page_size, int64_t num_pages, int32_t max_splits,
+                            int32_t min_pages_per_split, float softmax_scale, void *stream);
+
+int litekv_paged_decode_append_int8(const void *q, int64_t q_batch_stride, void *kv_pool_int8,
+                                   const float *scales, const int32_t *block_table,
+                                   int32_t block_table_stride, const int32_t *seq_lens,
+                                   const void *k_new, const void *v_new, int64_t k_new_stride,
+                                   int64_t v_new_stride, void *out, void *workspace,
+                                   size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+                                   int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                                   int64_t num_pages, int32_t max_splits,
+                                   int32_t min_pages_per_split, float softmax_scale, void *stream);
+
+int litekv_paged_decode_prefix_int8(const void *q, int64_t q_batch_stride, void *kv_pool_int8,
+                                   const float *scales, const int32_t *block_table,
+                                   const int32_t *seq_lens, void *plan, size_t plan_bytes,
+                                   const void *k_new, const void *v_new, int64_t k_new_stride,
+                                   int64_t v_new_stride, void *out, void *workspace,
+                                   size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+                                   int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                                   int64_t num_pages, int32_t block_table_stride, int32_t chunks,
+                                   int32_t shared_pages, float softmax_scale, void *stream);
+
+int litekv_paged_prefill_int8(const void *q, int64_t q_token_stride,
+                             const void *kv_pool, const float *kv_scales,
+                             const int32_t *block_table,
+                             int32_t block_table_stride,
+                             const int32_t *cu_q_lens,
+                             const int32_t *context_lens, void *out,
+                             int64_t out_token_stride, int32_t batch,
+                             int32_t num_q_heads, int32_t num_kv_heads,
+                             int32_t head_dim, int32_t page_size,
+                             int64_t num_pages, int32_t max_q_len,
+                             float softmax_scale, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

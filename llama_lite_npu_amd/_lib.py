@@ -61,6 +61,12 @@ SIGNATURES = {
          c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32, c_float,
          c_void_p],
     ),
+    "litekv_paged_decode_int8": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_size_t,
+         c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int32, c_float,
+         c_void_p],
+    ),
     "litekv_paged_decode_append": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
@@ -68,6 +74,12 @@ SIGNATURES = {
          c_int32, c_float, c_void_p],
     ),
     "litekv_paged_decode_append_fp8": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
+         c_int64, c_void_p, c_void_p, c_size_t, c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,
+         c_int32, c_int32, c_float, c_void_p],
+    ),
+    "litekv_paged_decode_append_int8": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
          c_int64, c_void_p, c_void_p, c_size_t, c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,
@@ -117,7 +129,18 @@ SIGNATURES = {
          c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_int32, c_int32, c_int32, c_int32, c_int32,
          c_int64, c_int32, c_int32, c_int32, c_float, c_void_p],
     ),
+    "litekv_paged_decode_prefix_int8": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p,
+         c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_int32, c_int32, c_int32, c_int32, c_int32,
+         c_int64, c_int32, c_int32, c_int32, c_float, c_void_p],
+    ),
     "litekv_kv_append_fp8": (
+        c_int32,
+        [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32,
+         c_int64, c_void_p],
+    ),
+    "litekv_kv_append_int8": (
         c_int32,
         [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32,
          c_int64, c_void_p],
@@ -127,12 +150,28 @@ SIGNATURES = {
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
          c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int64, c_float, c_void_p],
     ),
+    "litekv_qk_norm_rope_append_int8": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_int64, c_float, c_void_p],
+    ),
     "litekv_page_dequant": (
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_int32, c_int32, c_int32, c_int64,
          c_int64, c_void_p],
     ),
+    "litekv_page_dequant_int8": (
+        c_int32,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_int32, c_int32, c_int32, c_int64,
+         c_int64, c_void_p],
+    ),
     "litekv_paged_decode_balanced_fp8": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p, c_int64,
+         c_int64, c_void_p, c_void_p, c_size_t, c_int32, c_int32, c_int32, c_int32, c_int32,
+         c_int64, c_int32, c_int32, c_float, c_void_p],
+    ),
+    "litekv_paged_decode_balanced_int8": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_void_p, c_int64,
          c_int64, c_void_p, c_void_p, c_size_t, c_int32, c_int32, c_int32, c_int32, c_int32,
@@ -150,6 +189,11 @@ SIGNATURES = {
          c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_float, c_void_p],
     ),
     "litekv_paged_prefill_fp8": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
+         c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_float, c_void_p],
+    ),
+    "litekv_paged_prefill_int8": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
          c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_float, c_void_p],

@@ -12,7 +12,7 @@ arguments, driven by the same ``AttentionInfo``. Differences:
   chunks), so one kernel serves both branches of the reference;
 * ``qkv_epilogue`` folds the step before the append (QK RMSNorm, rotary embedding,
   qwen3.py:124-129) into the append itself; the forward calls are then made with ``xk=None``;
-* a layer whose pool holds fp8 codes (``atten_info.kv_scales[layer]`` set) quantises on append
+* a layer whose pool holds fp8 or int8 codes (``atten_info.kv_scales[layer]`` set) quantises on append
   and attends straight from the codes, in decode and in chunks over cached history; fresh
   prompts attend to their own fp16 K/V.
 
@@ -46,7 +46,7 @@ class Attention:
         ``context_forward`` / ``token_forward`` afterwards with ``xk=None, xv=None``."""
         cos, sin = position_embeddings if position_embeddings is not None else (None, None)
         pool = atten_info.kv_buffer[layer_index]
-        scales = atten_info.kv_scales[layer_index] if ops.is_fp8_pool(pool) else None
+        scales = atten_info.kv_scales[layer_index] if ops.is_quantised_pool(pool) else None
         return ops.qk_norm_rope_append(xq, xk, xv, atten_info.cur_select_index, pool, q_norm_weight,
                                        k_norm_weight, cos, sin, rms_eps, kv_scales=scales)
 
@@ -55,7 +55,7 @@ class Attention:
         (None when ``qkv_epilogue`` already stored them)."""
         pool = atten_info.kv_buffer[layer_index]
         scale = (1.0 / math.sqrt(self.head_dim)) if qk_scale is None else float(qk_scale) / LOG2E
-        if ops.is_fp8_pool(pool):
+        if ops.is_quantised_pool(pool):
             return self._context_forward_fp8(xq, xk, xv, atten_info, pool, atten_info.kv_scales[layer_index], scale)
         if xk is not None:
             ops.kv_append(xk, xv, atten_info.cur_select_index, pool)
@@ -68,7 +68,7 @@ class Attention:
     def _context_forward_fp8(self, xq, xk, xv, atten_info, pool, scales, scale) -> torch.Tensor:
         chunked = getattr(atten_info, "is_paged_chunk_prefill", False)
         if xk is not None:
-            ops.kv_append_fp8(xk, xv, atten_info.cur_select_index, pool, scales)
+            ops.kv_append_quantised(xk, xv, atten_info.cur_select_index, pool, scales)
             if not chunked:
                 # a fresh prompt attends to its own K/V as computed, not as stored
                 return ops.varlen_prefill(xq, xk, xv, atten_info.b_start_loc, atten_info.seq_lens_i32,
@@ -87,12 +87,12 @@ class Attention:
         pool = atten_info.kv_buffer[layer_index]
         scale = (1.0 / math.sqrt(self.head_dim)) if qk_scale is None else float(qk_scale)
         plan = getattr(atten_info, "decode_plan", None)
-        scales = atten_info.kv_scales[layer_index] if ops.is_fp8_pool(pool) else None
+        scales = atten_info.kv_scales[layer_index] if ops.is_quantised_pool(pool) else None
         if plan is not None:
             return ops.decode_step(xq, pool, plan, xk, xv, scale, kv_scales=scales)
         if xk is not None:
             if scales is not None:
-                ops.kv_append_fp8(xk, xv, atten_info.cur_select_index, pool, scales)
+                ops.kv_append_quantised(xk, xv, atten_info.cur_select_index, pool, scales)
             else:
                 ops.kv_append(xk, xv, atten_info.cur_select_index, pool)
         return ops.paged_decode(xq, pool, atten_info.block_table, atten_info.seq_lens_i32, scale, kv_scales=scales)

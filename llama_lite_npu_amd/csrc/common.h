@@ -52,7 +52,7 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
                          const int32_t *block_table, int32_t batch, int32_t num_q_heads,
                          int32_t num_kv_heads, int64_t num_pages, int32_t shared_pages,
                          int32_t page_shift, float *part_o, float *part_lse, float softmax_scale,
-                         hipStream_t stream, int *splits_out);
+                         hipStream_t stream, int *splits_out, int format);
 
 // ---- device side ---------------------------------------------------------
 

@@ -41,4 +41,59 @@ __device__ __forceinline__ uint2_t half8_to_fp8(half8_t x, float inv_scale) {
   return uint2_t{(uint32_t)lo, (uint32_t)hi};
 }
 
+// ---- int8 storage -----------------------------------------------------------------------------
+// The same pools and scales with signed 8-bit codes:
+//     stored code = clamp(round_to_nearest_even(x / scale), -127, 127)
+//     value used  = code * scale
+// Every code is an fp16 number, so attention over an int8 pool is fp16 attention over the codes
+// with the scales folded in where the fp8 pool folds them.
+
+// Eight codes -> eight fp16 values, exact: byte c ^ 0x80 = c + 128 under the exponent byte of
+// 1024.0 is the fp16 number 1024 + 128 + c, and 1152 is subtracted from pairs.
+__device__ __forceinline__ half8_t int8x8_to_half(uint2_t codes) {
+  const half2_t bias = half2_t{(_Float16)1152.0f, (_Float16)1152.0f};
+  half2_t h[4];
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    const uint32_t x = codes[w] ^ 0x80808080u;
+    h[2 * w] = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u)) - bias;
+    h[2 * w + 1] = __builtin_bit_cast(half2_t, __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u)) - bias;
+  }
+  return half8_t{h[0][0], h[0][1], h[1][0], h[1][1], h[2][0], h[2][1], h[3][0], h[3][1]};
+}
+
+// Eight fp16 values times `inv_scale` -> eight codes.
+__device__ __forceinline__ uint2_t half8_to_int8(half8_t x, float inv_scale) {
+  uint32_t w[2] = {0u, 0u};
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float f = __builtin_rintf((float)x[i] * inv_scale);  // v_rndne_f32: halves go to the even integer
+    f = __builtin_fminf(__builtin_fmaxf(f, -127.0f), 127.0f);
+    w[i >> 2] |= ((uint32_t)(int)f & 0xffu) << (8 * (i & 3));
+  }
+  return uint2_t{w[0], w[1]};
+}
+
+// The storage formats of a pool, as template arguments of the kernels that read or write one.
+constexpr int kKvF16 = 0, kKvFp8 = 1, kKvInt8 = 2;
+
+template <int KV>
+__device__ __forceinline__ half8_t codes_to_half(uint2_t codes) {
+  static_assert(KV == kKvFp8 || KV == kKvInt8, "an 8-bit format");
+  if constexpr (KV == kKvInt8) {
+    return int8x8_to_half(codes);
+  } else {
+    return fp8x8_to_half(codes);
+  }
+}
+template <int KV>
+__device__ __forceinline__ uint2_t half_to_codes(half8_t x, float inv_scale) {
+  static_assert(KV == kKvFp8 || KV == kKvInt8, "an 8-bit format");
+  if constexpr (KV == kKvInt8) {
+    return half8_to_int8(x, inv_scale);
+  } else {
+    return half8_to_fp8(x, inv_scale);
+  }
+}
+
 }  // namespace litekv

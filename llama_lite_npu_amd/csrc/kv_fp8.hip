@@ -1,5 +1,6 @@
-// FP8 KV pool: the append that quantises K/V rows on their way into the pages, and the page
-// dequantiser that turns pages back into fp16 rows (for the prefill kernels, which read fp16).
+// 8-bit KV pools (fp8 E4M3 or int8 codes, one fp32 scale per kv head): the append that quantises
+// K/V rows on their way into the pages, and the page dequantiser that turns pages back into fp16
+// rows.
 // The pool is [slots][2 * Hkv][128] bytes, K heads then V heads as in the fp16 pool, so a page is
 // one contiguous run of half the size; scales[2 * Hkv] holds the K-head scales, then the V-head
 // scales.
@@ -11,7 +12,8 @@
 
 namespace litekv {
 
-__global__ __launch_bounds__(256) void kv_append_fp8_kernel(
+template <int KV>
+__global__ __launch_bounds__(256) void kv_append_q8_kernel(
     const half8_t *__restrict__ k, const half8_t *__restrict__ v, int64_t k_stride8,
     int64_t v_stride8, const int32_t *__restrict__ slot_mapping, uint2_t *__restrict__ pool,
     const float *__restrict__ scales, int64_t total_items, int32_t items_per_half,
@@ -26,9 +28,10 @@ __global__ __launch_bounds__(256) void kv_append_fp8_kernel(
   const half8_t x = (c < items_per_half) ? k[token * k_stride8 + c]
                                          : v[token * v_stride8 + (c - items_per_half)];
   const float inv_scale = 1.0f / scales[c / (kHeadDim / 8)];  // head index over K heads then V heads
-  pool[slot * items_per_token + c] = half8_to_fp8(x, inv_scale);
+  pool[slot * items_per_token + c] = half_to_codes<KV>(x, inv_scale);
 }
 
+template <int KV>
 __global__ __launch_bounds__(256) void page_dequant_kernel(
     const uint2_t *__restrict__ src_pool, half8_t *__restrict__ dst_pool,
     const int32_t *__restrict__ src_ids, const int32_t *__restrict__ dst_ids,
@@ -40,7 +43,7 @@ __global__ __launch_bounds__(256) void page_dequant_kernel(
   if (sp < 0 || sp >= num_src_pages || dp < 0 || dp >= num_dst_pages) return;
   for (int c = blockIdx.y * 256 + threadIdx.x; c < page_items; c += gridDim.y * 256) {
     const float scale = scales[(c % items_per_slot) / (kHeadDim / 8)];
-    const half8_t raw = fp8x8_to_half(__builtin_nontemporal_load(src_pool + sp * page_items + c));
+    const half8_t raw = codes_to_half<KV>(__builtin_nontemporal_load(src_pool + sp * page_items + c));
     half8_t y;
 #pragma unroll
     for (int e = 0; e < 8; ++e) y[e] = (half_t)((float)raw[e] * scale);
@@ -56,15 +59,11 @@ static int check_scales_geometry(const char *what, int32_t num_kv_heads, int32_t
   return LITEKV_OK;
 }
 
-}  // namespace litekv
-
-extern "C" int litekv_kv_append_fp8(const void *k, const void *v, int64_t k_token_stride,
-                                    int64_t v_token_stride, const int32_t *slot_mapping,
-                                    void *kv_pool_fp8, const float *scales, int32_t num_tokens,
-                                    int32_t num_kv_heads, int32_t head_dim, int64_t num_slots,
-                                    void *stream) {
-  using namespace litekv;
-  const char *what = "kv_append_fp8";
+static int launch_kv_append_q8(const char *what, int format, const void *k, const void *v,
+                               int64_t k_token_stride, int64_t v_token_stride,
+                               const int32_t *slot_mapping, void *kv_pool_fp8, const float *scales,
+                               int32_t num_tokens, int32_t num_kv_heads, int32_t head_dim,
+                               int64_t num_slots, void *stream) {
   LITEKV_REQUIRE(num_tokens >= 0, "%s: num_tokens %d < 0", what, num_tokens);
   int rc = check_scales_geometry(what, num_kv_heads, head_dim);
   if (rc != LITEKV_OK) return rc;
@@ -85,20 +84,26 @@ extern "C" int litekv_kv_append_fp8(const void *k, const void *v, int64_t k_toke
   const int64_t total = (int64_t)num_tokens * 2 * items_per_half;
   const int64_t blocks = (total + 255) / 256;
   LITEKV_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many tokens", what);
-  hipLaunchKernelGGL(kv_append_fp8_kernel, dim3((unsigned)blocks), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const half8_t *>(k),
-                     static_cast<const half8_t *>(v), k_token_stride / 8, v_token_stride / 8,
-                     slot_mapping, static_cast<uint2_t *>(kv_pool_fp8), scales, total,
-                     items_per_half, num_slots);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const half8_t *>(k),
+                       static_cast<const half8_t *>(v), k_token_stride / 8, v_token_stride / 8,
+                       slot_mapping, static_cast<uint2_t *>(kv_pool_fp8), scales, total,
+                       items_per_half, num_slots);
+  };
+  if (format == kKvInt8) {
+    launch(kv_append_q8_kernel<kKvInt8>);
+  } else {
+    launch(kv_append_q8_kernel<kKvFp8>);
+  }
   return check_launch(what);
 }
 
-extern "C" int litekv_page_dequant(const void *kv_pool_fp8, void *dst_pool, const int32_t *src_ids,
-                                   const int32_t *dst_ids, int32_t n, const float *scales,
-                                   int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
-                                   int64_t num_src_pages, int64_t num_dst_pages, void *stream) {
-  using namespace litekv;
-  const char *what = "page_dequant";
+static int launch_page_dequant(const char *what, int format, const void *kv_pool_fp8,
+                               void *dst_pool, const int32_t *src_ids, const int32_t *dst_ids,
+                               int32_t n, const float *scales, int32_t num_kv_heads,
+                               int32_t head_dim, int32_t page_size, int64_t num_src_pages,
+                               int64_t num_dst_pages, void *stream) {
   LITEKV_REQUIRE(n >= 0, "%s: n %d < 0", what, n);
   int rc = check_scales_geometry(what, num_kv_heads, head_dim);
   if (rc != LITEKV_OK) return rc;
@@ -119,9 +124,57 @@ extern "C" int litekv_page_dequant(const void *kv_pool_fp8, void *dst_pool, cons
   LITEKV_REQUIRE(page_items <= 0x7fffffffLL, "%s: page too large", what);
   int64_t tiles = (page_items + 1023) / 1024;
   tiles = tiles < 1 ? 1 : (tiles > 64 ? 64 : tiles);
-  hipLaunchKernelGGL(page_dequant_kernel, dim3((unsigned)n, (unsigned)tiles), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const uint2_t *>(kv_pool_fp8),
-                     static_cast<half8_t *>(dst_pool), src_ids, dst_ids, scales, (int32_t)page_items,
-                     items_per_slot, num_src_pages, num_dst_pages);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)n, (unsigned)tiles), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const uint2_t *>(kv_pool_fp8),
+                       static_cast<half8_t *>(dst_pool), src_ids, dst_ids, scales,
+                       (int32_t)page_items, items_per_slot, num_src_pages, num_dst_pages);
+  };
+  if (format == kKvInt8) {
+    launch(page_dequant_kernel<kKvInt8>);
+  } else {
+    launch(page_dequant_kernel<kKvFp8>);
+  }
   return check_launch(what);
+}
+
+}  // namespace litekv
+
+extern "C" int litekv_kv_append_fp8(const void *k, const void *v, int64_t k_token_stride,
+                                    int64_t v_token_stride, const int32_t *slot_mapping,
+                                    void *kv_pool_fp8, const float *scales, int32_t num_tokens,
+                                    int32_t num_kv_heads, int32_t head_dim, int64_t num_slots,
+                                    void *stream) {
+  return litekv::launch_kv_append_q8("kv_append_fp8", litekv::kKvFp8, k, v, k_token_stride,
+                                     v_token_stride, slot_mapping, kv_pool_fp8, scales, num_tokens,
+                                     num_kv_heads, head_dim, num_slots, stream);
+}
+
+extern "C" int litekv_kv_append_int8(const void *k, const void *v, int64_t k_token_stride,
+                                     int64_t v_token_stride, const int32_t *slot_mapping,
+                                     void *kv_pool_int8, const float *scales, int32_t num_tokens,
+                                     int32_t num_kv_heads, int32_t head_dim, int64_t num_slots,
+                                     void *stream) {
+  return litekv::launch_kv_append_q8("kv_append_int8", litekv::kKvInt8, k, v, k_token_stride,
+                                     v_token_stride, slot_mapping, kv_pool_int8, scales, num_tokens,
+                                     num_kv_heads, head_dim, num_slots, stream);
+}
+
+extern "C" int litekv_page_dequant(const void *kv_pool_fp8, void *dst_pool, const int32_t *src_ids,
+                                   const int32_t *dst_ids, int32_t n, const float *scales,
+                                   int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                                   int64_t num_src_pages, int64_t num_dst_pages, void *stream) {
+  return litekv::launch_page_dequant("page_dequant", litekv::kKvFp8, kv_pool_fp8, dst_pool, src_ids,
+                                     dst_ids, n, scales, num_kv_heads, head_dim, page_size,
+                                     num_src_pages, num_dst_pages, stream);
+}
+
+extern "C" int litekv_page_dequant_int8(const void *kv_pool_int8, void *dst_pool,
+                                        const int32_t *src_ids, const int32_t *dst_ids, int32_t n,
+                                        const float *scales, int32_t num_kv_heads, int32_t head_dim,
+                                        int32_t page_size, int64_t num_src_pages,
+                                        int64_t num_dst_pages, void *stream) {
+  return litekv::launch_page_dequant("page_dequant_int8", litekv::kKvInt8, kv_pool_int8, dst_pool,
+                                     src_ids, dst_ids, n, scales, num_kv_heads, head_dim, page_size,
+                                     num_src_pages, num_dst_pages, stream);
 }

@@ -69,20 +69,20 @@ struct PageRegs {
   half8_t v[4];  // V rows 4*i + g, 16-byte column n
 };
 
-// One page of an fp8 pool: the same bytes per lane in half as many loads. The sum over d of a
+// One page of a pool of 8-bit codes (fp8 or int8): the same bytes per lane in half as many loads. The sum over d of a
 // dot product may run in any order as long as K and q agree, so a lane takes 16 consecutive
 // codes per load and MFMA step kk uses its lower or upper 8:
 //   k[j]: token n, d = 16*(g + 4*j) .. +15      step kk = 2*j + (0: lower, 1: upper 8 codes)
 //   v[i]: V row 8*i + 2*g + n/8, d = 16*(n%8) .. +15
-struct PageRegsFp8 {
+template <int KV>
+struct PageRegsQ8 {
   uint4_t k[2];
   uint4_t v[2];
 };
 
-// Storage of the pool a kernel reads.
-template <bool FP8> struct KvStore;
-template <> struct KvStore<false> { typedef half_t elem; typedef PageRegs page; };
-template <> struct KvStore<true> { typedef uint8_t elem; typedef PageRegsFp8 page; };
+// Storage of the pool a kernel reads: fp16, or the codes of format KV (kKvFp8, kKvInt8).
+template <int KV> struct KvStore { typedef uint8_t elem; typedef PageRegsQ8<KV> page; };
+template <> struct KvStore<kKvF16> { typedef half_t elem; typedef PageRegs page; };
 
 // Softmax state and output accumulator of the (up to 16) query heads of one kv head.
 // acc[j][i] is O^T[d = 16j + 4g + i][head n]; m is shared by the 4 lanes of a head, d is this
@@ -149,7 +149,8 @@ __device__ __forceinline__ void request_page(PageRegs &r, const half_t *k_lane,
 }
 
 // fp8 pool: k_lane points at token n, code 16*g; v_lane at row 2*g + n/8, code 16*(n%8).
-__device__ __forceinline__ void request_page(PageRegsFp8 &r, const uint8_t *k_lane,
+template <int KV>
+__device__ __forceinline__ void request_page(PageRegsQ8<KV> &r, const uint8_t *k_lane,
                                              const uint8_t *v_lane, int64_t page_off,
                                              int64_t row_stride, bool dummy = false,
                                              const uint8_t *pool = nullptr) {
@@ -240,21 +241,22 @@ __device__ __forceinline__ void attend_page(HeadState &st, const PageRegs &r,
   });
 }
 
-// The fp8 page: codes become fp16 exactly (the head's scales are applied by the caller).
-__device__ __forceinline__ void attend_page(HeadState &st, const PageRegsFp8 &r,
+// A page of codes: they become fp16 exactly (the head's scales are applied by the caller).
+template <int KV>
+__device__ __forceinline__ void attend_page(HeadState &st, const PageRegsQ8<KV> &r,
                                             const half8_t (&qf)[4], half_t *vstage,
                                             const half_t *vt_lane, int p, int len, int n, int g,
                                             float scale_log2) {
-  const half8_t kf[4] = {fp8x8_to_half(uint2_t{r.k[0][0], r.k[0][1]}),
-                         fp8x8_to_half(uint2_t{r.k[0][2], r.k[0][3]}),
-                         fp8x8_to_half(uint2_t{r.k[1][0], r.k[1][1]}),
-                         fp8x8_to_half(uint2_t{r.k[1][2], r.k[1][3]})};
+  const half8_t kf[4] = {codes_to_half<KV>(uint2_t{r.k[0][0], r.k[0][1]}),
+                         codes_to_half<KV>(uint2_t{r.k[0][2], r.k[0][3]}),
+                         codes_to_half<KV>(uint2_t{r.k[1][0], r.k[1][1]}),
+                         codes_to_half<KV>(uint2_t{r.k[1][2], r.k[1][3]})};
   attend_core(st, kf, qf, vt_lane, p, len, n, g, scale_log2, [&](bool tail) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int row = 8 * i + 2 * g + (n >> 3);
-      half8_t lo = fp8x8_to_half(uint2_t{r.v[i][0], r.v[i][1]});
-      half8_t hi = fp8x8_to_half(uint2_t{r.v[i][2], r.v[i][3]});
+      half8_t lo = codes_to_half<KV>(uint2_t{r.v[i][0], r.v[i][1]});
+      half8_t hi = codes_to_half<KV>(uint2_t{r.v[i][2], r.v[i][3]});
       if (tail && p * kPageSize + row >= len) {
         lo = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
         hi = lo;
@@ -405,10 +407,10 @@ __device__ __forceinline__ void load_new_rows(uint4_t (&kr)[4], uint4_t (&vr)[2]
 // ---------------------------------------------------------------------------------------------
 constexpr int kSplitWaves = 4;
 extern __shared__ __attribute__((aligned(16))) half_t split_vstage[];  // [waves][kPageSize * kVPitch]
-template <int DEPTH, bool FP8, bool APPEND>
+template <int DEPTH, int KV, bool APPEND>
 __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
     const half_t *__restrict__ q, int64_t q_batch_stride,
-    typename KvStore<FP8>::elem *__restrict__ kv, const float *__restrict__ scales,
+    typename KvStore<KV>::elem *__restrict__ kv, const float *__restrict__ scales,
     const int32_t *__restrict__ block_table, int32_t bt_stride,
     const int32_t *__restrict__ seq_lens, const half_t *__restrict__ k_new,
     const half_t *__restrict__ v_new, int64_t k_new_stride, int64_t v_new_stride,
@@ -441,8 +443,9 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
   const int p0 = (int)(((int64_t)split * pages) / n_splits);
   const int p1 = (int)(((int64_t)(split + 1) * pages) / n_splits);
 
-  typedef typename KvStore<FP8>::elem Elem;
-  typedef typename KvStore<FP8>::page Page;
+  constexpr bool FP8 = KV != kKvF16;  // 8-bit codes (either format): the layout they share
+  typedef typename KvStore<KV>::elem Elem;
+  typedef typename KvStore<KV>::page Page;
   half8_t qf[4];
   float v_scale = 1.0f, k_inv = 1.0f, v_inv = 1.0f;
   if constexpr (FP8) {  // the K scale joins the softmax scale, the V scale the normalisation
@@ -511,16 +514,16 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
               uint8_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 16 * g;
 #pragma unroll
               for (int j = 0; j < 2; ++j) {
-                const uint2_t lo = half8_to_fp8(__builtin_bit_cast(half8_t, k_row[2 * j]), k_inv);
-                const uint2_t hi = half8_to_fp8(__builtin_bit_cast(half8_t, k_row[2 * j + 1]), k_inv);
+                const uint2_t lo = half_to_codes<KV>(__builtin_bit_cast(half8_t, k_row[2 * j]), k_inv);
+                const uint2_t hi = half_to_codes<KV>(__builtin_bit_cast(half8_t, k_row[2 * j + 1]), k_inv);
                 const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
                 r.k[j] = x;
                 *(uint4_t *)(dst + 64 * j) = x;
               }
             }
             if (2 * g + (n >> 3) == (t_new & 7)) {
-              const uint2_t lo = half8_to_fp8(__builtin_bit_cast(half8_t, v_row[0]), v_inv);
-              const uint2_t hi = half8_to_fp8(__builtin_bit_cast(half8_t, v_row[1]), v_inv);
+              const uint2_t lo = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[0]), v_inv);
+              const uint2_t hi = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[1]), v_inv);
               const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
               *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7)) = x;
 #pragma unroll
@@ -961,10 +964,10 @@ __global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merg
   }
 }
 
-template <int DEPTH, bool FP8>
+template <int DEPTH, int KV>
 __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_kernel(
     const half_t *__restrict__ q, int64_t q_batch_stride,
-    typename KvStore<FP8>::elem *__restrict__ kv, const float *__restrict__ scales,
+    typename KvStore<KV>::elem *__restrict__ kv, const float *__restrict__ scales,
     const int32_t *__restrict__ seq_lens, const int32_t *__restrict__ plan,
     const half_t *__restrict__ k_new, const half_t *__restrict__ v_new, int64_t k_new_stride,
     int64_t v_new_stride, half_t *__restrict__ out, float *__restrict__ part_o,
@@ -1026,8 +1029,9 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   // second hop is under way while they are issued.
   int len_after = (cur_b + 1 < batch) ? lens[cur_b + 1] : 0;
 
-  typedef typename KvStore<FP8>::elem Elem;
-  typedef typename KvStore<FP8>::page Page;
+  constexpr bool FP8 = KV != kKvF16;  // 8-bit codes (either format): the layout they share
+  typedef typename KvStore<KV>::elem Elem;
+  typedef typename KvStore<KV>::page Page;
   // fp8 pool: the K scale joins the softmax scale, the V scale the final normalisation, and the
   // step's new rows are quantised with the reciprocals
   float k_inv = 1.0f, v_inv = 1.0f, v_scale = 1.0f;
@@ -1205,16 +1209,16 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
               uint8_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 16 * g;
 #pragma unroll
               for (int j = 0; j < 2; ++j) {
-                const uint2_t lo = half8_to_fp8(__builtin_bit_cast(half8_t, k_row[2 * j]), k_inv);
-                const uint2_t hi = half8_to_fp8(__builtin_bit_cast(half8_t, k_row[2 * j + 1]), k_inv);
+                const uint2_t lo = half_to_codes<KV>(__builtin_bit_cast(half8_t, k_row[2 * j]), k_inv);
+                const uint2_t hi = half_to_codes<KV>(__builtin_bit_cast(half8_t, k_row[2 * j + 1]), k_inv);
                 const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
                 buf[dd].k[j] = x;
                 *(uint4_t *)(dst + 64 * j) = x;
               }
             }
             if (2 * g + (n >> 3) == (t_new & 7)) {
-              const uint2_t lo = half8_to_fp8(__builtin_bit_cast(half8_t, v_row[0]), v_inv);
-              const uint2_t hi = half8_to_fp8(__builtin_bit_cast(half8_t, v_row[1]), v_inv);
+              const uint2_t lo = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[0]), v_inv);
+              const uint2_t hi = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[1]), v_inv);
               const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
               *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7)) = x;
 #pragma unroll
@@ -1352,9 +1356,12 @@ static int check_split_plan(const char *what, int32_t max_splits, int32_t min_pa
   return LITEKV_OK;
 }
 
+// fp8_scales: the scales of a pool of 8-bit codes of format `format` (kKvFp8, kKvInt8), or null.
 static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split,
-                        const float *fp8_scales = nullptr) {
-  const char *what = fp8_scales ? "paged_decode_split_fp8" : "paged_decode_split";
+                        const float *fp8_scales = nullptr, int format = kKvFp8) {
+  const char *what = !fp8_scales          ? "paged_decode_split"
+                     : format == kKvInt8 ? "paged_decode_split_int8"
+                                         : "paged_decode_split_fp8";
   int rc = check_split_plan(what, max_splits, min_pages_per_split);
   if (rc != LITEKV_OK) return rc;
   rc = validate_decode(what, a,
@@ -1400,16 +1407,22 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
                        min_16_token_pages(min_pages_per_split, a.page_size), (int32_t)a.num_pages,
                        page_shift_of(a.page_size), a.softmax_scale * kLog2e);
   };
-  if (fp8_scales != nullptr) {
+  if (fp8_scales != nullptr && format == kKvInt8) {
     if (a.k_new != nullptr) {
-      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, true, true>, static_cast<uint8_t *>(pool));
+      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvInt8, true>, static_cast<uint8_t *>(pool));
     } else {
-      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, true, false>, static_cast<uint8_t *>(pool));
+      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvInt8, false>, static_cast<uint8_t *>(pool));
+    }
+  } else if (fp8_scales != nullptr) {
+    if (a.k_new != nullptr) {
+      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvFp8, true>, static_cast<uint8_t *>(pool));
+    } else {
+      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvFp8, false>, static_cast<uint8_t *>(pool));
     }
   } else if (a.k_new != nullptr) {
-    launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, false, true>, static_cast<half_t *>(pool));
+    launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvF16, true>, static_cast<half_t *>(pool));
   } else {
-    launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, false, false>, static_cast<half_t *>(pool));
+    launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvF16, false>, static_cast<half_t *>(pool));
   }
   return check_launch(what);
 }
@@ -1600,7 +1613,8 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
                            size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
                            int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
                            int64_t num_pages, int32_t block_table_stride, int32_t chunks,
-                           int32_t shared_pages, float softmax_scale, void *stream) {
+                           int32_t shared_pages, float softmax_scale, void *stream,
+                           int format = kKvFp8) {
   const int shift = page_shift_of(page_size);
   LITEKV_REQUIRE(shift >= 0, "%s: page_size %d unsupported (16, 32 or 64)", what, page_size);
   LITEKV_REQUIRE(block_table_stride >= 1 && block_table_stride <= (0x7fffffff >> 4),
@@ -1650,7 +1664,7 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
     LITEKV_REQUIRE(block_table != nullptr, "%s: block_table is null", what);
     rc = launch_shared_prefix(q, q_batch_stride, kv_pool, fp8_scales, block_table, batch, num_q_heads,
                               num_kv_heads, num_pages, shared_pages, shift, pre_o, pre_lse,
-                              softmax_scale, static_cast<hipStream_t>(stream), &pre_splits);
+                              softmax_scale, static_cast<hipStream_t>(stream), &pre_splits, format);
     if (rc != LITEKV_OK) return rc;
   }
   const unsigned wgs = (unsigned)((chunks + s.replicas - 1) / s.replicas);
@@ -1658,26 +1672,21 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   g_profile_start = g_profile_stop = nullptr;
   const dim3 grid(wgs, (unsigned)s.head_groups);
   const dim3 block((unsigned)(kWave * s.heads_per_wg * s.replicas));
-  if (fp8_scales != nullptr) {
-    hipExtLaunchKernelGGL((paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, true>), grid, block, 0,
-                          static_cast<hipStream_t>(stream), ev0, ev1, 0,
-                          static_cast<const half_t *>(q), q_batch_stride,
-                          static_cast<uint8_t *>(kv_pool), fp8_scales, seq_lens,
+  auto launch = [&](auto kernel, auto *kv) {
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), ev0, ev1, 0,
+                          static_cast<const half_t *>(q), q_batch_stride, kv, fp8_scales, seq_lens,
                           static_cast<const int32_t *>(plan), static_cast<const half_t *>(k_new),
                           static_cast<const half_t *>(v_new), k_new_stride, v_new_stride,
                           static_cast<half_t *>(out), part_o, part_lse, sub_stride, batch,
                           num_q_heads, num_kv_heads, num_q_heads / num_kv_heads, s.heads_per_wg,
                           s.replicas, chunks, shared_pages << shift, softmax_scale * kLog2e);
+  };
+  if (fp8_scales != nullptr && format == kKvInt8) {
+    launch(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, kKvInt8>, static_cast<uint8_t *>(kv_pool));
+  } else if (fp8_scales != nullptr) {
+    launch(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, kKvFp8>, static_cast<uint8_t *>(kv_pool));
   } else {
-    hipExtLaunchKernelGGL((paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, false>), grid, block, 0,
-                          static_cast<hipStream_t>(stream), ev0, ev1, 0,
-                          static_cast<const half_t *>(q), q_batch_stride,
-                          static_cast<half_t *>(kv_pool), fp8_scales, seq_lens,
-                          static_cast<const int32_t *>(plan), static_cast<const half_t *>(k_new),
-                          static_cast<const half_t *>(v_new), k_new_stride, v_new_stride,
-                          static_cast<half_t *>(out), part_o, part_lse, sub_stride, batch,
-                          num_q_heads, num_kv_heads, num_q_heads / num_kv_heads, s.heads_per_wg,
-                          s.replicas, chunks, shared_pages << shift, softmax_scale * kLog2e);
+    launch(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, kKvF16>, static_cast<half_t *>(kv_pool));
   }
   rc = check_launch(what);
   if (rc != LITEKV_OK) return rc;
@@ -1743,6 +1752,23 @@ extern "C" int litekv_paged_decode_balanced_fp8(
                                  chunks, 0, softmax_scale, stream);
 }
 
+extern "C" int litekv_paged_decode_balanced_int8(
+    const void *q, int64_t q_batch_stride, void *kv_pool_int8, const float *scales,
+    const int32_t *seq_lens, void *plan, size_t plan_bytes, const void *k_new, const void *v_new,
+    int64_t k_new_stride, int64_t v_new_stride, void *out, void *workspace, size_t workspace_bytes,
+    int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+    int64_t num_pages, int32_t block_table_stride, int32_t chunks, float softmax_scale,
+    void *stream) {
+  if (scales == nullptr && batch > 0) {
+    return litekv::fail(LITEKV_ERR_INVALID_ARGUMENT, "paged_decode_balanced_int8: scales is null");
+  }
+  return litekv::launch_balanced("paged_decode_balanced_int8", q, q_batch_stride, kv_pool_int8, scales,
+                                 nullptr, seq_lens, plan, plan_bytes, k_new, v_new, k_new_stride,
+                                 v_new_stride, out, workspace, workspace_bytes, batch, num_q_heads,
+                                 num_kv_heads, head_dim, page_size, num_pages, block_table_stride,
+                                 chunks, 0, softmax_scale, stream, litekv::kKvInt8);
+}
+
 extern "C" size_t litekv_paged_decode_prefix_workspace_bytes(int32_t batch, int32_t num_q_heads,
                                                              int32_t head_dim, int32_t chunks) {
   return litekv::prefix_workspace_bytes(batch, num_q_heads, head_dim, chunks);
@@ -1778,6 +1804,24 @@ extern "C" int litekv_paged_decode_prefix_fp8(
                                  v_new_stride, out, workspace, workspace_bytes, batch, num_q_heads,
                                  num_kv_heads, head_dim, page_size, num_pages, block_table_stride,
                                  chunks, shared_pages, softmax_scale, stream);
+}
+
+extern "C" int litekv_paged_decode_prefix_int8(
+    const void *q, int64_t q_batch_stride, void *kv_pool_int8, const float *scales,
+    const int32_t *block_table, const int32_t *seq_lens, void *plan, size_t plan_bytes,
+    const void *k_new, const void *v_new, int64_t k_new_stride, int64_t v_new_stride, void *out,
+    void *workspace, size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+    int32_t num_kv_heads, int32_t head_dim, int32_t page_size, int64_t num_pages,
+    int32_t block_table_stride, int32_t chunks, int32_t shared_pages, float softmax_scale,
+    void *stream) {
+  if (scales == nullptr && batch > 0) {
+    return litekv::fail(LITEKV_ERR_INVALID_ARGUMENT, "paged_decode_prefix_int8: scales is null");
+  }
+  return litekv::launch_balanced("paged_decode_prefix_int8", q, q_batch_stride, kv_pool_int8, scales,
+                                 block_table, seq_lens, plan, plan_bytes, k_new, v_new, k_new_stride,
+                                 v_new_stride, out, workspace, workspace_bytes, batch, num_q_heads,
+                                 num_kv_heads, head_dim, page_size, num_pages, block_table_stride,
+                                 chunks, shared_pages, softmax_scale, stream, litekv::kKvInt8);
 }
 
 extern "C" size_t litekv_paged_decode_workspace_bytes(int32_t batch, int32_t num_q_heads,
@@ -1826,6 +1870,27 @@ extern "C" int litekv_paged_decode_fp8(const void *q, int64_t q_batch_stride,
                        workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim,
                        page_size, num_pages, softmax_scale, stream};
   int rc = litekv::launch_split(a, max_splits, min_pages_per_split, batch > 0 ? scales : nullptr);
+  if (rc != LITEKV_OK) return rc;
+  return litekv::launch_merge(a, max_splits, min_pages_per_split);
+}
+
+extern "C" int litekv_paged_decode_int8(const void *q, int64_t q_batch_stride,
+                                       const void *kv_pool_int8, const float *scales,
+                                       const int32_t *block_table, int32_t block_table_stride,
+                                       const int32_t *seq_lens, void *out, void *workspace,
+                                       size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+                                       int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
+                                       int64_t num_pages, int32_t max_splits,
+                                       int32_t min_pages_per_split, float softmax_scale,
+                                       void *stream) {
+  if (scales == nullptr && batch > 0) {
+    return litekv::fail(LITEKV_ERR_INVALID_ARGUMENT, "paged_decode_int8: scales is null");
+  }
+  litekv::DecodeArgs a{q, q_batch_stride, kv_pool_int8, block_table, block_table_stride, seq_lens, out,
+                       workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim,
+                       page_size, num_pages, softmax_scale, stream};
+  int rc = litekv::launch_split(a, max_splits, min_pages_per_split, batch > 0 ? scales : nullptr,
+                                litekv::kKvInt8);
   if (rc != LITEKV_OK) return rc;
   return litekv::launch_merge(a, max_splits, min_pages_per_split);
 }
@@ -1883,6 +1948,27 @@ extern "C" int litekv_paged_decode_append_fp8(
                        page_size, num_pages, softmax_scale, stream, k_new, v_new, k_new_stride,
                        v_new_stride};
   int rc = litekv::launch_split(a, max_splits, min_pages_per_split, batch > 0 ? scales : nullptr);
+  if (rc != LITEKV_OK) return rc;
+  return litekv::launch_merge(a, max_splits, min_pages_per_split);
+}
+
+extern "C" int litekv_paged_decode_append_int8(
+    const void *q, int64_t q_batch_stride, void *kv_pool_int8, const float *scales,
+    const int32_t *block_table, int32_t block_table_stride, const int32_t *seq_lens,
+    const void *k_new, const void *v_new, int64_t k_new_stride, int64_t v_new_stride, void *out,
+    void *workspace, size_t workspace_bytes, int32_t batch, int32_t num_q_heads,
+    int32_t num_kv_heads, int32_t head_dim, int32_t page_size, int64_t num_pages,
+    int32_t max_splits, int32_t min_pages_per_split, float softmax_scale, void *stream) {
+  if ((scales == nullptr || k_new == nullptr || v_new == nullptr) && batch > 0) {
+    return litekv::fail(LITEKV_ERR_INVALID_ARGUMENT,
+                        "paged_decode_append_int8: scales / k_new / v_new is null");
+  }
+  litekv::DecodeArgs a{q, q_batch_stride, kv_pool_int8, block_table, block_table_stride, seq_lens, out,
+                       workspace, workspace_bytes, batch, num_q_heads, num_kv_heads, head_dim,
+                       page_size, num_pages, softmax_scale, stream, k_new, v_new, k_new_stride,
+                       v_new_stride};
+  int rc = litekv::launch_split(a, max_splits, min_pages_per_split, batch > 0 ? scales : nullptr,
+                                litekv::kKvInt8);
   if (rc != LITEKV_OK) return rc;
   return litekv::launch_merge(a, max_splits, min_pages_per_split);
 }

@@ -106,7 +106,7 @@ __device__ __forceinline__ float vmax3(float a, float b, float c) {
 }
 __device__ __forceinline__ float vmax2(float a, float b) { return __builtin_fmaxf(a, b); }
 constexpr int kPagedPrefill = 0, kPackedPrefill = 1, kSharedPrefix = 2, kPagedPrefillFp8 = 3,
-              kSharedPrefixFp8 = 4;
+              kSharedPrefixFp8 = 4, kPagedPrefillInt8 = 5, kSharedPrefixInt8 = 6;
 
 template <int MODE>
 __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_kernel(
@@ -120,8 +120,10 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   // converted to fp16 (exactly) and written to LDS in the same swizzled layout, so everything
   // after the staging is shared. The K scale joins the softmax scale, the V scale the final
   // normalisation, as in the decode kernel.
-  constexpr bool FP8 = MODE == kPagedPrefillFp8 || MODE == kSharedPrefixFp8;
-  constexpr bool SHARED = MODE == kSharedPrefix || MODE == kSharedPrefixFp8;
+  constexpr bool FP8 = MODE == kPagedPrefillFp8 || MODE == kSharedPrefixFp8 ||
+                       MODE == kPagedPrefillInt8 || MODE == kSharedPrefixInt8;  // 8-bit codes
+  constexpr int KV = (MODE == kPagedPrefillInt8 || MODE == kSharedPrefixInt8) ? kKvInt8 : kKvFp8;
+  constexpr bool SHARED = MODE == kSharedPrefix || MODE == kSharedPrefixFp8 || MODE == kSharedPrefixInt8;
   // Two tiles of K and two of V: tile t sits in half t % 2.
   __shared__ __attribute__((aligned(1024))) half_t kbuf[2 * kTileHalfs];
   __shared__ __attribute__((aligned(1024))) half_t vbuf[2 * kTileHalfs];
@@ -496,8 +498,8 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       for (int j = 0; j < 4; ++j) {
         const int chunk = 4 * (lane & 3) + j;
         const uint4_t ck = raw_k[j >> 1], cv = raw_v[j >> 1];
-        const half8_t kh = fp8x8_to_half((j & 1) ? uint2_t{ck[2], ck[3]} : uint2_t{ck[0], ck[1]});
-        const half8_t vh = fp8x8_to_half((j & 1) ? uint2_t{cv[2], cv[3]} : uint2_t{cv[0], cv[1]});
+        const half8_t kh = codes_to_half<KV>((j & 1) ? uint2_t{ck[2], ck[3]} : uint2_t{ck[0], ck[1]});
+        const half8_t vh = codes_to_half<KV>((j & 1) ? uint2_t{cv[2], cv[3]} : uint2_t{cv[0], cv[1]});
         *(lds_half8_t *)(uintptr_t)(k_lds + row_at + 16u * (uint32_t)(chunk ^ r)) = kh;
         *(lds_half8_t *)(uintptr_t)(v_lds + row_at + 16u * (uint32_t)(chunk ^ (2 * (r & 7)))) = vh;
       }
@@ -780,7 +782,7 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
                          const float *fp8_scales, const int32_t *block_table, int32_t batch, int32_t num_q_heads,
                          int32_t num_kv_heads, int64_t num_pages, int32_t shared_pages,
                          int32_t page_shift, float *part_o, float *part_lse, float softmax_scale,
-                         hipStream_t stream, int *splits_out) {
+                         hipStream_t stream, int *splits_out, int format) {
   const char *what = "shared_prefix";
   const int group = num_q_heads / num_kv_heads;
   LITEKV_REQUIRE(group >= 1 && group <= 16, "%s: %d query heads per kv head unsupported", what, group);
@@ -805,18 +807,18 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
   PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
   PrefixTask task{part_o, part_lse, q_batch_stride, batch, num_q_heads, prefix_keys, keys_per_split};
   const dim3 grid((unsigned)num_kv_heads, (unsigned)col_blocks, (unsigned)splits);
-  if (fp8_scales != nullptr) {
-    hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kSharedPrefixFp8>, grid, dim3(kTiledWaves * kWave), 0,
-                       stream, static_cast<const half_t *>(q), (int64_t)0, (half_t *)nullptr,
-                       (int64_t)0, paged, packed, task, (const int32_t *)nullptr,
-                       (const int32_t *)nullptr, (const int32_t *)nullptr, group, 1, group, 1,
-                       softmax_scale * kLog2eP);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(kTiledWaves * kWave), 0, stream,
+                       static_cast<const half_t *>(q), (int64_t)0, (half_t *)nullptr, (int64_t)0,
+                       paged, packed, task, (const int32_t *)nullptr, (const int32_t *)nullptr,
+                       (const int32_t *)nullptr, group, 1, group, 1, softmax_scale * kLog2eP);
+  };
+  if (fp8_scales != nullptr && format == kKvInt8) {
+    launch(varlen_prefill_tiled_kernel<kSharedPrefixInt8>);
+  } else if (fp8_scales != nullptr) {
+    launch(varlen_prefill_tiled_kernel<kSharedPrefixFp8>);
   } else {
-    hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kSharedPrefix>, grid, dim3(kTiledWaves * kWave), 0,
-                       stream, static_cast<const half_t *>(q), (int64_t)0, (half_t *)nullptr,
-                       (int64_t)0, paged, packed, task, (const int32_t *)nullptr,
-                       (const int32_t *)nullptr, (const int32_t *)nullptr, group, 1, group, 1,
-                       softmax_scale * kLog2eP);
+    launch(varlen_prefill_tiled_kernel<kSharedPrefix>);
   }
   *splits_out = splits;
   return check_launch(what);
@@ -833,7 +835,8 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
                                 int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
                                 int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
                                 int64_t num_pages, int32_t max_q_len, float softmax_scale,
-                                void *stream, bool fp8) {
+                                void *stream, int format) {
+  const bool fp8 = format != kKvF16;  // a pool of 8-bit codes
   int rc = validate_prefill(what, q, q_token_stride, out, out_token_stride, batch, num_q_heads,
                             num_kv_heads, head_dim, max_q_len);
   if (rc != LITEKV_OK) return rc;
@@ -857,18 +860,19 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
   const PrefillShape s = prefill_shape(group, max_q_len);
   LITEKV_REQUIRE(s.row_blocks <= 65535u, "%s: max_q_len %d too large", what, max_q_len);
   const dim3 grid((unsigned)(num_kv_heads * s.head_splits), s.row_blocks, (unsigned)batch);
-  if (fp8) {
-    hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kPagedPrefillFp8>, grid, dim3(kTiledWaves * kWave),
-                       0, static_cast<hipStream_t>(stream), static_cast<const half_t *>(q),
-                       q_token_stride, static_cast<half_t *>(out), out_token_stride, paged, packed,
-                       PrefixTask{}, cu_q_lens, (const int32_t *)nullptr, context_lens, group,
-                       s.head_splits, s.heads_per_wg, s.row_tiles, softmax_scale * kLog2eP);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, grid, dim3(kTiledWaves * kWave), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
+                       out_token_stride, paged, packed, PrefixTask{}, cu_q_lens,
+                       (const int32_t *)nullptr, context_lens, group, s.head_splits, s.heads_per_wg,
+                       s.row_tiles, softmax_scale * kLog2eP);
+  };
+  if (format == kKvInt8) {
+    launch(varlen_prefill_tiled_kernel<kPagedPrefillInt8>);
+  } else if (format == kKvFp8) {
+    launch(varlen_prefill_tiled_kernel<kPagedPrefillFp8>);
   } else {
-    hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kPagedPrefill>, grid, dim3(kTiledWaves * kWave), 0,
-                       static_cast<hipStream_t>(stream), static_cast<const half_t *>(q),
-                       q_token_stride, static_cast<half_t *>(out), out_token_stride, paged, packed,
-                       PrefixTask{}, cu_q_lens, (const int32_t *)nullptr, context_lens, group,
-                       s.head_splits, s.heads_per_wg, s.row_tiles, softmax_scale * kLog2eP);
+    launch(varlen_prefill_tiled_kernel<kPagedPrefill>);
   }
   return check_launch(what);
 }
@@ -884,7 +888,8 @@ extern "C" int litekv_paged_prefill(const void *q, int64_t q_token_stride, const
   return litekv::launch_paged_prefill("paged_prefill", q, q_token_stride, kv_pool, nullptr, block_table,
                                       block_table_stride, cu_q_lens, context_lens, out,
                                       out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
-                                      page_size, num_pages, max_q_len, softmax_scale, stream, false);
+                                      page_size, num_pages, max_q_len, softmax_scale, stream,
+                                      litekv::kKvF16);
 }
 
 extern "C" int litekv_paged_prefill_fp8(const void *q, int64_t q_token_stride, const void *kv_pool,
@@ -898,7 +903,23 @@ extern "C" int litekv_paged_prefill_fp8(const void *q, int64_t q_token_stride, c
   return litekv::launch_paged_prefill("paged_prefill_fp8", q, q_token_stride, kv_pool, kv_scales,
                                       block_table, block_table_stride, cu_q_lens, context_lens, out,
                                       out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
-                                      page_size, num_pages, max_q_len, softmax_scale, stream, true);
+                                      page_size, num_pages, max_q_len, softmax_scale, stream,
+                                      litekv::kKvFp8);
+}
+
+extern "C" int litekv_paged_prefill_int8(const void *q, int64_t q_token_stride, const void *kv_pool,
+                                         const float *kv_scales, const int32_t *block_table,
+                                         int32_t block_table_stride, const int32_t *cu_q_lens,
+                                         const int32_t *context_lens, void *out,
+                                         int64_t out_token_stride, int32_t batch,
+                                         int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                         int32_t page_size, int64_t num_pages, int32_t max_q_len,
+                                         float softmax_scale, void *stream) {
+  return litekv::launch_paged_prefill("paged_prefill_int8", q, q_token_stride, kv_pool, kv_scales,
+                                      block_table, block_table_stride, cu_q_lens, context_lens, out,
+                                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
+                                      page_size, num_pages, max_q_len, softmax_scale, stream,
+                                      litekv::kKvInt8);
 }
 
 extern "C" int litekv_varlen_prefill(const void *q, int64_t q_token_stride, const void *k,

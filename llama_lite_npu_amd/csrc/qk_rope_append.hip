@@ -26,9 +26,10 @@ __device__ __forceinline__ float row_sum(float v) {
   return v;
 }
 
-// FP8: the pool holds E4M3 codes; `scales` are its per-head scales (K heads, then V heads) and a
-// row is quantised on its way in, exactly as kv_append_fp8_kernel would quantise the fp16 row.
-template <bool FP8>
+// KV kKvFp8 / kKvInt8: the pool holds 8-bit codes; `scales` are its per-head scales (K heads, then
+// V heads) and a row is quantised on its way in, exactly as kv_append_q8_kernel would quantise
+// the fp16 row.
+template <int KV>
 __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
     half_t *__restrict__ q, int64_t q_stride, const half_t *__restrict__ k, int64_t k_stride,
     const half_t *__restrict__ v, int64_t v_stride, const half_t *__restrict__ q_weight,
@@ -47,8 +48,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
   // stores 8 elements of head `kv_head` (K heads first, then V heads) of the token's slot
   auto store_row = [&](int kv_head, half8_t x) {
     const int64_t at = (slot * (int64_t)(2 * num_kv_heads) + kv_head) * kHeadDim + 8 * l16;
-    if constexpr (FP8) {
-      *(uint2_t *)(static_cast<uint8_t *>(pool_any) + at) = half8_to_fp8(x, 1.0f / scales[kv_head]);
+    if constexpr (KV != kKvF16) {
+      *(uint2_t *)(static_cast<uint8_t *>(pool_any) + at) =
+          half_to_codes<KV>(x, 1.0f / scales[kv_head]);
     } else {
       *(half8_t *)(static_cast<half_t *>(pool_any) + at) = x;
     }
@@ -119,7 +121,7 @@ static int launch_qk_epilogue(const char *what, void *q, int64_t q_token_stride,
                               const void *q_norm_weight, const void *k_norm_weight,
                               const void *cos_rows, const void *sin_rows,
                               int64_t cos_sin_token_stride, const int32_t *slot_mapping,
-                              void *kv_pool, const float *fp8_scales, bool fp8, int32_t num_tokens,
+                              void *kv_pool, const float *fp8_scales, int format, int32_t num_tokens,
                               int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                               int64_t num_slots, float rms_eps, void *stream) {
   LITEKV_REQUIRE(num_tokens >= 0, "%s: num_tokens %d < 0", what, num_tokens);
@@ -132,7 +134,7 @@ static int launch_qk_epilogue(const char *what, void *q, int64_t q_token_stride,
     return LITEKV_OK;
   }
   LITEKV_REQUIRE(q && k && v && slot_mapping && kv_pool, "%s: null pointer", what);
-  LITEKV_REQUIRE(!fp8 || fp8_scales != nullptr, "%s: scales is null", what);
+  LITEKV_REQUIRE(format == kKvF16 || fp8_scales != nullptr, "%s: scales is null", what);
   LITEKV_REQUIRE((q_norm_weight == nullptr) == (k_norm_weight == nullptr),
                  "%s: q_norm_weight and k_norm_weight go together", what);
   LITEKV_REQUIRE((cos_rows == nullptr) == (sin_rows == nullptr), "%s: cos and sin go together", what);
@@ -155,7 +157,9 @@ static int launch_qk_epilogue(const char *what, void *q, int64_t q_token_stride,
   const int64_t total_rows = (int64_t)num_tokens * (num_q_heads + 2 * num_kv_heads);
   const int64_t blocks = (total_rows * kLanesPerRow + 255) / 256;
   LITEKV_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many tokens", what);
-  auto kernel = fp8 ? qk_norm_rope_append_kernel<true> : qk_norm_rope_append_kernel<false>;
+  auto kernel = format == kKvFp8    ? qk_norm_rope_append_kernel<kKvFp8>
+                : format == kKvInt8 ? qk_norm_rope_append_kernel<kKvInt8>
+                                    : qk_norm_rope_append_kernel<kKvF16>;
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<half_t *>(q), q_token_stride, static_cast<const half_t *>(k),
                      k_token_stride, static_cast<const half_t *>(v), v_token_stride,
@@ -178,8 +182,8 @@ extern "C" int litekv_qk_norm_rope_append(void *q, int64_t q_token_stride, const
                                           float rms_eps, void *stream) {
   return litekv::launch_qk_epilogue("qk_norm_rope_append", q, q_token_stride, k, k_token_stride, v,
                                     v_token_stride, q_norm_weight, k_norm_weight, cos_rows, sin_rows,
-                                    cos_sin_token_stride, slot_mapping, kv_pool, nullptr, false,
-                                    num_tokens, num_q_heads, num_kv_heads, head_dim, num_slots,
+                                    cos_sin_token_stride, slot_mapping, kv_pool, nullptr,
+                                    litekv::kKvF16, num_tokens, num_q_heads, num_kv_heads, head_dim, num_slots,
                                     rms_eps, stream);
 }
 
@@ -196,6 +200,23 @@ extern "C" int litekv_qk_norm_rope_append_fp8(void *q, int64_t q_token_stride, c
   return litekv::launch_qk_epilogue("qk_norm_rope_append_fp8", q, q_token_stride, k, k_token_stride,
                                     v, v_token_stride, q_norm_weight, k_norm_weight, cos_rows,
                                     sin_rows, cos_sin_token_stride, slot_mapping, kv_pool_fp8, scales,
-                                    true, num_tokens, num_q_heads, num_kv_heads, head_dim, num_slots,
-                                    rms_eps, stream);
+                                    litekv::kKvFp8, num_tokens, num_q_heads, num_kv_heads, head_dim,
+                                    num_slots, rms_eps, stream);
+}
+
+extern "C" int litekv_qk_norm_rope_append_int8(void *q, int64_t q_token_stride, const void *k,
+                                               int64_t k_token_stride, const void *v,
+                                               int64_t v_token_stride, const void *q_norm_weight,
+                                               const void *k_norm_weight, const void *cos_rows,
+                                               const void *sin_rows, int64_t cos_sin_token_stride,
+                                               const int32_t *slot_mapping, void *kv_pool_int8,
+                                               const float *scales, int32_t num_tokens,
+                                               int32_t num_q_heads, int32_t num_kv_heads,
+                                               int32_t head_dim, int64_t num_slots, float rms_eps,
+                                               void *stream) {
+  return litekv::launch_qk_epilogue("qk_norm_rope_append_int8", q, q_token_stride, k, k_token_stride,
+                                    v, v_token_stride, q_norm_weight, k_norm_weight, cos_rows,
+                                    sin_rows, cos_sin_token_stride, slot_mapping, kv_pool_int8,
+                                    scales, litekv::kKvInt8, num_tokens, num_q_heads, num_kv_heads,
+                                    head_dim, num_slots, rms_eps, stream);
 }

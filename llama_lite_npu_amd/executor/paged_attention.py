@@ -57,7 +57,8 @@ class PagedKVCacheManager:
             torch.empty((self.max_tokens, 2 * self.num_kv_heads, self.head_dim), dtype=dtype, device=device)
             for _ in range(self.num_layers)
         ]
-        self.is_fp8 = dtype in (torch.uint8, torch.float8_e4m3fn)
+        # pools of 8-bit codes (fp8 E4M3 or int8) carry one scale per head
+        self.is_fp8 = dtype in (torch.uint8, torch.float8_e4m3fn, torch.int8)
         self.kv_scales = [
             torch.ones(2 * self.num_kv_heads, dtype=torch.float32, device=device) if self.is_fp8 else None
             for _ in range(self.num_layers)
@@ -71,7 +72,7 @@ class PagedKVCacheManager:
         self.num_free_pages = self.num_pages
 
     def set_kv_scales(self, layer: int, k_scales, v_scales) -> None:
-        """Per-head scales of an fp8 layer (value = code * scale); set them before anything is cached."""
+        """Per-head scales of an fp8 or int8 layer (value = code * scale); set them before anything is cached."""
         if not self.is_fp8:
             raise ValueError("fp16 pools have no scales")
         both = torch.cat([torch.as_tensor(k_scales, dtype=torch.float32).reshape(-1),

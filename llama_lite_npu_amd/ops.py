@@ -37,11 +37,13 @@ def _dev_half(name: str, t: torch.Tensor) -> None:
 
 
 FP8_DTYPES = (torch.uint8, torch.float8_e4m3fn)
+INT8_DTYPES = (torch.int8,)
 
 
 def _dev_pool(name: str, t: torch.Tensor) -> None:
     _need(t.is_cuda, f"{name} must live on the GPU")
-    _need(t.dtype == torch.float16 or t.dtype in FP8_DTYPES, f"{name} must be float16 or fp8, got {t.dtype}")
+    _need(t.dtype == torch.float16 or t.dtype in FP8_DTYPES + INT8_DTYPES,
+          f"{name} must be float16, fp8 or int8, got {t.dtype}")
 
 
 def is_fp8_pool(kv_pool: torch.Tensor) -> bool:
@@ -49,9 +51,25 @@ def is_fp8_pool(kv_pool: torch.Tensor) -> bool:
     return kv_pool.dtype in FP8_DTYPES
 
 
+def is_int8_pool(kv_pool: torch.Tensor) -> bool:
+    """An int8 pool holds one signed 8-bit code per element (a torch.int8 tensor)."""
+    return kv_pool.dtype in INT8_DTYPES
+
+
+def is_quantised_pool(kv_pool: torch.Tensor) -> bool:
+    """A pool of 8-bit codes (fp8 or int8) with one fp32 scale per kv head: value = code * scale."""
+    return is_fp8_pool(kv_pool) or is_int8_pool(kv_pool)
+
+
+def _q8_entry(lib, stem: str, kv_pool: torch.Tensor):
+    """The library's entry point `stem` for the pool's 8-bit format (litekv_<stem>_fp8 / _int8)."""
+    return getattr(lib, f"litekv_{stem}_{'int8' if is_int8_pool(kv_pool) else 'fp8'}")
+
+
 def _dev_fp8_pool(kv_pool: torch.Tensor, scales: Optional[torch.Tensor], num_kv_heads: int) -> None:
-    _need(kv_pool.is_cuda and is_fp8_pool(kv_pool), f"kv_pool must be an fp8 (uint8 / float8_e4m3fn) GPU tensor, got {kv_pool.dtype}")
-    _need(scales is not None, "an fp8 pool needs its per-head scales")
+    _need(kv_pool.is_cuda and is_quantised_pool(kv_pool),
+          f"kv_pool must be an fp8 (uint8 / float8_e4m3fn) or int8 GPU tensor, got {kv_pool.dtype}")
+    _need(scales is not None, "a pool of 8-bit codes needs its per-head scales")
     _need(scales.is_cuda and scales.dtype == torch.float32 and scales.is_contiguous()
           and scales.numel() == 2 * num_kv_heads, "scales must be float32 [2 * Hkv] on the GPU (K heads, then V heads)")
 
@@ -93,9 +111,10 @@ def kv_append(k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor, kv_p
                                     _ptr(kv_pool), t, hkv, d, slots, _stream()))
 
 
-def kv_append_fp8(k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor, kv_pool: torch.Tensor,
-                  scales: torch.Tensor) -> None:
-    """kv_pool[slot_mapping[t]] = e4m3(concat(k[t], v[t]) / scale of the head) for every token t;
+def kv_append_quantised(k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor, kv_pool: torch.Tensor,
+                        scales: torch.Tensor) -> None:
+    """kv_pool[slot_mapping[t]] = code(concat(k[t], v[t]) / scale of the head) for every token t, in the
+    pool's format (E4M3 for a uint8 / float8_e4m3fn pool, int8 for a torch.int8 pool);
     scales is float32 [2 * Hkv]: K-head scales, then V-head scales."""
     _dev_half("k", k), _dev_half("v", v)
     slots, hkv, d, _, _ = pool_geometry(kv_pool, 1)
@@ -105,8 +124,12 @@ def kv_append_fp8(k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor, 
     t = k.shape[0]
     _need(slot_mapping.numel() == t, "slot_mapping must hold one slot per token")
     lib = _lib.load()
-    _lib.check(lib.litekv_kv_append_fp8(_ptr(k), _ptr(v), _rows("k", k), _rows("v", v), _ptr(slot_mapping),
-                                        _ptr(kv_pool), _ptr(scales), t, hkv, d, slots, _stream()))
+    _lib.check(_q8_entry(lib, "kv_append", kv_pool)(_ptr(k), _ptr(v), _rows("k", k), _rows("v", v),
+                                                    _ptr(slot_mapping), _ptr(kv_pool), _ptr(scales), t, hkv, d,
+                                                    slots, _stream()))
+
+
+kv_append_fp8 = kv_append_quantised     # the name from before int8 pools
 
 
 def page_dequant(kv_pool: torch.Tensor, dst_pool: torch.Tensor, src_ids: torch.Tensor,
@@ -122,8 +145,9 @@ def page_dequant(kv_pool: torch.Tensor, dst_pool: torch.Tensor, src_ids: torch.T
         dst_ids = _dev_i32("dst_ids", dst_ids)
         _need(dst_ids.numel() == src_ids.numel(), "src_ids and dst_ids differ in length")
     lib = _lib.load()
-    _lib.check(lib.litekv_page_dequant(_ptr(kv_pool), _ptr(dst_pool), _ptr(src_ids), _ptr(dst_ids), src_ids.numel(),
-                                       _ptr(scales), hkv, d, page_size, n_src, n_dst, _stream()))
+    fn = lib.litekv_page_dequant_int8 if is_int8_pool(kv_pool) else lib.litekv_page_dequant
+    _lib.check(fn(_ptr(kv_pool), _ptr(dst_pool), _ptr(src_ids), _ptr(dst_ids), src_ids.numel(),
+                  _ptr(scales), hkv, d, page_size, n_src, n_dst, _stream()))
 
 
 def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor,
@@ -137,7 +161,7 @@ def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_
     each token's position. An fp8 pool (with its ``kv_scales``) receives the quantised rows. Returns q."""
     _dev_half("q", q), _dev_half("k", k), _dev_half("v", v)
     slots, hkv, d, _, _ = pool_geometry(kv_pool, 1)
-    fp8 = is_fp8_pool(kv_pool)
+    fp8 = is_quantised_pool(kv_pool)
     if fp8:
         _dev_fp8_pool(kv_pool, kv_scales, hkv)
     else:
@@ -163,7 +187,7 @@ def qk_norm_rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_
     _need(slot_mapping.numel() == t, "slot_mapping must hold one slot per token")
     lib = _lib.load()
     if fp8:
-        _lib.check(lib.litekv_qk_norm_rope_append_fp8(
+        _lib.check(_q8_entry(lib, "qk_norm_rope_append", kv_pool)(
             _ptr(q), _rows("q", q), _ptr(k), _rows("k", k), _ptr(v), _rows("v", v), _ptr(q_norm_weight),
             _ptr(k_norm_weight), _ptr(cos), _ptr(sin), cs_stride, _ptr(slot_mapping), _ptr(kv_pool),
             _ptr(kv_scales), t, hq, hkv, d, slots, float(rms_eps), _stream()))
@@ -395,7 +419,7 @@ def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
                             page_size=plan.page_size, schedule="splits", kv_scales=kv_scales,
                             k_new=k_new, v_new=v_new)
     _dev_half("q", q)
-    fp8 = is_fp8_pool(kv_pool)
+    fp8 = is_quantised_pool(kv_pool)
     if not fp8:
         _dev_half("kv_pool", kv_pool)
     _need(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2], "q must be [B, Hq, D] with contiguous heads")
@@ -422,13 +446,13 @@ def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
     if fp8:
         _dev_fp8_pool(kv_pool, kv_scales, hkv)
         if plan.shared_pages > 0:
-            _lib.check(lib.litekv_paged_decode_prefix_fp8(
+            _lib.check(_q8_entry(lib, "paged_decode_prefix", kv_pool)(
                 _ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(plan.block_table), _ptr(plan.seq_lens),
                 _ptr(plan.buffer), plan.plan_bytes, _ptr(k_new), _ptr(v_new), kn_stride, vn_stride, _ptr(out),
                 _ptr(plan.workspace), plan.workspace_bytes, b, hq, hkv, d, plan.page_size, n_pages, plan.bt_stride,
                 plan.chunks, plan.shared_pages, float(softmax_scale), _stream()))
             return out
-        _lib.check(lib.litekv_paged_decode_balanced_fp8(
+        _lib.check(_q8_entry(lib, "paged_decode_balanced", kv_pool)(
             _ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(plan.seq_lens), _ptr(plan.buffer),
             plan.plan_bytes, _ptr(k_new), _ptr(v_new), kn_stride, vn_stride, _ptr(out), _ptr(plan.workspace),
             plan.workspace_bytes, b, hq, hkv, d, plan.page_size, n_pages, plan.bt_stride, plan.chunks,
@@ -474,7 +498,7 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
     sequence is written at logical position seq_lens[b] - 1 by the same launch and attended.
     """
     _dev_half("q", q)
-    if not is_fp8_pool(kv_pool):
+    if not is_quantised_pool(kv_pool):
         _dev_half("kv_pool", kv_pool)
     _need(q.dim() == 3 and q.stride(2) == 1 and q.stride(1) == q.shape[2], "q must be [B, Hq, D] with contiguous heads")
     b, hq, d = q.shape
@@ -494,7 +518,7 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
             plan = DecodePlan(block_table, seq_lens, hq, hkv, n_pages, chunks, page_size, shared_pages)
         return decode_step(q, kv_pool, plan, None, None, softmax_scale, out, kv_scales)
 
-    fp8 = is_fp8_pool(kv_pool)
+    fp8 = is_quantised_pool(kv_pool)
     if fp8:
         _dev_fp8_pool(kv_pool, kv_scales, hkv)
         _need(stage == "both", "an fp8 pool is read by both stages in one call")
@@ -526,14 +550,14 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
         tail = (_ptr(out), _ptr(workspace), ws_bytes, b, hq, hkv, d, page_size, n_pages, max_splits,
                 min_pages_per_split, float(softmax_scale), _stream())
         if fp8:
-            _lib.check(lib.litekv_paged_decode_append_fp8(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales),
+            _lib.check(_q8_entry(lib, "paged_decode_append", kv_pool)(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales),
                                                           _ptr(block_table), block_table.stride(0), _ptr(seq_lens),
                                                           *rows, *tail))
         else:
             _lib.check(lib.litekv_paged_decode_append(_ptr(q), q_stride, _ptr(kv_pool), _ptr(block_table),
                                                       block_table.stride(0), _ptr(seq_lens), *rows, *tail))
     elif fp8:
-        _lib.check(lib.litekv_paged_decode_fp8(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(block_table),
+        _lib.check(_q8_entry(lib, "paged_decode", kv_pool)(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(block_table),
                                                block_table.stride(0), _ptr(seq_lens), _ptr(out), _ptr(workspace),
                                                ws_bytes, b, hq, hkv, d, page_size, n_pages, max_splits,
                                                min_pages_per_split, float(softmax_scale), _stream()))
@@ -585,7 +609,7 @@ def paged_prefill(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Ten
     """Causal varlen attention of packed q [T, Hq, D] over paged KV (history + the chunk itself).
     An fp8 pool (uint8 / float8_e4m3fn) comes with its per-head ``kv_scales``."""
     _dev_half("q", q)
-    fp8 = is_fp8_pool(kv_pool)
+    fp8 = is_quantised_pool(kv_pool)
     if not fp8:
         _dev_half("kv_pool", kv_pool)
         _need(kv_scales is None, "kv_scales belong to an fp8 pool")
@@ -608,7 +632,7 @@ def paged_prefill(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Ten
         out = torch.empty((t, hq, d), dtype=torch.float16, device=q.device)
     lib = _lib.load()
     if fp8:
-        _lib.check(lib.litekv_paged_prefill_fp8(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(block_table),
+        _lib.check(_q8_entry(lib, "paged_prefill", kv_pool)(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(block_table),
                                                 block_table.stride(0), _ptr(cu_q_lens), _ptr(context_lens),
                                                 _ptr(out), _rows("out", out), b, hq, hkv, d, page_size, n_pages,
                                                 int(max_q_len), float(softmax_scale), _stream()))

@@ -465,3 +465,58 @@ def test_fp8_append_uses_the_head_scales():
             assert np.all(np.abs(back[slot, 2 + h] - want_v) <= np.maximum(np.abs(want_v) * 2.0 ** -4,
                                                                            scales[2 + h] * 2.0 ** -10))
     assert np.all(np.abs(back[3, 3]) <= 448 * 0.004 + 1e-6)                    # a small scale saturates
+
+
+# ---- int8 storage ---------------------------------------------------------------------------------
+
+def test_int8_rounding_saturation_and_round_trip():
+    from oracle import int8
+
+    every = np.arange(-127, 128, dtype=np.float32)
+    assert np.array_equal(int8.encode(every), every.astype(np.int8))            # integers are fixed points
+    assert np.array_equal(int8.decode(int8.encode(every)), every)
+    ties = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, -126.5], dtype=np.float32)
+    assert int8.encode(ties).tolist() == [0, 2, 2, 0, -2, -2, 126, -126]        # halves go to the even integer
+    big = np.array([127.49, 127.5, 128.0, 1e9, -127.5, -128.0, -1e9], dtype=np.float32)
+    assert int8.encode(big).tolist() == [127, 127, 127, 127, -127, -127, -127]  # -128 is never produced
+    x = np.random.default_rng(5).normal(scale=60.0, size=4096).astype(np.float32)
+    back = int8.decode(int8.encode(x))
+    assert np.all(np.abs(back - np.clip(x, -127, 127)) <= 0.5)                  # half a step
+    assert np.all(np.diff(int8.decode(int8.encode(np.sort(x)))) >= 0)           # monotone
+
+
+def test_int8_encode_against_torch_round_and_clamp():
+    """An independent statement of the same rule: torch.round (half to even) then clamp, on every fp16
+    input of moderate size divided by a scale in fp32."""
+    import torch
+    from oracle import int8
+
+    halves = np.arange(0x10000, dtype=np.uint16).view(np.float16)
+    halves = halves[np.isfinite(halves) & (np.abs(halves.astype(np.float32)) <= 40.0)]
+    for scale in (1.0, 0.37, 0.011, 3.0):
+        y = halves.astype(np.float32) * (np.float32(1.0) / np.float32(scale))
+        want = torch.clamp(torch.round(torch.from_numpy(y)), -127, 127).to(torch.int8).numpy()
+        assert np.array_equal(int8.encode(y), want), scale
+
+
+def test_int8_append_uses_the_head_scales():
+    from oracle import int8
+
+    k = np.zeros((2, 2, 128), dtype=np.float16)
+    v = np.zeros((2, 2, 128), dtype=np.float16)
+    k[0, 0, :4] = [0.05, -0.05, 0.126, 10.0]       # scale 0.1: 0.5 -> 0, -0.5 -> 0, 1.26 -> 1, 100 -> 100
+    k[0, 1, :3] = [1.0, -3.0, 100.0]               # scale 0.5: 2, -6, 200 -> 127
+    v[1, 0, :2] = [0.25, -0.75]                    # scale 0.25: 1, -3
+    v[1, 1, :2] = [0.006, -2.0]                    # scale 0.004: 1.5 -> 2, -500 -> -127
+    scales = np.array([0.1, 0.5, 0.25, 0.004], dtype=np.float32)
+    pool = np.full((4, 4, 128), 0x55, dtype=np.int8)
+    int8.kv_append(k, v, np.array([2, 0]), pool, scales)
+    assert np.all(pool[[1, 3]] == 0x55)
+    # the fp16 inputs are not exactly the decimals written above: 0.05 (fp16) / 0.1 (fp32) is just
+    # under one half, -0.05 / 0.1 just above minus one half; both round to 0 either way
+    assert pool[2, 0, :4].tolist() == [0, 0, 1, 100]
+    assert pool[2, 1, :3].tolist() == [2, -6, 127]
+    assert pool[0, 2, :2].tolist() == [1, -3]
+    assert pool[0, 3, :2].tolist() == [2, -127]
+    back = int8.dequantize_pool(pool, scales)
+    assert back[2, 1, 2] == np.float32(127) * np.float32(0.5) and back[0, 3, 1] == np.float32(-127) * np.float32(0.004)
