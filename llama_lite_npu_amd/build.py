@@ -28,6 +28,7 @@ SOURCES = (
     "paged_decode.hip",
     "decode_advance.hip",
     "paged_prefill.hip",
+    "generic_attention.hip",
 )
 
 # Packed fp32 VALU forms are switched off for device code: the compiler would

@@ -54,6 +54,74 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
                          int32_t page_shift, float *part_o, float *part_lse, float softmax_scale,
                          hipStream_t stream, int *splits_out, int format);
 
+// ---- the plan of a balanced decode step (made by decode_plan_kernel in paged_decode.hip) -------
+// Plan buffer (int32 words): meta[kPlanMeta]; per sequence (first chunk, number of chunks it
+// spans); per sequence the position of its first 16-token page on the line; the chunk entries.
+constexpr int kPlanMeta = 16;      // int32 words of plan meta data
+constexpr int kEntryHeader = 8;    // int32 words of an entry before its page ids
+// plan meta words
+constexpr int kMetaTotal = 0, kMetaChunkPages = 1, kMetaChunks = 2, kMetaBatch = 3,
+              kMetaEntryStride = 4, kMetaKvHeads = 5, kMetaSkip = 6;
+
+__host__ __device__ __forceinline__ int round_up(int x, int m) { return (x + m - 1) / m * m; }
+__host__ __device__ __forceinline__ int plan_seq_info_offset() { return kPlanMeta; }
+__host__ __device__ __forceinline__ int plan_seq_before_offset(int batch) {
+  return kPlanMeta + round_up(2 * batch, 4);
+}
+__host__ __device__ __forceinline__ int plan_entries_offset(int batch) {
+  return plan_seq_before_offset(batch) + round_up(batch, 4);
+}
+
+// The cut of a line of `total` pages into `chunks` pieces whose sizes differ by at most one page:
+// the first `rem` chunks hold quot + 1 pages, the others quot (none when quot == 0).
+struct LineCut {
+  int quot, rem, big_end;  // big_end: pages covered by the larger chunks
+  __host__ __device__ LineCut(int total, int chunks)
+      : quot(total / chunks), rem(total - (total / chunks) * chunks), big_end(0) {
+    big_end = rem * (quot + 1);
+  }
+  __host__ __device__ int chunk_start(int c) const { return c * quot + (c < rem ? c : rem); }
+  __host__ __device__ int chunk_of(int f) const {
+    if (f < big_end) return f / (quot + 1);
+    return quot > 0 ? rem + (f - big_end) / quot : rem;
+  }
+};
+
+// Attention for the head dims the tuned kernels (128) do not take: 32, 64 and 256
+// (generic_attention.hip). A launch is a decode step (seq_lens), a paged prefill (cu_q_lens,
+// context_lens) or a packed prefill (kv_pool null; k, v, seq_starts, q_lens); `rows_per_seq` is
+// 1 for decode and the longest prompt or chunk otherwise. `format` is the pool's storage format
+// (kv_fp8.h); k_new / v_new fuse a decode step's append.
+struct GenericLaunch {
+  const void *q = nullptr;
+  int64_t q_row_stride = 0;
+  void *out = nullptr;
+  int64_t out_row_stride = 0;
+  void *kv_pool = nullptr;
+  const float *scales = nullptr;
+  int format = 0;
+  const int32_t *block_table = nullptr;  // or, for a balanced decode step, its plan:
+  const int32_t *plan = nullptr;
+  int32_t bt_stride = 0;
+  int32_t page_size = 16;
+  int64_t num_pages = 0;
+  const void *k = nullptr, *v = nullptr;
+  int64_t k_stride = 0, v_stride = 0;
+  const int32_t *seq_starts = nullptr;
+  const int32_t *seq_lens = nullptr;
+  const int32_t *cu_q_lens = nullptr;
+  const int32_t *q_lens = nullptr;
+  const int32_t *context_lens = nullptr;
+  const void *k_new = nullptr, *v_new = nullptr;
+  int64_t k_new_stride = 0, v_new_stride = 0;
+  int32_t batch = 0, rows_per_seq = 1;
+  int32_t num_q_heads = 0, num_kv_heads = 0, head_dim = 0;
+  float softmax_scale = 1.0f;
+  void *stream = nullptr;
+};
+bool generic_head_dim(int32_t head_dim);
+int launch_generic_attention(const char *what, const GenericLaunch &a);
+
 // ---- device side ---------------------------------------------------------
 
 // 2^x on the transcendental unit (v_exp_f32); exp2(-inf) == 0.

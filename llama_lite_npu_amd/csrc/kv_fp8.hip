@@ -1,12 +1,12 @@
 // 8-bit KV pools (fp8 E4M3 or int8 codes, one fp32 scale per kv head): the append that quantises
 // K/V rows on their way into the pages, and the page dequantiser that turns pages back into fp16
 // rows.
-// The pool is [slots][2 * Hkv][128] bytes, K heads then V heads as in the fp16 pool, so a page is
+// The pool is [slots][2 * Hkv][head_dim] bytes, K heads then V heads as in the fp16 pool, so a page is
 // one contiguous run of half the size; scales[2 * Hkv] holds the K-head scales, then the V-head
 // scales.
 //
 // One work item handles 8 elements: 16 bytes of fp16 in, 8 bytes of codes out (append), or the
-// reverse (dequantise); a head row of 128 elements is 16 consecutive items, so accesses are
+// reverse (dequantise); a head row of 128 elements is 16 consecutive items (head_dim / 8 in general), so accesses are
 // coalesced on both sides.
 #include "kv_fp8.h"
 
@@ -17,7 +17,7 @@ __global__ __launch_bounds__(256) void kv_append_q8_kernel(
     const half8_t *__restrict__ k, const half8_t *__restrict__ v, int64_t k_stride8,
     int64_t v_stride8, const int32_t *__restrict__ slot_mapping, uint2_t *__restrict__ pool,
     const float *__restrict__ scales, int64_t total_items, int32_t items_per_half,
-    int64_t num_slots) {
+    int32_t items_per_head, int64_t num_slots) {
   const int64_t item = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (item >= total_items) return;
   const int32_t items_per_token = 2 * items_per_half;
@@ -27,7 +27,7 @@ __global__ __launch_bounds__(256) void kv_append_q8_kernel(
   if (slot < 0 || slot >= num_slots) return;
   const half8_t x = (c < items_per_half) ? k[token * k_stride8 + c]
                                          : v[token * v_stride8 + (c - items_per_half)];
-  const float inv_scale = 1.0f / scales[c / (kHeadDim / 8)];  // head index over K heads then V heads
+  const float inv_scale = 1.0f / scales[c / items_per_head];  // head index over K heads then V heads
   pool[slot * items_per_token + c] = half_to_codes<KV>(x, inv_scale);
 }
 
@@ -36,13 +36,13 @@ __global__ __launch_bounds__(256) void page_dequant_kernel(
     const uint2_t *__restrict__ src_pool, half8_t *__restrict__ dst_pool,
     const int32_t *__restrict__ src_ids, const int32_t *__restrict__ dst_ids,
     const float *__restrict__ scales, int32_t page_items, int32_t items_per_slot,
-    int64_t num_src_pages, int64_t num_dst_pages) {
+    int32_t items_per_head, int64_t num_src_pages, int64_t num_dst_pages) {
   const int64_t i = blockIdx.x;
   const int64_t sp = src_ids[i];
   const int64_t dp = dst_ids ? (int64_t)dst_ids[i] : i;
   if (sp < 0 || sp >= num_src_pages || dp < 0 || dp >= num_dst_pages) return;
   for (int c = blockIdx.y * 256 + threadIdx.x; c < page_items; c += gridDim.y * 256) {
-    const float scale = scales[(c % items_per_slot) / (kHeadDim / 8)];
+    const float scale = scales[(c % items_per_slot) / items_per_head];
     const half8_t raw = codes_to_half<KV>(__builtin_nontemporal_load(src_pool + sp * page_items + c));
     half8_t y;
 #pragma unroll
@@ -52,8 +52,8 @@ __global__ __launch_bounds__(256) void page_dequant_kernel(
 }
 
 static int check_scales_geometry(const char *what, int32_t num_kv_heads, int32_t head_dim) {
-  LITEKV_REQUIRE(head_dim == kHeadDim, "%s: head_dim %d unsupported (only %d)", what, head_dim,
-                 kHeadDim);
+  LITEKV_REQUIRE(head_dim == kHeadDim || generic_head_dim(head_dim),
+                 "%s: head_dim %d unsupported (32, 64, 128 or 256)", what, head_dim);
   LITEKV_REQUIRE(num_kv_heads > 0 && num_kv_heads <= 65535, "%s: num_kv_heads %d out of range", what,
                  num_kv_heads);
   return LITEKV_OK;
@@ -89,7 +89,7 @@ static int launch_kv_append_q8(const char *what, int format, const void *k, cons
                        static_cast<hipStream_t>(stream), static_cast<const half8_t *>(k),
                        static_cast<const half8_t *>(v), k_token_stride / 8, v_token_stride / 8,
                        slot_mapping, static_cast<uint2_t *>(kv_pool_fp8), scales, total,
-                       items_per_half, num_slots);
+                       items_per_half, head_dim / 8, num_slots);
   };
   if (format == kKvInt8) {
     launch(kv_append_q8_kernel<kKvInt8>);
@@ -128,7 +128,8 @@ static int launch_page_dequant(const char *what, int format, const void *kv_pool
     hipLaunchKernelGGL(kernel, dim3((unsigned)n, (unsigned)tiles), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<const uint2_t *>(kv_pool_fp8),
                        static_cast<half8_t *>(dst_pool), src_ids, dst_ids, scales,
-                       (int32_t)page_items, items_per_slot, num_src_pages, num_dst_pages);
+                       (int32_t)page_items, items_per_slot, head_dim / 8, num_src_pages,
+                       num_dst_pages);
   };
   if (format == kKvInt8) {
     launch(page_dequant_kernel<kKvInt8>);

@@ -701,13 +701,8 @@ __global__ __launch_bounds__(kWave) void paged_decode_merge_kernel(
 // more than the 3 us of a launch boundary.
 // ---------------------------------------------------------------------------------------------
 constexpr int kMaxWavesPerWg = 8;
-constexpr int kPlanMeta = 16;      // int32 words of plan meta data
-constexpr int kEntryHeader = 8;    // int32 words of an entry before its page ids
-// plan meta words
-constexpr int kMetaTotal = 0, kMetaChunkPages = 1, kMetaChunks = 2, kMetaBatch = 3,
-              kMetaEntryStride = 4, kMetaKvHeads = 5, kMetaSkip = 6;
-
-__host__ __device__ __forceinline__ int round_up(int x, int m) { return (x + m - 1) / m * m; }
+// (the layout of a plan buffer -- kPlanMeta, kEntryHeader, the meta words, plan_entries_offset,
+// LineCut -- is in common.h: the kernel for other head dims reads page ids from a plan too)
 
 // Step metadata that no launch of the decode kernel modifies (plan entries, sequence lengths) is
 // read through the constant address space: with a wavefront-uniform address such a load is
@@ -724,12 +719,6 @@ __host__ __device__ __forceinline__ int plan_entry_stride(int batch, int bt_stri
   const int64_t max_total = (int64_t)batch * bt_stride;
   const int max_chunk_pages = (int)((max_total + chunks - 1) / chunks);
   return round_up(kEntryHeader + max_chunk_pages, 4);
-}
-// Plan buffer (int32 words): meta[kPlanMeta], then per sequence (first chunk, number of
-// chunks it spans), then the chunk entries.
-__host__ __device__ __forceinline__ int plan_seq_info_offset() { return kPlanMeta; }
-__host__ __device__ __forceinline__ int plan_entries_offset(int batch) {
-  return kPlanMeta + round_up(2 * batch, 4);
 }
 
 // One block per sequence: places the sequence's pages on the line, fills the entries they fall
@@ -775,14 +764,10 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
   // the first `rem` chunks hold quot + 1 pages, the others quot (none when quot == 0). With a
   // fixed ceil(total / chunks) pages per chunk the last chunks would stay empty whenever total is
   // just above a multiple of chunks (5 % of the compute units idle at 18.004 pages per chunk).
-  const int quot = total / chunks;
-  const int rem = total - quot * chunks;
-  const int big_end = rem * (quot + 1);  // pages covered by the larger chunks
-  auto chunk_start = [&](int c) { return c * quot + (c < rem ? c : rem); };
-  auto chunk_of = [&](int f) {
-    if (f < big_end) return f / (quot + 1);
-    return quot > 0 ? rem + (f - big_end) / quot : rem;
-  };
+  const LineCut cut(total, chunks);
+  const int quot = cut.quot, rem = cut.rem;
+  auto chunk_start = [&](int c) { return cut.chunk_start(c); };
+  auto chunk_of = [&](int f) { return cut.chunk_of(f); };
   int32_t *entries = plan + plan_entries_offset(batch);
 
   if (b == 0) {
@@ -808,6 +793,7 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(
   my_pages = my_pages > 0 ? my_pages : 0;
   if (tid == 0) {
     const int c_first = chunk_of(before);
+    plan[plan_seq_before_offset(batch) + b] = before;
     plan[plan_seq_info_offset() + 2 * b] = c_first;
     plan[plan_seq_info_offset() + 2 * b + 1] =
         my_pages > 0 ? chunk_of(before + my_pages - 1) - c_first + 1 : 0;
@@ -1296,8 +1282,8 @@ static int page_shift_of(int32_t page_size) {
 static int validate_decode(const char *what, const DecodeArgs &a, size_t workspace_needed,
                            bool need_inputs) {
   LITEKV_REQUIRE(a.batch >= 0 && a.batch <= 65535, "%s: batch %d out of [0, 65535]", what, a.batch);
-  LITEKV_REQUIRE(a.head_dim == kHeadDim, "%s: head_dim %d unsupported (only %d)", what, a.head_dim,
-                 kHeadDim);
+  LITEKV_REQUIRE(a.head_dim == kHeadDim, "%s: head_dim %d unsupported (32, 64, 128 or 256)", what,
+                 a.head_dim);
   LITEKV_REQUIRE(page_shift_of(a.page_size) >= 0, "%s: page_size %d unsupported (16, 32 or 64)",
                  what, a.page_size);
   LITEKV_REQUIRE(a.num_q_heads > 0 && a.num_q_heads <= 65535, "%s: num_q_heads %d out of range",
@@ -1334,6 +1320,42 @@ static int validate_decode(const char *what, const DecodeArgs &a, size_t workspa
   return LITEKV_OK;
 }
 
+// A decode step at a head dim the tuned kernels do not take (32, 64, 256): one launch of the
+// kernel of generic_attention.hip writes the final rows, whatever the schedule asked for; no
+// workspace is used. `plan` replaces the block table for the balanced entry points, which are
+// not given one.
+static int launch_generic_decode(const char *what, const DecodeArgs &a, const float *scales,
+                                 int format, const int32_t *plan = nullptr) {
+  LITEKV_REQUIRE(a.batch == 0 || a.seq_lens != nullptr, "%s: null pointer", what);
+  GenericLaunch g;
+  g.q = a.q;
+  g.q_row_stride = a.q_batch_stride;
+  g.out = a.out;
+  g.out_row_stride = (int64_t)a.num_q_heads * a.head_dim;
+  g.kv_pool = const_cast<void *>(a.kv_pool);
+  g.scales = scales;
+  g.format = scales != nullptr ? format : kKvF16;
+  g.block_table = plan != nullptr ? nullptr : a.block_table;
+  g.plan = plan;
+  g.bt_stride = a.block_table_stride;
+  g.page_size = a.page_size;
+  g.num_pages = a.num_pages;
+  g.seq_lens = a.seq_lens;
+  g.k_new = a.k_new;
+  g.v_new = a.v_new;
+  g.k_new_stride = a.k_new_stride;
+  g.v_new_stride = a.v_new_stride;
+  g.batch = a.batch;
+  g.rows_per_seq = 1;
+  g.num_q_heads = a.num_q_heads;
+  g.num_kv_heads = a.num_kv_heads;
+  g.head_dim = a.head_dim;
+  g.softmax_scale = a.softmax_scale;
+  g.stream = a.stream;
+  LITEKV_REQUIRE(a.kv_pool != nullptr || a.batch == 0, "%s: null pointer", what);
+  return launch_generic_attention(what, g);
+}
+
 // ---- schedule "splits" ----
 
 static size_t splits_workspace_bytes(int64_t batch, int64_t hq, int64_t d, int64_t s) {
@@ -1364,6 +1386,7 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
                                          : "paged_decode_split_fp8";
   int rc = check_split_plan(what, max_splits, min_pages_per_split);
   if (rc != LITEKV_OK) return rc;
+  if (a.head_dim != kHeadDim) return launch_generic_decode(what, a, fp8_scales, format);
   rc = validate_decode(what, a,
                        splits_workspace_bytes(a.batch, a.num_q_heads, a.head_dim, max_splits), true);
   if (rc != LITEKV_OK) return rc;
@@ -1431,6 +1454,10 @@ static int launch_merge(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   const char *what = "paged_decode_merge";
   int rc = check_split_plan(what, max_splits, min_pages_per_split);
   if (rc != LITEKV_OK) return rc;
+  if (a.head_dim != kHeadDim && generic_head_dim(a.head_dim)) {  // launch_generic_decode wrote the rows
+    clear_error();
+    return LITEKV_OK;
+  }
   rc = validate_decode(what, a,
                        splits_workspace_bytes(a.batch, a.num_q_heads, a.head_dim, max_splits),
                        false);
@@ -1626,6 +1653,23 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   DecodeArgs a{q, q_batch_stride, kv_pool, block_table ? block_table : &dummy_table,
                block_table_stride, seq_lens, out, workspace, workspace_bytes, batch, num_q_heads,
                num_kv_heads, head_dim, page_size, num_pages, softmax_scale, stream};
+  if (head_dim != kHeadDim) {
+    // other head dims: the generic kernel, which takes its page ids from the block table where
+    // the caller gave one (then shared pages are attended like any others), else from the plan
+    a.k_new = k_new;
+    a.v_new = v_new;
+    a.k_new_stride = k_new_stride;
+    a.v_new_stride = v_new_stride;
+    if (block_table == nullptr && batch > 0) {
+      LITEKV_REQUIRE(plan != nullptr && aligned16(plan), "%s: plan must be a 16-byte aligned buffer",
+                     what);
+      const size_t need_plan = plan_bytes_for(batch, sub_stride, num_kv_heads, chunks);
+      LITEKV_REQUIRE(plan_bytes >= need_plan, "%s: plan buffer of %zu bytes needed, got %zu", what,
+                     need_plan, plan_bytes);
+    }
+    return launch_generic_decode(what, a, fp8_scales, format,
+                                 block_table == nullptr ? static_cast<const int32_t *>(plan) : nullptr);
+  }
   const size_t ws_need = shared_pages > 0
                              ? prefix_workspace_bytes(batch, num_q_heads, head_dim, chunks)
                              : balanced_workspace_bytes(batch, num_q_heads, head_dim, chunks);

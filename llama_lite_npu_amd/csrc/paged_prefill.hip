@@ -747,8 +747,8 @@ static int validate_prefill(const char *what, const void *q, int64_t q_stride, c
                             int64_t out_stride, int32_t batch, int32_t hq, int32_t hkv,
                             int32_t head_dim, int32_t max_q_len) {
   LITEKV_REQUIRE(batch >= 0 && batch <= 65535, "%s: batch %d out of [0, 65535]", what, batch);
-  LITEKV_REQUIRE(head_dim == kHeadDim, "%s: head_dim %d unsupported (only %d)", what, head_dim,
-                 kHeadDim);
+  LITEKV_REQUIRE(head_dim == kHeadDim, "%s: head_dim %d unsupported (32, 64, 128 or 256)", what,
+                 head_dim);
   LITEKV_REQUIRE(hq > 0 && hkv > 0 && hq % hkv == 0 && hq <= 65535,
                  "%s: num_q_heads %d / num_kv_heads %d invalid", what, hq, hkv);
   LITEKV_REQUIRE(hq / hkv <= 16, "%s: %d query heads per kv head unsupported (max 16)", what,
@@ -837,6 +837,34 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
                                 int64_t num_pages, int32_t max_q_len, float softmax_scale,
                                 void *stream, int format) {
   const bool fp8 = format != kKvF16;  // a pool of 8-bit codes
+  if (head_dim != kHeadDim && generic_head_dim(head_dim)) {  // see generic_attention.hip
+    LITEKV_REQUIRE(max_q_len >= 0, "%s: max_q_len %d < 0", what, max_q_len);
+    LITEKV_REQUIRE(batch == 0 || max_q_len == 0 || (kv_pool && block_table && cu_q_lens),
+                   "%s: null pointer", what);
+    LITEKV_REQUIRE(!fp8 || kv_scales, "%s: null pointer (kv_scales)", what);
+    GenericLaunch g;
+    g.q = q;
+    g.q_row_stride = q_token_stride;
+    g.out = out;
+    g.out_row_stride = out_token_stride;
+    g.kv_pool = const_cast<void *>(kv_pool);
+    g.scales = kv_scales;
+    g.format = format;
+    g.block_table = block_table;
+    g.bt_stride = block_table_stride;
+    g.page_size = page_size;
+    g.num_pages = num_pages;
+    g.cu_q_lens = cu_q_lens;
+    g.context_lens = context_lens;
+    g.batch = batch;
+    g.rows_per_seq = max_q_len;
+    g.num_q_heads = num_q_heads;
+    g.num_kv_heads = num_kv_heads;
+    g.head_dim = head_dim;
+    g.softmax_scale = softmax_scale;
+    g.stream = stream;
+    return launch_generic_attention(what, g);
+  }
   int rc = validate_prefill(what, q, q_token_stride, out, out_token_stride, batch, num_q_heads,
                             num_kv_heads, head_dim, max_q_len);
   if (rc != LITEKV_OK) return rc;
@@ -929,6 +957,28 @@ extern "C" int litekv_varlen_prefill(const void *q, int64_t q_token_stride, cons
                                      int32_t num_kv_heads, int32_t head_dim, int32_t max_seq_len,
                                      int64_t num_tokens, float softmax_scale, void *stream) {
   using namespace litekv;
+  if (head_dim != kHeadDim && generic_head_dim(head_dim)) {  // see generic_attention.hip
+    LITEKV_REQUIRE(max_seq_len >= 0, "varlen_prefill: max_seq_len %d < 0", max_seq_len);
+    GenericLaunch g;
+    g.q = q;
+    g.q_row_stride = q_token_stride;
+    g.out = out;
+    g.out_row_stride = out_token_stride;
+    g.k = k;
+    g.v = v;
+    g.k_stride = k_token_stride;
+    g.v_stride = v_token_stride;
+    g.seq_starts = seq_starts;
+    g.q_lens = seq_lens;
+    g.batch = num_tokens == 0 ? 0 : batch;
+    g.rows_per_seq = max_seq_len;
+    g.num_q_heads = num_q_heads;
+    g.num_kv_heads = num_kv_heads;
+    g.head_dim = head_dim;
+    g.softmax_scale = softmax_scale;
+    g.stream = stream;
+    return launch_generic_attention("varlen_prefill", g);
+  }
   int rc = validate_prefill("varlen_prefill", q, q_token_stride, out, out_token_stride, batch,
                             num_q_heads, num_kv_heads, head_dim, max_seq_len);
   if (rc != LITEKV_OK) return rc;

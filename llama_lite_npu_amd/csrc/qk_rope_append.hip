@@ -6,30 +6,29 @@
 //
 // A head row (128 fp16) is held by 16 lanes, 8 elements each; a wavefront works on 4 rows. The
 // sum of squares is reduced across the 16 lanes; the rotation pairs element i with i + 64, which
-// lives 8 lanes away. Rounding follows the reference where it is specified: the normalised value
+// lives 8 lanes away. (Head dims 32, 64 and 256: 4, 8 and 32 lanes per row, template argument L.) Rounding follows the reference where it is specified: the normalised value
 // is rounded to fp16 before the weight multiply, and that product to fp16
 // (`(x * rrms).to(fp16) * w`, lite_llama/kernels/skip_rmsnorm.py:137-145); the rotation
 // x1*cos - x2*sin, x2*cos + x1*sin (lite_llama/kernels/rope_emb.py:79-87) is evaluated in fp32
 // from fp16 inputs and rounded once.
+#include <type_traits>
+
 #include "common.h"
 #include "kv_fp8.h"
 
 namespace litekv {
 
-constexpr int kLanesPerRow = 16;
-
+template <int L>
 __device__ __forceinline__ float row_sum(float v) {
-  v += __shfl_xor(v, 1, kLanesPerRow);
-  v += __shfl_xor(v, 2, kLanesPerRow);
-  v += __shfl_xor(v, 4, kLanesPerRow);
-  v += __shfl_xor(v, 8, kLanesPerRow);
+#pragma unroll
+  for (int off = 1; off < L; off <<= 1) v += __shfl_xor(v, off, L);
   return v;
 }
 
 // KV kKvFp8 / kKvInt8: the pool holds 8-bit codes; `scales` are its per-head scales (K heads, then
 // V heads) and a row is quantised on its way in, exactly as kv_append_q8_kernel would quantise
 // the fp16 row.
-template <int KV>
+template <int KV, int L>
 __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
     half_t *__restrict__ q, int64_t q_stride, const half_t *__restrict__ k, int64_t k_stride,
     const half_t *__restrict__ v, int64_t v_stride, const half_t *__restrict__ q_weight,
@@ -37,8 +36,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
     const half_t *__restrict__ sin_rows, int64_t cs_stride, const int32_t *__restrict__ slot_mapping,
     void *__restrict__ pool_any, const float *__restrict__ scales, int64_t total_rows,
     int32_t num_q_heads, int32_t num_kv_heads, int64_t num_slots, float eps) {
-  const int l16 = threadIdx.x & 15;
-  const int64_t row = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+  constexpr int kDim = 8 * L;       // the head dim
+  const int l16 = threadIdx.x & (L - 1);  // lane inside the row
+  const int64_t row = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / L;
   if (row >= total_rows) return;  // whole 16-lane groups leave together
   const int rows_per_token = num_q_heads + 2 * num_kv_heads;
   const int64_t token = row / rows_per_token;
@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
   const bool slot_ok = slot >= 0 && slot < num_slots;
   // stores 8 elements of head `kv_head` (K heads first, then V heads) of the token's slot
   auto store_row = [&](int kv_head, half8_t x) {
-    const int64_t at = (slot * (int64_t)(2 * num_kv_heads) + kv_head) * kHeadDim + 8 * l16;
+    const int64_t at = (slot * (int64_t)(2 * num_kv_heads) + kv_head) * kDim + 8 * l16;
     if constexpr (KV != kKvF16) {
       *(uint2_t *)(static_cast<uint8_t *>(pool_any) + at) =
           half_to_codes<KV>(x, 1.0f / scales[kv_head]);
@@ -60,14 +60,14 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
     const int head = r - num_q_heads - num_kv_heads;
     if (slot_ok) {
       store_row(num_kv_heads + head,
-                *(const half8_t *)(v + token * v_stride + (int64_t)head * kHeadDim + 8 * l16));
+                *(const half8_t *)(v + token * v_stride + (int64_t)head * kDim + 8 * l16));
     }
     return;
   }
   const bool is_q = r < num_q_heads;
   const int head = is_q ? r : r - num_q_heads;
-  const half_t *src = is_q ? q + token * q_stride + (int64_t)head * kHeadDim
-                           : k + token * k_stride + (int64_t)head * kHeadDim;
+  const half_t *src = is_q ? q + token * q_stride + (int64_t)head * kDim
+                           : k + token * k_stride + (int64_t)head * kDim;
   const half_t *weight = is_q ? q_weight : k_weight;
   half8_t x = *(const half8_t *)(src + 8 * l16);
 
@@ -78,8 +78,8 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
       xf[i] = (float)x[i];
       ss += xf[i] * xf[i];
     }
-    ss = row_sum(ss);
-    const float rrms = 1.0f / sqrtf(ss * (1.0f / kHeadDim) + eps);
+    ss = row_sum<L>(ss);
+    const float rrms = 1.0f / sqrtf(ss * (1.0f / kDim) + eps);
     const half8_t w = *(const half8_t *)(weight + 8 * l16);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -89,17 +89,17 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
   }
 
   if (cos_rows != nullptr) {
-    // partner: element i + 64 for the first half of the row, i - 64 for the second
+    // partner: element i + dim / 2 for the first half of the row, i - dim / 2 for the second
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     u32x4 bits = __builtin_bit_cast(u32x4, x);
     u32x4 other;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) other[i] = __shfl_xor(bits[i], 8, kLanesPerRow);
+    for (int i = 0; i < 4; ++i) other[i] = __shfl_xor(bits[i], L / 2, L);
     const half8_t p = __builtin_bit_cast(half8_t, other);
-    const int j = 8 * (l16 & 7);  // index into the first 64 entries of the cos / sin row
+    const int j = 8 * (l16 & (L / 2 - 1));  // index into the first dim / 2 entries of the cos / sin row
     const half8_t c = *(const half8_t *)(cos_rows + token * cs_stride + j);
     const half8_t s = *(const half8_t *)(sin_rows + token * cs_stride + j);
-    const float sign = l16 < 8 ? -1.0f : 1.0f;
+    const float sign = l16 < L / 2 ? -1.0f : 1.0f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       x[i] = (half_t)((float)x[i] * (float)c[i] + sign * ((float)p[i] * (float)s[i]));
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
   }
 
   if (is_q) {
-    *(half8_t *)(q + token * q_stride + (int64_t)head * kHeadDim + 8 * l16) = x;
+    *(half8_t *)(q + token * q_stride + (int64_t)head * kDim + 8 * l16) = x;
   } else if (slot_ok) {
     store_row(head, x);
   }
@@ -125,8 +125,8 @@ static int launch_qk_epilogue(const char *what, void *q, int64_t q_token_stride,
                               int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                               int64_t num_slots, float rms_eps, void *stream) {
   LITEKV_REQUIRE(num_tokens >= 0, "%s: num_tokens %d < 0", what, num_tokens);
-  LITEKV_REQUIRE(head_dim == kHeadDim, "%s: head_dim %d unsupported (only %d)", what, head_dim,
-                 kHeadDim);
+  LITEKV_REQUIRE(head_dim == kHeadDim || generic_head_dim(head_dim),
+                 "%s: head_dim %d unsupported (32, 64, 128 or 256)", what, head_dim);
   LITEKV_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads <= 65535 && num_kv_heads <= 65535,
                  "%s: num_q_heads %d / num_kv_heads %d invalid", what, num_q_heads, num_kv_heads);
   if (num_tokens == 0) {
@@ -155,18 +155,34 @@ static int launch_qk_epilogue(const char *what, void *q, int64_t q_token_stride,
   LITEKV_REQUIRE(num_slots > 0, "%s: num_slots %lld <= 0", what, (long long)num_slots);
   LITEKV_REQUIRE(rms_eps >= 0.f, "%s: rms_eps %g < 0", what, (double)rms_eps);
   const int64_t total_rows = (int64_t)num_tokens * (num_q_heads + 2 * num_kv_heads);
-  const int64_t blocks = (total_rows * kLanesPerRow + 255) / 256;
+  const int64_t blocks = (total_rows * (head_dim / 8) + 255) / 256;
   LITEKV_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many tokens", what);
-  auto kernel = format == kKvFp8    ? qk_norm_rope_append_kernel<kKvFp8>
-                : format == kKvInt8 ? qk_norm_rope_append_kernel<kKvInt8>
-                                    : qk_norm_rope_append_kernel<kKvF16>;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<half_t *>(q), q_token_stride, static_cast<const half_t *>(k),
-                     k_token_stride, static_cast<const half_t *>(v), v_token_stride,
-                     static_cast<const half_t *>(q_norm_weight),
-                     static_cast<const half_t *>(k_norm_weight), static_cast<const half_t *>(cos_rows),
-                     static_cast<const half_t *>(sin_rows), cos_sin_token_stride, slot_mapping, kv_pool,
-                     fp8_scales, total_rows, num_q_heads, num_kv_heads, num_slots, rms_eps);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<half_t *>(q), q_token_stride, static_cast<const half_t *>(k),
+                       k_token_stride, static_cast<const half_t *>(v), v_token_stride,
+                       static_cast<const half_t *>(q_norm_weight),
+                       static_cast<const half_t *>(k_norm_weight),
+                       static_cast<const half_t *>(cos_rows), static_cast<const half_t *>(sin_rows),
+                       cos_sin_token_stride, slot_mapping, kv_pool, fp8_scales, total_rows,
+                       num_q_heads, num_kv_heads, num_slots, rms_eps);
+  };
+  auto by_format = [&](auto lanes) {
+    constexpr int L = decltype(lanes)::value;
+    if (format == kKvFp8) {
+      launch(qk_norm_rope_append_kernel<kKvFp8, L>);
+    } else if (format == kKvInt8) {
+      launch(qk_norm_rope_append_kernel<kKvInt8, L>);
+    } else {
+      launch(qk_norm_rope_append_kernel<kKvF16, L>);
+    }
+  };
+  switch (head_dim) {
+    case 32: by_format(std::integral_constant<int, 4>{}); break;
+    case 64: by_format(std::integral_constant<int, 8>{}); break;
+    case 256: by_format(std::integral_constant<int, 32>{}); break;
+    default: by_format(std::integral_constant<int, 16>{}); break;
+  }
   return check_launch(what);
 }
 }  // namespace litekv

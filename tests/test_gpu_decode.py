@@ -255,7 +255,7 @@ def test_invalid_arguments_raise():
     case = workloads.make_decode_case("err", 99, [10], 16, 8, device=DEV)
     from llama_lite_npu_amd._lib import LiteKVError
     with pytest.raises(LiteKVError, match="head_dim"):
-        ops.paged_decode(case.q[..., :64].contiguous(), case.kv_pool[..., :64].contiguous(), case.block_table,
+        ops.paged_decode(case.q[..., :96].contiguous(), case.kv_pool[..., :96].contiguous(), case.block_table,
                          case.seq_lens)
     with pytest.raises(LiteKVError, match="workspace"):
         ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, max_splits=4,
@@ -394,3 +394,60 @@ def test_unsupported_page_size_is_refused():
         ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, page_size=48, num_splits=1)
     with pytest.raises((LiteKVError, ValueError), match="page_size"):
         ops.paged_decode(case.q, case.kv_pool, case.block_table, case.seq_lens, page_size=48, schedule="balanced")
+
+
+# ---- head dims other than 128 (the reference kernels take any block size, flashdecoding.py:305) ----
+
+@pytest.mark.parametrize("head_dim", [64, 32, 256])
+@pytest.mark.parametrize("hq,hkv,page_size", [(64, 8, 16), (14, 2, 16), (16, 4, 64), (8, 8, 32)])
+def test_head_dims_every_schedule(head_dim, hq, hkv, page_size):
+    """Decode at head dims 32, 64 and 256 through every entry point: both schedules, the plan made
+    on the device, the fused append, a shared prefix, empty rows."""
+    print(f"decode head_dim {head_dim} heads {hq}/{hkv} page_size {page_size}", flush=True)
+    case = workloads.make_decode_case("dims", 500 + head_dim + hq, [0, 1, 15, 16, 17, 63, 64, 65, 255, 700], hq, hkv,
+                                      device=DEV, page_size=page_size, head_dim=head_dim)
+    lens = case.seq_lens.clone()
+    lens[4] = 0
+    pool_ref = case.kv_pool.clone()
+    ops.kv_append(case.k_new, case.v_new, case.slot_mapping, pool_ref)
+    ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool_ref), case.block_table.cpu().numpy(),
+                                lens.cpu().numpy(), case.softmax_scale, page_size=page_size)
+    for kw in ({"num_splits": 1}, {"num_splits": 3}, {"schedule": "balanced"}, {"schedule": "balanced", "chunks": 7}):
+        out = ops.paged_decode(case.q, pool_ref, case.block_table, lens, case.softmax_scale, page_size=page_size, **kw)
+        torch.cuda.synchronize()
+        assert_attention_close(out, ref, f"head_dim {head_dim} {kw}")
+        assert float(out[4].abs().max()) == 0.0
+    keep = torch.ones(case.kv_pool.shape[0], dtype=torch.bool, device=DEV)
+    keep[case.slot_mapping[4].long()] = False           # the empty sequence appends nothing
+    # fused append, balanced entry (page ids from the plan) and per-sequence entry
+    pool = case.kv_pool.clone()
+    plan = ops.DecodePlan(case.block_table, lens, hq, hkv, case.num_pages, 5, page_size=page_size)
+    out = ops.decode_step(case.q, pool, plan, case.k_new, case.v_new, case.softmax_scale)
+    torch.cuda.synchronize()
+    assert torch.equal(pool[keep].view(torch.int16), pool_ref[keep].view(torch.int16))
+    assert_attention_close(out, ref, f"head_dim {head_dim} fused step")
+    pool = case.kv_pool.clone()
+    out = ops.paged_decode(case.q, pool, case.block_table, lens, case.softmax_scale, num_splits=1,
+                           page_size=page_size, k_new=case.k_new, v_new=case.v_new)
+    torch.cuda.synchronize()
+    assert torch.equal(pool[keep].view(torch.int16), pool_ref[keep].view(torch.int16))
+    assert_attention_close(out, ref, f"head_dim {head_dim} per-sequence fused step")
+
+
+@pytest.mark.parametrize("head_dim", [64, 256])
+def test_head_dims_shared_prefix(head_dim):
+    print(f"decode shared prefix head_dim {head_dim}", flush=True)
+    shared_pages, suffix = 5, [0, 5, 15, 16, 40, 300]
+    ctx = [shared_pages * 16 + s for s in suffix]
+    priv = [(c + 1 + 15) // 16 - shared_pages for c in ctx]
+    num_pages = shared_pages + sum(priv) + 7
+    perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(head_dim)).to(torch.int32)
+    shared, cur, lists = perm[:shared_pages], shared_pages, []
+    for n in priv:
+        lists.append(torch.cat([shared, perm[cur:cur + n]]))
+        cur += n
+    case = workloads.make_decode_case("shared-dims", 560 + head_dim, ctx, 32, 4, num_pages=num_pages, device=DEV,
+                                      page_lists=lists, head_dim=head_dim)
+    ref = _oracle(case)
+    out = _run(case, schedule="balanced", shared_pages=shared_pages)
+    assert_attention_close(out, ref, f"shared prefix head_dim {head_dim}")

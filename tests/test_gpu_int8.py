@@ -328,3 +328,54 @@ def test_executor_on_int8_pools_with_a_shared_system_prompt():
         info = ex.atten_info
         ref = cpu_ref.paged_decode_ref(qd.cpu(), decoded(), info.block_table.cpu(), info.seq_lens_i32.cpu(), SCALE).numpy()
         assert_attention_close(out, ref, f"int8 decode step {step} over a shared system prompt")
+
+
+@pytest.mark.parametrize("dtype", [torch.int8, torch.uint8])
+def test_quantised_pools_at_head_dim_64(dtype):
+    """8-bit pools (int8 and fp8) at head dim 64: quantising append, decode through both schedules
+    with the fused append, and a chunk over cached history."""
+    from oracle import fp8
+    codec = int8 if dtype == torch.int8 else fp8
+    print(f"head_dim 64, pool dtype {dtype}", flush=True)
+    d, hq, hkv = 64, 16, 4
+    scale = 1.0 / math.sqrt(d)
+    case = workloads.make_decode_case("q64", 77, [0, 15, 16, 17, 200, 63], hq, hkv, device=DEV, head_dim=d)
+    scales = _head_scales(hkv) if dtype == torch.int8 else _head_scales(hkv, 0.02, 0.015)
+    pool = torch.zeros(case.kv_pool.shape, dtype=dtype, device=DEV)
+    every_slot = torch.arange(pool.shape[0], dtype=torch.int32, device=DEV)
+    ops.kv_append_quantised(case.kv_pool[:, :hkv], case.kv_pool[:, hkv:], every_slot, pool, scales)
+    want_codes = np.zeros(pool.shape, dtype=np.int8 if dtype == torch.int8 else np.uint8)
+    codec.kv_append(case.kv_pool[:, :hkv].cpu().numpy(), case.kv_pool[:, hkv:].cpu().numpy(), every_slot.cpu().numpy(),
+                    want_codes, scales.cpu().numpy())
+    got = pool.cpu().numpy()
+    if dtype == torch.int8:
+        assert np.array_equal(got, want_codes)
+    else:
+        assert (((got == want_codes) | (((got & 0x7F) == 0) & ((want_codes & 0x7F) == 0)))).all()
+    ref_pool = pool.clone()
+    ops.kv_append_quantised(case.k_new, case.v_new, case.slot_mapping, ref_pool, scales)
+    values = torch.from_numpy(codec.dequantize_pool(ref_pool.cpu().numpy(), scales.cpu().numpy()))
+    ref = cpu_ref.paged_decode_ref(case.q.cpu(), values, case.block_table.cpu(), case.seq_lens.cpu(), scale).numpy()
+    for kw in ({"num_splits": 1}, {"schedule": "balanced", "chunks": 3}):
+        fused = pool.clone()
+        if "schedule" in kw:
+            plan = ops.DecodePlan(case.block_table, case.seq_lens, hq, hkv, case.num_pages, 3)
+            out = ops.decode_step(case.q, fused, plan, case.k_new, case.v_new, scale, kv_scales=scales)
+        else:
+            out = ops.paged_decode(case.q, fused, case.block_table, case.seq_lens, scale, kv_scales=scales,
+                                   k_new=case.k_new, v_new=case.v_new, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(fused, ref_pool)
+        assert_attention_close(out, ref, f"head_dim 64 {dtype} {kw}")
+    pre = workloads.make_prefill_case("q64p", 78, [40, 7, 65], hq, hkv, context_lens=[33, 0, 100], device=DEV, head_dim=d)
+    pool = torch.zeros(pre.kv_pool.shape, dtype=dtype, device=DEV)
+    every_slot = torch.arange(pool.shape[0], dtype=torch.int32, device=DEV)
+    ops.kv_append_quantised(pre.kv_pool[:, :hkv], pre.kv_pool[:, hkv:], every_slot, pool, scales)
+    ops.kv_append_quantised(pre.k, pre.v, pre.slot_mapping, pool, scales)
+    out = ops.paged_prefill(pre.q, pool, pre.block_table, pre.cu_q_lens, pre.context_lens, pre.max_q_len, scale,
+                            kv_scales=scales)
+    torch.cuda.synchronize()
+    values = torch.from_numpy(codec.dequantize_pool(pool.cpu().numpy(), scales.cpu().numpy()))
+    ref = cpu_ref.paged_prefill_ref(pre.q.cpu(), values, pre.block_table.cpu(), pre.cu_q_lens.cpu(),
+                                    pre.context_lens.cpu(), scale).numpy()
+    assert_attention_close(out, ref, f"head_dim 64 {dtype} chunk prefill")

@@ -176,3 +176,29 @@ def test_paged_prefill_page_sizes(page_size, hq, hkv, lens, ctx):
                             page_size=page_size)
     torch.cuda.synchronize()
     assert_attention_close(out, _oracle_paged(case), f"paged prefill page_size {page_size}")
+
+
+@pytest.mark.parametrize("head_dim", [64, 32, 256])
+@pytest.mark.parametrize("hq,hkv,lens,ctx,page_size", [
+    (16, 8, [1, 2, 15, 16, 17, 33, 64, 65], None, 16),
+    (14, 2, [128, 77], None, 16),
+    (32, 4, [100, 5, 96], [100, 31, 64], 32),       # chunks over cached history
+    (16, 1, [70, 40], [17, 200], 64),
+])
+def test_prefill_head_dims(head_dim, hq, hkv, lens, ctx, page_size):
+    """Prefill at head dims 32, 64 and 256: prompts (paged and packed entry points agree bit for
+    bit) and chunks over cached history."""
+    print(f"prefill head_dim {head_dim} {hq}/{hkv} {lens} ctx {ctx} page_size {page_size}", flush=True)
+    case = workloads.make_prefill_case("pd", 950 + head_dim + hq, lens, hq, hkv, context_lens=ctx, device=DEV,
+                                       page_size=page_size, head_dim=head_dim)
+    _append(case)
+    out = ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens,
+                            case.context_lens if ctx is not None else None, case.max_q_len, case.softmax_scale,
+                            page_size=page_size)
+    torch.cuda.synchronize()
+    assert_attention_close(out, _oracle_paged(case), f"paged prefill head_dim {head_dim}")
+    if ctx is None:
+        out2 = ops.varlen_prefill(case.q, case.k, case.v, case.cu_q_lens[:-1], case.seq_lens, case.max_q_len,
+                                  case.softmax_scale)
+        torch.cuda.synchronize()
+        assert torch.equal(out, out2)

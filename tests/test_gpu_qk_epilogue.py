@@ -17,7 +17,7 @@ MAX_ABS = 4e-3
 MIN_EXACT = 0.995
 
 
-def _inputs(seed, t, hq, hkv):
+def _inputs(seed, t, hq, hkv, D=D):
     slots_in_pool = max(256, 2 * t)
     g = torch.Generator(device=DEV).manual_seed(seed)
     qkv = torch.randn((t, hq + 2 * hkv, D), generator=g, device=DEV, dtype=torch.float16) * 1.7
@@ -50,8 +50,18 @@ def _check(got16, want16, what):
     (5, 8, 8, False, False),        # degenerates to the plain append
 ])
 def test_fused_epilogue_matches_oracle(t, hq, hkv, norm, rope):
-    print(f"qk epilogue T={t} {hq}/{hkv} norm={norm} rope={rope}", flush=True)
-    q, k, v, wq, wk, cos, sin, pool, slots = _inputs(900 + t, t, hq, hkv)
+    _epilogue_case(t, hq, hkv, norm, rope, D)
+
+
+@pytest.mark.parametrize("head_dim", [64, 32, 256])
+@pytest.mark.parametrize("t,hq,hkv,norm,rope", [(33, 14, 2, True, True), (7, 16, 8, False, True), (9, 8, 1, True, False)])
+def test_fused_epilogue_other_head_dims(head_dim, t, hq, hkv, norm, rope):
+    _epilogue_case(t, hq, hkv, norm, rope, head_dim)
+
+
+def _epilogue_case(t, hq, hkv, norm, rope, head_dim):
+    print(f"qk epilogue T={t} {hq}/{hkv} norm={norm} rope={rope} head_dim={head_dim}", flush=True)
+    q, k, v, wq, wk, cos, sin, pool, slots = _inputs(900 + t, t, hq, hkv, head_dim)
     slots[t // 2] = -1                              # a padding row: q still processed, nothing stored
     if t > 3:
         slots[3] = pool.shape[0] + 5
