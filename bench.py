@@ -127,13 +127,18 @@ class DecodeLayerSet:
         b, hq, hkv = c.batch, c.num_q_heads, c.num_kv_heads
         slots = c.num_pages * 16
         gen = torch.Generator(device=device).manual_seed(4242)
-        self.fp8 = kv_dtype == "fp8"
+        self.fp8 = kv_dtype in ("fp8", "int8")       # 8-bit codes with one scale per head
+        self.q8 = kv_dtype
         if self.fp8:
             if schedule != "balanced":
-                raise ValueError("fp8 pools are read by the balanced schedule")
-            # E4M3 codes (no NaN codes) and one scale per head
-            pools = torch.randint(0, 0x7F, (layers, slots, 2 * hkv, 128), generator=gen, device=device,
-                                  dtype=torch.uint8)
+                raise ValueError("8-bit pools are read by the balanced schedule in this benchmark")
+            # E4M3 codes (no NaN codes) or int8 codes (no -128), and one scale per head
+            if kv_dtype == "fp8":
+                pools = torch.randint(0, 0x7F, (layers, slots, 2 * hkv, 128), generator=gen, device=device,
+                                      dtype=torch.uint8)
+            else:
+                pools = torch.randint(-127, 128, (layers, slots, 2 * hkv, 128), generator=gen, device=device,
+                                      dtype=torch.int8)
             self.scales = torch.full((2 * hkv,), 0.02, dtype=torch.float32, device=device)
         else:
             pools = torch.empty((layers, slots, 2 * hkv, 128), dtype=torch.float16, device=device)
@@ -215,7 +220,8 @@ class DecodeLayerSet:
             on = (lambda a: a) if stream is None else (lambda a: a[:-1] + (stream,))
             rc |= lib.litekv_decode_advance(*on(self.advance_args))
             rc |= lib.litekv_decode_plan_prefix(*on(self.plan_args))
-            dec = lib.litekv_paged_decode_prefix_fp8 if self.fp8 else lib.litekv_paged_decode_prefix
+            dec = (getattr(lib, "litekv_paged_decode_prefix_" + self.q8) if self.fp8
+                   else lib.litekv_paged_decode_prefix)
             prof = lib.litekv_profile_next_decode
             for l in range(self.layers):
                 if events is not None:
@@ -285,7 +291,7 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
     ms_per_step = wall * 1e3 / steps
     decode_bytes = case.decode_bytes()
     append_bytes = case.append_bytes()
-    if kv_dtype == "fp8":
+    if kv_dtype in ("fp8", "int8"):
         # one byte per cached element: K/V traffic halves; the appended rows arrive as fp16
         kv_read = int(case.seq_lens.sum()) * case.tok_bytes
         decode_bytes -= kv_read // 2
@@ -337,7 +343,7 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
         res["roofline"]["kernel"] = "shared prefix (varlen_prefill_tiled_kernel<2>) + paged_decode_balanced_kernel + merge"
         res["roofline"]["duration_us"] = k_mean * 1e3
     unique = case.unique_decode_bytes() + (append_bytes if balanced else 0)
-    if kv_dtype == "fp8":
+    if kv_dtype in ("fp8", "int8"):
         unique -= (case.unique_decode_bytes() - (case.decode_bytes() - int(case.seq_lens.sum()) * case.tok_bytes)) // 2
     if unique < kernel_bytes:
         # Pages shared between block tables: the roofline fraction is taken on the bytes that must
@@ -741,8 +747,9 @@ def main() -> int:
                     help="balanced schedule: pieces per kv head (default: one workgroup per compute unit)")
     ap.add_argument("--no-shared-prefix", action="store_true",
                     help="c4: read the shared prefix pages once per sequence like any other page")
-    ap.add_argument("--kv-dtype", default="f16", choices=["f16", "fp8"],
-                    help="storage of the KV pools (fp8: E4M3 codes with per-head scales; decode configs only)")
+    ap.add_argument("--kv-dtype", default="f16", choices=["f16", "fp8", "int8"],
+                    help="storage of the KV pools (fp8: E4M3 codes, int8: signed codes, both with per-head "
+                         "scales; decode configs only)")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the leg that replays the decode step as one HIP graph")
     ap.add_argument("--out-dir", default="bench_out",
