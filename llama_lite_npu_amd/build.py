@@ -26,6 +26,7 @@ SOURCES = (
     "qk_rope_append.hip",
     "page_ops.hip",
     "paged_decode.hip",
+    "paged_decode_hd64.hip",
     "decode_advance.hip",
     "paged_prefill.hip",
     "generic_attention.hip",

@@ -87,6 +87,41 @@ struct LineCut {
   }
 };
 
+// One decode call, as the launchers of paged_decode.hip take it.
+struct DecodeArgs {
+  const void *q;
+  int64_t q_batch_stride;
+  const void *kv_pool;
+  const int32_t *block_table;
+  int32_t block_table_stride;
+  const int32_t *seq_lens;
+  void *out;
+  void *workspace;
+  size_t workspace_bytes;
+  int32_t batch, num_q_heads, num_kv_heads, head_dim, page_size;
+  int64_t num_pages;
+  float softmax_scale;
+  void *stream;
+  // the step's new rows [B][Hkv][D] for the append fused into the splits schedule (or null)
+  const void *k_new = nullptr;
+  const void *v_new = nullptr;
+  int64_t k_new_stride = 0, v_new_stride = 0;
+};
+
+// The launchers of the head dim 64 build of paged_decode.hip (paged_decode_hd64.hip), to which the
+// head dim 128 build, which owns the C ABI, hands calls with head_dim == 64. `scales` marks a pool
+// of 8-bit codes of format `format` (kv_fp8.h).
+int hd64_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split,
+               const float *scales, int format);
+int hd64_merge(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split);
+int hd64_balanced(const char *what, const void *q, int64_t q_batch_stride, void *kv_pool,
+                  const float *scales, const int32_t *seq_lens, void *plan, size_t plan_bytes,
+                  const void *k_new, const void *v_new, int64_t k_new_stride, int64_t v_new_stride,
+                  void *out, void *workspace, size_t workspace_bytes, int32_t batch,
+                  int32_t num_q_heads, int32_t num_kv_heads, int32_t page_size, int64_t num_pages,
+                  int32_t block_table_stride, int32_t chunks, float softmax_scale, void *stream,
+                  int format);
+
 // Attention for the head dims the tuned kernels (128) do not take: 32, 64 and 256
 // (generic_attention.hip). A launch is a decode step (seq_lens), a paged prefill (cu_q_lens,
 // context_lens) or a packed prefill (kv_pool null; k, v, seq_starts, q_lens); `rows_per_seq` is

@@ -35,9 +35,33 @@
 #include "common.h"
 #include "kv_fp8.h"
 
-namespace litekv {
+// This file is compiled once per head dim its kernels are tuned for: as itself for 128, and
+// through paged_decode_hd64.hip (which defines LITEKV_HD and includes it) for 64. Everything
+// below lives in an inline namespace named after the head dim, so the two sets of kernels and
+// launchers are distinct symbols; the extern "C" entry points exist in the 128 build only and hand
+// head dim 64 to the launchers of the other build (litekv::hd64_*, declared in common.h).
+// At 64 the lane maps are those of 128 with half the MFMA k-steps and half the output column
+// tiles; lanes whose 16-byte column of a V row would lie past the row re-read the column of
+// their twin (n % 8) and stage it in a part of the LDS row nobody reads.
+#ifndef LITEKV_HD
+#define LITEKV_HD 128
+#endif
+#if LITEKV_HD == 128
+#define LITEKV_HD_NS hd128
+#elif LITEKV_HD == 64
+#define LITEKV_HD_NS hd64
+#else
+#error "paged_decode.hip is written for head dims 64 and 128"
+#endif
 
-constexpr int kVPitch = kHeadDim + 8;  // fp16 elements per staged V row (272 bytes)
+namespace litekv {
+inline namespace LITEKV_HD_NS {
+
+constexpr int kHD = LITEKV_HD;       // head dim of this build of the file
+constexpr int kKSteps = kHD / 32;    // MFMA k-steps of a score product (fp16 fragments of 8)
+constexpr int kJTiles = kHD / 16;    // 16-column tiles of an output row
+constexpr int kVCols = kHD / 8;      // 16-byte columns of an fp16 row
+constexpr int kVPitch = 128 + 8;     // fp16 elements per staged V row (272 bytes), whatever kHD
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -93,7 +117,7 @@ struct HeadState {
   float d;
   __device__ __forceinline__ void reset() {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < kJTiles; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
     m = -INFINITY;
     d = 0.f;
   }
@@ -110,9 +134,9 @@ __device__ __forceinline__ void wave_lds_fence() {
 // Q^T as B operand: lane (n, g) holds q[head n][32*kk + 8*g .. +7]; lanes past the group get 0.
 __device__ __forceinline__ void load_q(half8_t (&qf)[4], const half_t *q_row0, int n, int g,
                                        int group) {
-  const half_t *qrow = q_row0 + (int64_t)n * kHeadDim + 8 * g;
+  const half_t *qrow = q_row0 + (int64_t)n * kHD + 8 * g;
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) {
+  for (int kk = 0; kk < kKSteps; ++kk) {
     qf[kk] = (n < group) ? *(const half8_t *)(qrow + 32 * kk) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
   }
 }
@@ -120,9 +144,9 @@ __device__ __forceinline__ void load_q(half8_t (&qf)[4], const half_t *q_row0, i
 // The same for an fp8 pool, in the d order of PageRegsFp8::k.
 __device__ __forceinline__ void load_q_fp8_order(half8_t (&qf)[4], const half_t *q_row0, int n, int g,
                                                  int group) {
-  const half_t *qrow = q_row0 + (int64_t)n * kHeadDim + 16 * g;
+  const half_t *qrow = q_row0 + (int64_t)n * kHD + 16 * g;
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) {
+  for (int kk = 0; kk < kKSteps; ++kk) {
     qf[kk] = (n < group) ? *(const half8_t *)(qrow + 64 * (kk >> 1) + 8 * (kk & 1))
                          : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
   }
@@ -141,7 +165,7 @@ __device__ __forceinline__ void request_page(PageRegs &r, const half_t *k_lane,
   const half_t *kr = dummy ? pool + page_off : k_lane + page_off;
   const int64_t k_step = dummy ? 0 : 32;
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) r.k[kk] = __builtin_nontemporal_load((const half8_t *)(kr + kk * k_step));
+  for (int kk = 0; kk < kKSteps; ++kk) r.k[kk] = __builtin_nontemporal_load((const half8_t *)(kr + kk * k_step));
   const half_t *vr = dummy ? pool + page_off : v_lane + page_off;
   const int64_t v_step = dummy ? 0 : 4 * row_stride;
 #pragma unroll
@@ -157,7 +181,7 @@ __device__ __forceinline__ void request_page(PageRegsQ8<KV> &r, const uint8_t *k
   const uint8_t *kr = dummy ? pool + page_off : k_lane + page_off;
   const int64_t k_step = dummy ? 0 : 64;
 #pragma unroll
-  for (int j = 0; j < 2; ++j) r.k[j] = __builtin_nontemporal_load((const uint4_t *)(kr + j * k_step));
+  for (int j = 0; j < kHD / 64; ++j) r.k[j] = __builtin_nontemporal_load((const uint4_t *)(kr + j * k_step));
   const uint8_t *vr = dummy ? pool + page_off : v_lane + page_off;
   const int64_t v_step = dummy ? 0 : 8 * row_stride;
 #pragma unroll
@@ -179,9 +203,11 @@ __device__ __forceinline__ void attend_core(HeadState &st, const half8_t (&kf)[4
 
   // two accumulators: the dependent MFMA chain is two deep instead of four
   float4_t s = mfma_16x16x32(kf[0], qf[0], float4_t{0.f, 0.f, 0.f, 0.f});
-  float4_t s1 = mfma_16x16x32(kf[2], qf[2], float4_t{0.f, 0.f, 0.f, 0.f});
-  s = mfma_16x16x32(kf[1], qf[1], s);
-  s1 = mfma_16x16x32(kf[3], qf[3], s1);
+  float4_t s1 = mfma_16x16x32(kf[kKSteps / 2], qf[kKSteps / 2], float4_t{0.f, 0.f, 0.f, 0.f});
+  if constexpr (kKSteps == 4) {
+    s = mfma_16x16x32(kf[1], qf[1], s);
+    s1 = mfma_16x16x32(kf[3], qf[3], s1);
+  }
 
   float sv[4];
 #pragma unroll
@@ -200,7 +226,7 @@ __device__ __forceinline__ void attend_core(HeadState &st, const half8_t (&kf)[4
     const float alpha = fast_exp2(st.m - m_new);
     st.d *= alpha;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < kJTiles; ++j) {
       st.acc[j][0] *= alpha;
       st.acc[j][1] *= alpha;
       st.acc[j][2] *= alpha;
@@ -215,7 +241,7 @@ __device__ __forceinline__ void attend_core(HeadState &st, const half8_t (&kf)[4
   const half4_t pt = half4_t{(half_t)pr[0], (half_t)pr[1], (half_t)pr[2], (half_t)pr[3]};
 
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
+  for (int j = 0; j < kJTiles; ++j) {
     // V^T fragment: lane (n, g) receives V[4g .. 4g+3][16j + n] from the transposing LDS read
     // (lane i of a 16-lane group passes the address of row i/4, columns 4*(i%4) .. +3).
     const half4_t vt = __builtin_bit_cast(
@@ -280,9 +306,9 @@ __device__ __forceinline__ void store_state(const HeadState &st, bool final_row,
   const float inv = out_scale / d_tot;  // out_scale: the V scale of an fp8 pool
   if (n >= group) return;
   if (final_row) {
-    half_t *o = out_row + (int64_t)n * kHeadDim + 4 * g;
+    half_t *o = out_row + (int64_t)n * kHD + 4 * g;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < kJTiles; ++j) {
       *(half4_t *)(o + 16 * j) =
           half4_t{(half_t)(st.acc[j][0] * inv), (half_t)(st.acc[j][1] * inv),
                   (half_t)(st.acc[j][2] * inv), (half_t)(st.acc[j][3] * inv)};
@@ -292,7 +318,7 @@ __device__ __forceinline__ void store_state(const HeadState &st, bool final_row,
     const float lse = (st.m + fast_log2(d_tot)) * kLn2;
     {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < kJTiles; ++j) {
         // Partials are read once, by the merge launch: streaming stores leave for memory as they
         // are issued instead of waiting in L2 for the write-back at the end of the kernel
         // (C2: 0.6 us per layer).
@@ -312,7 +338,7 @@ __device__ __forceinline__ void store_state(const HeadState &st, bool final_row,
 // (normalised fp32 and the log-sum-exp); unpark_state writes them out at the end of the chunk,
 // each lane reading back what it wrote itself.
 constexpr int kParkHeads = 8;                                  // query heads per kv head that fit
-constexpr int kParkFloats = kParkHeads * kHeadDim + 16;        // rows, then one log-sum-exp per head
+constexpr int kParkFloats = kParkHeads * kHD + 16;        // rows, then one log-sum-exp per head
 
 __device__ __forceinline__ void park_state(const HeadState &st, float *park, int n, int g,
                                            int group, float out_scale) {
@@ -320,13 +346,13 @@ __device__ __forceinline__ void park_state(const HeadState &st, float *park, int
   d_tot += xor_lane(d_tot, 32);
   const float inv = out_scale / d_tot;
   if (n >= group) return;
-  float *row = park + n * kHeadDim + 4 * g;
+  float *row = park + n * kHD + 4 * g;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
+  for (int j = 0; j < kJTiles; ++j) {
     *(float4_t *)(row + 16 * j) = float4_t{st.acc[j][0] * inv, st.acc[j][1] * inv,
                                            st.acc[j][2] * inv, st.acc[j][3] * inv};
   }
-  if (g == 0) park[kParkHeads * kHeadDim + n] = (st.m + fast_log2(d_tot)) * kLn2;
+  if (g == 0) park[kParkHeads * kHD + n] = (st.m + fast_log2(d_tot)) * kLn2;
 }
 
 __device__ __forceinline__ void unpark_state(const float *park, bool final_row, half_t *out_row,
@@ -334,10 +360,10 @@ __device__ __forceinline__ void unpark_state(const float *park, bool final_row, 
                                              int group) {
   if (final_row) {
     if (n >= group) return;
-    const float *row = park + n * kHeadDim + 4 * g;
-    half_t *o = out_row + (int64_t)n * kHeadDim + 4 * g;
+    const float *row = park + n * kHD + 4 * g;
+    half_t *o = out_row + (int64_t)n * kHD + 4 * g;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < kJTiles; ++j) {
       const float4_t x = *(const float4_t *)(row + 16 * j);
       *(half4_t *)(o + 16 * j) = half4_t{(half_t)x[0], (half_t)x[1], (half_t)x[2], (half_t)x[3]};
     }
@@ -347,13 +373,13 @@ __device__ __forceinline__ void unpark_state(const float *park, bool final_row, 
     wave_lds_fence();
     const int lane = 16 * g + n;
 #pragma unroll
-    for (int i = 0; i < kParkHeads / 2; ++i) {
+    for (int i = 0; i < kParkHeads * kHD / 256; ++i) {
       const int at = 4 * (64 * i + lane);
-      if (at < group * kHeadDim) {
+      if (at < group * kHD) {
         __builtin_nontemporal_store(*(const float4_t *)(park + at), (float4_t *)(part_row + at));
       }
     }
-    if (lane < group) __builtin_nontemporal_store(park[kParkHeads * kHeadDim + lane], part_lse_cell + lane);
+    if (lane < group) __builtin_nontemporal_store(park[kParkHeads * kHD + lane], part_lse_cell + lane);
   }
 }
 
@@ -381,16 +407,16 @@ __device__ __forceinline__ void load_new_rows(uint4_t (&kr)[4], uint4_t (&vr)[2]
                                               const half_t *vn, int n, int g) {
   if constexpr (FP8) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < kHD / 64; ++j) {
       kr[2 * j] = *(const uint4_t *)(kn + 64 * j + 16 * g);
       kr[2 * j + 1] = *(const uint4_t *)(kn + 64 * j + 16 * g + 8);
     }
-    vr[0] = *(const uint4_t *)(vn + 16 * (n & 7));
-    vr[1] = *(const uint4_t *)(vn + 16 * (n & 7) + 8);
+    vr[0] = *(const uint4_t *)(vn + 16 * (n & (kHD / 16 - 1)));
+    vr[1] = *(const uint4_t *)(vn + 16 * (n & (kHD / 16 - 1)) + 8);
   } else {
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) kr[kk] = *(const uint4_t *)(kn + 32 * kk + 8 * g);
-    vr[0] = *(const uint4_t *)(vn + 8 * n);
+    for (int kk = 0; kk < kKSteps; ++kk) kr[kk] = *(const uint4_t *)(kn + 32 * kk + 8 * g);
+    vr[0] = *(const uint4_t *)(vn + 8 * (n & (kVCols - 1)));
     vr[1] = uint4_t{0, 0, 0, 0};  // fp8 only
   }
 }
@@ -428,12 +454,12 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
 
   const int len = seq_lens[b];
   const int hq0 = h * group;
-  half_t *out_row = out + ((int64_t)b * num_q_heads + hq0) * kHeadDim;
+  half_t *out_row = out + ((int64_t)b * num_q_heads + hq0) * kHD;
   if (len <= 0) {
     if (split == 0 && n < group) {
-      half_t *o = out_row + (int64_t)n * kHeadDim;
+      half_t *o = out_row + (int64_t)n * kHD;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) *(half4_t *)(o + 16 * j + 4 * g) = half4_t{0, 0, 0, 0};
+      for (int j = 0; j < kJTiles; ++j) *(half4_t *)(o + 16 * j + 4 * g) = half4_t{0, 0, 0, 0};
     }
     return;
   }
@@ -449,29 +475,29 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
   half8_t qf[4];
   float v_scale = 1.0f, k_inv = 1.0f, v_inv = 1.0f;
   if constexpr (FP8) {  // the K scale joins the softmax scale, the V scale the normalisation
-    load_q_fp8_order(qf, q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
+    load_q_fp8_order(qf, q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHD, n, g, group);
     const float ks = scales[h];
     scale_log2 *= ks;
     v_scale = scales[num_kv_heads + h];
     k_inv = 1.0f / ks;  // the step's new rows are quantised with the reciprocals
     v_inv = 1.0f / v_scale;
   } else {
-    load_q(qf, q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHeadDim, n, g, group);
+    load_q(qf, q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHD, n, g, group);
   }
   // Fused append: the wavefront that attends the sequence's last page writes the step's token
   // into it. Its rows are requested here, before the pages.
   uint4_t k_row[4] = {}, v_row[2] = {};
   if constexpr (APPEND) {
-    load_new_rows<FP8>(k_row, v_row, k_new + (int64_t)b * k_new_stride + (int64_t)h * kHeadDim,
-                       v_new + (int64_t)b * v_new_stride + (int64_t)h * kHeadDim, n, g);
+    load_new_rows<FP8>(k_row, v_row, k_new + (int64_t)b * k_new_stride + (int64_t)h * kHD,
+                       v_new + (int64_t)b * v_new_stride + (int64_t)h * kHD, n, g);
   }
 
-  const int64_t row_stride = (int64_t)2 * num_kv_heads * kHeadDim;  // elements per slot
+  const int64_t row_stride = (int64_t)2 * num_kv_heads * kHD;  // elements per slot
   // this lane's row and column inside page 0 (see PageRegs / PageRegsFp8)
-  Elem *k_lane = kv + (int64_t)h * kHeadDim + (FP8 ? 16 : 8) * g + n * row_stride;
-  Elem *v_lane = FP8 ? kv + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7) +
+  Elem *k_lane = kv + (int64_t)h * kHD + (FP8 ? 16 : 8) * g + n * row_stride;
+  Elem *v_lane = FP8 ? kv + (int64_t)(num_kv_heads + h) * kHD + 16 * (n & (kHD / 16 - 1)) +
                            (2 * g + (n >> 3)) * row_stride
-                     : kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
+                     : kv + (int64_t)(num_kv_heads + h) * kHD + 8 * (n & (kVCols - 1)) + g * row_stride;
   const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
   const int32_t *table = block_table + (int64_t)b * bt_stride;
 
@@ -511,9 +537,9 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
           Page &r = buf[dd];
           if constexpr (FP8) {
             if (n == t_new) {
-              uint8_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 16 * g;
+              uint8_t *dst = kv + slot_off + (int64_t)h * kHD + 16 * g;
 #pragma unroll
-              for (int j = 0; j < 2; ++j) {
+              for (int j = 0; j < kHD / 64; ++j) {
                 const uint2_t lo = half_to_codes<KV>(__builtin_bit_cast(half8_t, k_row[2 * j]), k_inv);
                 const uint2_t hi = half_to_codes<KV>(__builtin_bit_cast(half8_t, k_row[2 * j + 1]), k_inv);
                 const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
@@ -525,7 +551,7 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
               const uint2_t lo = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[0]), v_inv);
               const uint2_t hi = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[1]), v_inv);
               const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
-              *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7)) = x;
+              *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHD + 16 * (n & (kHD / 16 - 1))) = x;
 #pragma unroll
               for (int i = 0; i < 2; ++i) {
                 if (i == (t_new >> 3)) r.v[i] = x;
@@ -533,9 +559,9 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
             }
           } else {
             if (n == t_new) {
-              half_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 8 * g;
+              half_t *dst = kv + slot_off + (int64_t)h * kHD + 8 * g;
 #pragma unroll
-              for (int kk = 0; kk < 4; ++kk) {
+              for (int kk = 0; kk < kKSteps; ++kk) {
                 const half8_t x = __builtin_bit_cast(half8_t, k_row[kk]);
                 r.k[kk] = x;
                 *(half8_t *)(dst + 32 * kk) = x;
@@ -543,7 +569,7 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
             }
             if (g == (t_new & 3)) {
               const half8_t x = __builtin_bit_cast(half8_t, v_row[0]);
-              *(half8_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n) = x;
+              *(half8_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHD + 8 * (n & (kVCols - 1))) = x;
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
                 if (i == (t_new >> 2)) r.v[i] = x;
@@ -558,7 +584,7 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
   }
 
   const int64_t cell = ((int64_t)b * num_q_heads + hq0) * max_splits + split;
-  store_state(st, n_splits == 1, out_row, part_o + cell * kHeadDim, (int64_t)max_splits * kHeadDim,
+  store_state(st, n_splits == 1, out_row, part_o + cell * kHD, (int64_t)max_splits * kHD,
               part_lse + cell, max_splits, n, g, group, v_scale);
 }
 
@@ -574,6 +600,10 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_
                                           const float *__restrict__ po2, int64_t po2_stride, int n2,
                                           half_t *out_row, int lane) {
   const int n_parts = TWO_RUNS ? n1 + n2 : n1;
+  // lane l holds elements 2l, 2l + 1 of the row; with a row of 64 the upper lanes re-read
+  // element 0 and store nothing
+  const bool live_col = 2 * lane < kHD;
+  const int mcol = live_col ? 2 * lane : 0;
   auto lse_of = [&](int s) {
     if (!TWO_RUNS || s < n1) return lse1[(int64_t)s * lse1_stride];
     return lse2[(int64_t)(s - n1) * lse2_stride];
@@ -591,7 +621,7 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_
 #pragma unroll
     for (int s = 0; s < 16; ++s) {
       r[s] = float2{0.f, 0.f};
-      if (s < n_parts) r[s] = *(const float2 *)(row_of(s) + 2 * lane);
+      if (s < n_parts) r[s] = *(const float2 *)(row_of(s) + mcol);
     }
     const float l = lane < n_parts ? lse_of(lane) : -INFINITY;
     float mx = l;
@@ -612,7 +642,7 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_
     }
     const float inv = 1.0f / den;
     typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-    *(half2_t *)(out_row + 2 * lane) = half2_t{(half_t)(num0 * inv), (half_t)(num1 * inv)};
+    if (live_col) *(half2_t *)(out_row + mcol) = half2_t{(half_t)(num0 * inv), (half_t)(num1 * inv)};
     return;
   }
   float mx = -INFINITY;
@@ -632,7 +662,7 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_
     for (; s + 4 <= cnt; s += 4) {
       float2 r[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) r[u] = *(const float2 *)(row_of(s0 + s + u) + 2 * lane);
+      for (int u = 0; u < 4; ++u) r[u] = *(const float2 *)(row_of(s0 + s + u) + mcol);
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const float wu = __shfl(w, s + u, kWave);
@@ -641,7 +671,7 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_
       }
     }
     for (; s < cnt; ++s) {
-      const float2 r = *(const float2 *)(row_of(s0 + s) + 2 * lane);
+      const float2 r = *(const float2 *)(row_of(s0 + s) + mcol);
       const float wu = __shfl(w, s, kWave);
       num0 += wu * r.x;
       num1 += wu * r.y;
@@ -651,7 +681,7 @@ __device__ __forceinline__ void merge_row(const float *__restrict__ lse1, int64_
   for (int off = 32; off > 0; off >>= 1) den += xor_lane(den, off);
   const float inv = 1.0f / den;
   typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-  *(half2_t *)(out_row + 2 * lane) = half2_t{(half_t)(num0 * inv), (half_t)(num1 * inv)};
+  if (live_col) *(half2_t *)(out_row + mcol) = half2_t{(half_t)(num0 * inv), (half_t)(num1 * inv)};
 }
 
 // Schedule "splits" merge: one wavefront per (query head, sequence).
@@ -666,8 +696,8 @@ __global__ __launch_bounds__(kWave) void paged_decode_merge_kernel(
   const int n_splits = splits_for_pages(pages_of(len), max_splits, min_pages_per_split);
   if (n_splits == 1) return;  // the split kernel already wrote the final row
   const int64_t cell0 = ((int64_t)b * num_q_heads + hq) * max_splits;
-  merge_row<false>(part_lse + cell0, 1, part_o + cell0 * kHeadDim, kHeadDim, n_splits, nullptr, 0,
-                   nullptr, 0, 0, out + ((int64_t)b * num_q_heads + hq) * kHeadDim, threadIdx.x);
+  merge_row<false>(part_lse + cell0, 1, part_o + cell0 * kHD, kHD, n_splits, nullptr, 0,
+                   nullptr, 0, 0, out + ((int64_t)b * num_q_heads + hq) * kHD, threadIdx.x);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -834,6 +864,8 @@ __device__ __forceinline__ void merge_row_wide(const float *__restrict__ lse, in
                                                int n_parts, half_t *out_row, int tid, float *red) {
   const int lane = tid & 63;
   const int wave = tid >> 6;
+  const bool live_col = 2 * lane < kHD;  // see merge_row
+  const int mcol = live_col ? 2 * lane : 0;
   float mx = -INFINITY;
   for (int s = tid; s < n_parts; s += kMergeWaves * kWave) mx = fmaxf(mx, lse[(int64_t)s * lse_stride]);
 #pragma unroll
@@ -855,7 +887,7 @@ __device__ __forceinline__ void merge_row_wide(const float *__restrict__ lse, in
     for (; s + 16 <= cnt; s += 16) {
       float2 r[16];
 #pragma unroll
-      for (int u = 0; u < 16; ++u) r[u] = *(const float2 *)(po + (int64_t)(base + s + u) * po_stride + 2 * lane);
+      for (int u = 0; u < 16; ++u) r[u] = *(const float2 *)(po + (int64_t)(base + s + u) * po_stride + mcol);
 #pragma unroll
       for (int u = 0; u < 16; ++u) {
         const float wu = __shfl(w, s + u, kWave);
@@ -864,7 +896,7 @@ __device__ __forceinline__ void merge_row_wide(const float *__restrict__ lse, in
       }
     }
     for (; s < cnt; ++s) {
-      const float2 r = *(const float2 *)(po + (int64_t)(base + s) * po_stride + 2 * lane);
+      const float2 r = *(const float2 *)(po + (int64_t)(base + s) * po_stride + mcol);
       const float wu = __shfl(w, s, kWave);
       num0 += wu * r.x;
       num1 += wu * r.y;
@@ -872,22 +904,24 @@ __device__ __forceinline__ void merge_row_wide(const float *__restrict__ lse, in
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) den += xor_lane(den, off);
-  float *sums = red + 8;  // [kMergeWaves][kHeadDim], then the denominators
-  sums[wave * kHeadDim + 2 * lane] = num0;
-  sums[wave * kHeadDim + 2 * lane + 1] = num1;
-  if (lane == 0) sums[kMergeWaves * kHeadDim + wave] = den;
+  float *sums = red + 8;  // [kMergeWaves][kHD], then the denominators
+  if (live_col) {
+    sums[wave * kHD + mcol] = num0;
+    sums[wave * kHD + mcol + 1] = num1;
+  }
+  if (lane == 0) sums[kMergeWaves * kHD + wave] = den;
   __syncthreads();
   if (wave != 0) return;
   float d = 0.f, o0 = 0.f, o1 = 0.f;
 #pragma unroll
   for (int w2 = 0; w2 < kMergeWaves; ++w2) {
-    o0 += sums[w2 * kHeadDim + 2 * lane];
-    o1 += sums[w2 * kHeadDim + 2 * lane + 1];
-    d += sums[kMergeWaves * kHeadDim + w2];
+    o0 += sums[w2 * kHD + mcol];
+    o1 += sums[w2 * kHD + mcol + 1];
+    d += sums[kMergeWaves * kHD + w2];
   }
   const float inv = 1.0f / d;
   typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-  *(half2_t *)(out_row + 2 * lane) = half2_t{(half_t)(o0 * inv), (half_t)(o1 * inv)};
+  if (live_col) *(half2_t *)(out_row + mcol) = half2_t{(half_t)(o0 * inv), (half_t)(o1 * inv)};
 }
 
 // Balanced-schedule merge, one workgroup per (query head, sequence) -- or, without a shared
@@ -902,7 +936,7 @@ __global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merg
     const float *__restrict__ part_lse, const float *__restrict__ pre_o,
     const float *__restrict__ pre_lse, int32_t pre_splits, int32_t batch, int32_t num_q_heads,
     int32_t by_boundary, int32_t bt_stride, int32_t chunks, int32_t heads_per_wg) {
-  __shared__ float red[8 + kMergeWaves * kHeadDim + kMergeWaves];
+  __shared__ float red[8 + kMergeWaves * kHD + kMergeWaves];
   // heads_per_wg 1: the workgroup has one row (query head); 4: each wavefront has its own
   const int hq = blockIdx.x * heads_per_wg + (heads_per_wg > 1 ? (int)(threadIdx.x >> 6) : 0);
   int b = blockIdx.y;
@@ -925,13 +959,13 @@ __global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merg
   const int64_t cell0 = (int64_t)(c_first + b) * num_q_heads + hq;
   const int64_t pre0 = (int64_t)b * num_q_heads + hq;
   const int64_t pre_step = (int64_t)batch * num_q_heads;
-  half_t *out_row = out + ((int64_t)b * num_q_heads + hq) * kHeadDim;
+  half_t *out_row = out + ((int64_t)b * num_q_heads + hq) * kHD;
   if (pre_splits == 0 && n_parts > 16 && blockDim.x == kMergeWaves * kWave) {  // uniform in the workgroup
     // a long row takes the whole workgroup; with a row per wavefront the rows take turns
     for (int r = 0; r < heads_per_wg; ++r) {
       const int shift = heads_per_wg > 1 ? r - (int)(threadIdx.x >> 6) : 0;  // from this wavefront's row to row r
-      merge_row_wide(part_lse + cell0 + shift, num_q_heads, part_o + (cell0 + shift) * kHeadDim,
-                     (int64_t)num_q_heads * kHeadDim, n_parts, out_row + (int64_t)shift * kHeadDim,
+      merge_row_wide(part_lse + cell0 + shift, num_q_heads, part_o + (cell0 + shift) * kHD,
+                     (int64_t)num_q_heads * kHD, n_parts, out_row + (int64_t)shift * kHD,
                      threadIdx.x, red);
       __syncthreads();
     }
@@ -940,13 +974,13 @@ __global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merg
   if (heads_per_wg == 1 && threadIdx.x >= kWave) return;
   const int lane = threadIdx.x & (kWave - 1);
   if (pre_splits == 0) {
-    merge_row<false>(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
-                     (int64_t)num_q_heads * kHeadDim, n_parts, nullptr, 0, nullptr, 0, 0, out_row,
+    merge_row<false>(part_lse + cell0, num_q_heads, part_o + cell0 * kHD,
+                     (int64_t)num_q_heads * kHD, n_parts, nullptr, 0, nullptr, 0, 0, out_row,
                      lane);
   } else {
-    merge_row<true>(part_lse + cell0, num_q_heads, part_o + cell0 * kHeadDim,
-                    (int64_t)num_q_heads * kHeadDim, n_parts, pre_lse + pre0, pre_step,
-                    pre_o + pre0 * kHeadDim, pre_step * kHeadDim, pre_splits, out_row, lane);
+    merge_row<true>(part_lse + cell0, num_q_heads, part_o + cell0 * kHD,
+                    (int64_t)num_q_heads * kHD, n_parts, pre_lse + pre0, pre_step,
+                    pre_o + pre0 * kHD, pre_step * kHD, pre_splits, out_row, lane);
   }
 }
 
@@ -977,9 +1011,9 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   auto zero_empty_rows = [&]() {
     for (int bz = cidx; bz < batch; bz += chunks) {
       if (seq_lens[bz] <= 0 && n < group) {
-        half_t *o = out + ((int64_t)bz * num_q_heads + h * group + n) * kHeadDim + 4 * g;
+        half_t *o = out + ((int64_t)bz * num_q_heads + h * group + n) * kHD + 4 * g;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) *(half4_t *)(o + 16 * j) = half4_t{0, 0, 0, 0};
+        for (int j = 0; j < kJTiles; ++j) *(half4_t *)(o + 16 * j) = half4_t{0, 0, 0, 0};
       }
     }
   };
@@ -1030,16 +1064,16 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   }
 
   const int hq0 = h * group;
-  const int64_t row_stride = (int64_t)2 * num_kv_heads * kHeadDim;
+  const int64_t row_stride = (int64_t)2 * num_kv_heads * kHD;
   // this lane's row and column inside page 0 (see PageRegs / PageRegsFp8)
-  Elem *k_lane = kv + (int64_t)h * kHeadDim + (FP8 ? 16 : 8) * g + n * row_stride;
-  Elem *v_lane = FP8 ? kv + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7) +
+  Elem *k_lane = kv + (int64_t)h * kHD + (FP8 ? 16 : 8) * g + n * row_stride;
+  Elem *v_lane = FP8 ? kv + (int64_t)(num_kv_heads + h) * kHD + 16 * (n & (kHD / 16 - 1)) +
                            (2 * g + (n >> 3)) * row_stride
-                     : kv + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n + g * row_stride;
+                     : kv + (int64_t)(num_kv_heads + h) * kHD + 8 * (n & (kVCols - 1)) + g * row_stride;
   const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
   half8_t qf[4];
   auto fetch_q_into = [&](half8_t (&dst)[4], int b) {
-    const half_t *row0 = q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHeadDim;
+    const half_t *row0 = q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHD;
     if constexpr (FP8) {
       load_q_fp8_order(dst, row0, n, g, group);
     } else {
@@ -1048,20 +1082,20 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   };
   // This lane's parts of the step's new K and V rows of sequence b (see the fused append below).
   auto fetch_new_rows = [&](uint4_t (&kr)[4], uint4_t (&vr)[2], int b) {
-    const half_t *kn = k_new + (int64_t)b * k_new_stride + (int64_t)h * kHeadDim;
-    const half_t *vn = v_new + (int64_t)b * v_new_stride + (int64_t)h * kHeadDim;
+    const half_t *kn = k_new + (int64_t)b * k_new_stride + (int64_t)h * kHD;
+    const half_t *vn = v_new + (int64_t)b * v_new_stride + (int64_t)h * kHD;
     if constexpr (FP8) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < kHD / 64; ++j) {
         kr[2 * j] = *(const uint4_t *)(kn + 64 * j + 16 * g);
         kr[2 * j + 1] = *(const uint4_t *)(kn + 64 * j + 16 * g + 8);
       }
-      vr[0] = *(const uint4_t *)(vn + 16 * (n & 7));
-      vr[1] = *(const uint4_t *)(vn + 16 * (n & 7) + 8);
+      vr[0] = *(const uint4_t *)(vn + 16 * (n & (kHD / 16 - 1)));
+      vr[1] = *(const uint4_t *)(vn + 16 * (n & (kHD / 16 - 1)) + 8);
     } else {
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) kr[kk] = *(const uint4_t *)(kn + 32 * kk + 8 * g);
-      vr[0] = *(const uint4_t *)(vn + 8 * n);
+      for (int kk = 0; kk < kKSteps; ++kk) kr[kk] = *(const uint4_t *)(kn + 32 * kk + 8 * g);
+      vr[0] = *(const uint4_t *)(vn + 8 * (n & (kVCols - 1)));
       vr[1] = uint4_t{0, 0, 0, 0};  // fp8 only
     }
   };
@@ -1093,9 +1127,9 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     // register copies that wait for it, here in front of the first page requests.
     const int nn = n < group ? n : group - 1;
     const half_t *row = q + (int64_t)(ahead_b < batch ? ahead_b : cur_b) * q_batch_stride +
-                        (int64_t)(hq0 + nn) * kHeadDim + (FP8 ? 16 : 8) * g;
+                        (int64_t)(hq0 + nn) * kHD + (FP8 ? 16 : 8) * g;
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {  // the d order of load_q / load_q_fp8_order
+    for (int kk = 0; kk < kKSteps; ++kk) {  // the d order of load_q / load_q_fp8_order
       q_ahead[kk] = *(const uint4_t *)(row + (FP8 ? 64 * (kk >> 1) + 8 * (kk & 1) : 32 * kk));
     }
   }
@@ -1106,8 +1140,8 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     // the sequence lies inside this chunk and has no shared-prefix partials to merge with
     const bool whole = cu_lo >= f0 && cu_hi <= f1 && skip == 0;
     const int64_t cell = (int64_t)(cidx + cur_b) * num_q_heads + hq0;
-    half_t *out_row = out + ((int64_t)cur_b * num_q_heads + hq0) * kHeadDim;
-    store_state(st, whole, out_row, part_o + cell * kHeadDim, kHeadDim, part_lse + cell, 1, n, g,
+    half_t *out_row = out + ((int64_t)cur_b * num_q_heads + hq0) * kHD;
+    store_state(st, whole, out_row, part_o + cell * kHD, kHD, part_lse + cell, 1, n, g,
                 group, v_scale);
   };
   // A sequence that ends inside the chunk is parked (see park_state) and written with the
@@ -1117,8 +1151,8 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   bool parked_whole = false;
   auto unpark = [&]() {
     const int64_t cell = (int64_t)(cidx + parked_b) * num_q_heads + hq0;
-    half_t *out_row = out + ((int64_t)parked_b * num_q_heads + hq0) * kHeadDim;
-    unpark_state(park, parked_whole, out_row, part_o + cell * kHeadDim, part_lse + cell, n, g, group);
+    half_t *out_row = out + ((int64_t)parked_b * num_q_heads + hq0) * kHD;
+    unpark_state(park, parked_whole, out_row, part_o + cell * kHD, part_lse + cell, n, g, group);
     parked_b = -1;
   };
   auto flush_at_crossing = [&]() {
@@ -1164,7 +1198,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
           st.reset();
           if (cur_b == ahead_b) {
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) qf[kk] = __builtin_bit_cast(half8_t, q_ahead[kk]);
+            for (int kk = 0; kk < kKSteps; ++kk) qf[kk] = __builtin_bit_cast(half8_t, q_ahead[kk]);
           } else {
             fetch_q_into(qf, cur_b);
             wait_vector_loads();
@@ -1180,7 +1214,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
           uint4_t v_row[2];
           if (cur_b == rows_b) {
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) k_row[kk] = k_ahead[kk];
+            for (int kk = 0; kk < kKSteps; ++kk) k_row[kk] = k_ahead[kk];
             v_row[0] = v_ahead[0];
             v_row[1] = v_ahead[1];
           } else {
@@ -1192,9 +1226,9 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
           if constexpr (FP8) {
             // the rows are quantised as the append kernel would, stored, and attended as stored
             if (n == t_new) {
-              uint8_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 16 * g;
+              uint8_t *dst = kv + slot_off + (int64_t)h * kHD + 16 * g;
 #pragma unroll
-              for (int j = 0; j < 2; ++j) {
+              for (int j = 0; j < kHD / 64; ++j) {
                 const uint2_t lo = half_to_codes<KV>(__builtin_bit_cast(half8_t, k_row[2 * j]), k_inv);
                 const uint2_t hi = half_to_codes<KV>(__builtin_bit_cast(half8_t, k_row[2 * j + 1]), k_inv);
                 const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
@@ -1206,7 +1240,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
               const uint2_t lo = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[0]), v_inv);
               const uint2_t hi = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[1]), v_inv);
               const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
-              *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 16 * (n & 7)) = x;
+              *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHD + 16 * (n & (kHD / 16 - 1))) = x;
 #pragma unroll
               for (int i = 0; i < 2; ++i) {
                 if (i == (t_new >> 3)) buf[dd].v[i] = x;
@@ -1214,9 +1248,9 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
             }
           } else {
             if (n == t_new) {
-              half_t *dst = kv + slot_off + (int64_t)h * kHeadDim + 8 * g;
+              half_t *dst = kv + slot_off + (int64_t)h * kHD + 8 * g;
 #pragma unroll
-              for (int kk = 0; kk < 4; ++kk) {
+              for (int kk = 0; kk < kKSteps; ++kk) {
                 const half8_t x = __builtin_bit_cast(half8_t, k_row[kk]);
                 buf[dd].k[kk] = x;
                 *(half8_t *)(dst + 32 * kk) = x;
@@ -1224,7 +1258,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
             }
             if (g == (t_new & 3)) {
               const half8_t x = __builtin_bit_cast(half8_t, v_row[0]);
-              *(half8_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHeadDim + 8 * n) = x;
+              *(half8_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHD + 8 * (n & (kVCols - 1))) = x;
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
                 if (i == (t_new >> 2)) buf[dd].v[i] = x;
@@ -1246,32 +1280,15 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   zero_empty_rows();
 }
 
+}  // namespace LITEKV_HD_NS
 }  // namespace litekv
 
 // ---------------------------------------------------------------------------------------------
 // Host side: argument checks and launches.
 // ---------------------------------------------------------------------------------------------
 namespace litekv {
+inline namespace LITEKV_HD_NS {
 
-struct DecodeArgs {
-  const void *q;
-  int64_t q_batch_stride;
-  const void *kv_pool;
-  const int32_t *block_table;
-  int32_t block_table_stride;
-  const int32_t *seq_lens;
-  void *out;
-  void *workspace;
-  size_t workspace_bytes;
-  int32_t batch, num_q_heads, num_kv_heads, head_dim, page_size;
-  int64_t num_pages;
-  float softmax_scale;
-  void *stream;
-  // the step's new rows [B][Hkv][D] for the append fused into the splits schedule (or null)
-  const void *k_new = nullptr;
-  const void *v_new = nullptr;
-  int64_t k_new_stride = 0, v_new_stride = 0;
-};
 
 // log2(page_size / 16) for the page sizes the kernels take (16, 32, 64 tokens), or -1.
 static int page_shift_of(int32_t page_size) {
@@ -1282,7 +1299,7 @@ static int page_shift_of(int32_t page_size) {
 static int validate_decode(const char *what, const DecodeArgs &a, size_t workspace_needed,
                            bool need_inputs) {
   LITEKV_REQUIRE(a.batch >= 0 && a.batch <= 65535, "%s: batch %d out of [0, 65535]", what, a.batch);
-  LITEKV_REQUIRE(a.head_dim == kHeadDim, "%s: head_dim %d unsupported (32, 64, 128 or 256)", what,
+  LITEKV_REQUIRE(a.head_dim == kHD, "%s: head_dim %d unsupported (32, 64, 128 or 256)", what,
                  a.head_dim);
   LITEKV_REQUIRE(page_shift_of(a.page_size) >= 0, "%s: page_size %d unsupported (16, 32 or 64)",
                  what, a.page_size);
@@ -1386,7 +1403,10 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
                                          : "paged_decode_split_fp8";
   int rc = check_split_plan(what, max_splits, min_pages_per_split);
   if (rc != LITEKV_OK) return rc;
-  if (a.head_dim != kHeadDim) return launch_generic_decode(what, a, fp8_scales, format);
+#if LITEKV_HD == 128
+  if (a.head_dim == 64) return hd64_split(a, max_splits, min_pages_per_split, fp8_scales, format);
+#endif
+  if (a.head_dim != kHD) return launch_generic_decode(what, a, fp8_scales, format);
   rc = validate_decode(what, a,
                        splits_workspace_bytes(a.batch, a.num_q_heads, a.head_dim, max_splits), true);
   if (rc != LITEKV_OK) return rc;
@@ -1454,7 +1474,10 @@ static int launch_merge(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   const char *what = "paged_decode_merge";
   int rc = check_split_plan(what, max_splits, min_pages_per_split);
   if (rc != LITEKV_OK) return rc;
-  if (a.head_dim != kHeadDim && generic_head_dim(a.head_dim)) {  // launch_generic_decode wrote the rows
+#if LITEKV_HD == 128
+  if (a.head_dim == 64) return hd64_merge(a, max_splits, min_pages_per_split);
+#endif
+  if (a.head_dim != kHD && generic_head_dim(a.head_dim)) {  // launch_generic_decode wrote the rows
     clear_error();
     return LITEKV_OK;
   }
@@ -1545,8 +1568,10 @@ static int check_chunks(const char *what, int32_t batch, int32_t bt_stride, int3
 static thread_local hipEvent_t g_profile_start = nullptr;
 static thread_local hipEvent_t g_profile_stop = nullptr;
 
+}  // namespace LITEKV_HD_NS
 }  // namespace litekv
 
+#if LITEKV_HD == 128  // the C ABI lives in the head dim 128 build of this file
 extern "C" int32_t litekv_paged_decode_balanced_chunks(int32_t num_kv_heads) {
   return num_kv_heads > 0 ? litekv::auto_chunks(num_kv_heads) : 0;
 }
@@ -1569,7 +1594,9 @@ extern "C" size_t litekv_decode_plan_bytes_paged(int32_t batch, int32_t block_ta
   return litekv::plan_bytes_for(batch, (int64_t)block_table_stride << shift, num_kv_heads, chunks);
 }
 
+#endif  // LITEKV_HD == 128
 namespace litekv {
+inline namespace LITEKV_HD_NS {
 static int launch_plan(const char *what, const int32_t *block_table, int32_t block_table_stride,
                        const int32_t *seq_lens, int32_t batch, int32_t num_kv_heads,
                        int32_t page_size, int64_t num_pages, int32_t chunks, int32_t shared_pages,
@@ -1603,8 +1630,10 @@ static int launch_plan(const char *what, const int32_t *block_table, int32_t blo
                      shared_pages << shift, static_cast<int32_t *>(plan));
   return check_launch(what);
 }
+}  // namespace LITEKV_HD_NS
 }  // namespace litekv
 
+#if LITEKV_HD == 128  // the C ABI lives in the head dim 128 build of this file
 extern "C" int litekv_decode_plan(const int32_t *block_table, int32_t block_table_stride,
                                   const int32_t *seq_lens, int32_t batch, int32_t num_kv_heads,
                                   int32_t page_size, int64_t num_pages, int32_t chunks, void *plan,
@@ -1630,7 +1659,9 @@ extern "C" int litekv_profile_next_decode(void *start_event, void *stop_event) {
   return LITEKV_OK;
 }
 
+#endif  // LITEKV_HD == 128
 namespace litekv {
+inline namespace LITEKV_HD_NS {
 // The balanced decode step; with shared_pages > 0 preceded by the shared-prefix launch.
 static int launch_balanced(const char *what, const void *q, int64_t q_batch_stride, void *kv_pool,
                            const float *fp8_scales, const int32_t *block_table,
@@ -1653,8 +1684,16 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   DecodeArgs a{q, q_batch_stride, kv_pool, block_table ? block_table : &dummy_table,
                block_table_stride, seq_lens, out, workspace, workspace_bytes, batch, num_q_heads,
                num_kv_heads, head_dim, page_size, num_pages, softmax_scale, stream};
-  if (head_dim != kHeadDim) {
-    // other head dims: the generic kernel, which takes its page ids from the block table where
+#if LITEKV_HD == 128
+  if (head_dim == 64 && shared_pages == 0) {
+    return hd64_balanced(what, q, q_batch_stride, kv_pool, fp8_scales, seq_lens, plan, plan_bytes,
+                         k_new, v_new, k_new_stride, v_new_stride, out, workspace, workspace_bytes,
+                         batch, num_q_heads, num_kv_heads, page_size, num_pages, block_table_stride,
+                         chunks, softmax_scale, stream, format);
+  }
+#endif
+  if (head_dim != kHD) {
+    // other head dims (and 64 over a shared prefix): the generic kernel, which takes its page ids from the block table where
     // the caller gave one (then shared pages are attended like any others), else from the plan
     a.k_new = k_new;
     a.v_new = v_new;
@@ -1763,8 +1802,10 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
                      batch, num_q_heads, by_boundary ? 1 : 0, sub_stride, chunks, merge_heads);
   return check_launch("paged_decode_balanced_merge");
 }
+}  // namespace LITEKV_HD_NS
 }  // namespace litekv
 
+#if LITEKV_HD == 128  // the C ABI lives in the head dim 128 build of this file
 extern "C" int litekv_paged_decode_balanced(
     const void *q, int64_t q_batch_stride, void *kv_pool, const int32_t *seq_lens, void *plan,
     size_t plan_bytes, const void *k_new, const void *v_new, int64_t k_new_stride,
@@ -2023,7 +2064,10 @@ extern "C" int litekv_paged_decode_append_int8(
 // caller's workspace. Every device the library runs on holds its own copy of the array until
 // the process ends; its address on a device is looked up once, with that device current.
 // ---------------------------------------------------------------------------------------------
+#endif  // LITEKV_HD == 128
+#if LITEKV_HD == 128
 namespace litekv {
+inline namespace LITEKV_HD_NS {
 
 static __device__ __align__(256) unsigned char scratch[LITEKV_STATIC_SCRATCH_BYTES];
 
@@ -2053,8 +2097,11 @@ static int static_scratch(const char *what, void **ptr_out) {
   return LITEKV_OK;
 }
 
+}  // namespace LITEKV_HD_NS
 }  // namespace litekv
+#endif  // LITEKV_HD == 128
 
+#if LITEKV_HD == 128  // the C ABI lives in the head dim 128 build of this file
 extern "C" int litekv_paged_decode_static(const void *q, int64_t q_batch_stride, const void *kv_pool,
                                           const int32_t *block_table, int32_t block_table_stride,
                                           const int32_t *seq_lens, void *out, int32_t batch,
@@ -2089,3 +2136,30 @@ extern "C" int litekv_paged_decode_static(const void *q, int64_t q_batch_stride,
   if (rc != LITEKV_OK) return rc;
   return litekv::launch_merge(a, max_splits, min_pages_per_split);
 }
+
+#endif  // LITEKV_HD == 128
+
+#if LITEKV_HD == 64
+// What the head dim 128 build, which owns the C ABI, calls for head_dim == 64 (see common.h).
+namespace litekv {
+int hd64_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split,
+               const float *scales, int format) {
+  return launch_split(a, max_splits, min_pages_per_split, scales, format);
+}
+int hd64_merge(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split) {
+  return launch_merge(a, max_splits, min_pages_per_split);
+}
+int hd64_balanced(const char *what, const void *q, int64_t q_batch_stride, void *kv_pool,
+                  const float *scales, const int32_t *seq_lens, void *plan, size_t plan_bytes,
+                  const void *k_new, const void *v_new, int64_t k_new_stride, int64_t v_new_stride,
+                  void *out, void *workspace, size_t workspace_bytes, int32_t batch,
+                  int32_t num_q_heads, int32_t num_kv_heads, int32_t page_size, int64_t num_pages,
+                  int32_t block_table_stride, int32_t chunks, float softmax_scale, void *stream,
+                  int format) {
+  return launch_balanced(what, q, q_batch_stride, kv_pool, scales, nullptr, seq_lens, plan,
+                         plan_bytes, k_new, v_new, k_new_stride, v_new_stride, out, workspace,
+                         workspace_bytes, batch, num_q_heads, num_kv_heads, kHD, page_size, num_pages,
+                         block_table_stride, chunks, 0, softmax_scale, stream, format);
+}
+}  // namespace litekv
+#endif  // LITEKV_HD == 64

@@ -451,3 +451,28 @@ def test_head_dims_shared_prefix(head_dim):
     ref = _oracle(case)
     out = _run(case, schedule="balanced", shared_pages=shared_pages)
     assert_attention_close(out, ref, f"shared prefix head_dim {head_dim}")
+
+
+def test_head_dim_64_at_a_larger_size():
+    """Head dim 64 on the MFMA kernels at a size where chunks cross many sequences and sequences
+    span many chunks: both schedules against the oracle, fused append bit exact, repeatable."""
+    print("decode head_dim 64, larger batch", flush=True)
+    lens = workloads.uniform_lens(641, 24, 1, 3000) + [0, 15, 16, 4095]
+    case = workloads.make_decode_case("d64-large", 642, lens, 32, 8, device=DEV, head_dim=64)
+    pool_ref = case.kv_pool.clone()
+    ops.kv_append(case.k_new, case.v_new, case.slot_mapping, pool_ref)
+    ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool_ref), case.block_table.cpu().numpy(),
+                                case.seq_lens.cpu().numpy(), case.softmax_scale)
+    plan = ops.DecodePlan(case.block_table, case.seq_lens, 32, 8, case.num_pages)
+    pool = case.kv_pool.clone()
+    out = ops.decode_step(case.q, pool, plan, case.k_new, case.v_new, case.softmax_scale)
+    again = ops.decode_step(case.q, pool, plan, None, None, case.softmax_scale)
+    torch.cuda.synchronize()
+    assert torch.equal(pool.view(torch.int16), pool_ref.view(torch.int16))
+    assert_attention_close(out, ref, "head_dim 64 balanced, fused append")
+    assert_attention_close(again, ref, "head_dim 64 balanced")
+    for kw in ({"num_splits": 1}, {"num_splits": 5}, {"max_splits": 16, "min_pages_per_split": 4},
+               {"schedule": "balanced", "chunks": 37}):
+        got = ops.paged_decode(case.q, pool_ref, case.block_table, case.seq_lens, case.softmax_scale, **kw)
+        torch.cuda.synchronize()
+        assert_attention_close(got, ref, f"head_dim 64 {kw}")
