@@ -31,6 +31,11 @@ from . import ops
 LOG2E = 1.4426950408889634
 
 
+def _page_size(atten_info) -> int:
+    """Tokens per page of the step's pools (metadata built by other code may not carry it: 16)."""
+    return int(getattr(atten_info, "page_size", 16) or 16)
+
+
 class Attention:
     def __init__(self, num_q_heads: int, num_kv_heads: int, head_dim: int):
         self.num_q_heads = num_q_heads
@@ -61,9 +66,10 @@ class Attention:
             ops.kv_append(xk, xv, atten_info.cur_select_index, pool)
         if getattr(atten_info, "is_paged_chunk_prefill", False):
             return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens,
-                                     atten_info.context_lens_i32, int(atten_info.max_actual_q_seq_len), scale)
+                                     atten_info.context_lens_i32, int(atten_info.max_actual_q_seq_len), scale,
+                                     page_size=_page_size(atten_info))
         return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens, None,
-                                 int(atten_info.max_actual_seq_len), scale)
+                                 int(atten_info.max_actual_seq_len), scale, page_size=_page_size(atten_info))
 
     def _context_forward_fp8(self, xq, xk, xv, atten_info, pool, scales, scale) -> torch.Tensor:
         chunked = getattr(atten_info, "is_paged_chunk_prefill", False)
@@ -77,9 +83,10 @@ class Attention:
         if chunked:
             return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens,
                                      atten_info.context_lens_i32, int(atten_info.max_actual_q_seq_len), scale,
-                                     kv_scales=scales)
+                                     kv_scales=scales, page_size=_page_size(atten_info))
         return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens, None,
-                                 int(atten_info.max_actual_seq_len), scale, kv_scales=scales)
+                                 int(atten_info.max_actual_seq_len), scale, kv_scales=scales,
+                                 page_size=_page_size(atten_info))
 
     def token_forward(self, xq, xk, xv, atten_info, layer_index: int, qk_scale=None) -> torch.Tensor:
         """Decode: xq [B, Hq, D], xk / xv [B, Hkv, D], one new token per sequence (None when
@@ -95,4 +102,5 @@ class Attention:
                 ops.kv_append_quantised(xk, xv, atten_info.cur_select_index, pool, scales)
             else:
                 ops.kv_append(xk, xv, atten_info.cur_select_index, pool)
-        return ops.paged_decode(xq, pool, atten_info.block_table, atten_info.seq_lens_i32, scale, kv_scales=scales)
+        return ops.paged_decode(xq, pool, atten_info.block_table, atten_info.seq_lens_i32, scale, kv_scales=scales,
+                                page_size=_page_size(atten_info))

@@ -52,6 +52,7 @@ class ModelExecutor:
         self.atten_info = AttentionInfo()
         self.atten_info.kv_buffer = self.kv_mem_manager.gpu_kv_buffer
         self.atten_info.kv_scales = self.kv_mem_manager.kv_scales
+        self.atten_info.page_size = self.page_size
         self.build_decode_plans = build_decode_plans and torch.device(device).type == "cuda"
         # K + V bytes of one token in a layer's pool (what a decode step reads per token attended)
         self.kv_token_bytes = 2 * self.local_kv_heads * head_dim * torch.empty((), dtype=dtype).element_size()

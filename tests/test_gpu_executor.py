@@ -341,3 +341,53 @@ def test_static_batch_prefill_then_decode_equals_the_packed_flow():
         torch.cuda.synchronize()
         assert float((o_s.float() - o_p.float()).abs().max()) <= 1e-3, f"decode step {step}"
         assert_attention_close(o_s, _oracle_decode(static, qd, 0), f"static batch decode step {step}")
+
+
+@pytest.mark.parametrize("page_size,head_dim", [(32, 128), (64, 64), (16, 64), (16, 256)])
+def test_executor_flow_at_other_page_sizes_and_head_dims(page_size, head_dim):
+    """The same host flow -- packed prefill, a chunk over cached history, fused decode steps --
+    on pools with larger pages and other head dims."""
+    print(f"executor: page_size {page_size}, head_dim {head_dim}", flush=True)
+    hq, hkv = 16, 4
+    scale = 1.0 / math.sqrt(head_dim)
+    ex = ModelExecutor(num_layers=1, num_q_heads=hq, num_kv_heads=hkv, head_dim=head_dim, num_pages=64,
+                       max_seq_len=512, max_requests=8, device=DEV, page_size=page_size)
+    ex.kv_mem_manager.gpu_kv_buffer[0].normal_()
+    attn = Attention(hq, hkv, head_dim)
+
+    def rows(tokens, heads, seed):
+        g = torch.Generator(device=DEV).manual_seed(seed)
+        return torch.randn((tokens, heads, head_dim), generator=g, device=DEV, dtype=torch.float16)
+
+    lens = [37, 16, 90, 5]
+    ids = ex.reserve_paged_requests(lens, reserved_lengths=[n + 60 for n in lens])
+    ex.activate_paged_packed_prefill_batch(ids, lens)
+    info = ex.atten_info
+    assert info.page_size == page_size
+    q, k, v = rows(sum(lens), hq, 1), rows(sum(lens), hkv, 2), rows(sum(lens), hkv, 3)
+    out = attn.context_forward(q, k, v, info, 0, scale * LOG2E)
+    torch.cuda.synchronize()
+    ref = c_oracle.varlen_prefill(to_np16(q), to_np16(k), to_np16(v), info.b_start_loc.cpu().numpy(),
+                                  np.asarray(lens, dtype=np.int32), scale)
+    assert_attention_close(out, ref, "prefill")
+    # a chunk of 30 more tokens for request 2, over its 90 cached ones
+    ex.activate_paged_chunk_prefill_batch((ids[2],), [90], [30])
+    info = ex.atten_info
+    q, k, v = rows(30, hq, 4), rows(30, hkv, 5), rows(30, hkv, 6)
+    out = attn.context_forward(q, k, v, info, 0, scale * LOG2E)
+    torch.cuda.synchronize()
+    ref = c_oracle.paged_prefill(to_np16(q), to_np16(info.kv_buffer[0]), info.block_table.cpu().numpy(),
+                                 info.cu_q_lens.cpu().numpy(), info.context_lens_i32.cpu().numpy(), scale,
+                                 page_size=page_size)
+    assert_attention_close(out, ref, "chunk over history")
+    for step in range(20):
+        ex.extend_paged_requests(ids)
+        info = ex.atten_info
+        q, k, v = rows(len(ids), hq, 100 + step), rows(len(ids), hkv, 200 + step), rows(len(ids), hkv, 300 + step)
+        out = attn.token_forward(q, k, v, info, 0, qk_scale=scale)
+        torch.cuda.synchronize()
+        sel = info.cur_select_index.long()
+        assert_bit_exact(info.kv_buffer[0][sel][:, :hkv], k, "appended K")
+        ref = c_oracle.paged_decode(to_np16(q), to_np16(info.kv_buffer[0]), info.block_table.cpu().numpy(),
+                                    info.seq_lens_i32.cpu().numpy(), scale, page_size=page_size)
+        assert_attention_close(out, ref, f"decode step {step}")
