@@ -43,6 +43,12 @@
 // exponentials of one half run beside the MFMAs of the other; the next tile's HBM -> LDS loads
 // leave a quarter at a time between MFMA pairs instead of in one burst behind the barrier.
 //
+// q and the output move as whole 256-byte rows: q comes in through the direct HBM -> LDS load
+// (into the half that tile 1 takes later) and is read back as fragments; the accumulators, which
+// hold O^T (4 consecutive d of one row per lane), are transposed through LDS after the last tile
+// and leave 4 rows per store instruction. Straight from registers, every q load and output store
+// touched 16 rows with 64 / 32 bytes each.
+//
 // About 235 registers per lane leave two wavefronts per SIMD: two workgroups share a compute
 // unit and drift apart, so one's softmax (vector ALU) overlaps the other's MFMAs and a
 // finishing block's prologue/epilogue hides behind its neighbour. Grid: x = kv head (times the
@@ -280,6 +286,33 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     }
   };
 
+  // q rows come in as whole 256-byte rows, 4 per direct-load instruction, into a region of the
+  // LDS half that tile 1 will take (8 KiB per wavefront, private to it), swizzled like a K tile;
+  // the fragments are read back from there. Requested before tile 0: vmcnt counts in order.
+  uint32_t q_lds = 0;
+  if constexpr (!SHARED) {
+    q_lds = ((wave & 2) ? v_lds : k_lds) + (uint32_t)(kTileHalfs * 2 + (wave & 1) * 8192);
+#pragma unroll
+    for (int u = 0; u < kColTiles; ++u) {
+      const int t = wave * kColTiles + u;
+      const int head = t / row_tiles;
+      const int row0 = m0 + (t - head * row_tiles) * 16;
+      const int hq = h * group + head0 + (head < heads_here ? head : 0);
+      const int first = row0 < q_len ? row0 : q_len - 1;
+      const char *base = (const char *)(q + (int64_t)(q_start + first) * q_stride + (int64_t)hq * kHeadDim);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int rip = 4 * i + r_loc;
+        const int chunk = slot ^ rip;
+        rip = first + rip < q_len ? rip : q_len - 1 - first;  // rows past the end re-read the last one
+        const uint32_t off = (uint32_t)rip * (uint32_t)q_stride * 2u + 16u * (uint32_t)chunk;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(q_lds + 4096u * u + 1024u * i), "v"(off), "s"(base)
+                     : "memory", "m0");
+      }
+    }
+  }
   issue_tile(0);
 
   // ---- this wavefront's columns: tile t = head (t / row_tiles), rows 16 * (t % row_tiles) ..
@@ -312,11 +345,30 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       qrow = q + (int64_t)(q_start + (ok ? row : 0)) * q_stride + (int64_t)hq * kHeadDim + 8 * g;
     }
     out_head[u] = hq;
+    if constexpr (!SHARED) continue;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
       const half8_t raw = ok ? *(const half8_t *)(qrow + 32 * kk) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
       typedef float float8_t __attribute__((ext_vector_type(8)));
       qf[u][kk] = __builtin_convertvector(__builtin_convertvector(raw, float8_t) * scale_log2, half8_t);
+    }
+  }
+  if constexpr (!SHARED) {
+    // the eight loads of tile 0 (four of an 8-bit pool) were requested after q's
+    if constexpr (FP8) {
+      __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+    }
+#pragma unroll
+    for (int u = 0; u < kColTiles; ++u) {
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const half8_t raw = *(const lds_half8_t *)(uintptr_t)(
+            q_lds + 4096u * u + (uint32_t)(n * 2 * kHeadDim + 16 * ((4 * kk + g) ^ n)));
+        typedef float float8_t __attribute__((ext_vector_type(8)));
+        qf[u][kk] = __builtin_convertvector(__builtin_convertvector(raw, float8_t) * scale_log2, half8_t);
+      }
     }
   }
 
@@ -709,6 +761,43 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     }
   }
 
+  if constexpr (!SHARED) {
+    // The accumulators hold O^T: a lane has 4 consecutive d of one row, so stored directly every
+    // store instruction would touch 16 rows with 32 bytes each. The rows go through LDS instead
+    // (the K/V tiles are done with) and leave as whole 256-byte rows, 4 rows per instruction.
+    constexpr int kOutPitch = 2 * kHeadDim + 16;  // bytes; 68 dwords: a half-wave's 8-byte writes hit 64 banks
+    __syncthreads();                              // every wavefront is done reading the last tile
+    const uint32_t mine = ((wave & 2) ? v_lds : k_lds) + (uint32_t)((wave & 1) * kColTiles * 16 * kOutPitch);
+#pragma unroll
+    for (int u = 0; u < kColTiles; ++u) {
+      const float inv = v_scale / dsum[u][0];
+      const uint32_t at = mine + (uint32_t)((u * 16 + n) * kOutPitch + 8 * g);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        *(__attribute__((address_space(3))) half4_t *)(uintptr_t)(at + 32u * j) =
+            half4_t{(half_t)(acc[j][u][0] * inv), (half_t)(acc[j][u][1] * inv),
+                    (half_t)(acc[j][u][2] * inv), (half_t)(acc[j][u][3] * inv)};
+      }
+    }
+    // lane l carries chunk l % 16 of row l / 16 + 4 * step
+    const int chunk = lane & 15, r4 = lane >> 4;
+#pragma unroll
+    for (int u = 0; u < kColTiles; ++u) {
+#pragma unroll
+      for (int step = 0; step < 4; ++step) {
+        const int r = 4 * step + r4;
+        const half8_t row = *(const lds_half8_t *)(uintptr_t)(mine + (uint32_t)((u * 16 + r) * kOutPitch + 16 * chunk));
+        const int t = wave * kColTiles + u;
+        const int head = t / row_tiles;
+        const int qrow_idx = m0 + (t - head * row_tiles) * 16 + r;
+        if (head < heads_here && qrow_idx < q_len) {
+          *(half8_t *)(out + (int64_t)(q_start + qrow_idx) * out_stride + (int64_t)out_head[u] * kHeadDim +
+                       8 * chunk) = row;
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int u = 0; u < kColTiles; ++u) {
     const float inv = v_scale / dsum[u][0];
