@@ -29,6 +29,7 @@ SOURCES = (
     "paged_decode_hd64.hip",
     "decode_advance.hip",
     "paged_prefill.hip",
+    "paged_prefill_hd64.hip",
     "generic_attention.hip",
 )
 
@@ -53,6 +54,7 @@ HIPCC_FLAGS = (
 # remarks on every such statement that m0 is a reserved register, which is the point of listing it.
 PER_FILE_FLAGS = {
     "paged_prefill.hip": ("-fno-honor-nans", "-Wno-inline-asm"),
+    "paged_prefill_hd64.hip": ("-fno-honor-nans", "-Wno-inline-asm"),
 }
 
 

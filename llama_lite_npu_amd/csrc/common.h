@@ -108,6 +108,19 @@ struct DecodeArgs {
   int64_t k_new_stride = 0, v_new_stride = 0;
 };
 
+// The launchers of the head dim 64 build of paged_prefill.hip (paged_prefill_hd64.hip; fp16 K/V).
+int hd64_paged_prefill(const char *what, const void *q, int64_t q_token_stride, const void *kv_pool,
+                       const int32_t *block_table, int32_t block_table_stride,
+                       const int32_t *cu_q_lens, const int32_t *context_lens, void *out,
+                       int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
+                       int32_t num_kv_heads, int32_t page_size, int64_t num_pages,
+                       int32_t max_q_len, float softmax_scale, void *stream);
+int hd64_varlen_prefill(const void *q, int64_t q_token_stride, const void *k, int64_t k_token_stride,
+                        const void *v, int64_t v_token_stride, const int32_t *seq_starts,
+                        const int32_t *seq_lens, void *out, int64_t out_token_stride, int32_t batch,
+                        int32_t num_q_heads, int32_t num_kv_heads, int32_t max_seq_len,
+                        int64_t num_tokens, float softmax_scale, void *stream);
+
 // The launchers of the head dim 64 build of paged_decode.hip (paged_decode_hd64.hip), to which the
 // head dim 128 build, which owns the C ABI, hands calls with head_dim == 64. `scales` marks a pool
 // of 8-bit codes of format `format` (kv_fp8.h).

@@ -59,7 +59,37 @@
 #include "common.h"
 #include "kv_fp8.h"
 
+// This file is compiled twice: as it stands for head dim 128, and through paged_prefill_hd64.hip
+// (which defines LITEKV_HD and includes it) for head dim 64 with fp16 K/V (paged or packed).
+// Everything sits in an inline namespace named after the head dim, so the two builds link side by
+// side; the C ABI and the shared-prefix launcher are in the 128 build, which hands 64-wide calls
+// to hd64_paged_prefill / hd64_varlen_prefill.
+#ifndef LITEKV_HD
+#define LITEKV_HD 128
+#endif
+#if LITEKV_HD == 128
+#define LITEKV_HD_NS hd128
+#elif LITEKV_HD == 64
+#define LITEKV_HD_NS hd64
+#else
+#error "paged_prefill.hip: LITEKV_HD must be 128 or 64"
+#endif
+
 namespace litekv {
+inline namespace LITEKV_HD_NS {
+
+constexpr int kHD = LITEKV_HD;              // head dim of this build of the file
+constexpr int kKSteps = kHD / 32;           // MFMA k steps of the first product
+constexpr int kJTiles = kHD / 16;           // 16-row tiles of O^T; also K fragments per 32-key half
+constexpr int kChunks = kHD / 8;            // 16-byte chunks of a staged row
+constexpr int kRowsPerLoad = 64 / kChunks;  // rows one direct-load instruction (64 x 16 bytes) fills
+constexpr int kLoadsPerWave = 16 / kRowsPerLoad;  // such instructions per wavefront, tile and operand
+
+// XOR applied to the 16-byte chunk index of staged row r, for K (and q) and for V. A row of 256
+// bytes covers all 64 banks, so consecutive rows must differ in the chunk; rows of 128 bytes
+// alternate between the bank halves, so it is every second row that must.
+__device__ __forceinline__ int k_swz(int r) { return kHD == 128 ? (r & 15) : ((r >> 1) & 7); }
+__device__ __forceinline__ int v_swz(int r) { return kHD == 128 ? 2 * (r & 7) : 2 * ((r >> 1) & 3); }
 
 constexpr float kLog2eP = 1.4426950408889634f;
 
@@ -96,7 +126,7 @@ constexpr int kKvTile = 64;
 constexpr int kColTiles = 2;      // 16-column tiles per wavefront
 constexpr int kTiledWaves = 4;
 constexpr int kWgColTiles = kColTiles * kTiledWaves;
-constexpr int kTileHalfs = kKvTile * kHeadDim;  // one staged tile: 64 rows of 256 bytes
+constexpr int kTileHalfs = kKvTile * kHD;  // one staged tile: 64 rows of 2 * kHD bytes
 
 typedef __attribute__((address_space(3))) half_t lds_half_t;
 typedef __attribute__((address_space(3))) half8_t lds_half8_t;
@@ -115,7 +145,7 @@ constexpr int kPagedPrefill = 0, kPackedPrefill = 1, kSharedPrefix = 2, kPagedPr
               kSharedPrefixFp8 = 4, kPagedPrefillInt8 = 5, kSharedPrefixInt8 = 6;
 
 template <int MODE>
-__global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_kernel(
+__global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_prefill_tiled_kernel(
     const half_t *__restrict__ q, int64_t q_stride, half_t *__restrict__ out, int64_t out_stride,
     PagedSource paged, PackedSource packed, PrefixTask prefix,
     const int32_t *__restrict__ q_starts_or_cu, const int32_t *__restrict__ q_lens_or_null,
@@ -192,20 +222,20 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   // ---- staging addresses -------------------------------------------------------------------
   // Direct-load instruction i of wavefront w fills tile rows 16w + 4i .. +3 (one page per
   // wavefront): lane l writes slot l % 16 of row 4i + l / 16.
-  const int r_loc = lane >> 4;
-  const int slot = lane & 15;
-  const uint32_t k_pitch = PAGED ? 2u * paged.num_kv_heads * kHeadDim * (FP8 ? 1u : 2u)
+  const int r_loc = lane / kChunks;
+  const int slot = lane % kChunks;
+  const uint32_t k_pitch = PAGED ? 2u * paged.num_kv_heads * kHD * (FP8 ? 1u : 2u)
                                  : (uint32_t)packed.k_stride * 2u;
   const uint32_t v_pitch = PAGED ? k_pitch : (uint32_t)packed.v_stride * 2u;
-  uint32_t koff[4], voff[4];  // byte offsets from the wavefront's 16-row base
+  uint32_t koff[kLoadsPerWave], voff[kLoadsPerWave];  // byte offsets from the wavefront's 16-row base
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int rip = 4 * i + r_loc;
-    const int ck = slot ^ rip;              // K: f(r) = r % 16
-    const int cv = slot ^ (2 * (rip & 7));  // V: f(r) = 2 * (r % 8)
-    koff[i] = rip * k_pitch + (uint32_t)(h * kHeadDim + 8 * ck) * 2u;
+  for (int i = 0; i < kLoadsPerWave; ++i) {
+    const int rip = kRowsPerLoad * i + r_loc;
+    const int ck = slot ^ k_swz(rip);
+    const int cv = slot ^ v_swz(rip);
+    koff[i] = rip * k_pitch + (uint32_t)(h * kHD + 8 * ck) * 2u;
     voff[i] = rip * v_pitch +
-              (uint32_t)(((PAGED ? paged.num_kv_heads : 0) + h) * kHeadDim + 8 * cv) * 2u;
+              (uint32_t)(((PAGED ? paged.num_kv_heads : 0) + h) * kHD + 8 * cv) * 2u;
   }
   const int32_t *table =
       PAGED ? paged.block_table + (SHARED ? 0 : (int64_t)b * paged.bt_stride) : nullptr;
@@ -234,8 +264,8 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       const int src_row = tok - pidx * kPageSize;
       const uint8_t *base = (const uint8_t *)paged.kv +
                             ((int64_t)pid * kPageSize + src_row) * (int64_t)k_pitch + 32 * (lane & 3);
-      const uint8_t *kp = base + h * kHeadDim;
-      const uint8_t *vp = base + (paged.num_kv_heads + h) * kHeadDim;
+      const uint8_t *kp = base + h * kHD;
+      const uint8_t *vp = base + (paged.num_kv_heads + h) * kHD;
       raw_k[0] = *(const uint4_t *)kp;
       raw_k[1] = *(const uint4_t *)(kp + 16);
       raw_v[0] = *(const uint4_t *)vp;
@@ -257,7 +287,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       vbase = (const char *)packed.v + (int64_t)(q_start + first) * v_pitch;
       src0 = first;
     }
-    const uint32_t dst = (uint32_t)((kt & 1) * kTileHalfs + 16 * wave * kHeadDim) * 2u;
+    const uint32_t dst = (uint32_t)((kt & 1) * kTileHalfs + 16 * wave * kHD) * 2u;
     auto load_rows = [&](uint32_t i, uint32_t ko, uint32_t vo) {
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                    :
@@ -270,13 +300,13 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     };
     if (row0 + 15 <= last_key) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) load_rows(i, koff[i], voff[i]);
+      for (int i = 0; i < kLoadsPerWave; ++i) load_rows(i, koff[i], voff[i]);
     } else {
       // Only in the last tile of a sequence. Rows past the last key re-read it: finite values
       // that zero probabilities multiply.
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int rip = 4 * i + r_loc;
+      for (int i = 0; i < kLoadsPerWave; ++i) {
+        const int rip = kRowsPerLoad * i + r_loc;
         int tok = row0 + rip;
         tok = tok < last_key ? tok : last_key;
         const uint32_t back = (uint32_t)(row0 + rip - tok) - (uint32_t)(row0 - src0);
@@ -291,7 +321,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   // the fragments are read back from there. Requested before tile 0: vmcnt counts in order.
   uint32_t q_lds = 0;
   if constexpr (!SHARED) {
-    q_lds = ((wave & 2) ? v_lds : k_lds) + (uint32_t)(kTileHalfs * 2 + (wave & 1) * 8192);
+    q_lds = ((wave & 2) ? v_lds : k_lds) + (uint32_t)(kTileHalfs * 2 + (wave & 1) * (64 * kHD));
 #pragma unroll
     for (int u = 0; u < kColTiles; ++u) {
       const int t = wave * kColTiles + u;
@@ -299,16 +329,16 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       const int row0 = m0 + (t - head * row_tiles) * 16;
       const int hq = h * group + head0 + (head < heads_here ? head : 0);
       const int first = row0 < q_len ? row0 : q_len - 1;
-      const char *base = (const char *)(q + (int64_t)(q_start + first) * q_stride + (int64_t)hq * kHeadDim);
+      const char *base = (const char *)(q + (int64_t)(q_start + first) * q_stride + (int64_t)hq * kHD);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        int rip = 4 * i + r_loc;
-        const int chunk = slot ^ rip;
+      for (int i = 0; i < kLoadsPerWave; ++i) {
+        int rip = kRowsPerLoad * i + r_loc;
+        const int chunk = slot ^ k_swz(rip);
         rip = first + rip < q_len ? rip : q_len - 1 - first;  // rows past the end re-read the last one
         const uint32_t off = (uint32_t)rip * (uint32_t)q_stride * 2u + 16u * (uint32_t)chunk;
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                      :
-                     : "s"(q_lds + 4096u * u + 1024u * i), "v"(off), "s"(base)
+                     : "s"(q_lds + (uint32_t)(32 * kHD) * u + 1024u * i), "v"(off), "s"(base)
                      : "memory", "m0");
       }
     }
@@ -316,7 +346,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   issue_tile(0);
 
   // ---- this wavefront's columns: tile t = head (t / row_tiles), rows 16 * (t % row_tiles) ..
-  half8_t qf[kColTiles][4];
+  half8_t qf[kColTiles][kKSteps];
   int q_pos[kColTiles];
   int out_row[kColTiles];   // packed row index, or -1
   int out_head[kColTiles];
@@ -333,7 +363,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       hq = h * group + (ok ? col - seq * group : 0);
       q_pos[u] = kv_end - 1;
       out_row[u] = ok ? seq : -1;
-      qrow = q + (int64_t)seq * prefix.q_batch_stride + (int64_t)hq * kHeadDim + 8 * g;
+      qrow = q + (int64_t)seq * prefix.q_batch_stride + (int64_t)hq * kHD + 8 * g;
     } else {
       const int head = t / row_tiles;
       const int row = m0 + (t - head * row_tiles) * 16 + n;
@@ -342,37 +372,37 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       const int last = q_len - 1;
       q_pos[u] = ctx + (row < last ? row : last);
       out_row[u] = ok ? q_start + row : -1;
-      qrow = q + (int64_t)(q_start + (ok ? row : 0)) * q_stride + (int64_t)hq * kHeadDim + 8 * g;
+      qrow = q + (int64_t)(q_start + (ok ? row : 0)) * q_stride + (int64_t)hq * kHD + 8 * g;
     }
     out_head[u] = hq;
     if constexpr (!SHARED) continue;
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
+    for (int kk = 0; kk < kKSteps; ++kk) {
       const half8_t raw = ok ? *(const half8_t *)(qrow + 32 * kk) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
       typedef float float8_t __attribute__((ext_vector_type(8)));
       qf[u][kk] = __builtin_convertvector(__builtin_convertvector(raw, float8_t) * scale_log2, half8_t);
     }
   }
   if constexpr (!SHARED) {
-    // the eight loads of tile 0 (four of an 8-bit pool) were requested after q's
+    // the loads of tile 0 (K and V; four of an 8-bit pool) were requested after q's
     if constexpr (FP8) {
       __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
     } else {
-      __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kLoadsPerWave));
     }
 #pragma unroll
     for (int u = 0; u < kColTiles; ++u) {
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
+      for (int kk = 0; kk < kKSteps; ++kk) {
         const half8_t raw = *(const lds_half8_t *)(uintptr_t)(
-            q_lds + 4096u * u + (uint32_t)(n * 2 * kHeadDim + 16 * ((4 * kk + g) ^ n)));
+            q_lds + (uint32_t)(32 * kHD) * u + (uint32_t)(n * 2 * kHD + 16 * ((4 * kk + g) ^ k_swz(n))));
         typedef float float8_t __attribute__((ext_vector_type(8)));
         qf[u][kk] = __builtin_convertvector(__builtin_convertvector(raw, float8_t) * scale_log2, half8_t);
       }
     }
   }
 
-  float4_t acc[8][kColTiles];
+  float4_t acc[kJTiles][kColTiles];
   float4_t dsum[kColTiles];
   float m_run[kColTiles];
   // Seed of the score accumulators in the fast tiles: -m_run (divided by k_mul), in all four
@@ -384,31 +414,31 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     seed[u] = float4_t{0.f, 0.f, 0.f, 0.f};
     dsum[u] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < kJTiles; ++j) acc[j][u] = float4_t{0.f, 0.f, 0.f, 0.f};
   }
   const half8_t ones = half8_t{1, 1, 1, 1, 1, 1, 1, 1};
 
   // Swizzled read addresses (LDS bytes) for the tile half in use; they flip between the halves
   // once per tile.
   // K, A operand of S^T: row 16m + n, chunk (4kk + g) ^ n.
-  uint32_t k_addr[4];
+  uint32_t k_addr[kKSteps];
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) {
-    k_addr[kk] = k_lds + 2u * (uint32_t)(n * kHeadDim + 8 * ((4 * kk + g) ^ n));
+  for (int kk = 0; kk < kKSteps; ++kk) {
+    k_addr[kk] = k_lds + 2u * (uint32_t)(n * kHD + 8 * ((4 * kk + g) ^ k_swz(n)));
   }
   // V^T, A operand of O^T: row 32 s2 + 4g + n/4 (+16), halfs 16j + 4(n%4); chunk pair j ^ (r%8).
   const int v_row = 4 * g + (n >> 2);
-  uint32_t v_addr[8];
+  uint32_t v_addr[kJTiles];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    v_addr[j] = v_lds + 2u * (uint32_t)(v_row * kHeadDim + 16 * (j ^ (v_row & 7)) + 4 * (n & 3));
+  for (int j = 0; j < kJTiles; ++j) {
+    v_addr[j] = v_lds + 2u * (uint32_t)(v_row * kHD + 8 * ((2 * j) ^ v_swz(v_row)) + 4 * (n & 3));
   }
   int flip = kTileHalfs * 2;  // bytes to the other half
   auto flip_halves = [&]() {
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) k_addr[kk] += flip;
+    for (int kk = 0; kk < kKSteps; ++kk) k_addr[kk] += flip;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v_addr[j] += flip;
+    for (int j = 0; j < kJTiles; ++j) v_addr[j] += flip;
     flip = -flip;
   };
 
@@ -423,9 +453,9 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
 #pragma unroll
       for (int u = 0; u < kColTiles; ++u) st[m][u] = SEEDED ? seed[u] : float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
+      for (int kk = 0; kk < kKSteps; ++kk) {
         const half8_t a =
-            *(const lds_half8_t *)(uintptr_t)(k_addr[kk] + 2u * (32 * s2 + 16 * m) * kHeadDim);
+            *(const lds_half8_t *)(uintptr_t)(k_addr[kk] + 2u * (32 * s2 + 16 * m) * kHD);
 #pragma unroll
         for (int u = 0; u < kColTiles; ++u) st[m][u] = mfma_16x16x32(a, qf[u][kk], st[m][u]);
       }
@@ -512,11 +542,11 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
 #pragma unroll
     for (int u = 0; u < kColTiles; ++u) dsum[u] = mfma_16x16x32(ones, pk[u], dsum[u]);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const uint32_t at = v_addr[j] + 2u * 32 * s2 * kHeadDim;
+    for (int j = 0; j < kJTiles; ++j) {
+      const uint32_t at = v_addr[j] + 2u * 32 * s2 * kHD;
       const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t *)(uintptr_t)at);
       const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-          (lds_short4_t *)(uintptr_t)(at + 2u * 16 * kHeadDim));
+          (lds_short4_t *)(uintptr_t)(at + 2u * 16 * kHD));
       const short8_t both = short8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
       const half8_t a = __builtin_bit_cast(half8_t, both);
 #pragma unroll
@@ -525,10 +555,10 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
   };
   // V^T fragment j (A operand: d rows 16j.., keys 32 s2 + {4g..4g+3, 16+4g..}) of the staged tile.
   auto load_vfrag = [&](int j, int s2) -> half8_t {
-    const uint32_t at = v_addr[j] + 2u * 32 * s2 * kHeadDim;
+    const uint32_t at = v_addr[j] + 2u * 32 * s2 * kHD;
     const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_t *)(uintptr_t)at);
     const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (lds_short4_t *)(uintptr_t)(at + 2u * 16 * kHeadDim));
+        (lds_short4_t *)(uintptr_t)(at + 2u * 16 * kHD));
     const short8_t both = short8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     return __builtin_bit_cast(half8_t, both);
   };
@@ -545,7 +575,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       // The codes of tile kt (requested a tile ago) become fp16 rows in its LDS half: 16-byte
       // chunk c of row r goes where the direct load of the fp16 path would have put it.
       const int r = lane >> 2;
-      const uint32_t row_at = (uint32_t)((kt & 1) * kTileHalfs + (16 * wave + r) * kHeadDim) * 2u;
+      const uint32_t row_at = (uint32_t)((kt & 1) * kTileHalfs + (16 * wave + r) * kHD) * 2u;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int chunk = 4 * (lane & 3) + j;
@@ -575,7 +605,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       next_kbase = (const char *)packed.k + (int64_t)(q_start + row0) * k_pitch;
       next_vbase = (const char *)packed.v + (int64_t)(q_start + row0) * v_pitch;
     }
-    next_dst = (uint32_t)((kt & 1) * kTileHalfs + 16 * wave * kHeadDim) * 2u;
+    next_dst = (uint32_t)((kt & 1) * kTileHalfs + 16 * wave * kHD) * 2u;
   };
   auto issue_rows = [&](int i) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -609,7 +639,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
         seed[u] = float4_t{sd, sd, sd, sd};
         dsum[u] *= alpha;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j][u] *= alpha;
+        for (int j = 0; j < kJTiles; ++j) acc[j][u] *= alpha;
         exponentials(u);
       }
       accumulate_sub(s2);
@@ -657,11 +687,11 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       // MFMAs, and the first half's V fragments requested before the block ends.
       // Region 1: all eight K fragments of the first half are requested at once.
       auto load_kfrag = [&](int s2, int i) -> half8_t {   // fragment i = (kk = i / 2, m = i % 2)
-        return *(const lds_half8_t *)(uintptr_t)(k_addr[i >> 1] + 2u * (32 * s2 + 16 * (i & 1)) * kHeadDim);
+        return *(const lds_half8_t *)(uintptr_t)(k_addr[i >> 1] + 2u * (32 * s2 + 16 * (i & 1)) * kHD);
       };
-      half8_t kf[8];
+      half8_t kf[kJTiles];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) kf[i] = load_kfrag(0, i);
+      for (int i = 0; i < kJTiles; ++i) kf[i] = load_kfrag(0, i);
 #pragma unroll
       for (int m = 0; m < 2; ++m) {
 #pragma unroll
@@ -671,9 +701,9 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       // Region 2: the first half's MFMAs; each fragment register takes the second half's
       // fragment once its pair is issued. Four accumulators in rotation: no MFMA waits for
       // the one before it.
-      half8_t kf1[8];
+      half8_t kf1[kJTiles];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < kJTiles; ++i) {
 #pragma unroll
         for (int u = 0; u < kColTiles; ++u) st[i & 1][u] = mfma_16x16x32(kf[i], qf[u][i >> 1], st[i & 1][u]);
         kf1[i] = load_kfrag(1, i);
@@ -682,7 +712,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
         }
       }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < kJTiles; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         if (!FP8 && (i & 1)) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
@@ -690,9 +720,9 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       __builtin_amdgcn_sched_barrier(0);
       // Region 3: the second half's MFMAs beside the first half's exponentials; the first
       // half's V fragments are requested on the way.
-      half8_t vf[8];
+      half8_t vf[kJTiles];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < kJTiles; ++i) {
 #pragma unroll
         for (int u = 0; u < kColTiles; ++u) st1[i & 1][u] = mfma_16x16x32(kf1[i], qf[u][i >> 1], st1[i & 1][u]);
         vf[i] = load_vfrag(i, 0);
@@ -701,7 +731,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       exponentials_seeded(st, pk, 1);
       const bool over_a = overflowed(pk);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < kJTiles; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
@@ -709,11 +739,11 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       if (over_a) return 1;
       // Block 2: second product of the first half beside the second half's exponentials; each
       // fragment register takes the second half's fragment as soon as its MFMAs are issued.
-      half8_t vf2[8];
+      half8_t vf2[kJTiles];
 #pragma unroll
       for (int u = 0; u < kColTiles; ++u) dsum[u] = mfma_16x16x32(ones, pk[u], dsum[u]);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < kJTiles; ++j) {
 #pragma unroll
         for (int u = 0; u < kColTiles; ++u) acc[j][u] = mfma_16x16x32(vf[j], pk[u], acc[j][u]);
         vf2[j] = load_vfrag(j, 1);
@@ -722,7 +752,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       exponentials_seeded(st1, pk1, 1);
       const bool over_b = overflowed(pk1);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < kJTiles; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
@@ -734,7 +764,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
 #pragma unroll
       for (int u = 0; u < kColTiles; ++u) dsum[u] = mfma_16x16x32(ones, pk1[u], dsum[u]);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < kJTiles; ++j) {
 #pragma unroll
         for (int u = 0; u < kColTiles; ++u) acc[j][u] = mfma_16x16x32(vf2[j], pk1[u], acc[j][u]);
       }
@@ -765,7 +795,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
     // The accumulators hold O^T: a lane has 4 consecutive d of one row, so stored directly every
     // store instruction would touch 16 rows with 32 bytes each. The rows go through LDS instead
     // (the K/V tiles are done with) and leave as whole 256-byte rows, 4 rows per instruction.
-    constexpr int kOutPitch = 2 * kHeadDim + 16;  // bytes; 68 dwords: a half-wave's 8-byte writes hit 64 banks
+    constexpr int kOutPitch = 2 * kHD + 16;  // bytes; at 128: 68 dwords, a half-wave's 8-byte writes hit 64 banks
     __syncthreads();                              // every wavefront is done reading the last tile
     const uint32_t mine = ((wave & 2) ? v_lds : k_lds) + (uint32_t)((wave & 1) * kColTiles * 16 * kOutPitch);
 #pragma unroll
@@ -773,25 +803,25 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       const float inv = v_scale / dsum[u][0];
       const uint32_t at = mine + (uint32_t)((u * 16 + n) * kOutPitch + 8 * g);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < kJTiles; ++j) {
         *(__attribute__((address_space(3))) half4_t *)(uintptr_t)(at + 32u * j) =
             half4_t{(half_t)(acc[j][u][0] * inv), (half_t)(acc[j][u][1] * inv),
                     (half_t)(acc[j][u][2] * inv), (half_t)(acc[j][u][3] * inv)};
       }
     }
-    // lane l carries chunk l % 16 of row l / 16 + 4 * step
-    const int chunk = lane & 15, r4 = lane >> 4;
+    // lane l carries chunk l % kChunks of row l / kChunks + kRowsPerLoad * step
+    const int chunk = slot, r4 = r_loc;
 #pragma unroll
     for (int u = 0; u < kColTiles; ++u) {
 #pragma unroll
-      for (int step = 0; step < 4; ++step) {
-        const int r = 4 * step + r4;
+      for (int step = 0; step < kLoadsPerWave; ++step) {
+        const int r = kRowsPerLoad * step + r4;
         const half8_t row = *(const lds_half8_t *)(uintptr_t)(mine + (uint32_t)((u * 16 + r) * kOutPitch + 16 * chunk));
         const int t = wave * kColTiles + u;
         const int head = t / row_tiles;
         const int qrow_idx = m0 + (t - head * row_tiles) * 16 + r;
         if (head < heads_here && qrow_idx < q_len) {
-          *(half8_t *)(out + (int64_t)(q_start + qrow_idx) * out_stride + (int64_t)out_head[u] * kHeadDim +
+          *(half8_t *)(out + (int64_t)(q_start + qrow_idx) * out_stride + (int64_t)out_head[u] * kHD +
                        8 * chunk) = row;
         }
       }
@@ -805,9 +835,9 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       if (out_row[u] >= 0) {
         const int64_t cell =
             ((int64_t)blockIdx.z * prefix.batch + out_row[u]) * prefix.num_q_heads + out_head[u];
-        float *po = prefix.part_o + cell * kHeadDim + 4 * g;
+        float *po = prefix.part_o + cell * kHD + 4 * g;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < kJTiles; ++j) {
           // read once, by the merge launch: streaming stores (see store_state in paged_decode.hip)
           __builtin_nontemporal_store(float4_t{acc[j][u][0] * inv, acc[j][u][1] * inv,
                                                acc[j][u][2] * inv, acc[j][u][3] * inv},
@@ -821,9 +851,9 @@ __global__ __launch_bounds__(kTiledWaves *kWave, 2) void varlen_prefill_tiled_ke
       continue;
     }
     if (out_row[u] >= 0) {
-      half_t *o = out + (int64_t)out_row[u] * out_stride + (int64_t)out_head[u] * kHeadDim + 4 * g;
+      half_t *o = out + (int64_t)out_row[u] * out_stride + (int64_t)out_head[u] * kHD + 4 * g;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < kJTiles; ++j) {
         *(half4_t *)(o + 16 * j) =
             half4_t{(half_t)(acc[j][u][0] * inv), (half_t)(acc[j][u][1] * inv),
                     (half_t)(acc[j][u][2] * inv), (half_t)(acc[j][u][3] * inv)};
@@ -836,7 +866,7 @@ static int validate_prefill(const char *what, const void *q, int64_t q_stride, c
                             int64_t out_stride, int32_t batch, int32_t hq, int32_t hkv,
                             int32_t head_dim, int32_t max_q_len) {
   LITEKV_REQUIRE(batch >= 0 && batch <= 65535, "%s: batch %d out of [0, 65535]", what, batch);
-  LITEKV_REQUIRE(head_dim == kHeadDim, "%s: head_dim %d unsupported (32, 64, 128 or 256)", what,
+  LITEKV_REQUIRE(head_dim == kHD, "%s: head_dim %d unsupported (32, 64, 128 or 256)", what,
                  head_dim);
   LITEKV_REQUIRE(hq > 0 && hkv > 0 && hq % hkv == 0 && hq <= 65535,
                  "%s: num_q_heads %d / num_kv_heads %d invalid", what, hq, hkv);
@@ -867,6 +897,8 @@ static PrefillShape prefill_shape(int group, int max_q_len) {
   return s;
 }
 
+}  // namespace LITEKV_HD_NS
+#if LITEKV_HD == 128
 int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_pool,
                          const float *fp8_scales, const int32_t *block_table, int32_t batch, int32_t num_q_heads,
                          int32_t num_kv_heads, int64_t num_pages, int32_t shared_pages,
@@ -912,10 +944,12 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
   *splits_out = splits;
   return check_launch(what);
 }
+#endif  // LITEKV_HD == 128
 
 }  // namespace litekv
 
 namespace litekv {
+inline namespace LITEKV_HD_NS {
 // Causal chunk attention over paged KV; `kv_scales` selects the fp8 pool.
 static int launch_paged_prefill(const char *what, const void *q, int64_t q_token_stride,
                                 const void *kv_pool, const float *kv_scales,
@@ -926,7 +960,14 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
                                 int64_t num_pages, int32_t max_q_len, float softmax_scale,
                                 void *stream, int format) {
   const bool fp8 = format != kKvF16;  // a pool of 8-bit codes
-  if (head_dim != kHeadDim && generic_head_dim(head_dim)) {  // see generic_attention.hip
+#if LITEKV_HD == 128
+  if (head_dim == 64 && !fp8) {  // the head dim 64 build of this file
+    return hd64_paged_prefill(what, q, q_token_stride, kv_pool, block_table, block_table_stride,
+                              cu_q_lens, context_lens, out, out_token_stride, batch, num_q_heads,
+                              num_kv_heads, page_size, num_pages, max_q_len, softmax_scale, stream);
+  }
+#endif
+  if (head_dim != kHD && generic_head_dim(head_dim)) {  // see generic_attention.hip
     LITEKV_REQUIRE(max_q_len >= 0, "%s: max_q_len %d < 0", what, max_q_len);
     LITEKV_REQUIRE(batch == 0 || max_q_len == 0 || (kv_pool && block_table && cu_q_lens),
                    "%s: null pointer", what);
@@ -984,6 +1025,7 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
                        (const int32_t *)nullptr, context_lens, group, s.head_splits, s.heads_per_wg,
                        s.row_tiles, softmax_scale * kLog2eP);
   };
+#if LITEKV_HD == 128
   if (format == kKvInt8) {
     launch(varlen_prefill_tiled_kernel<kPagedPrefillInt8>);
   } else if (format == kKvFp8) {
@@ -991,62 +1033,28 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
   } else {
     launch(varlen_prefill_tiled_kernel<kPagedPrefill>);
   }
+#else
+  LITEKV_REQUIRE(!fp8, "%s: 8-bit pools at head dim %d take the general kernel", what, kHD);
+  launch(varlen_prefill_tiled_kernel<kPagedPrefill>);
+#endif
   return check_launch(what);
 }
-}  // namespace litekv
 
-extern "C" int litekv_paged_prefill(const void *q, int64_t q_token_stride, const void *kv_pool,
-                                    const int32_t *block_table, int32_t block_table_stride,
-                                    const int32_t *cu_q_lens, const int32_t *context_lens,
-                                    void *out, int64_t out_token_stride, int32_t batch,
-                                    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
-                                    int32_t page_size, int64_t num_pages, int32_t max_q_len,
-                                    float softmax_scale, void *stream) {
-  return litekv::launch_paged_prefill("paged_prefill", q, q_token_stride, kv_pool, nullptr, block_table,
-                                      block_table_stride, cu_q_lens, context_lens, out,
-                                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
-                                      page_size, num_pages, max_q_len, softmax_scale, stream,
-                                      litekv::kKvF16);
-}
-
-extern "C" int litekv_paged_prefill_fp8(const void *q, int64_t q_token_stride, const void *kv_pool,
-                                        const float *kv_scales, const int32_t *block_table,
-                                        int32_t block_table_stride, const int32_t *cu_q_lens,
-                                        const int32_t *context_lens, void *out,
-                                        int64_t out_token_stride, int32_t batch,
-                                        int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
-                                        int32_t page_size, int64_t num_pages, int32_t max_q_len,
-                                        float softmax_scale, void *stream) {
-  return litekv::launch_paged_prefill("paged_prefill_fp8", q, q_token_stride, kv_pool, kv_scales,
-                                      block_table, block_table_stride, cu_q_lens, context_lens, out,
-                                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
-                                      page_size, num_pages, max_q_len, softmax_scale, stream,
-                                      litekv::kKvFp8);
-}
-
-extern "C" int litekv_paged_prefill_int8(const void *q, int64_t q_token_stride, const void *kv_pool,
-                                         const float *kv_scales, const int32_t *block_table,
-                                         int32_t block_table_stride, const int32_t *cu_q_lens,
-                                         const int32_t *context_lens, void *out,
-                                         int64_t out_token_stride, int32_t batch,
-                                         int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
-                                         int32_t page_size, int64_t num_pages, int32_t max_q_len,
-                                         float softmax_scale, void *stream) {
-  return litekv::launch_paged_prefill("paged_prefill_int8", q, q_token_stride, kv_pool, kv_scales,
-                                      block_table, block_table_stride, cu_q_lens, context_lens, out,
-                                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
-                                      page_size, num_pages, max_q_len, softmax_scale, stream,
-                                      litekv::kKvInt8);
-}
-
-extern "C" int litekv_varlen_prefill(const void *q, int64_t q_token_stride, const void *k,
-                                     int64_t k_token_stride, const void *v, int64_t v_token_stride,
-                                     const int32_t *seq_starts, const int32_t *seq_lens, void *out,
-                                     int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
-                                     int32_t num_kv_heads, int32_t head_dim, int32_t max_seq_len,
-                                     int64_t num_tokens, float softmax_scale, void *stream) {
-  using namespace litekv;
-  if (head_dim != kHeadDim && generic_head_dim(head_dim)) {  // see generic_attention.hip
+// Causal attention over packed, contiguous K/V.
+static int launch_varlen_prefill(const void *q, int64_t q_token_stride, const void *k,
+                                 int64_t k_token_stride, const void *v, int64_t v_token_stride,
+                                 const int32_t *seq_starts, const int32_t *seq_lens, void *out,
+                                 int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
+                                 int32_t num_kv_heads, int32_t head_dim, int32_t max_seq_len,
+                                 int64_t num_tokens, float softmax_scale, void *stream) {
+#if LITEKV_HD == 128
+  if (head_dim == 64) {  // the head dim 64 build of this file
+    return hd64_varlen_prefill(q, q_token_stride, k, k_token_stride, v, v_token_stride, seq_starts,
+                               seq_lens, out, out_token_stride, batch, num_q_heads, num_kv_heads,
+                               max_seq_len, num_tokens, softmax_scale, stream);
+  }
+#endif
+  if (head_dim != kHD && generic_head_dim(head_dim)) {  // see generic_attention.hip
     LITEKV_REQUIRE(max_seq_len >= 0, "varlen_prefill: max_seq_len %d < 0", max_seq_len);
     GenericLaunch g;
     g.q = q;
@@ -1100,3 +1108,87 @@ extern "C" int litekv_varlen_prefill(const void *q, int64_t q_token_stride, cons
                      softmax_scale * kLog2eP);
   return check_launch("varlen_prefill");
 }
+}  // namespace LITEKV_HD_NS
+
+#if LITEKV_HD == 64
+int hd64_paged_prefill(const char *what, const void *q, int64_t q_token_stride, const void *kv_pool,
+                       const int32_t *block_table, int32_t block_table_stride,
+                       const int32_t *cu_q_lens, const int32_t *context_lens, void *out,
+                       int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
+                       int32_t num_kv_heads, int32_t page_size, int64_t num_pages,
+                       int32_t max_q_len, float softmax_scale, void *stream) {
+  return launch_paged_prefill(what, q, q_token_stride, kv_pool, nullptr, block_table,
+                              block_table_stride, cu_q_lens, context_lens, out, out_token_stride,
+                              batch, num_q_heads, num_kv_heads, 64, page_size, num_pages, max_q_len,
+                              softmax_scale, stream, kKvF16);
+}
+int hd64_varlen_prefill(const void *q, int64_t q_token_stride, const void *k, int64_t k_token_stride,
+                        const void *v, int64_t v_token_stride, const int32_t *seq_starts,
+                        const int32_t *seq_lens, void *out, int64_t out_token_stride, int32_t batch,
+                        int32_t num_q_heads, int32_t num_kv_heads, int32_t max_seq_len,
+                        int64_t num_tokens, float softmax_scale, void *stream) {
+  return launch_varlen_prefill(q, q_token_stride, k, k_token_stride, v, v_token_stride, seq_starts,
+                               seq_lens, out, out_token_stride, batch, num_q_heads, num_kv_heads, 64,
+                               max_seq_len, num_tokens, softmax_scale, stream);
+}
+#endif  // LITEKV_HD == 64
+}  // namespace litekv
+
+#if LITEKV_HD == 128  // the C ABI lives in the head dim 128 build of this file
+
+extern "C" int litekv_paged_prefill(const void *q, int64_t q_token_stride, const void *kv_pool,
+                                    const int32_t *block_table, int32_t block_table_stride,
+                                    const int32_t *cu_q_lens, const int32_t *context_lens,
+                                    void *out, int64_t out_token_stride, int32_t batch,
+                                    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                    int32_t page_size, int64_t num_pages, int32_t max_q_len,
+                                    float softmax_scale, void *stream) {
+  return litekv::launch_paged_prefill("paged_prefill", q, q_token_stride, kv_pool, nullptr, block_table,
+                                      block_table_stride, cu_q_lens, context_lens, out,
+                                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
+                                      page_size, num_pages, max_q_len, softmax_scale, stream,
+                                      litekv::kKvF16);
+}
+
+extern "C" int litekv_paged_prefill_fp8(const void *q, int64_t q_token_stride, const void *kv_pool,
+                                        const float *kv_scales, const int32_t *block_table,
+                                        int32_t block_table_stride, const int32_t *cu_q_lens,
+                                        const int32_t *context_lens, void *out,
+                                        int64_t out_token_stride, int32_t batch,
+                                        int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                        int32_t page_size, int64_t num_pages, int32_t max_q_len,
+                                        float softmax_scale, void *stream) {
+  return litekv::launch_paged_prefill("paged_prefill_fp8", q, q_token_stride, kv_pool, kv_scales,
+                                      block_table, block_table_stride, cu_q_lens, context_lens, out,
+                                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
+                                      page_size, num_pages, max_q_len, softmax_scale, stream,
+                                      litekv::kKvFp8);
+}
+
+extern "C" int litekv_paged_prefill_int8(const void *q, int64_t q_token_stride, const void *kv_pool,
+                                         const float *kv_scales, const int32_t *block_table,
+                                         int32_t block_table_stride, const int32_t *cu_q_lens,
+                                         const int32_t *context_lens, void *out,
+                                         int64_t out_token_stride, int32_t batch,
+                                         int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                         int32_t page_size, int64_t num_pages, int32_t max_q_len,
+                                         float softmax_scale, void *stream) {
+  return litekv::launch_paged_prefill("paged_prefill_int8", q, q_token_stride, kv_pool, kv_scales,
+                                      block_table, block_table_stride, cu_q_lens, context_lens, out,
+                                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
+                                      page_size, num_pages, max_q_len, softmax_scale, stream,
+                                      litekv::kKvInt8);
+}
+
+extern "C" int litekv_varlen_prefill(const void *q, int64_t q_token_stride, const void *k,
+                                     int64_t k_token_stride, const void *v, int64_t v_token_stride,
+                                     const int32_t *seq_starts, const int32_t *seq_lens, void *out,
+                                     int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
+                                     int32_t num_kv_heads, int32_t head_dim, int32_t max_seq_len,
+                                     int64_t num_tokens, float softmax_scale, void *stream) {
+  return litekv::launch_varlen_prefill(q, q_token_stride, k, k_token_stride, v, v_token_stride,
+                                       seq_starts, seq_lens, out, out_token_stride, batch,
+                                       num_q_heads, num_kv_heads, head_dim, max_seq_len, num_tokens,
+                                       softmax_scale, stream);
+}
+#endif  // LITEKV_HD == 128

@@ -202,3 +202,30 @@ def test_prefill_head_dims(head_dim, hq, hkv, lens, ctx, page_size):
                                   case.softmax_scale)
         torch.cuda.synchronize()
         assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize("hq,hkv,lens,ctx,page_size", [
+    (32, 8, [700, 333, 1500], None, 16),            # Llama-3.2-1B's heads; many key tiles, ragged ends
+    (64, 4, [257, 1023], None, 16),                 # 16 query heads per kv head: two workgroups per group
+    (24, 8, [129, 64, 900], [513, 1, 250], 32),     # 3 heads per kv head; chunks over long histories
+    (8, 8, [1100], [2000], 64),                     # no grouping
+])
+def test_prefill_head_dim_64_on_the_tiled_kernel(hq, hkv, lens, ctx, page_size):
+    """Head dim 64 with fp16 K/V runs on the MFMA-tiled kernel (rows of 128 bytes, their own LDS
+    swizzle): sequences long enough for the pipelined loop, the masked diagonal and rescales, and
+    repeated launches agree bit for bit."""
+    print(f"prefill head_dim 64 tiled {hq}/{hkv} {lens} ctx {ctx} page_size {page_size}", flush=True)
+    case = workloads.make_prefill_case("p64", 4200 + hq, lens, hq, hkv, context_lens=ctx, device=DEV,
+                                       page_size=page_size, head_dim=64)
+    _append(case)
+    outs = [ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens,
+                              case.context_lens if ctx is not None else None, case.max_q_len,
+                              case.softmax_scale, page_size=page_size) for _ in range(3)]
+    torch.cuda.synchronize()
+    assert_attention_close(outs[0], _oracle_paged(case), "paged prefill head_dim 64")
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    if ctx is None:
+        out2 = ops.varlen_prefill(case.q, case.k, case.v, case.cu_q_lens[:-1], case.seq_lens, case.max_q_len,
+                                  case.softmax_scale)
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0], out2)
