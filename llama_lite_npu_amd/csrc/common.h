@@ -108,9 +108,10 @@ struct DecodeArgs {
   int64_t k_new_stride = 0, v_new_stride = 0;
 };
 
-// The launchers of the head dim 64 build of paged_prefill.hip (paged_prefill_hd64.hip; fp16 K/V).
+// The launchers of the head dim 64 build of paged_prefill.hip (paged_prefill_hd64.hip).
 int hd64_paged_prefill(const char *what, const void *q, int64_t q_token_stride, const void *kv_pool,
-                       const int32_t *block_table, int32_t block_table_stride,
+                       const float *kv_scales, int format, const int32_t *block_table,
+                       int32_t block_table_stride,
                        const int32_t *cu_q_lens, const int32_t *context_lens, void *out,
                        int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
                        int32_t num_kv_heads, int32_t page_size, int64_t num_pages,

@@ -60,7 +60,7 @@
 #include "kv_fp8.h"
 
 // This file is compiled twice: as it stands for head dim 128, and through paged_prefill_hd64.hip
-// (which defines LITEKV_HD and includes it) for head dim 64 with fp16 K/V (paged or packed).
+// (which defines LITEKV_HD and includes it) for head dim 64 (paged in every pool format, or packed).
 // Everything sits in an inline namespace named after the head dim, so the two builds link side by
 // side; the C ABI and the shared-prefix launcher are in the 128 build, which hands 64-wide calls
 // to hd64_paged_prefill / hd64_varlen_prefill.
@@ -251,11 +251,12 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
   // Starts the loads of tile kt into its LDS half. The instruction is written as asm so that the
   // compiler does not make later LDS reads of the *other* half wait for it; the wait is the
   // explicit vmcnt(0) before the barrier that publishes the tile.
-  uint4_t raw_k[2], raw_v[2];  // fp8: this lane's 32 codes of K and of V of the tile requested last
+  constexpr int kRawVecs = kHD / 64;    // 8-bit pools: 16-byte vectors of codes per lane and operand
+  uint4_t raw_k[kRawVecs], raw_v[kRawVecs];  // this lane's codes of K and of V of the tile requested last
   auto issue_tile = [&](int kt) {
     const int row0 = (tile0 + kt) * kKvTile + 16 * wave;  // first key of this wavefront's 16 rows
     if constexpr (FP8) {
-      // lane l: row l / 4 of the wavefront's page, codes 32 * (l % 4) .. +31 of the head's row
+      // lane l: row l / 4 of the wavefront's page, a quarter of the head's row (kHD / 4 codes)
       int pidx = (tile0 + kt) * 4 + wave;
       pidx = pidx < last_page ? pidx : last_page;
       const int pid = page_of(pidx);
@@ -263,13 +264,14 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
       tok = tok < last_key ? tok : last_key;  // rows past the last key re-read it
       const int src_row = tok - pidx * kPageSize;
       const uint8_t *base = (const uint8_t *)paged.kv +
-                            ((int64_t)pid * kPageSize + src_row) * (int64_t)k_pitch + 32 * (lane & 3);
+                            ((int64_t)pid * kPageSize + src_row) * (int64_t)k_pitch + (kHD / 4) * (lane & 3);
       const uint8_t *kp = base + h * kHD;
       const uint8_t *vp = base + (paged.num_kv_heads + h) * kHD;
-      raw_k[0] = *(const uint4_t *)kp;
-      raw_k[1] = *(const uint4_t *)(kp + 16);
-      raw_v[0] = *(const uint4_t *)vp;
-      raw_v[1] = *(const uint4_t *)(vp + 16);
+#pragma unroll
+      for (int i = 0; i < kRawVecs; ++i) {
+        raw_k[i] = *(const uint4_t *)(kp + 16 * i);
+        raw_v[i] = *(const uint4_t *)(vp + 16 * i);
+      }
       return;
     }
     const char *kbase, *vbase;
@@ -384,9 +386,9 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
     }
   }
   if constexpr (!SHARED) {
-    // the loads of tile 0 (K and V; four of an 8-bit pool) were requested after q's
+    // the loads of tile 0 (K and V) were requested after q's
     if constexpr (FP8) {
-      __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kRawVecs));
     } else {
       __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kLoadsPerWave));
     }
@@ -577,13 +579,13 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
       const int r = lane >> 2;
       const uint32_t row_at = (uint32_t)((kt & 1) * kTileHalfs + (16 * wave + r) * kHD) * 2u;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int chunk = 4 * (lane & 3) + j;
+      for (int j = 0; j < kHD / 32; ++j) {
+        const int chunk = (kHD / 32) * (lane & 3) + j;
         const uint4_t ck = raw_k[j >> 1], cv = raw_v[j >> 1];
         const half8_t kh = codes_to_half<KV>((j & 1) ? uint2_t{ck[2], ck[3]} : uint2_t{ck[0], ck[1]});
         const half8_t vh = codes_to_half<KV>((j & 1) ? uint2_t{cv[2], cv[3]} : uint2_t{cv[0], cv[1]});
-        *(lds_half8_t *)(uintptr_t)(k_lds + row_at + 16u * (uint32_t)(chunk ^ r)) = kh;
-        *(lds_half8_t *)(uintptr_t)(v_lds + row_at + 16u * (uint32_t)(chunk ^ (2 * (r & 7)))) = vh;
+        *(lds_half8_t *)(uintptr_t)(k_lds + row_at + 16u * (uint32_t)(chunk ^ k_swz(r))) = kh;
+        *(lds_half8_t *)(uintptr_t)(v_lds + row_at + 16u * (uint32_t)(chunk ^ v_swz(r))) = vh;
       }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wavefront's part of tile kt is in LDS
@@ -961,8 +963,8 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
                                 void *stream, int format) {
   const bool fp8 = format != kKvF16;  // a pool of 8-bit codes
 #if LITEKV_HD == 128
-  if (head_dim == 64 && !fp8) {  // the head dim 64 build of this file
-    return hd64_paged_prefill(what, q, q_token_stride, kv_pool, block_table, block_table_stride,
+  if (head_dim == 64) {  // the head dim 64 build of this file
+    return hd64_paged_prefill(what, q, q_token_stride, kv_pool, kv_scales, format, block_table, block_table_stride,
                               cu_q_lens, context_lens, out, out_token_stride, batch, num_q_heads,
                               num_kv_heads, page_size, num_pages, max_q_len, softmax_scale, stream);
   }
@@ -1025,7 +1027,6 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
                        (const int32_t *)nullptr, context_lens, group, s.head_splits, s.heads_per_wg,
                        s.row_tiles, softmax_scale * kLog2eP);
   };
-#if LITEKV_HD == 128
   if (format == kKvInt8) {
     launch(varlen_prefill_tiled_kernel<kPagedPrefillInt8>);
   } else if (format == kKvFp8) {
@@ -1033,10 +1034,6 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
   } else {
     launch(varlen_prefill_tiled_kernel<kPagedPrefill>);
   }
-#else
-  LITEKV_REQUIRE(!fp8, "%s: 8-bit pools at head dim %d take the general kernel", what, kHD);
-  launch(varlen_prefill_tiled_kernel<kPagedPrefill>);
-#endif
   return check_launch(what);
 }
 
@@ -1112,15 +1109,16 @@ static int launch_varlen_prefill(const void *q, int64_t q_token_stride, const vo
 
 #if LITEKV_HD == 64
 int hd64_paged_prefill(const char *what, const void *q, int64_t q_token_stride, const void *kv_pool,
-                       const int32_t *block_table, int32_t block_table_stride,
+                       const float *kv_scales, int format, const int32_t *block_table,
+                       int32_t block_table_stride,
                        const int32_t *cu_q_lens, const int32_t *context_lens, void *out,
                        int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
                        int32_t num_kv_heads, int32_t page_size, int64_t num_pages,
                        int32_t max_q_len, float softmax_scale, void *stream) {
-  return launch_paged_prefill(what, q, q_token_stride, kv_pool, nullptr, block_table,
+  return launch_paged_prefill(what, q, q_token_stride, kv_pool, kv_scales, block_table,
                               block_table_stride, cu_q_lens, context_lens, out, out_token_stride,
                               batch, num_q_heads, num_kv_heads, 64, page_size, num_pages, max_q_len,
-                              softmax_scale, stream, kKvF16);
+                              softmax_scale, stream, format);
 }
 int hd64_varlen_prefill(const void *q, int64_t q_token_stride, const void *k, int64_t k_token_stride,
                         const void *v, int64_t v_token_stride, const int32_t *seq_starts,

@@ -1,4 +1,4 @@
-// The head dim 64 build of paged_prefill.hip (fp16 K/V, paged or packed): see the note at the top
+// The head dim 64 build of paged_prefill.hip (paged in every pool format, or packed): see the note at the top
 // of that file.
 #define LITEKV_HD 64
 #include "paged_prefill.hip"

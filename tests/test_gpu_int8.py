@@ -379,3 +379,30 @@ def test_quantised_pools_at_head_dim_64(dtype):
     ref = cpu_ref.paged_prefill_ref(pre.q.cpu(), values, pre.block_table.cpu(), pre.cu_q_lens.cpu(),
                                     pre.context_lens.cpu(), scale).numpy()
     assert_attention_close(out, ref, f"head_dim 64 {dtype} chunk prefill")
+
+
+@pytest.mark.parametrize("dtype", [torch.int8, torch.uint8])
+@pytest.mark.parametrize("page_size", [16, 32])
+def test_quantised_chunk_prefill_at_head_dim_64_many_tiles(dtype, page_size):
+    """Chunks over long 8-bit histories at head dim 64 (the MFMA-tiled kernel's staging of 64-wide
+    code rows): many key tiles, ragged ends, 3 and 8 query heads per KV head."""
+    from oracle import fp8
+    codec = int8 if dtype == torch.int8 else fp8
+    d = 64
+    scale = 1.0 / math.sqrt(d)
+    for hq, hkv, lens, ctx in ((24, 8, [300, 65, 129], [700, 1, 450]), (32, 4, [513], [1000])):
+        print(f"head_dim 64 {dtype} page_size {page_size} {hq}/{hkv} {lens} ctx {ctx}", flush=True)
+        pre = workloads.make_prefill_case("q64t", 91 + hq, lens, hq, hkv, context_lens=ctx, device=DEV, head_dim=d,
+                                          page_size=page_size)
+        scales = _head_scales(hkv) if dtype == torch.int8 else _head_scales(hkv, 0.02, 0.015)
+        pool = torch.zeros(pre.kv_pool.shape, dtype=dtype, device=DEV)
+        every_slot = torch.arange(pool.shape[0], dtype=torch.int32, device=DEV)
+        ops.kv_append_quantised(pre.kv_pool[:, :hkv], pre.kv_pool[:, hkv:], every_slot, pool, scales)
+        ops.kv_append_quantised(pre.k, pre.v, pre.slot_mapping, pool, scales)
+        out = ops.paged_prefill(pre.q, pool, pre.block_table, pre.cu_q_lens, pre.context_lens, pre.max_q_len, scale,
+                                kv_scales=scales, page_size=page_size)
+        torch.cuda.synchronize()
+        values = torch.from_numpy(codec.dequantize_pool(pool.cpu().numpy(), scales.cpu().numpy()))
+        ref = cpu_ref.paged_prefill_ref(pre.q.cpu(), values, pre.block_table.cpu(), pre.cu_q_lens.cpu(),
+                                        pre.context_lens.cpu(), scale, page_size=page_size).numpy()
+        assert_attention_close(out, ref, f"head_dim 64 {dtype} chunk prefill over {ctx}")
