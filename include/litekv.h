@@ -25,11 +25,12 @@
  * Supported shapes: Hq % Hkv == 0, Hq / Hkv <= 16; page_size 16, 32 or 64
  * (the reference's --page_size, lite_llama/server.py:1038-1161): the attention
  * kernels walk a page of 32 or 64 tokens as two or four consecutive 16-token
- * pieces; head_dim 128 and 64 on the MFMA-tiled kernels, and 32, 64 or 256 (the reference kernels take the head dim as a block
- * size, lite_llama/kernels/flashdecoding.py:305, 393-396) through the same
- * entry points on one general kernel with fp32 arithmetic where no tiled kernel
- * exists: it writes the final rows in a single launch whatever schedule was
- * asked for, and uses no workspace.
+ * pieces; head_dim 128 and 64 on the MFMA-tiled kernels, and 32, 64 or 256
+ * (the reference kernels take the head dim as a block size,
+ * lite_llama/kernels/flashdecoding.py:305, 393-396) through the same entry
+ * points on one general kernel with fp32 arithmetic where no tiled kernel
+ * exists (32 and 256; a shared prefix at 64): it writes the final rows in a
+ * single launch whatever schedule was asked for, and uses no workspace.
  */
 #ifndef LITEKV_H
 #define LITEKV_H
