@@ -34,82 +34,94 @@ __global__ __launch_bounds__(256) void qk_norm_rope_append_kernel(
     const half_t *__restrict__ v, int64_t v_stride, const half_t *__restrict__ q_weight,
     const half_t *__restrict__ k_weight, const half_t *__restrict__ cos_rows,
     const half_t *__restrict__ sin_rows, int64_t cs_stride, const int32_t *__restrict__ slot_mapping,
-    void *__restrict__ pool_any, const float *__restrict__ scales, int64_t total_rows,
+    void *__restrict__ pool_any, const float *__restrict__ scales, int64_t num_tokens,
     int32_t num_q_heads, int32_t num_kv_heads, int64_t num_slots, float eps) {
+  // grid: x = group of four tokens, y = block of 256 / L consecutive head rows of a token (q heads,
+  // k heads, v heads): no division on the way to an address, a workgroup's rows are one
+  // contiguous run per token, and a lane has the loads of four tokens in flight.
   constexpr int kDim = 8 * L;       // the head dim
+  constexpr int kTok = 4;
   const int l16 = threadIdx.x & (L - 1);  // lane inside the row
-  const int64_t row = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / L;
-  if (row >= total_rows) return;  // whole 16-lane groups leave together
-  const int rows_per_token = num_q_heads + 2 * num_kv_heads;
-  const int64_t token = row / rows_per_token;
-  const int r = (int)(row - token * rows_per_token);
-  const int64_t slot = slot_mapping[token];
-  const bool slot_ok = slot >= 0 && slot < num_slots;
-  // stores 8 elements of head `kv_head` (K heads first, then V heads) of the token's slot
-  auto store_row = [&](int kv_head, half8_t x) {
-    const int64_t at = (slot * (int64_t)(2 * num_kv_heads) + kv_head) * kDim + 8 * l16;
+  const int r = (int)blockIdx.y * (256 / L) + (int)(threadIdx.x / L);
+  if (r >= num_q_heads + 2 * num_kv_heads) return;  // whole L-lane groups leave together
+  const bool is_v = r >= num_q_heads + num_kv_heads;
+  const bool is_q = r < num_q_heads;
+  const int head = is_q ? r : (is_v ? r - num_q_heads - num_kv_heads : r - num_q_heads);
+  int64_t token[kTok], slot[kTok];
+  bool live[kTok];
+  half8_t x[kTok], c[kTok], sn[kTok];
+#pragma unroll
+  for (int t = 0; t < kTok; ++t) {
+    token[t] = (int64_t)blockIdx.x * kTok + t;
+    live[t] = token[t] < num_tokens;
+    if (!live[t]) token[t] = num_tokens - 1;  // loads repeat the last token; nothing is stored
+    const half_t *src = is_q   ? q + token[t] * q_stride + (int64_t)head * kDim
+                        : is_v ? v + token[t] * v_stride + (int64_t)head * kDim
+                               : k + token[t] * k_stride + (int64_t)head * kDim;
+    x[t] = *(const half8_t *)(src + 8 * l16);
+    slot[t] = slot_mapping[token[t]];
+    if (cos_rows != nullptr && !is_v) {
+      const int j = 8 * (l16 & (L / 2 - 1));  // index into the first dim / 2 entries of the cos / sin row
+      c[t] = *(const half8_t *)(cos_rows + token[t] * cs_stride + j);
+      sn[t] = *(const half8_t *)(sin_rows + token[t] * cs_stride + j);
+    }
+  }
+  // stores 8 elements of head `kv_head` (K heads first, then V heads) of a slot
+  auto store_row = [&](int64_t slot_t, int kv_head, half8_t y) {
+    const int64_t at = (slot_t * (int64_t)(2 * num_kv_heads) + kv_head) * kDim + 8 * l16;
     if constexpr (KV != kKvF16) {
       *(uint2_t *)(static_cast<uint8_t *>(pool_any) + at) =
-          half_to_codes<KV>(x, 1.0f / scales[kv_head]);
+          half_to_codes<KV>(y, 1.0f / scales[kv_head]);
     } else {
-      *(half8_t *)(static_cast<half_t *>(pool_any) + at) = x;
+      *(half8_t *)(static_cast<half_t *>(pool_any) + at) = y;
     }
   };
-
-  if (r >= num_q_heads + num_kv_heads) {  // a v row: plain copy into the slot
-    const int head = r - num_q_heads - num_kv_heads;
-    if (slot_ok) {
-      store_row(num_kv_heads + head,
-                *(const half8_t *)(v + token * v_stride + (int64_t)head * kDim + 8 * l16));
-    }
-    return;
-  }
-  const bool is_q = r < num_q_heads;
-  const int head = is_q ? r : r - num_q_heads;
-  const half_t *src = is_q ? q + token * q_stride + (int64_t)head * kDim
-                           : k + token * k_stride + (int64_t)head * kDim;
   const half_t *weight = is_q ? q_weight : k_weight;
-  half8_t x = *(const half8_t *)(src + 8 * l16);
+  half8_t w = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+  if (weight != nullptr && !is_v) w = *(const half8_t *)(weight + 8 * l16);
 
-  if (weight != nullptr) {
-    float xf[8], ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      xf[i] = (float)x[i];
-      ss += xf[i] * xf[i];
+  for (int t = 0; t < kTok; ++t) {
+    const bool slot_ok = live[t] && slot[t] >= 0 && slot[t] < num_slots;
+    if (is_v) {  // a v row: plain copy into the slot
+      if (slot_ok) store_row(slot[t], num_kv_heads + head, x[t]);
+      continue;
     }
-    ss = row_sum<L>(ss);
-    const float rrms = 1.0f / sqrtf(ss * (1.0f / kDim) + eps);
-    const half8_t w = *(const half8_t *)(weight + 8 * l16);
+    half8_t y = x[t];
+    if (weight != nullptr) {
+      float xf[8], ss = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const half_t y = (half_t)(xf[i] * rrms);
-      x[i] = (half_t)((float)y * (float)w[i]);
+      for (int i = 0; i < 8; ++i) {
+        xf[i] = (float)y[i];
+        ss += xf[i] * xf[i];
+      }
+      ss = row_sum<L>(ss);
+      const float rrms = 1.0f / sqrtf(ss * (1.0f / kDim) + eps);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const half_t z = (half_t)(xf[i] * rrms);
+        y[i] = (half_t)((float)z * (float)w[i]);
+      }
     }
-  }
-
-  if (cos_rows != nullptr) {
-    // partner: element i + dim / 2 for the first half of the row, i - dim / 2 for the second
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    u32x4 bits = __builtin_bit_cast(u32x4, x);
-    u32x4 other;
+    if (cos_rows != nullptr) {
+      // partner: element i + dim / 2 for the first half of the row, i - dim / 2 for the second
+      typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+      u32x4 bits = __builtin_bit_cast(u32x4, y);
+      u32x4 other;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) other[i] = __shfl_xor(bits[i], L / 2, L);
-    const half8_t p = __builtin_bit_cast(half8_t, other);
-    const int j = 8 * (l16 & (L / 2 - 1));  // index into the first dim / 2 entries of the cos / sin row
-    const half8_t c = *(const half8_t *)(cos_rows + token * cs_stride + j);
-    const half8_t s = *(const half8_t *)(sin_rows + token * cs_stride + j);
-    const float sign = l16 < L / 2 ? -1.0f : 1.0f;
+      for (int i = 0; i < 4; ++i) other[i] = __shfl_xor(bits[i], L / 2, L);
+      const half8_t p = __builtin_bit_cast(half8_t, other);
+      const float sign = l16 < L / 2 ? -1.0f : 1.0f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      x[i] = (half_t)((float)x[i] * (float)c[i] + sign * ((float)p[i] * (float)s[i]));
+      for (int i = 0; i < 8; ++i) {
+        y[i] = (half_t)((float)y[i] * (float)c[t][i] + sign * ((float)p[i] * (float)sn[t][i]));
+      }
     }
-  }
-
-  if (is_q) {
-    *(half8_t *)(q + token * q_stride + (int64_t)head * kDim + 8 * l16) = x;
-  } else if (slot_ok) {
-    store_row(head, x);
+    if (is_q) {
+      if (live[t]) *(half8_t *)(q + token[t] * q_stride + (int64_t)head * kDim + 8 * l16) = y;
+    } else if (slot_ok) {
+      store_row(slot[t], head, y);
+    }
   }
 }
 
@@ -154,17 +166,18 @@ static int launch_qk_epilogue(const char *what, void *q, int64_t q_token_stride,
   }
   LITEKV_REQUIRE(num_slots > 0, "%s: num_slots %lld <= 0", what, (long long)num_slots);
   LITEKV_REQUIRE(rms_eps >= 0.f, "%s: rms_eps %g < 0", what, (double)rms_eps);
-  const int64_t total_rows = (int64_t)num_tokens * (num_q_heads + 2 * num_kv_heads);
-  const int64_t blocks = (total_rows * (head_dim / 8) + 255) / 256;
-  LITEKV_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many tokens", what);
+  const int rows_per_block = 256 / (head_dim / 8);
+  const int row_blocks = (num_q_heads + 2 * num_kv_heads + rows_per_block - 1) / rows_per_block;
+  LITEKV_REQUIRE(row_blocks <= 65535, "%s: too many heads", what);
   auto launch = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+    hipLaunchKernelGGL(kernel, dim3((unsigned)((num_tokens + 3) / 4), (unsigned)row_blocks), dim3(256), 0,
+                       static_cast<hipStream_t>(stream),
                        static_cast<half_t *>(q), q_token_stride, static_cast<const half_t *>(k),
                        k_token_stride, static_cast<const half_t *>(v), v_token_stride,
                        static_cast<const half_t *>(q_norm_weight),
                        static_cast<const half_t *>(k_norm_weight),
                        static_cast<const half_t *>(cos_rows), static_cast<const half_t *>(sin_rows),
-                       cos_sin_token_stride, slot_mapping, kv_pool, fp8_scales, total_rows,
+                       cos_sin_token_stride, slot_mapping, kv_pool, fp8_scales, (int64_t)num_tokens,
                        num_q_heads, num_kv_heads, num_slots, rms_eps);
   };
   auto by_format = [&](auto lanes) {
