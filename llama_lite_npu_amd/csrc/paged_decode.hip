@@ -425,7 +425,7 @@ __device__ __forceinline__ void load_new_rows(uint4_t (&kr)[4], uint4_t (&vr)[2]
 // Schedule "splits": one wavefront per (kv head, split, sequence).
 // Partials: part_o[b][hq][split][D], part_lse[b][hq][split].
 // The wavefronts are independent (no barrier). A workgroup holds 1, 2 or 4 of them (blockDim.x /
-// 64; neighbouring kv heads of one sequence), chosen by the host: few wavefronts want
+// 64; neighbouring kv heads of one sequence and split), chosen by the host: few wavefronts want
 // one per workgroup so that they spread over all compute units, many short ones want four,
 // because the dispatcher places workgroups at a fixed rate whatever their size (512 sequences of
 // 32 tokens, 8 kv heads: 30.5 us as 4096 workgroups). Not eight: at three wavefronts per SIMD a
@@ -1419,11 +1419,12 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   float *part_o = max_splits > 1 ? static_cast<float *>(a.workspace) : nullptr;
   float *part_lse =
       max_splits > 1 ? part_o + (size_t)a.batch * a.num_q_heads * max_splits * a.head_dim : nullptr;
-  // Wavefronts per workgroup: one where sequences are split (long chains: a workgroup would
-  // hold its slots until its longest wavefront is done), else as many heads of a sequence as
-  // leave at least two workgroups per compute unit.
-  const int64_t units = (int64_t)a.batch * a.num_kv_heads;
-  int waves = max_splits == 1 ? kSplitWaves : 1;
+  // Wavefronts per workgroup: as many kv heads of one (sequence, split) -- they have the same
+  // pages and the same trip count, and a token's K and V rows are contiguous over the heads -- as
+  // leave at least two workgroups per compute unit (C5, 16 splits: 1011 us per layer with one
+  // wavefront per workgroup, 930 with its four kv heads together).
+  const int64_t units = (int64_t)a.batch * a.num_kv_heads * max_splits;
+  int waves = kSplitWaves;
   while (waves > 1 && (units / waves < 512 || a.num_kv_heads % waves != 0)) waves >>= 1;
   const dim3 grid((unsigned)(a.num_kv_heads / waves), (unsigned)max_splits, (unsigned)a.batch);
   const dim3 block((unsigned)(waves * kWave));
