@@ -597,10 +597,20 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
   // tile_bases() reads the page id (scalar), issue_rows(i) requests row group i of K and of V.
   const char *next_kbase = nullptr, *next_vbase = nullptr;
   uint32_t next_dst = 0;
+  // The page ids of a tile's four pages, one per lane (lane l: page l % 4 of the tile), requested a
+  // whole tile before tile_bases() needs them: as a scalar value read on the spot the id cost
+  // every tile a round trip to memory in front of its first MFMA.
+  auto page_ids_of_tile = [&](int kt) -> int {
+    if constexpr (!PAGED) return 0;
+    int pidx = (tile0 + kt) * 4 + (lane & 3);
+    pidx = pidx < last_page ? pidx : last_page;
+    return page_of(pidx);
+  };
+  int ids_ahead = 0;  // of the tile after the one being staged
   auto tile_bases = [&](int kt) {
     const int row0 = (tile0 + kt) * kKvTile + 16 * wave;
     if (PAGED) {
-      const int pid = page_of((tile0 + kt) * 4 + wave);
+      const int pid = __builtin_amdgcn_readlane(ids_ahead, wave);
       next_kbase = (const char *)paged.kv + (int64_t)pid * ((int64_t)kPageSize * k_pitch);
       next_vbase = next_kbase;
     } else {
@@ -681,10 +691,16 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
   // beside the vector ALU work of the other. Returns like fast_tiles (a grown tile is redone
   // from its first half).
   auto fast_plain_tiles = [&](int kt_end) -> int {
+    if constexpr (!FP8) {
+      if (kt < kt_end) ids_ahead = page_ids_of_tile(kt + 1);
+    }
     for (; kt < kt_end; ++kt) {
       sync_and_prefetch(kt, FP8);
       flip_halves();
-      if constexpr (!FP8) tile_bases(kt + 1);
+      if constexpr (!FP8) {
+        tile_bases(kt + 1);
+        ids_ahead = page_ids_of_tile(kt + 2);
+      }
       // Block 1: scores of both halves, the first half's exponentials beside the second half's
       // MFMAs, and the first half's V fragments requested before the block ends.
       // Region 1: all eight K fragments of the first half are requested at once.
