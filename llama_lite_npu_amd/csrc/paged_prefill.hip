@@ -898,6 +898,8 @@ static int validate_prefill(const char *what, const void *q, int64_t q_stride, c
   LITEKV_REQUIRE(q_stride >= row && q_stride % 8 == 0 && out_stride >= row && out_stride % 8 == 0,
                  "%s: token strides (%lld, %lld) invalid", what, (long long)q_stride,
                  (long long)out_stride);
+  // q rows are staged with 32-bit byte offsets from the block's first row
+  LITEKV_REQUIRE(q_stride < (1 << 25), "%s: q token stride %lld too large", what, (long long)q_stride);
   return LITEKV_OK;
 }
 
