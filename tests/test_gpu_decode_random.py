@@ -174,3 +174,48 @@ def test_large_batches_take_the_packed_merge(batch):
     assert float(out[11].abs().max()) == 0.0
     live = [i for i in range(batch) if i != 11]
     assert torch.equal(again[live], out[live])
+
+
+@pytest.mark.parametrize("seed", range(2))
+def test_random_fused_steps_at_head_dim_64_and_larger_pages(seed):
+    """The same at head dim 64 (the second build of the decode kernels) with pages of 16, 32 or 64
+    tokens, both schedules."""
+    rng = random.Random(700 + seed)
+    for case_no in range(10):
+        hq, hkv = rng.choice(HEADS)
+        page_size = rng.choice([16, 32, 64])
+        b = rng.choice([1, 2, 3, 5, 8, 13, 32])
+        kind = rng.choice(["short", "mixed", "long", "tiny"])
+        lens = _lengths(rng, kind, b)
+        chunks = rng.choice(CHUNKS)
+        case = workloads.make_decode_case("random64", 5000 + 100 * seed + case_no, lens, hq, hkv, device=DEV,
+                                          head_dim=64, page_size=page_size)
+        empty = [i for i in range(b) if rng.random() < 0.1]
+        live = [i for i in range(b) if i not in empty]
+        for i in empty:
+            case.seq_lens[i] = 0
+        print(f"random step hd64 {seed}.{case_no}: heads {hq}/{hkv} page {page_size} batch {b} {kind} chunks {chunks} "
+              f"empty {empty}", flush=True)
+        pool_ref = case.kv_pool.clone()
+        ops.kv_append(case.k_new, case.v_new, case.slot_mapping, pool_ref)
+        keep = torch.ones(case.kv_pool.shape[0], dtype=torch.bool, device=DEV)
+        for i in empty:
+            keep[case.slot_mapping[i].long()] = False
+        ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool_ref), case.block_table.cpu().numpy(),
+                                    case.seq_lens.cpu().numpy(), case.softmax_scale, page_size=page_size)
+        plan = ops.DecodePlan(case.block_table, case.seq_lens, hq, hkv, case.num_pages, chunks, page_size=page_size)
+        pool = case.kv_pool.clone()
+        out = ops.decode_step(case.q, pool, plan, case.k_new, case.v_new, case.softmax_scale)
+        again = ops.decode_step(case.q, pool, plan, None, None, case.softmax_scale)
+        split_pool = case.kv_pool.clone()
+        split = ops.paged_decode(case.q, split_pool, case.block_table, case.seq_lens, case.softmax_scale,
+                                 max_splits=rng.choice([1, 3, 8]), min_pages_per_split=rng.choice([1, 4]),
+                                 k_new=case.k_new, v_new=case.v_new, page_size=page_size)
+        torch.cuda.synchronize()
+        assert torch.equal(pool[keep].view(torch.int16), pool_ref[keep].view(torch.int16))
+        assert torch.equal(split_pool[keep].view(torch.int16), pool_ref[keep].view(torch.int16))
+        assert_attention_close(out, ref, f"random step hd64 {seed}.{case_no}")
+        assert_attention_close(split, ref, f"random step hd64 {seed}.{case_no}, splits schedule")
+        for i in empty:
+            assert float(out[i].abs().max()) == 0.0
+        assert torch.equal(again[live], out[live])
