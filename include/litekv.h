@@ -29,8 +29,8 @@
  * (the reference kernels take the head dim as a block size,
  * lite_llama/kernels/flashdecoding.py:305, 393-396) through the same entry
  * points on one general kernel with fp32 arithmetic where no tiled kernel
- * exists (32 and 256; a shared prefix at 64): it writes the final rows in a
- * single launch whatever schedule was asked for, and uses no workspace.
+ * exists (32 and 256): it writes the final rows in a single launch whatever
+ * schedule was asked for, and uses no workspace.
  */
 #ifndef LITEKV_H
 #define LITEKV_H

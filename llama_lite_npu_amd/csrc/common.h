@@ -53,6 +53,13 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
                          int32_t num_kv_heads, int64_t num_pages, int32_t shared_pages,
                          int32_t page_shift, float *part_o, float *part_lse, float softmax_scale,
                          hipStream_t stream, int *splits_out, int format);
+// The same for head dim 64 (defined in the head dim 64 build of paged_prefill.hip).
+int launch_shared_prefix_hd64(const void *q, int64_t q_batch_stride, const void *kv_pool,
+                              const float *fp8_scales, const int32_t *block_table, int32_t batch,
+                              int32_t num_q_heads, int32_t num_kv_heads, int64_t num_pages,
+                              int32_t shared_pages, int32_t page_shift, float *part_o,
+                              float *part_lse, float softmax_scale, hipStream_t stream,
+                              int *splits_out, int format);
 
 // ---- the plan of a balanced decode step (made by decode_plan_kernel in paged_decode.hip) -------
 // Plan buffer (int32 words): meta[kPlanMeta]; per sequence (first chunk, number of chunks it
@@ -129,7 +136,8 @@ int hd64_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_sp
                const float *scales, int format);
 int hd64_merge(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split);
 int hd64_balanced(const char *what, const void *q, int64_t q_batch_stride, void *kv_pool,
-                  const float *scales, const int32_t *seq_lens, void *plan, size_t plan_bytes,
+                  const float *scales, const int32_t *block_table, int32_t shared_pages,
+                  const int32_t *seq_lens, void *plan, size_t plan_bytes,
                   const void *k_new, const void *v_new, int64_t k_new_stride, int64_t v_new_stride,
                   void *out, void *workspace, size_t workspace_bytes, int32_t batch,
                   int32_t num_q_heads, int32_t num_kv_heads, int32_t page_size, int64_t num_pages,

@@ -1686,15 +1686,16 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
                block_table_stride, seq_lens, out, workspace, workspace_bytes, batch, num_q_heads,
                num_kv_heads, head_dim, page_size, num_pages, softmax_scale, stream};
 #if LITEKV_HD == 128
-  if (head_dim == 64 && shared_pages == 0) {
-    return hd64_balanced(what, q, q_batch_stride, kv_pool, fp8_scales, seq_lens, plan, plan_bytes,
+  if (head_dim == 64) {
+    return hd64_balanced(what, q, q_batch_stride, kv_pool, fp8_scales, block_table, shared_pages,
+                         seq_lens, plan, plan_bytes,
                          k_new, v_new, k_new_stride, v_new_stride, out, workspace, workspace_bytes,
                          batch, num_q_heads, num_kv_heads, page_size, num_pages, block_table_stride,
                          chunks, softmax_scale, stream, format);
   }
 #endif
   if (head_dim != kHD) {
-    // other head dims (and 64 over a shared prefix): the generic kernel, which takes its page ids from the block table where
+    // other head dims: the generic kernel, which takes its page ids from the block table where
     // the caller gave one (then shared pages are attended like any others), else from the plan
     a.k_new = k_new;
     a.v_new = v_new;
@@ -1746,7 +1747,12 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   int pre_splits = 0;
   if (shared_pages > 0) {
     LITEKV_REQUIRE(block_table != nullptr, "%s: block_table is null", what);
-    rc = launch_shared_prefix(q, q_batch_stride, kv_pool, fp8_scales, block_table, batch, num_q_heads,
+#if LITEKV_HD == 64
+    rc = launch_shared_prefix_hd64(
+#else
+    rc = launch_shared_prefix(
+#endif
+                              q, q_batch_stride, kv_pool, fp8_scales, block_table, batch, num_q_heads,
                               num_kv_heads, num_pages, shared_pages, shift, pre_o, pre_lse,
                               softmax_scale, static_cast<hipStream_t>(stream), &pre_splits, format);
     if (rc != LITEKV_OK) return rc;
@@ -2151,16 +2157,17 @@ int hd64_merge(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_sp
   return launch_merge(a, max_splits, min_pages_per_split);
 }
 int hd64_balanced(const char *what, const void *q, int64_t q_batch_stride, void *kv_pool,
-                  const float *scales, const int32_t *seq_lens, void *plan, size_t plan_bytes,
+                  const float *scales, const int32_t *block_table, int32_t shared_pages,
+                  const int32_t *seq_lens, void *plan, size_t plan_bytes,
                   const void *k_new, const void *v_new, int64_t k_new_stride, int64_t v_new_stride,
                   void *out, void *workspace, size_t workspace_bytes, int32_t batch,
                   int32_t num_q_heads, int32_t num_kv_heads, int32_t page_size, int64_t num_pages,
                   int32_t block_table_stride, int32_t chunks, float softmax_scale, void *stream,
                   int format) {
-  return launch_balanced(what, q, q_batch_stride, kv_pool, scales, nullptr, seq_lens, plan,
+  return launch_balanced(what, q, q_batch_stride, kv_pool, scales, block_table, seq_lens, plan,
                          plan_bytes, k_new, v_new, k_new_stride, v_new_stride, out, workspace,
                          workspace_bytes, batch, num_q_heads, num_kv_heads, kHD, page_size, num_pages,
-                         block_table_stride, chunks, 0, softmax_scale, stream, format);
+                         block_table_stride, chunks, shared_pages, softmax_scale, stream, format);
 }
 }  // namespace litekv
 #endif  // LITEKV_HD == 64

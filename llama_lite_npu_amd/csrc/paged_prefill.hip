@@ -62,7 +62,7 @@
 // This file is compiled twice: as it stands for head dim 128, and through paged_prefill_hd64.hip
 // (which defines LITEKV_HD and includes it) for head dim 64 (paged in every pool format, or packed).
 // Everything sits in an inline namespace named after the head dim, so the two builds link side by
-// side; the C ABI and the shared-prefix launcher are in the 128 build, which hands 64-wide calls
+// side; the C ABI is in the 128 build, which hands 64-wide calls
 // to hd64_paged_prefill / hd64_varlen_prefill.
 #ifndef LITEKV_HD
 #define LITEKV_HD 128
@@ -919,7 +919,11 @@ static PrefillShape prefill_shape(int group, int max_q_len) {
 
 }  // namespace LITEKV_HD_NS
 #if LITEKV_HD == 128
-int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_pool,
+int launch_shared_prefix(
+#else
+int launch_shared_prefix_hd64(
+#endif
+                         const void *q, int64_t q_batch_stride, const void *kv_pool,
                          const float *fp8_scales, const int32_t *block_table, int32_t batch, int32_t num_q_heads,
                          int32_t num_kv_heads, int64_t num_pages, int32_t shared_pages,
                          int32_t page_shift, float *part_o, float *part_lse, float softmax_scale,
@@ -964,7 +968,6 @@ int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_p
   *splits_out = splits;
   return check_launch(what);
 }
-#endif  // LITEKV_HD == 128
 
 }  // namespace litekv
 

@@ -476,3 +476,28 @@ def test_head_dim_64_at_a_larger_size():
         got = ops.paged_decode(case.q, pool_ref, case.block_table, case.seq_lens, case.softmax_scale, **kw)
         torch.cuda.synchronize()
         assert_attention_close(got, ref, f"head_dim 64 {kw}")
+
+
+@pytest.mark.parametrize("page_size,shared_tokens", [(16, 1040), (32, 640), (64, 2048)])
+def test_head_dim_64_long_shared_prefix(page_size, shared_tokens):
+    """Head dim 64 behind a long shared prefix: the prefix goes through the tiled prefix kernel in
+    several key slices, the private pages through the balanced kernel, and the merge joins them."""
+    print(f"decode head_dim 64 shared prefix of {shared_tokens} tokens, page_size {page_size}", flush=True)
+    shared_pages = shared_tokens // page_size
+    suffix = [0, 1, page_size - 1, page_size, 3 * page_size + 5, 700, 64, 333]
+    ctx = [shared_tokens + s for s in suffix]
+    priv = [(c + 1 + page_size - 1) // page_size - shared_pages for c in ctx]
+    num_pages = shared_pages + sum(priv) + 5
+    perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(page_size)).to(torch.int32)
+    shared, cur, lists = perm[:shared_pages], shared_pages, []
+    for n in priv:
+        lists.append(torch.cat([shared, perm[cur:cur + n]]))
+        cur += n
+    case = workloads.make_decode_case("shared-64", 1560 + page_size, ctx, 32, 8, num_pages=num_pages, device=DEV,
+                                      page_lists=lists, head_dim=64, page_size=page_size)
+    ref = _oracle(case)
+    out = _run(case, schedule="balanced", shared_pages=shared_pages)
+    assert_attention_close(out, ref, "shared prefix at head_dim 64")
+    partly = _run(case, schedule="balanced", shared_pages=shared_pages // 2)
+    assert_attention_close(partly, ref, "half the shared prefix declared, head_dim 64")
+    assert torch.equal(out, _run(case, schedule="balanced", shared_pages=shared_pages))
