@@ -1047,7 +1047,20 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
 
   // Read ahead for the crossing. Everything the first requests need came with the entry: this
   // second hop is under way while they are issued.
-  int len_after = (cur_b + 1 < batch) ? lens[cur_b + 1] : 0;
+  // (the lengths of the next kLensAhead sequences: a scalar load issued at a crossing is waited
+  // for by the next LDS wait of the page loop, its whole latency exposed)
+  constexpr int kLensAhead = 2;
+  int lens_ahead[kLensAhead];
+  auto fetch_lens_ahead = [&]() {
+#pragma unroll
+    for (int i = 0; i < kLensAhead; ++i) {
+      lens_ahead[i] = lens[cur_b + 1 + i < batch ? cur_b + 1 + i : batch - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < kLensAhead; ++i) lens_ahead[i] = cur_b + 1 + i < batch ? lens_ahead[i] : 0;
+  };
+  fetch_lens_ahead();
+  int lens_left = kLensAhead;
 
   constexpr bool FP8 = KV != kKvF16;  // 8-bit codes (either format): the layout they share
   typedef typename KvStore<KV>::elem Elem;
@@ -1102,7 +1115,9 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
 
   // Page ids travel through scalar loads, one request ahead of their use.
   int pid_next = 0;
-  auto request = [&](int i, Page &r) {  // i = page index inside the chunk
+  int pid_held[DEPTH];  // the ids of the pages in flight, by buffer (the fused append needs one)
+  auto request = [&](int i, Page &r, int &held) {  // i = page index inside the chunk
+    held = pid_next;
     const int64_t page_off = (int64_t)pid_next * kPageSize * row_stride;
     const int nx = i + 1 < f1 - f0 ? i + 1 : f1 - f0 - 1;
     pid_next = page_ids[nx];
@@ -1166,11 +1181,33 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     parked_whole = cu_lo >= f0 && cu_hi <= f1 && skip == 0;
   };
 
+  // Stores the step's new fp16 rows (the lanes that own them in a page's registers).
+  auto store_new_rows = [&](const uint4_t (&k_row)[4], const uint4_t (&v_row)[2], int64_t slot_off,
+                            int t_new) {
+    if constexpr (!FP8) {
+      if (n == t_new) {
+        half_t *dst = kv + slot_off + (int64_t)h * kHD + 8 * g;
+#pragma unroll
+        for (int kk = 0; kk < kKSteps; ++kk) *(uint4_t *)(dst + 32 * kk) = k_row[kk];
+      }
+      if (g == (t_new & 3)) {
+        *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHD + 8 * (n & (kVCols - 1))) = v_row[0];
+      }
+    }
+  };
+  // In an fp16 pool the rows requested ahead (the chunk's first sequence) are stored after the
+  // page loop, for the reason a finished state is parked: a store in the middle of the chunk
+  // delays every later counted wait by its acknowledgement (C2: -0.25 us per layer). The page's
+  // registers are patched where it is attended. With 8-bit codes the rows kept for the end cost
+  // 30 registers and the step is 0.3 to 1.5 us slower: those are stored where they are appended.
+  int late_row = -1;  // the pool row (page * 16 + token) they go to
+
   Page buf[DEPTH];
 #pragma unroll
   for (int dd = 0; dd < DEPTH; ++dd) {
     pid_next = first_ids[dd];
-    if (dd < f1 - f0) request(dd, buf[dd]);
+    pid_held[dd] = 0;
+    if (dd < f1 - f0) request(dd, buf[dd], pid_held[dd]);
   }
   // after the prologue pid_next holds the id of page DEPTH (clamped), as the loop expects
   for (int f = f0; f < f1; f += DEPTH) {
@@ -1186,9 +1223,15 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
         if (ff >= cu_hi) {  // the line enters the next non-empty sequence
           flush_at_crossing();
           do {
+            if (lens_left == 0) {
+              fetch_lens_ahead();
+              lens_left = kLensAhead;
+            }
             ++cur_b;
-            len_b = len_after;
-            len_after = (cur_b + 1 < batch) ? lens[cur_b + 1] : 0;
+            --lens_left;
+            len_b = lens_ahead[0];
+#pragma unroll
+            for (int i = 0; i + 1 < kLensAhead; ++i) lens_ahead[i] = lens_ahead[i + 1];
             int pg = pages_of(len_b);
             pg = (pg < bt_stride ? pg : bt_stride) - skip;
             pg = pg > 0 ? pg : 0;
@@ -1221,8 +1264,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
             fetch_new_rows(k_row, v_row, cur_b);
             wait_vector_loads();
           }
-          const int pid = page_ids[ff - f0];
-          const int64_t slot_off = ((int64_t)pid * kPageSize + t_new) * row_stride;
+          const int64_t slot_off = ((int64_t)pid_held[dd] * kPageSize + t_new) * row_stride;
           if constexpr (FP8) {
             // the rows are quantised as the append kernel would, stored, and attended as stored
             if (n == t_new) {
@@ -1248,21 +1290,20 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
             }
           } else {
             if (n == t_new) {
-              half_t *dst = kv + slot_off + (int64_t)h * kHD + 8 * g;
 #pragma unroll
-              for (int kk = 0; kk < kKSteps; ++kk) {
-                const half8_t x = __builtin_bit_cast(half8_t, k_row[kk]);
-                buf[dd].k[kk] = x;
-                *(half8_t *)(dst + 32 * kk) = x;
-              }
+              for (int kk = 0; kk < kKSteps; ++kk) buf[dd].k[kk] = __builtin_bit_cast(half8_t, k_row[kk]);
             }
             if (g == (t_new & 3)) {
               const half8_t x = __builtin_bit_cast(half8_t, v_row[0]);
-              *(half8_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHD + 8 * (n & (kVCols - 1))) = x;
 #pragma unroll
               for (int i = 0; i < 4; ++i) {
                 if (i == (t_new >> 2)) buf[dd].v[i] = x;
               }
+            }
+            if (cur_b == rows_b) {  // from k_ahead / v_ahead, after the page loop
+              late_row = pid_held[dd] * kPageSize + t_new;
+            } else {
+              store_new_rows(k_row, v_row, slot_off, t_new);
             }
           }
         }
@@ -1272,8 +1313,11 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
       // of 16 bytes, so that the number of loads in flight was a compile-time constant and every
       // wait named exactly the page it needed; with the condition the compiler's waits also
       // cover part of the next page's loads, and the launch is still faster: C2 0.65 us per layer.)
-      if (ff + DEPTH < f1) request(ff - f0 + DEPTH, buf[dd]);
+      if (ff + DEPTH < f1) request(ff - f0 + DEPTH, buf[dd], pid_held[dd]);
     }
+  }
+  if (late_row >= 0) {
+    store_new_rows(k_ahead, v_ahead, (int64_t)late_row * row_stride, late_row & (kPageSize - 1));
   }
   flush();
   if (parked_b >= 0) unpark();
