@@ -22,10 +22,14 @@
  * (lite_llama/executor/paged_attention.py:141-146, 347-354), so a page is one
  * contiguous run of page_size * 2 * Hkv * head_dim * 2 bytes.
  *
- * Supported shapes: Hq % Hkv == 0, Hq / Hkv <= 16; page_size 16, 32 or 64
- * (the reference's --page_size, lite_llama/server.py:1038-1161): the attention
- * kernels walk a page of 32 or 64 tokens as two or four consecutive 16-token
- * pieces; head_dim 128 and 64 on the MFMA-tiled kernels, and 32, 64 or 256
+ * Supported shapes: Hq % Hkv == 0, Hq / Hkv <= 64 (the decode kernels hold the
+ * query heads of a kv head in the 16 columns of a tile; a larger group runs as
+ * slices of up to 16, each reading the head's K/V; the reference's grids are
+ * per query head, lite_llama/kernels/flashdecoding.py:44, 170-175); page_size
+ * 16, 32, 64, 128 or 256 (the reference's --page_size,
+ * lite_llama/server.py:1038-1161, "typically 16-256",
+ * lite_llama/executor/paged_attention.py:27): the attention kernels walk a
+ * larger page as 2 .. 16 consecutive 16-token pieces; head_dim 128 and 64 on the MFMA-tiled kernels, and 32, 64 or 256
  * (the reference kernels take the head dim as a block size,
  * lite_llama/kernels/flashdecoding.py:305, 393-396) through the same entry
  * points on one general kernel with fp32 arithmetic where no tiled kernel
@@ -46,7 +50,7 @@ extern "C" {
 #define LITEKV_ERR_INVALID_ARGUMENT 1
 #define LITEKV_ERR_LAUNCH 2
 
-#define LITEKV_ABI_VERSION 1
+#define LITEKV_ABI_VERSION 2
 
 /* ABI version of the loaded library (LITEKV_ABI_VERSION at build time). */
 int litekv_abi_version(void);
@@ -209,9 +213,14 @@ int litekv_paged_decode_merge(const int32_t *seq_lens, void *out,
  *           in time on one GPU (two streams, two threads) race; calls on one
  *           stream are ordered. Nothing in it has to start at zero: the merge
  *           reads only the cells the split launch of the same call wrote.
+ *           A host thread that enters while another is still enqueueing its
+ *           launches on the same GPU gets LITEKV_ERR_INVALID_ARGUMENT; overlap
+ *           on the GPU between streams is the caller's to exclude.
  *   set-up  the array's address on a device is looked up on the first call
- *           made with that device current (no allocation, but make that first
- *           call outside a graph capture).
+ *           made with that device current (no allocation). Any call does it,
+ *           also one with batch 0: make that call before capturing a graph. A
+ *           first call that finds its stream capturing returns
+ *           LITEKV_ERR_INVALID_ARGUMENT and leaves the capture intact.
  */
 #define LITEKV_STATIC_SCRATCH_BYTES (32u << 20)
 
@@ -264,7 +273,7 @@ size_t litekv_paged_decode_balanced_workspace_bytes(int32_t batch, int32_t num_q
 
 size_t litekv_decode_plan_bytes(int32_t batch, int32_t block_table_stride,
                                 int32_t num_kv_heads, int32_t chunks);
-/* The same for a pool whose pages hold page_size (16, 32 or 64) tokens: the plan
+/* The same for a pool whose pages hold page_size (16 .. 256) tokens: the plan
  * lists 16-token pages, page_size / 16 per block-table entry.
  * litekv_decode_plan_bytes is the page_size 16 case. 0 for another page_size. */
 size_t litekv_decode_plan_bytes_paged(int32_t batch, int32_t block_table_stride,

@@ -29,6 +29,17 @@ constexpr int kWave = 64;       // lanes per wavefront on CDNA
 int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 void clear_error();
 
+// log2(page_size / 16) for the page sizes the kernels take (16, 32, 64, 128, 256 tokens: the
+// reference documents "typically 16-256", lite_llama/executor/paged_attention.py:27), or -1. The
+// attention kernels keep their 16-token page step and walk a larger page as 2 .. 16 consecutive
+// 16-token pieces.
+inline int page_shift_of(int32_t page_size) {
+  for (int shift = 0; shift <= 4; ++shift) {
+    if (page_size == (16 << shift)) return shift;
+  }
+  return -1;
+}
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // Turns the status of the launch just issued into an ABI status.
@@ -38,6 +49,26 @@ int check_launch(const char *what);
   do {                                                                    \
     if (!(cond)) return ::litekv::fail(LITEKV_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
   } while (0)
+
+// Query heads per kv head the kernels take. The decode kernels hold the query heads of a kv head
+// in the 16 columns of an MFMA tile; a larger group is served as `head_slices(group)` slices of
+// the kv head, each a wavefront of its own with up to 16 of the group's query heads (the
+// reference's grid is per query head with no bound, lite_llama/kernels/flashdecoding.py:44,
+// 170-175). K/V of such a head is then read once per slice.
+constexpr int kMaxGroup = 64;
+__host__ __device__ __forceinline__ int head_slices(int group) { return (group + 15) / 16; }
+struct HeadSlice {
+  int kv_head;   // whose K/V rows and scales the slice reads
+  int q_head0;   // first query head of the slice
+  int q_heads;   // query heads in the slice (columns in use)
+};
+// Slice `hv` of the launch's kv_heads * slices slices (slices of one kv head are neighbours).
+__host__ __device__ __forceinline__ HeadSlice head_slice(int hv, int slices, int group) {
+  const int kv = hv / slices, sub = hv - kv * slices;
+  const int per = (group + slices - 1) / slices;
+  const int left = group - sub * per;
+  return HeadSlice{kv, kv * group + sub * per, left < per ? left : per};
+}
 
 // Most key slices the shared-prefix kernel may cut the prefix into (bounds its workspace).
 constexpr int kMaxPrefixSplits = 8;

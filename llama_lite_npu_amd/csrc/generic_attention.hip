@@ -84,17 +84,19 @@ __device__ __forceinline__ void store8(void *row, int d8, half8_t x, float inv_s
   }
 }
 
-// grid (kv heads, query rows per sequence, sequences), one wavefront each
+// grid (head slices, query rows per sequence, sequences), one wavefront each; a head slice is a
+// kv head, or up to 16 of its query heads when it has more than 16 (see head_slice)
 template <int KV>
 __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t) {
   __shared__ float qs[kGenericMaxGroup][kGenericMaxDim];
   __shared__ float ps[kWave][kGenericMaxGroup + 1];
   const int lane = threadIdx.x;
-  const int h = blockIdx.x;
+  const HeadSlice hs = head_slice((int)blockIdx.x, head_slices(t.group), t.group);
+  const int h = hs.kv_head;
   const int row_in_seq = blockIdx.y;
   const int b = blockIdx.z;
   const int D = t.head_dim;
-  const int group = t.group;
+  const int group = hs.q_heads;
   const bool paged = t.kv_pool != nullptr;
 
   // the query row, the number of keys it sees, and where its sequence's packed keys start
@@ -115,7 +117,7 @@ __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t)
     q_row = b;
     n_keys = t.seq_lens[b];
   }
-  const int hq0 = h * group;
+  const int hq0 = hs.q_head0;
   half_t *out_row = t.out + q_row * t.out_row_stride + (int64_t)hq0 * D;
   if (n_keys <= 0) {  // an empty sequence of a decode step
     for (int i = lane; i < group * D; i += kWave) out_row[i] = (half_t)0.f;
@@ -145,7 +147,9 @@ __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t)
   // the K row of key `tok` (V: + num_kv_heads * D elements in a pool)
   auto k_row_of = [&](int tok) -> const char * {
     if (planned) {
-      const int f = before + (tok >> 4);
+      // the plan holds at most a block-table row's worth of 16-token pages per sequence
+      const int cap16 = t.bt_stride * (t.page_size >> 4);
+      const int f = before + ((tok >> 4) < cap16 ? (tok >> 4) : cap16 - 1);
       const int c = cut.chunk_of(f);
       const int pid16 = t.plan[plan_entries_offset(plan_batch) + (int64_t)c * entry_stride + kEntryHeader +
                                (f - cut.chunk_start(c))];
@@ -153,7 +157,9 @@ __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t)
       return (const char *)t.kv_pool + slot * slot_bytes + (int64_t)h * D * elem;
     }
     if (paged) {
-      int pid = table[tok / t.page_size];
+      int at = tok / t.page_size;
+      at = at < t.bt_stride ? at : t.bt_stride - 1;  // a length beyond the row re-reads its last entry
+      int pid = table[at];
       pid = pid < 0 ? 0 : (pid >= t.num_pages ? t.num_pages - 1 : pid);
       const int64_t slot = (int64_t)pid * t.page_size + tok % t.page_size;
       return (const char *)t.kv_pool + slot * slot_bytes + (int64_t)h * D * elem;
@@ -167,8 +173,10 @@ __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t)
     return (const char *)(t.v + (packed0 + tok) * t.v_stride + (int64_t)h * D);
   };
 
-  // the step's new rows of this head, if this launch appends them
-  const bool appends = t.k_new != nullptr;
+  // the step's new rows of this head, if this launch appends them (not for a length beyond what
+  // the block-table row can name: the row's last page is not where that token belongs)
+  const bool appends = t.k_new != nullptr &&
+                       (int64_t)n_keys <= (int64_t)t.bt_stride * t.page_size;
   const half_t *k_new = appends ? t.k_new + (int64_t)b * t.k_new_stride + (int64_t)h * D : nullptr;
   const half_t *v_new = appends ? t.v_new + (int64_t)b * t.v_new_stride + (int64_t)h * D : nullptr;
 
@@ -280,8 +288,8 @@ int launch_generic_attention(const char *what, const GenericLaunch &a) {
                      a.num_q_heads <= 65535,
                  "%s: num_q_heads %d / num_kv_heads %d invalid", what, a.num_q_heads, a.num_kv_heads);
   const int group = a.num_q_heads / a.num_kv_heads;
-  LITEKV_REQUIRE(group <= kGenericMaxGroup, "%s: %d query heads per kv head unsupported (max 16)",
-                 what, group);
+  LITEKV_REQUIRE(group <= kMaxGroup, "%s: %d query heads per kv head unsupported (max %d)", what,
+                 group, kMaxGroup);
   LITEKV_REQUIRE(a.rows_per_seq >= 0 && a.rows_per_seq <= 65535, "%s: %d query rows per sequence",
                  what, a.rows_per_seq);
   if (a.batch == 0 || a.rows_per_seq == 0) {
@@ -298,8 +306,8 @@ int launch_generic_attention(const char *what, const GenericLaunch &a) {
   if (a.kv_pool != nullptr) {
     LITEKV_REQUIRE((a.block_table != nullptr && a.bt_stride >= 1) || a.plan != nullptr,
                    "%s: block table missing", what);
-    LITEKV_REQUIRE(a.page_size == 16 || a.page_size == 32 || a.page_size == 64,
-                   "%s: page_size %d unsupported (16, 32 or 64)", what, a.page_size);
+    LITEKV_REQUIRE(page_shift_of(a.page_size) >= 0,
+                   "%s: page_size %d unsupported (16, 32, 64, 128 or 256)", what, a.page_size);
     LITEKV_REQUIRE(a.num_pages >= 1 && a.num_pages <= 0x7fffffffLL / a.page_size,
                    "%s: num_pages %lld out of range", what, (long long)a.num_pages);
     LITEKV_REQUIRE(aligned16(a.kv_pool), "%s: kv_pool must be 16-byte aligned", what);
@@ -352,8 +360,9 @@ int launch_generic_attention(const char *what, const GenericLaunch &a) {
   t.group = group;
   t.head_dim = a.head_dim;
   t.scale_log2 = a.softmax_scale * 1.4426950408889634f;
-  LITEKV_REQUIRE(a.num_kv_heads <= 65535, "%s: num_kv_heads %d > 65535", what, a.num_kv_heads);
-  const dim3 grid((unsigned)a.num_kv_heads, (unsigned)a.rows_per_seq, (unsigned)a.batch);
+  const int slice_heads = a.num_kv_heads * head_slices(group);
+  LITEKV_REQUIRE(slice_heads <= 65535, "%s: num_q_heads %d too large", what, a.num_q_heads);
+  const dim3 grid((unsigned)slice_heads, (unsigned)a.rows_per_seq, (unsigned)a.batch);
   const hipStream_t stream = static_cast<hipStream_t>(a.stream);
   const int format = a.kv_pool != nullptr ? a.format : kKvF16;
   if (format == kKvInt8) {

@@ -441,19 +441,22 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
     const int32_t *__restrict__ seq_lens, const half_t *__restrict__ k_new,
     const half_t *__restrict__ v_new, int64_t k_new_stride, int64_t v_new_stride,
     half_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_lse,
-    int32_t num_q_heads, int32_t num_kv_heads, int32_t group, int32_t max_splits,
+    int32_t num_q_heads, int32_t num_kv_heads, int32_t group_all, int32_t slices, int32_t max_splits,
     int32_t min_pages_per_split, int32_t num_pages, int32_t page_shift, float scale_log2) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
-  const int n = lane & 15;   // query head inside the group (column of S^T)
+  const int n = lane & 15;   // query head inside the slice (column of S^T)
   const int g = lane >> 4;   // lane group: owns tokens 4g..4g+3 of a page
-  const int h = blockIdx.x * (blockDim.x >> 6) + wave;  // kv head
+  // a kv head with more than 16 query heads is served in slices of up to 16 (see head_slice)
+  const HeadSlice hs = head_slice(blockIdx.x * (blockDim.x >> 6) + wave, slices, group_all);
+  const int h = hs.kv_head;
+  const int group = hs.q_heads;
   const int split = blockIdx.y;
   const int b = blockIdx.z;
   half_t *vstage = split_vstage + wave * (kPageSize * kVPitch);
 
   const int len = seq_lens[b];
-  const int hq0 = h * group;
+  const int hq0 = hs.q_head0;
   half_t *out_row = out + ((int64_t)b * num_q_heads + hq0) * kHD;
   if (len <= 0) {
     if (split == 0 && n < group) {
@@ -509,9 +512,14 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
   // use. Requests past the range still issue their loads (16 bytes of its last page), which keeps
   // the number of vector loads in flight a compile-time constant, so each wait names exactly the
   // page it needs and never drains the younger prefetches.
+  // A length beyond what a block-table row can name (the host cannot check lengths that live on
+  // the device) re-reads the row's last entry instead of reading past it, and appends nothing.
+  const bool fits_table = pages <= (bt_stride << page_shift);
   auto page_id = [&](int p) {
     const int pp = p < p1 ? p : p1 - 1;
-    return sub_page_id(table[pp >> page_shift], pp, page_shift, num_pages);
+    int at = pp >> page_shift;
+    at = at < bt_stride ? at : bt_stride - 1;
+    return sub_page_id(table[at], pp, page_shift, num_pages);
   };
   int pid_next = page_id(p0);
   auto request = [&](int p, Page &r) {
@@ -526,7 +534,7 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
 #pragma unroll
     for (int dd = 0; dd < DEPTH; ++dd) {
       if (p + dd < p1) {
-        if (APPEND && (p + dd + 1) * kPageSize >= len) {
+        if (APPEND && fits_table && (p + dd + 1) * kPageSize >= len) {
           // The sequence's last page: the step's new token (logical position len - 1) goes to
           // the pool and replaces the stale values this wavefront loaded before the write; an
           // fp8 pool gets the codes the append kernel would store and is attended as stored.
@@ -991,8 +999,9 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     const int32_t *__restrict__ seq_lens, const int32_t *__restrict__ plan,
     const half_t *__restrict__ k_new, const half_t *__restrict__ v_new, int64_t k_new_stride,
     int64_t v_new_stride, half_t *__restrict__ out, float *__restrict__ part_o,
-    float *__restrict__ part_lse, int32_t bt_stride, int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t group,
-    int32_t heads_per_wg, int32_t replicas, int32_t chunks, int32_t skip, float scale_log2) {
+    float *__restrict__ part_lse, int32_t bt_stride, int32_t batch, int32_t num_q_heads,
+    int32_t num_kv_heads, int32_t group_all, int32_t slices, int32_t heads_per_wg,
+    int32_t replicas, int32_t chunks, int32_t skip, float scale_log2) {
   __shared__ __attribute__((aligned(16))) half_t vstage_all[kMaxWavesPerWg][kPageSize * kVPitch];
   __shared__ __attribute__((aligned(16))) float park_all[kMaxWavesPerWg][kParkFloats];
 
@@ -1001,9 +1010,14 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   const int lane = threadIdx.x & 63;
   const int n = lane & 15;
   const int g = lane >> 4;
-  const int h = blockIdx.y * heads_per_wg + wave % heads_per_wg;
+  // a wavefront per head slice: the kv head itself, or up to 16 of its query heads when it has
+  // more than 16 (see head_slice)
+  const int hv = blockIdx.y * heads_per_wg + wave % heads_per_wg;
   const int cidx = blockIdx.x * replicas + wave / heads_per_wg;
-  if (h >= num_kv_heads || cidx >= chunks) return;  // whole wavefront; no workgroup barriers below
+  if (hv >= num_kv_heads * slices || cidx >= chunks) return;  // whole wavefront; no workgroup barriers below
+  const HeadSlice hs = head_slice(hv, slices, group_all);
+  const int h = hs.kv_head;
+  const int group = hs.q_heads;
   half_t *vstage = vstage_all[wave];
 
   // Empty sequences are on no chunk's line: chunk c zeroes the rows of sequences c, c + chunks, ...
@@ -1011,7 +1025,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   auto zero_empty_rows = [&]() {
     for (int bz = cidx; bz < batch; bz += chunks) {
       if (seq_lens[bz] <= 0 && n < group) {
-        half_t *o = out + ((int64_t)bz * num_q_heads + h * group + n) * kHD + 4 * g;
+        half_t *o = out + ((int64_t)bz * num_q_heads + hs.q_head0 + n) * kHD + 4 * g;
 #pragma unroll
         for (int j = 0; j < kJTiles; ++j) *(half4_t *)(o + 16 * j) = half4_t{0, 0, 0, 0};
       }
@@ -1076,7 +1090,7 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     v_inv = 1.0f / v_scale;
   }
 
-  const int hq0 = h * group;
+  const int hq0 = hs.q_head0;
   const int64_t row_stride = (int64_t)2 * num_kv_heads * kHD;
   // this lane's row and column inside page 0 (see PageRegs / PageRegsFp8)
   Elem *k_lane = kv + (int64_t)h * kHD + (FP8 ? 16 : 8) * g + n * row_stride;
@@ -1334,10 +1348,6 @@ namespace litekv {
 inline namespace LITEKV_HD_NS {
 
 
-// log2(page_size / 16) for the page sizes the kernels take (16, 32, 64 tokens), or -1.
-static int page_shift_of(int32_t page_size) {
-  return page_size == 16 ? 0 : page_size == 32 ? 1 : page_size == 64 ? 2 : -1;
-}
 
 // Checks shared by every decode entry point; `need_inputs` is false for the merge-only calls.
 static int validate_decode(const char *what, const DecodeArgs &a, size_t workspace_needed,
@@ -1345,7 +1355,7 @@ static int validate_decode(const char *what, const DecodeArgs &a, size_t workspa
   LITEKV_REQUIRE(a.batch >= 0 && a.batch <= 65535, "%s: batch %d out of [0, 65535]", what, a.batch);
   LITEKV_REQUIRE(a.head_dim == kHD, "%s: head_dim %d unsupported (32, 64, 128 or 256)", what,
                  a.head_dim);
-  LITEKV_REQUIRE(page_shift_of(a.page_size) >= 0, "%s: page_size %d unsupported (16, 32 or 64)",
+  LITEKV_REQUIRE(page_shift_of(a.page_size) >= 0, "%s: page_size %d unsupported (16, 32, 64, 128 or 256)",
                  what, a.page_size);
   LITEKV_REQUIRE(a.num_q_heads > 0 && a.num_q_heads <= 65535, "%s: num_q_heads %d out of range",
                  what, a.num_q_heads);
@@ -1363,9 +1373,9 @@ static int validate_decode(const char *what, const DecodeArgs &a, size_t workspa
     LITEKV_REQUIRE(a.num_kv_heads > 0 && a.num_q_heads % a.num_kv_heads == 0,
                    "%s: num_q_heads %d not a multiple of num_kv_heads %d", what, a.num_q_heads,
                    a.num_kv_heads);
-    LITEKV_REQUIRE(a.num_q_heads / a.num_kv_heads <= 16,
-                   "%s: %d query heads per kv head unsupported (max 16)", what,
-                   a.num_q_heads / a.num_kv_heads);
+    LITEKV_REQUIRE(a.num_q_heads / a.num_kv_heads <= kMaxGroup,
+                   "%s: %d query heads per kv head unsupported (max %d)", what,
+                   a.num_q_heads / a.num_kv_heads, kMaxGroup);
     LITEKV_REQUIRE(a.q_batch_stride >= (int64_t)a.num_q_heads * a.head_dim &&
                        a.q_batch_stride % 8 == 0,
                    "%s: q_batch_stride %lld invalid", what, (long long)a.q_batch_stride);
@@ -1460,6 +1470,9 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   }
   LITEKV_REQUIRE(a.num_kv_heads <= 65535, "%s: num_kv_heads %d > 65535", what, a.num_kv_heads);
   const int group = a.num_q_heads / a.num_kv_heads;
+  const int slices = head_slices(group);           // wavefronts per kv head
+  const int slice_heads = a.num_kv_heads * slices;
+  LITEKV_REQUIRE(slice_heads <= 65535, "%s: num_q_heads %d too large", what, a.num_q_heads);
   float *part_o = max_splits > 1 ? static_cast<float *>(a.workspace) : nullptr;
   float *part_lse =
       max_splits > 1 ? part_o + (size_t)a.batch * a.num_q_heads * max_splits * a.head_dim : nullptr;
@@ -1467,10 +1480,10 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   // pages and the same trip count, and a token's K and V rows are contiguous over the heads -- as
   // leave at least two workgroups per compute unit (C5, 16 splits: 1011 us per layer with one
   // wavefront per workgroup, 930 with its four kv heads together).
-  const int64_t units = (int64_t)a.batch * a.num_kv_heads * max_splits;
+  const int64_t units = (int64_t)a.batch * slice_heads * max_splits;
   int waves = kSplitWaves;
-  while (waves > 1 && (units / waves < 512 || a.num_kv_heads % waves != 0)) waves >>= 1;
-  const dim3 grid((unsigned)(a.num_kv_heads / waves), (unsigned)max_splits, (unsigned)a.batch);
+  while (waves > 1 && (units / waves < 512 || slice_heads % waves != 0)) waves >>= 1;
+  const dim3 grid((unsigned)(slice_heads / waves), (unsigned)max_splits, (unsigned)a.batch);
   const dim3 block((unsigned)(waves * kWave));
   const size_t lds = (size_t)waves * kPageSize * kVPitch * sizeof(half_t);
   LITEKV_REQUIRE((a.k_new == nullptr) == (a.v_new == nullptr), "%s: k_new and v_new go together", what);
@@ -1491,7 +1504,7 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
                        a.block_table, a.block_table_stride, a.seq_lens,
                        static_cast<const half_t *>(a.k_new), static_cast<const half_t *>(a.v_new),
                        a.k_new_stride, a.v_new_stride, static_cast<half_t *>(a.out), part_o, part_lse,
-                       a.num_q_heads, a.num_kv_heads, group, max_splits,
+                       a.num_q_heads, a.num_kv_heads, group, slices, max_splits,
                        min_16_token_pages(min_pages_per_split, a.page_size), (int32_t)a.num_pages,
                        page_shift_of(a.page_size), a.softmax_scale * kLog2e);
   };
@@ -1648,7 +1661,7 @@ static int launch_plan(const char *what, const int32_t *block_table, int32_t blo
                        void *plan, size_t plan_bytes, void *stream) {
   LITEKV_REQUIRE(batch >= 0 && batch <= 65535, "%s: batch %d out of [0, 65535]", what, batch);
   const int shift = page_shift_of(page_size);
-  LITEKV_REQUIRE(shift >= 0, "%s: page_size %d unsupported (16, 32 or 64)", what, page_size);
+  LITEKV_REQUIRE(shift >= 0, "%s: page_size %d unsupported (16, 32, 64, 128 or 256)", what, page_size);
   LITEKV_REQUIRE(block_table_stride >= 1 && block_table_stride <= (0x7fffffff >> 4),
                  "%s: block_table_stride %d out of range", what, block_table_stride);
   const int32_t sub_stride = block_table_stride << shift;  // a row in 16-token pages
@@ -1719,7 +1732,7 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
                            int32_t shared_pages, float softmax_scale, void *stream,
                            int format = kKvFp8) {
   const int shift = page_shift_of(page_size);
-  LITEKV_REQUIRE(shift >= 0, "%s: page_size %d unsupported (16, 32 or 64)", what, page_size);
+  LITEKV_REQUIRE(shift >= 0, "%s: page_size %d unsupported (16, 32, 64, 128 or 256)", what, page_size);
   LITEKV_REQUIRE(block_table_stride >= 1 && block_table_stride <= (0x7fffffff >> 4),
                  "%s: block_table_stride %d out of range", what, block_table_stride);
   const int32_t sub_stride = block_table_stride << shift;  // a block-table row in 16-token pages
@@ -1782,7 +1795,8 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
                    "%s: k_new/v_new strides (%lld, %lld) invalid", what, (long long)k_new_stride,
                    (long long)v_new_stride);
   }
-  const BalancedShape s = balanced_shape(num_kv_heads);
+  const int slices = head_slices(num_q_heads / num_kv_heads);  // wavefronts per kv head and chunk
+  const BalancedShape s = balanced_shape(num_kv_heads * slices);
   LITEKV_REQUIRE(s.head_groups <= 65535, "%s: num_kv_heads %d too large", what, num_kv_heads);
   float *part_o = static_cast<float *>(workspace);
   float *part_lse = part_o + (size_t)(chunks + batch) * num_q_heads * head_dim;
@@ -1812,8 +1826,9 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
                           static_cast<const int32_t *>(plan), static_cast<const half_t *>(k_new),
                           static_cast<const half_t *>(v_new), k_new_stride, v_new_stride,
                           static_cast<half_t *>(out), part_o, part_lse, sub_stride, batch,
-                          num_q_heads, num_kv_heads, num_q_heads / num_kv_heads, s.heads_per_wg,
-                          s.replicas, chunks, shared_pages << shift, softmax_scale * kLog2e);
+                          num_q_heads, num_kv_heads, num_q_heads / num_kv_heads, slices,
+                          s.heads_per_wg, s.replicas, chunks, shared_pages << shift,
+                          softmax_scale * kLog2e);
   };
   if (fp8_scales != nullptr && format == kKvInt8) {
     launch(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, kKvInt8>, static_cast<uint8_t *>(kv_pool));
@@ -2127,7 +2142,11 @@ constexpr int kMaxStaticDevices = 64;
 // device; a race between two first calls stores the same address twice.
 static std::atomic<void *> g_scratch_ptr[kMaxStaticDevices];
 
-static int static_scratch(const char *what, void **ptr_out) {
+// Set while a call is enqueueing its two launches on a device: a second host thread that enters
+// meanwhile would interleave its launches with them on the shared array and is turned away.
+static std::atomic<bool> g_scratch_busy[kMaxStaticDevices];
+
+static int static_scratch(const char *what, hipStream_t stream, void **ptr_out, int *dev_out) {
   int dev = -1;
   hipError_t err = hipGetDevice(&dev);
   if (err != hipSuccess) {
@@ -2135,8 +2154,19 @@ static int static_scratch(const char *what, void **ptr_out) {
   }
   LITEKV_REQUIRE(dev >= 0 && dev < kMaxStaticDevices, "%s: device ordinal %d out of [0, %d)", what,
                  dev, kMaxStaticDevices);
+  *dev_out = dev;
   void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
   if (ptr == nullptr) {
+    // The lookup is not a stream operation: under a capture it would either fail or end the
+    // capture with an error that the next, unrelated call reports.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) == hipSuccess &&
+        capturing != hipStreamCaptureStatusNone) {
+      return fail(LITEKV_ERR_INVALID_ARGUMENT,
+                  "%s: first call on device %d is inside a stream capture; call once with batch 0 "
+                  "before capturing",
+                  what, dev);
+    }
     err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (err != hipSuccess || ptr == nullptr) {
       return fail(LITEKV_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) failed on device %d: %s", what,
@@ -2175,17 +2205,25 @@ extern "C" int litekv_paged_decode_static(const void *q, int64_t q_batch_stride,
                  "%s: batch %d x %d query heads x %d splits needs %zu bytes of partial results, the "
                  "built-in scratch holds %zu; use litekv_paged_decode with a workspace",
                  what, batch, num_q_heads, max_splits, need, (size_t)LITEKV_STATIC_SCRATCH_BYTES);
+  // Every call resolves the array's address on its device, also one with batch 0: that is the
+  // warm-up a caller makes before it starts capturing.
   void *ws = nullptr;
-  if (need > 0) {
-    int rc = litekv::static_scratch(what, &ws);
-    if (rc != LITEKV_OK) return rc;
+  int dev = 0;
+  int rc = litekv::static_scratch(what, static_cast<hipStream_t>(stream), &ws, &dev);
+  if (rc != LITEKV_OK) return rc;
+  if (litekv::g_scratch_busy[dev].exchange(true, std::memory_order_acquire)) {
+    return litekv::fail(LITEKV_ERR_INVALID_ARGUMENT,
+                        "%s: another thread is inside this call on device %d; calls that share the "
+                        "built-in scratch must not overlap",
+                        what, dev);
   }
   litekv::DecodeArgs a{q, q_batch_stride, kv_pool, block_table, block_table_stride, seq_lens, out,
-                       ws, need, batch, num_q_heads, num_kv_heads, head_dim,
+                       need > 0 ? ws : nullptr, need, batch, num_q_heads, num_kv_heads, head_dim,
                        page_size, num_pages, softmax_scale, stream};
-  int rc = litekv::launch_split(a, max_splits, min_pages_per_split);
-  if (rc != LITEKV_OK) return rc;
-  return litekv::launch_merge(a, max_splits, min_pages_per_split);
+  rc = litekv::launch_split(a, max_splits, min_pages_per_split);
+  if (rc == LITEKV_OK) rc = litekv::launch_merge(a, max_splits, min_pages_per_split);
+  litekv::g_scratch_busy[dev].store(false, std::memory_order_release);
+  return rc;
 }
 
 #endif  // LITEKV_HD == 128

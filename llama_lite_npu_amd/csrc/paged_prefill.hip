@@ -27,10 +27,11 @@
 // back as 16-byte rows by 16 lanes of different rows) and V (read back transposed, 8 rows x
 // 32 bytes at a time); both reads are then free of bank conflicts.
 //
-// The softmax scale (times log2 e) is folded into q when it is loaded, and in the fast tiles the
-// score accumulators start from -m (the running maximum of their column) instead of zero, so the
-// MFMA result is already the exponent: a probability costs one v_exp_f32 and half a packed
-// conversion. Whether the running maximum still holds is checked on the packed fp16
+// In the fast tiles the score accumulators start from -m / c (m the running maximum of their
+// column, c the softmax scale times log2 e) instead of zero, so the MFMA result times c is the
+// exponent: a probability costs one multiply, one v_exp_f32 and half a packed conversion. q is not
+// pre-multiplied by c: rounding q * c to fp16 would cost the scores 2^-12 of every channel's
+// share. Whether the running maximum still holds is checked on the packed fp16
 // probabilities (any above 2^8, or not finite, sends the sub-tile to general_tile), not by a
 // column maximum over the fp32 scores.
 //
@@ -175,12 +176,15 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
   const int head0 = ((int)blockIdx.x - h * head_splits) * heads_per_wg;
   const int heads_here = (group - head0) < heads_per_wg ? (group - head0) : heads_per_wg;
   const int b = blockIdx.z;
-  // The softmax scale (times log2 e) is folded into q when it is loaded, so a score leaves the
-  // MFMA in the exponent's unit. An fp8 pool's K scale stays a multiplier of the scores
-  // (k_mul): folded into fp16 q it could push small elements into the subnormal range.
-  float v_scale = 1.0f, k_mul = 1.0f;
+  // q reaches the MFMA as the caller gave it: the products of fp16 q and K elements are exact and
+  // summed in fp32, and the softmax scale (times log2 e, times the K scale of a pool of 8-bit
+  // codes) multiplies the finished score in fp32 (k_mul). Folded into q instead, the product
+  // would be rounded to fp16 once more: an error of 2^-12 of every channel's share of a score,
+  // which rows with a few large channels of q and K (scores tens of log2 units apart) turn into
+  // percent-level errors of their probabilities.
+  float v_scale = 1.0f, k_mul = scale_log2;
   if constexpr (FP8) {
-    k_mul = paged.scales[h];
+    k_mul *= paged.scales[h];
     v_scale = paged.scales[paged.num_kv_heads + h];
   }
   const float k_mul_inv = 1.0f / k_mul;
@@ -243,7 +247,9 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
   // The kernel works on 16-token pages: page j of them is part j % (1 << page_shift) of the
   // sequence's page j >> page_shift, whose tokens are contiguous in the pool.
   auto page_of = [&](int pidx) {
-    int pid = table[pidx >> paged.page_shift];
+    int at = pidx >> paged.page_shift;
+    at = at < paged.bt_stride ? at : paged.bt_stride - 1;  // a length beyond the row re-reads its last entry
+    int pid = table[at];
     pid = pid < 0 ? 0 : (pid >= paged.num_pages ? paged.num_pages - 1 : pid);
     return (pid << paged.page_shift) + (pidx & ((1 << paged.page_shift) - 1));
   };
@@ -380,9 +386,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
     if constexpr (!SHARED) continue;
 #pragma unroll
     for (int kk = 0; kk < kKSteps; ++kk) {
-      const half8_t raw = ok ? *(const half8_t *)(qrow + 32 * kk) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      typedef float float8_t __attribute__((ext_vector_type(8)));
-      qf[u][kk] = __builtin_convertvector(__builtin_convertvector(raw, float8_t) * scale_log2, half8_t);
+      qf[u][kk] = ok ? *(const half8_t *)(qrow + 32 * kk) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
     }
   }
   if constexpr (!SHARED) {
@@ -396,10 +400,8 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
     for (int u = 0; u < kColTiles; ++u) {
 #pragma unroll
       for (int kk = 0; kk < kKSteps; ++kk) {
-        const half8_t raw = *(const lds_half8_t *)(uintptr_t)(
+        qf[u][kk] = *(const lds_half8_t *)(uintptr_t)(
             q_lds + (uint32_t)(32 * kHD) * u + (uint32_t)(n * 2 * kHD + 16 * ((4 * kk + g) ^ k_swz(n))));
-        typedef float float8_t __attribute__((ext_vector_type(8)));
-        qf[u][kk] = __builtin_convertvector(__builtin_convertvector(raw, float8_t) * scale_log2, half8_t);
       }
     }
   }
@@ -492,31 +494,21 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
     for (int m = 0; m < 2; ++m) {
 #pragma unroll
       for (int i = 0; i < 4; i += 2) {
-        float2_t p;
-        if constexpr (FP8) {
-          p = float2_t{fast_exp2(__builtin_fmaf(st[m][u][i], k_mul, neg_m)),
-                       fast_exp2(__builtin_fmaf(st[m][u][i + 1], k_mul, neg_m))};
-        } else {
-          p = float2_t{fast_exp2(st[m][u][i] + neg_m), fast_exp2(st[m][u][i + 1] + neg_m)};
-        }
+        const float2_t p = float2_t{fast_exp2(__builtin_fmaf(st[m][u][i], k_mul, neg_m)),
+                                    fast_exp2(__builtin_fmaf(st[m][u][i + 1], k_mul, neg_m))};
         const half2_t ph = __builtin_convertvector(p, half2_t);
         pk[u][4 * m + i] = ph[0];
         pk[u][4 * m + i + 1] = ph[1];
       }
     }
   };
-  // Fast path: the scores were seeded with -m, so they are the exponents themselves.
+  // Fast path: the scores were seeded with -m / k_mul, so they are the exponents up to that factor.
   auto exponentials_seeded = [&](const float4_t (&st)[2][kColTiles], half8_t (&pk)[kColTiles], int u) {
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
 #pragma unroll
       for (int i = 0; i < 4; i += 2) {
-        float2_t p;
-        if constexpr (FP8) {
-          p = float2_t{fast_exp2(st[m][u][i] * k_mul), fast_exp2(st[m][u][i + 1] * k_mul)};
-        } else {
-          p = float2_t{fast_exp2(st[m][u][i]), fast_exp2(st[m][u][i + 1])};
-        }
+        const float2_t p = float2_t{fast_exp2(st[m][u][i] * k_mul), fast_exp2(st[m][u][i + 1] * k_mul)};
         const half2_t ph = __builtin_convertvector(p, half2_t);
         pk[u][4 * m + i] = ph[0];
         pk[u][4 * m + i + 1] = ph[1];
@@ -888,8 +880,8 @@ static int validate_prefill(const char *what, const void *q, int64_t q_stride, c
                  head_dim);
   LITEKV_REQUIRE(hq > 0 && hkv > 0 && hq % hkv == 0 && hq <= 65535,
                  "%s: num_q_heads %d / num_kv_heads %d invalid", what, hq, hkv);
-  LITEKV_REQUIRE(hq / hkv <= 16, "%s: %d query heads per kv head unsupported (max 16)", what,
-                 hq / hkv);
+  LITEKV_REQUIRE(hq / hkv <= kMaxGroup, "%s: %d query heads per kv head unsupported (max %d)", what,
+                 hq / hkv, kMaxGroup);
   LITEKV_REQUIRE(max_q_len >= 0, "%s: max_q_len %d < 0", what, max_q_len);
   if (batch == 0 || max_q_len == 0) return LITEKV_OK;
   LITEKV_REQUIRE(q && out, "%s: null pointer", what);
@@ -930,7 +922,7 @@ int launch_shared_prefix_hd64(
                          hipStream_t stream, int *splits_out, int format) {
   const char *what = "shared_prefix";
   const int group = num_q_heads / num_kv_heads;
-  LITEKV_REQUIRE(group >= 1 && group <= 16, "%s: %d query heads per kv head unsupported", what, group);
+  LITEKV_REQUIRE(group >= 1 && group <= kMaxGroup, "%s: %d query heads per kv head unsupported", what, group);
   LITEKV_REQUIRE(num_kv_heads <= 1024, "%s: num_kv_heads %d > 1024", what, num_kv_heads);
   LITEKV_REQUIRE(shared_pages >= 1 && shared_pages <= (1 << 24), "%s: shared_pages %d out of range",
                  what, shared_pages);
@@ -947,7 +939,8 @@ int launch_shared_prefix_hd64(
   int keys_per_split = (prefix_keys + splits - 1) / splits;
   keys_per_split = (keys_per_split + kKvTile - 1) / kKvTile * kKvTile;
   splits = (prefix_keys + keys_per_split - 1) / keys_per_split;
-  PagedSource paged{static_cast<const half_t *>(kv_pool), block_table, 0, num_kv_heads,
+  // only the first shared_pages entries of block-table row 0 are read
+  PagedSource paged{static_cast<const half_t *>(kv_pool), block_table, shared_pages, num_kv_heads,
                     (int32_t)num_pages, fp8_scales, page_shift};
   PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
   PrefixTask task{part_o, part_lse, q_batch_stride, batch, num_q_heads, prefix_keys, keys_per_split};
@@ -1021,8 +1014,8 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
   int rc = validate_prefill(what, q, q_token_stride, out, out_token_stride, batch, num_q_heads,
                             num_kv_heads, head_dim, max_q_len);
   if (rc != LITEKV_OK) return rc;
-  const int page_shift = page_size == 16 ? 0 : page_size == 32 ? 1 : page_size == 64 ? 2 : -1;
-  LITEKV_REQUIRE(page_shift >= 0, "%s: page_size %d unsupported (16, 32 or 64)", what, page_size);
+  const int page_shift = page_shift_of(page_size);
+  LITEKV_REQUIRE(page_shift >= 0, "%s: page_size %d unsupported (16, 32, 64, 128 or 256)", what, page_size);
   if (batch == 0 || max_q_len == 0) {
     clear_error();
     return LITEKV_OK;

@@ -33,6 +33,6 @@ class AttentionInfo:
     seq_lens_i32: Optional[torch.Tensor] = None          # b_seq_len as int32
     cu_q_lens: Optional[torch.Tensor] = None             # [B+1] int32 packed-row offsets (prefill)
     context_lens_i32: Optional[torch.Tensor] = None      # chunk_context_len as int32
-    page_size: int = 16                                  # tokens per page of the pools (16, 32 or 64)
+    page_size: int = 16                                  # tokens per page of the pools (16, 32, 64, 128 or 256)
     decode_plan: Any = None                              # ops.DecodePlan of the step (decode only)
     device_decode: Any = None                            # DeviceDecodeBatch that owns the tensors above, if any

@@ -321,7 +321,7 @@ class DecodePlan:
         dev = self.block_table.device
         self.plan_bytes = int(lib.litekv_decode_plan_bytes_paged(self.batch, self.bt_stride, self.num_kv_heads,
                                                                  self.chunks, self.page_size))
-        _need(self.plan_bytes > 0 or self.batch == 0, f"page_size {self.page_size} unsupported (16, 32 or 64)")
+        _need(self.plan_bytes > 0 or self.batch == 0, f"page_size {self.page_size} unsupported (16, 32, 64, 128 or 256)")
         self.buffer = torch.empty(max(4, self.plan_bytes // 4), dtype=torch.int32, device=dev)
         ws_fn = (lib.litekv_paged_decode_prefix_workspace_bytes if self.shared_pages > 0
                  else lib.litekv_paged_decode_balanced_workspace_bytes)

@@ -9,11 +9,15 @@ subnormals at exponent 0, largest finite value 448 (S.1111.110), S.1111.111 = Na
 conversion rounds to nearest even and saturates:
     encode(x, scale) = e4m3(clamp(x * (1 / scale), -448, 448))
     decode(code, scale) = value(code) * scale
+Inputs that are not finite: +-Inf saturate to +-448; the clamp is maxNum(x, -448) then
+minNum(., 448) (IEEE 754-2008: a quiet NaN operand is dropped), so NaN is stored as -448 (0xFE),
+never as one of the format's NaN codes.
 Numeric parity with the reference is **parity unpinned** (nothing to compare with).
 
 Pinned in tests/test_oracle.py by: the closed form of all 256 code values; PyTorch's independent
 float8_e4m3fn conversion on the CPU for every fp16 input in range (both directions); ties going to
-the even code; saturation at +-448; decode(encode(v)) == v for every representable v; monotonicity.
+the even code; saturation at +-448; decode(encode(v)) == v for every representable v; monotonicity;
+the codes of NaN and +-Inf.
 Attention over an fp8 pool is the fp16 oracle applied to the decoded pool (decoding is exact in
 fp16 before the scale; the scale is applied in fp32).
 """
@@ -41,7 +45,8 @@ def code_values() -> np.ndarray:
 def encode(x: np.ndarray) -> np.ndarray:
     """float32 (already divided by the scale) -> uint8 codes: clamp to +-448, round to nearest even."""
     x = np.asarray(x, dtype=np.float32)
-    a = np.minimum(np.abs(x.astype(np.float64)), FP8_MAX)
+    x = np.fmin(np.fmax(x, np.float32(-FP8_MAX)), np.float32(FP8_MAX))   # maxNum / minNum: NaN -> -448
+    a = np.abs(x.astype(np.float64))
     # spacing of the representable numbers around a: 2^(floor(log2 a) - 3), at least 2^-9
     with np.errstate(divide="ignore"):
         exp = np.floor(np.log2(np.where(a > 0, a, 1.0)))
@@ -58,7 +63,6 @@ def encode(x: np.ndarray) -> np.ndarray:
     m_field = np.where(is_sub, np.round(a_q / np.exp2(-9.0)), np.round((a_q / np.exp2(e_q) - 1.0) * 8.0)).astype(np.int64)
     code = (e_field << 3) | m_field
     code = np.where(np.signbit(x), code | 0x80, code)
-    code = np.where(np.isnan(x), 0x7F, code)
     return code.astype(np.uint8)
 
 

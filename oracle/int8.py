@@ -6,11 +6,15 @@ reads int8 K/V as they are, without scales, and has no quantising append to foll
 states the scheme in closed form -- the one the fp8 pools use, with integer codes:
     encode(x, scale) = clamp(round_half_to_even(x * (1 / scale)), -127, 127)      (x * (1/scale) in fp32)
     decode(code, scale) = code * scale
+Inputs that are not finite: +-Inf saturate like any large value; the clamp is maxNum(x, -127) then
+minNum(., 127) (IEEE 754-2008: a quiet NaN operand is dropped), so NaN is stored as -127. An int8
+pool cannot hold a NaN; the rule only makes what is stored a function of the input.
 Numeric parity with the reference is **parity unpinned** (nothing to compare with).
 
 Pinned in tests/test_oracle.py by: halves going to the even integer, saturation at +-127 (-128 is
 never produced), decode(encode(v)) == v for every integer in range, monotonicity, PyTorch's
-independent round + clamp on every fp16 input in range, and hand-computed examples with scales.
+independent round + clamp on every fp16 input in range, hand-computed examples with scales, and
+the codes of NaN and +-Inf.
 Attention over an int8 pool is the fp16 oracle applied to the decoded pool (codes are exact in
 fp16; the scale is applied in fp32).
 """
@@ -26,7 +30,7 @@ def encode(x: np.ndarray) -> np.ndarray:
     """float32 (already divided by the scale) -> int8 codes: round half to even, clamp to +-127."""
     x = np.asarray(x, dtype=np.float32)
     r = np.rint(x)                                   # numpy rounds halves to even
-    r = np.minimum(np.maximum(r, -INT8_MAX), INT8_MAX)
+    r = np.fmin(np.fmax(r, -INT8_MAX), INT8_MAX)     # maxNum / minNum: NaN -> -127, +-Inf -> +-127
     return r.astype(np.int8)
 
 

@@ -125,3 +125,35 @@ def test_static_batch_prefill_then_decode_select_indices():
     else:
         raise AssertionError("allocation beyond the pool did not fail")
     assert small.kv_mem_manager.num_free_pages == 2
+
+
+def test_static_batch_decode_steps_never_attend_a_padding_row():
+    """After the padded static-batch prefill every decode step writes request r's token at
+    slots(r)[tokens so far] (the first one over the first padding row) and attends exactly the
+    prompt's own tokens plus the tokens decoded so far: the slots a step can reach never include
+    a padding row that has not been overwritten. The reference's paged branch counts the padded
+    length instead (model_executor.py:450-455); this pins the behaviour chosen here."""
+    page = 4
+    lens = [3, 7, 1, 5]
+    longest = 7
+    executor = ModelExecutor(num_layers=1, num_q_heads=2, num_kv_heads=1, head_dim=8, num_pages=16,
+                             max_seq_len=16, max_requests=4, page_size=page, device="cpu")
+    select, _ = executor.prefill_alloc_kv_cache(longest, torch.tensor(lens), torch.arange(4, dtype=torch.int32))
+    mgr = executor.req_tokens_manager
+    rows = select.reshape(4, longest)
+    written = [set(rows[r, :lens[r]].tolist()) for r in range(4)]           # slots holding real tokens
+    padding = [set(rows[r, lens[r]:].tolist()) for r in range(4)]
+    info = executor.atten_info
+    for step in range(1, 6):
+        slots = executor.decode_alloc_kv_cache(4).tolist()
+        for r in range(4):
+            have = lens[r] + step
+            assert slots[r] == mgr.slots(r, 0, have)[have - 1]                # right behind what the request holds
+            assert int(info.b_seq_len[r]) == have
+            written[r].add(slots[r])
+            padding[r].discard(slots[r])
+            # what a kernel reaches: the first `have` tokens of the step's block-table row
+            pages = info.block_table[r].tolist()
+            attended = {pages[t // page] * page + t % page for t in range(int(info.seq_lens_i32[r]))}
+            assert attended == written[r], (r, step)
+            assert not (attended & padding[r])

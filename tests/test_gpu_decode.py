@@ -316,10 +316,11 @@ def test_shared_prefix_fused_append_and_empty_rows():
     assert float(out[2].abs().max()) == 0.0
 
 
-# ---- pools with pages of 32 and 64 tokens (the reference's --page_size, server.py:1038-1161) ----
+# ---- pools with pages of 32 to 256 tokens (the reference's --page_size, server.py:1038-1161;
+# "typically 16-256", executor/paged_attention.py:27) ----
 
-PAGE_SIZES = [32, 64]
-EDGE_CONTEXTS = [0, 1, 15, 16, 17, 31, 32, 33, 47, 48, 63, 64, 65, 127, 128, 255, 700, 1200]
+PAGE_SIZES = [32, 64, 128, 256]
+EDGE_CONTEXTS = [0, 1, 15, 16, 17, 31, 32, 33, 47, 48, 63, 64, 65, 127, 128, 129, 255, 256, 257, 700, 1200]
 
 
 @pytest.mark.parametrize("page_size", PAGE_SIZES)
@@ -501,3 +502,99 @@ def test_head_dim_64_long_shared_prefix(page_size, shared_tokens):
     partly = _run(case, schedule="balanced", shared_pages=shared_pages // 2)
     assert_attention_close(partly, ref, "half the shared prefix declared, head_dim 64")
     assert torch.equal(out, _run(case, schedule="balanced", shared_pages=shared_pages))
+
+
+# ---- more than 16 query heads per kv head (the reference's grid is per query head,
+# flashdecoding.py:44, 170-175: no bound on the group) ----
+
+@pytest.mark.parametrize("head_dim", [128, 64, 32])
+@pytest.mark.parametrize("hq,hkv", [(32, 1), (64, 2), (96, 4), (20, 1), (51, 3)])
+def test_more_than_16_query_heads_per_kv_head(head_dim, hq, hkv):
+    """Groups of 17 to 32 query heads run as two slices of their kv head (up to 16 columns each):
+    both schedules, the fused append (written once per slice, the same bits), a shared prefix."""
+    print(f"decode {hq}/{hkv} heads, head_dim {head_dim}", flush=True)
+    lens = [0, 1, 15, 16, 17, 255, 256, 700, 40]
+    case = workloads.make_decode_case("wide-group", 1700 + hq + head_dim, lens, hq, hkv, device=DEV,
+                                      head_dim=head_dim)
+    seq = case.seq_lens.clone()
+    seq[8] = 0
+    pool_ref = case.kv_pool.clone()
+    ops.kv_append(case.k_new, case.v_new, case.slot_mapping, pool_ref)
+    ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool_ref), case.block_table.cpu().numpy(),
+                                seq.cpu().numpy(), case.softmax_scale)
+    keep = torch.ones(case.kv_pool.shape[0], dtype=torch.bool, device=DEV)
+    keep[case.slot_mapping[8].long()] = False           # the empty sequence appends nothing
+    for kw in ({"num_splits": 1}, {"num_splits": 3}, {"max_splits": 16, "min_pages_per_split": 2},
+               {"schedule": "balanced"}, {"schedule": "balanced", "chunks": 5}):
+        out = ops.paged_decode(case.q, pool_ref, case.block_table, seq, case.softmax_scale, **kw)
+        torch.cuda.synchronize()
+        assert_attention_close(out, ref, f"{hq}/{hkv} d={head_dim} {kw}")
+        assert float(out[8].abs().max()) == 0.0
+    for chunks in (None, 3):
+        pool = case.kv_pool.clone()
+        plan = ops.DecodePlan(case.block_table, seq, hq, hkv, case.num_pages, chunks)
+        out = ops.decode_step(case.q, pool, plan, case.k_new, case.v_new, case.softmax_scale)
+        torch.cuda.synchronize()
+        assert torch.equal(pool[keep].view(torch.int16), pool_ref[keep].view(torch.int16))
+        assert_attention_close(out, ref, f"{hq}/{hkv} d={head_dim} fused step chunks={chunks}")
+    pool = case.kv_pool.clone()
+    out = ops.paged_decode(case.q, pool, case.block_table, seq, case.softmax_scale, num_splits=1,
+                           k_new=case.k_new, v_new=case.v_new)
+    torch.cuda.synchronize()
+    assert torch.equal(pool[keep].view(torch.int16), pool_ref[keep].view(torch.int16))
+    assert_attention_close(out, ref, f"{hq}/{hkv} d={head_dim} per-sequence fused step")
+
+
+@pytest.mark.parametrize("head_dim", [128, 64])
+def test_more_than_16_query_heads_per_kv_head_behind_a_shared_prefix(head_dim):
+    print(f"decode 64/2 heads behind a shared prefix, head_dim {head_dim}", flush=True)
+    shared_pages, suffix = 13, [0, 5, 15, 16, 40, 300]
+    ctx = [shared_pages * 16 + s for s in suffix]
+    priv = [(c + 1 + 15) // 16 - shared_pages for c in ctx]
+    num_pages = shared_pages + sum(priv) + 7
+    perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(head_dim + 3)).to(torch.int32)
+    shared, cur, lists = perm[:shared_pages], shared_pages, []
+    for n in priv:
+        lists.append(torch.cat([shared, perm[cur:cur + n]]))
+        cur += n
+    case = workloads.make_decode_case("wide-shared", 1760 + head_dim, ctx, 64, 2, num_pages=num_pages, device=DEV,
+                                      page_lists=lists, head_dim=head_dim)
+    ref = _oracle(case)
+    for chunks in (None, 5):
+        out = _run(case, schedule="balanced", chunks=chunks, shared_pages=shared_pages)
+        assert_attention_close(out, ref, f"64/2 shared prefix d={head_dim} chunks={chunks}")
+
+
+# ---- a length beyond what the block table can name (lengths live on the device: no host check) ----
+
+@pytest.mark.parametrize("head_dim", [128, 32])
+def test_length_beyond_the_block_table_row_touches_no_other_page(head_dim):
+    """Sequence 1 claims 100 tokens against a table whose rows name 4 pages (64 tokens): the
+    kernels re-read the row's last entry instead of reading past the row, and the fused append
+    writes nothing for it; the other sequences are attended and appended as usual."""
+    print(f"decode length beyond the table, head_dim {head_dim}", flush=True)
+    hq, hkv = 16, 4
+    case = workloads.make_decode_case("beyond", 1790 + head_dim, [39, 63, 63, 20], hq, hkv, device=DEV,
+                                      head_dim=head_dim)
+    assert case.block_table.shape[1] == 4
+    seq = case.seq_lens.clone()
+    seq[1] = 100
+    good = [0, 2, 3]
+    pool_ref = case.kv_pool.clone()
+    ops.kv_append(case.k_new[good], case.v_new[good], case.slot_mapping[good], pool_ref)
+    ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool_ref), case.block_table.cpu().numpy(),
+                                case.seq_lens.cpu().numpy(), case.softmax_scale)
+    for kw in ({"num_splits": 1}, {"num_splits": 3}):
+        pool = case.kv_pool.clone()
+        out = ops.paged_decode(case.q, pool, case.block_table, seq, case.softmax_scale, k_new=case.k_new,
+                               v_new=case.v_new, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(pool.view(torch.int16), pool_ref.view(torch.int16)), f"pool changed elsewhere {kw}"
+        assert_attention_close(out[good], ref[good], f"length beyond the table {kw}")
+        assert bool(torch.isfinite(out).all())
+    pool = case.kv_pool.clone()
+    plan = ops.DecodePlan(case.block_table, seq, hq, hkv, case.num_pages, 3)
+    out = ops.decode_step(case.q, pool, plan, case.k_new, case.v_new, case.softmax_scale)
+    torch.cuda.synchronize()
+    assert torch.equal(pool.view(torch.int16), pool_ref.view(torch.int16)), "pool changed elsewhere (balanced)"
+    assert_attention_close(out[good], ref[good], "length beyond the table, balanced")

@@ -406,3 +406,50 @@ def test_quantised_chunk_prefill_at_head_dim_64_many_tiles(dtype, page_size):
         ref = cpu_ref.paged_prefill_ref(pre.q.cpu(), values, pre.block_table.cpu(), pre.cu_q_lens.cpu(),
                                         pre.context_lens.cpu(), scale, page_size=page_size).numpy()
         assert_attention_close(out, ref, f"head_dim 64 {dtype} chunk prefill over {ctx}")
+
+
+@pytest.mark.parametrize("dtype", [torch.int8, torch.uint8])
+def test_codes_of_rows_that_are_not_finite(dtype):
+    """NaN and +-Inf elements of a row: +-Inf saturate, NaN is stored as the most negative code
+    (the clamp drops a NaN operand), by the append kernel and by the appends fused into decode;
+    no other element's code changes."""
+    from oracle import fp8
+    codec = int8 if dtype == torch.int8 else fp8
+    print(f"codes of non-finite inputs, pool dtype {dtype}", flush=True)
+    hq, hkv = 8, 2
+    case = workloads.make_decode_case("nonfinite", 88, [20, 47, 15], hq, hkv, device=DEV)
+    for row in (case.k_new, case.v_new):
+        row[0, 0, 3], row[0, 1, 64], row[1, 0, 127] = float("nan"), float("inf"), float("-inf")
+        row[2, 1, 0] = float("nan")
+    scales = _head_scales(hkv) if dtype == torch.int8 else _head_scales(hkv, 0.02, 0.015)
+    pool0 = torch.zeros(case.kv_pool.shape, dtype=dtype, device=DEV)
+    every_slot = torch.arange(pool0.shape[0], dtype=torch.int32, device=DEV)
+    ops.kv_append_quantised(case.kv_pool[:, :hkv], case.kv_pool[:, hkv:], every_slot, pool0, scales)
+    want = pool0.cpu().numpy().copy()
+    codec.kv_append(case.k_new.cpu().numpy(), case.v_new.cpu().numpy(), case.slot_mapping.cpu().numpy(), want,
+                    scales.cpu().numpy())
+    lowest, highest = (-127, 127) if dtype == torch.int8 else (0xFE, 0x7E)
+    slot0 = int(case.slot_mapping[0])
+    assert want[slot0, 0, 3] == lowest and want[slot0, 1, 64] == highest
+    pool = pool0.clone()
+    ops.kv_append_quantised(case.k_new, case.v_new, case.slot_mapping, pool, scales)
+    torch.cuda.synchronize()
+
+    def same_codes(got):
+        got = got.cpu().numpy()
+        if dtype == torch.int8:
+            return np.array_equal(got, want)
+        return bool((((got == want) | (((got & 0x7F) == 0) & ((want & 0x7F) == 0)))).all())   # zero's sign is free
+
+    assert same_codes(pool), "append kernel"
+    for chunks in (None, 2):
+        fused = pool0.clone()
+        plan = ops.DecodePlan(case.block_table, case.seq_lens, hq, hkv, case.num_pages, chunks)
+        ops.decode_step(case.q, fused, plan, case.k_new, case.v_new, SCALE, kv_scales=scales)
+        torch.cuda.synchronize()
+        assert same_codes(fused), f"append fused into the balanced step, chunks={chunks}"
+    fused = pool0.clone()
+    ops.paged_decode(case.q, fused, case.block_table, case.seq_lens, SCALE, kv_scales=scales, num_splits=1,
+                     k_new=case.k_new, v_new=case.v_new)
+    torch.cuda.synchronize()
+    assert same_codes(fused), "append fused into the per-sequence step"

@@ -157,15 +157,15 @@ def test_prefill_repeats_bit_for_bit():
         assert torch.equal(outs[0], o)
 
 
-@pytest.mark.parametrize("page_size", [32, 64])
+@pytest.mark.parametrize("page_size", [32, 64, 128, 256])
 @pytest.mark.parametrize("hq,hkv,lens,ctx", [
-    (16, 8, [1, 2, 15, 16, 17, 33, 47, 48, 63, 64, 65], None),
+    (16, 8, [1, 2, 15, 16, 17, 33, 47, 48, 63, 64, 65, 127, 128, 129, 255, 256, 257], None),
     (64, 8, [128, 77, 200], None),
     (32, 4, [300, 5, 96], [100, 31, 64]),       # chunks over cached history
     (16, 1, [130, 40], [17, 700]),
 ])
 def test_paged_prefill_page_sizes(page_size, hq, hkv, lens, ctx):
-    """Pools with pages of 32 and 64 tokens (the reference's --page_size): prompts and chunks over
+    """Pools with pages of 32 to 256 tokens (the reference's --page_size): prompts and chunks over
     history whose ends fall on every kind of boundary inside and between pages."""
     print(f"prefill page_size {page_size} {hq}/{hkv} {lens} ctx {ctx}", flush=True)
     case = workloads.make_prefill_case("pp", 900 + page_size + hq, lens, hq, hkv, context_lens=ctx, device=DEV,
@@ -229,3 +229,44 @@ def test_prefill_head_dim_64_on_the_tiled_kernel(hq, hkv, lens, ctx, page_size):
                                   case.softmax_scale)
         torch.cuda.synchronize()
         assert torch.equal(outs[0], out2)
+
+
+@pytest.mark.parametrize("head_dim", [128, 64])
+@pytest.mark.parametrize("hq,hkv,lens,ctx", [
+    (32, 1, [130, 40], None),                  # 32 heads per kv head: four workgroups per kv head
+    (96, 4, [70, 200], None),                  # 24
+    (40, 2, [260, 31], [100, 700]),            # 20, chunks over history
+])
+def test_prefill_more_than_16_query_heads_per_kv_head(head_dim, hq, hkv, lens, ctx):
+    """The reference's grid is per query head (flashattention2_nopad.py:195): no bound on the group."""
+    print(f"prefill {hq}/{hkv} heads d={head_dim} {lens} ctx {ctx}", flush=True)
+    case = workloads.make_prefill_case("wg", 1300 + hq + head_dim, lens, hq, hkv, context_lens=ctx, device=DEV,
+                                       head_dim=head_dim)
+    _append(case)
+    out = ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens,
+                            case.context_lens if ctx is not None else None, case.max_q_len, case.softmax_scale)
+    torch.cuda.synchronize()
+    assert_attention_close(out, _oracle_paged(case), f"prefill {hq}/{hkv}")
+    if ctx is None:
+        out2 = ops.varlen_prefill(case.q, case.k, case.v, case.cu_q_lens[:-1], case.seq_lens, case.max_q_len,
+                                  case.softmax_scale)
+        torch.cuda.synchronize()
+        assert torch.equal(out, out2)
+
+
+def test_prefill_length_beyond_the_block_table_row():
+    """A chunk whose history claims more tokens than its block-table row names: the row's last
+    entry is re-read instead of the memory behind the row; the other sequences are unaffected."""
+    print("prefill length beyond the table", flush=True)
+    case = workloads.make_prefill_case("pb", 1390, [20, 30, 17], 16, 4, context_lens=[40, 30, 0], device=DEV)
+    _append(case)
+    ref = _oracle_paged(case)
+    ctx = case.context_lens.clone()
+    ctx[1] = 500                                # the table has 4 entries per row
+    assert case.block_table.shape[1] == 4
+    out = ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, ctx, case.max_q_len,
+                            case.softmax_scale)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    rows = torch.cat([torch.arange(0, 20), torch.arange(50, 67)])
+    assert_attention_close(out[rows.to(DEV)], ref[rows.numpy()], "rows of the other sequences")

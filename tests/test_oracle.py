@@ -485,6 +485,30 @@ def test_int8_rounding_saturation_and_round_trip():
     assert np.all(np.diff(int8.decode(int8.encode(np.sort(x)))) >= 0)           # monotone
 
 
+def test_codes_of_inputs_that_are_not_finite():
+    """+-Inf saturate; NaN is dropped by the clamp's maxNum (IEEE 754-2008) and stored as the most
+    negative code. Stated independently of the oracle's own expression: through torch.fmax / fmin,
+    which implement maxNum / minNum, and as literal codes."""
+    import torch
+    from oracle import fp8, int8
+
+    x = np.array([np.nan, -np.nan, np.inf, -np.inf, 1.0], dtype=np.float32)
+    assert int8.encode(x).tolist() == [-127, -127, 127, -127, 1]
+    assert fp8.encode(x).tolist() == [0xFE, 0xFE, 0x7E, 0xFE, 0x38]
+    t = torch.from_numpy(x)
+    clamped = torch.fmin(torch.fmax(t, torch.tensor(-127.0)), torch.tensor(127.0))
+    assert clamped.tolist() == [-127.0, -127.0, 127.0, -127.0, 1.0]
+    # through the append: a NaN / Inf element of a row changes no other element's code
+    k = np.ones((1, 1, 128), dtype=np.float16)
+    k[0, 0, 5], k[0, 0, 9], k[0, 0, 11] = np.nan, np.inf, -np.inf
+    for codec, dtype, lowest, highest, one in ((int8, np.int8, -127, 127, 2), (fp8, np.uint8, 0xFE, 0x7E, 0x40)):
+        pool = np.zeros((1, 2, 128), dtype=dtype)
+        codec.kv_append(k, k, np.array([0]), pool, np.array([0.5, 0.5], dtype=np.float32))
+        row = pool[0, 0].tolist()
+        assert (row[5], row[9], row[11]) == (lowest, highest, lowest)
+        assert all(c == one for i, c in enumerate(row) if i not in (5, 9, 11))
+
+
 def test_int8_encode_against_torch_round_and_clamp():
     """An independent statement of the same rule: torch.round (half to even) then clamp, on every fp16
     input of moderate size divided by a scale in fp32."""

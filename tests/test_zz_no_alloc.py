@@ -68,3 +68,65 @@ def test_static_scratch_limit_is_enforced():
     ref_out = ops.paged_decode(case.q, case.kv_pool, bt, sl, case.softmax_scale, max_splits=too_many - 1,
                                min_pages_per_split=1)
     assert_bit_exact(out, ref_out, "static vs workspace at the limit")
+
+
+_CAPTURE_SCRIPT = r"""
+import sys
+import torch
+sys.path.insert(0, sys.argv[1])
+from llama_lite_npu_amd import _lib, ops, workloads
+
+dev = "cuda:0"
+case = workloads.make_decode_case("static-capture", 7201, [300, 17, 64, 900], 16, 8, device=dev)
+bt = case.block_table.to(torch.int32).contiguous()
+sl = case.seq_lens.to(torch.int32).contiguous()
+want = ops.paged_decode(case.q, case.kv_pool, bt, sl, case.softmax_scale, max_splits=3, min_pages_per_split=2)
+out = torch.zeros_like(want)
+torch.cuda.synchronize()
+
+# the very first call of this process on the device, inside a capture: refused, capture intact
+g = torch.cuda.CUDAGraph()
+refused = ""
+with torch.cuda.graph(g):
+    out.add_(0)
+    try:
+        ops.paged_decode_static(case.q, case.kv_pool, bt, sl, out, 3, 2, case.softmax_scale)
+    except _lib.LiteKVError as e:
+        refused = str(e)
+assert "capture" in refused, refused
+g.replay()
+torch.cuda.synchronize()
+assert float(out.abs().max()) == 0.0
+print("refused:", refused, flush=True)
+
+# the warm-up call (batch 0) resolves the array's address; then the same capture holds the step
+empty = torch.empty((0,) + tuple(case.q.shape[1:]), dtype=torch.float16, device=dev)
+ops.paged_decode_static(empty, case.kv_pool, bt[:0], sl[:0], empty.clone(), 3, 2, case.softmax_scale)
+g2 = torch.cuda.CUDAGraph()
+with torch.cuda.graph(g2):
+    ops.paged_decode_static(case.q, case.kv_pool, bt, sl, out, 3, 2, case.softmax_scale)
+for replay in range(3):
+    out.fill_(float("nan"))
+    torch.cuda.synchronize()
+    g2.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want), f"replay {replay} differs"
+print("captured after warm-up: ok", flush=True)
+"""
+
+
+def test_first_static_call_inside_a_capture_is_refused_and_a_warm_up_call_enables_it():
+    """The array's address is looked up on the first call on a device, which a stream capture
+    cannot hold: such a call is refused with a message, and a call with batch 0 beforehand makes
+    the entry point capturable. Needs a process that has not called the entry point yet."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    print("static decode: first call under capture (own process)", flush=True)
+    root = str(Path(__file__).resolve().parents[1])
+    proc = subprocess.run([sys.executable, "-u", "-c", _CAPTURE_SCRIPT, root], capture_output=True, text=True,
+                          timeout=300)
+    print(proc.stdout, proc.stderr[-2000:], flush=True)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "captured after warm-up: ok" in proc.stdout
