@@ -68,6 +68,11 @@
 #ifndef LITEKV_HD
 #define LITEKV_HD 128
 #endif
+// Wavefronts per workgroup of the fp16 prefill launches: 4, or 8 (twice the query rows on every
+// staged K/V tile, one workgroup per compute unit instead of two).
+#ifndef LITEKV_PREFILL_WAVES
+#define LITEKV_PREFILL_WAVES 4
+#endif
 #if LITEKV_HD == 128
 #define LITEKV_HD_NS hd128
 #elif LITEKV_HD == 64
@@ -125,7 +130,8 @@ struct PackedSource {
 
 constexpr int kKvTile = 64;
 constexpr int kColTiles = 2;      // 16-column tiles per wavefront
-constexpr int kTiledWaves = 4;
+constexpr int kTiledWaves = 4;    // wavefronts of a workgroup, unless the kernel is built for kWideWaves
+constexpr int kWideWaves = 8;     // fp16 prefill only: twice the columns on every staged K/V tile
 constexpr int kWgColTiles = kColTiles * kTiledWaves;
 constexpr int kTileHalfs = kKvTile * kHD;  // one staged tile: 64 rows of 2 * kHD bytes
 
@@ -145,8 +151,8 @@ __device__ __forceinline__ float vmax2(float a, float b) { return __builtin_fmax
 constexpr int kPagedPrefill = 0, kPackedPrefill = 1, kSharedPrefix = 2, kPagedPrefillFp8 = 3,
               kSharedPrefixFp8 = 4, kPagedPrefillInt8 = 5, kSharedPrefixInt8 = 6;
 
-template <int MODE>
-__global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_prefill_tiled_kernel(
+template <int MODE, int W = kTiledWaves>
+__global__ __launch_bounds__(W *kWave, W == kWideWaves ? 1 : (kHD == 64 ? 3 : 2)) void varlen_prefill_tiled_kernel(
     const half_t *__restrict__ q, int64_t q_stride, half_t *__restrict__ out, int64_t out_stride,
     PagedSource paged, PackedSource packed, PrefixTask prefix,
     const int32_t *__restrict__ q_starts_or_cu, const int32_t *__restrict__ q_lens_or_null,
@@ -161,11 +167,18 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
                        MODE == kPagedPrefillInt8 || MODE == kSharedPrefixInt8;  // 8-bit codes
   constexpr int KV = (MODE == kPagedPrefillInt8 || MODE == kSharedPrefixInt8) ? kKvInt8 : kKvFp8;
   constexpr bool SHARED = MODE == kSharedPrefix || MODE == kSharedPrefixFp8 || MODE == kSharedPrefixInt8;
-  // Two tiles of K and two of V: tile t sits in half t % 2.
-  __shared__ __attribute__((aligned(1024))) half_t kbuf[2 * kTileHalfs];
-  __shared__ __attribute__((aligned(1024))) half_t vbuf[2 * kTileHalfs];
-  const uint32_t k_lds = (uint32_t)(uintptr_t)(lds_half_t *)kbuf;  // LDS byte addresses
-  const uint32_t v_lds = (uint32_t)(uintptr_t)(lds_half_t *)vbuf;
+  static_assert(W == kTiledWaves || (W == kWideWaves && !FP8 && !SHARED),
+                "eight wavefronts: fp16 prefill only");
+  // Rows of a 64-key tile one wavefront stages (a page, or half of one), and the direct-load
+  // instructions that takes per operand.
+  constexpr int kRowsPerWave = kKvTile / W;
+  constexpr int kLoads = kRowsPerWave / kRowsPerLoad;
+  // Two tiles of K, then two of V: tile t sits in half t % 2. Eight wavefronts have a third
+  // region of the same size behind them: q of wavefronts 4..7, and room for the output rows.
+  __shared__ __attribute__((aligned(1024))) half_t lds_all[(W == kWideWaves ? 6 : 4) * kTileHalfs];
+  const uint32_t k_lds = (uint32_t)(uintptr_t)(lds_half_t *)lds_all;  // LDS byte addresses
+  const uint32_t v_lds = k_lds + 4u * kTileHalfs;
+  const uint32_t x_lds = v_lds + 4u * kTileHalfs;
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -224,21 +237,24 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
   const int n_tiles = (kv_end + kKvTile - 1) / kKvTile - tile0;
 
   // ---- staging addresses -------------------------------------------------------------------
-  // Direct-load instruction i of wavefront w fills tile rows 16w + 4i .. +3 (one page per
-  // wavefront): lane l writes slot l % 16 of row 4i + l / 16.
+  // Direct-load instruction i of wavefront w fills tile rows kRowsPerWave * w + 4i .. +3 (one
+  // page per wavefront, or half of one): lane l writes slot l % 16 of row 4i + l / 16.
   const int r_loc = lane / kChunks;
   const int slot = lane % kChunks;
+  const int sub = (kRowsPerWave * wave) & 15;   // first row of this wavefront's rows inside their page
   const uint32_t k_pitch = PAGED ? 2u * paged.num_kv_heads * kHD * (FP8 ? 1u : 2u)
                                  : (uint32_t)packed.k_stride * 2u;
   const uint32_t v_pitch = PAGED ? k_pitch : (uint32_t)packed.v_stride * 2u;
-  uint32_t koff[kLoadsPerWave], voff[kLoadsPerWave];  // byte offsets from the wavefront's 16-row base
+  // byte offsets from the page (paged) or from the wavefront's first row (packed)
+  uint32_t koff[kLoadsPerWave], voff[kLoadsPerWave];
 #pragma unroll
-  for (int i = 0; i < kLoadsPerWave; ++i) {
-    const int rip = kRowsPerLoad * i + r_loc;
-    const int ck = slot ^ k_swz(rip);
-    const int cv = slot ^ v_swz(rip);
-    koff[i] = rip * k_pitch + (uint32_t)(h * kHD + 8 * ck) * 2u;
-    voff[i] = rip * v_pitch +
+  for (int i = 0; i < kLoads; ++i) {
+    const int rip = kRowsPerLoad * i + r_loc;   // row among this wavefront's rows
+    const int ck = slot ^ k_swz(sub + rip);      // the swizzle goes by the row of the tile
+    const int cv = slot ^ v_swz(sub + rip);
+    const int src_row = (PAGED ? sub : 0) + rip;
+    koff[i] = src_row * k_pitch + (uint32_t)(h * kHD + 8 * ck) * 2u;
+    voff[i] = src_row * v_pitch +
               (uint32_t)(((PAGED ? paged.num_kv_heads : 0) + h) * kHD + 8 * cv) * 2u;
   }
   const int32_t *table =
@@ -260,7 +276,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
   constexpr int kRawVecs = kHD / 64;    // 8-bit pools: 16-byte vectors of codes per lane and operand
   uint4_t raw_k[kRawVecs], raw_v[kRawVecs];  // this lane's codes of K and of V of the tile requested last
   auto issue_tile = [&](int kt) {
-    const int row0 = (tile0 + kt) * kKvTile + 16 * wave;  // first key of this wavefront's 16 rows
+    const int row0 = (tile0 + kt) * kKvTile + kRowsPerWave * wave;  // first key of this wavefront's rows
     if constexpr (FP8) {
       // lane l: row l / 4 of the wavefront's page, a quarter of the head's row (kHD / 4 codes)
       int pidx = (tile0 + kt) * 4 + wave;
@@ -283,7 +299,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
     const char *kbase, *vbase;
     int src0;  // key index the bases point at
     if (PAGED) {
-      int pidx = (tile0 + kt) * 4 + wave;
+      int pidx = (tile0 + kt) * 4 + (kRowsPerWave * wave) / 16;
       pidx = pidx < last_page ? pidx : last_page;
       const int pid = page_of(pidx);
       kbase = (const char *)paged.kv + (int64_t)pid * ((int64_t)kPageSize * k_pitch);
@@ -295,7 +311,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
       vbase = (const char *)packed.v + (int64_t)(q_start + first) * v_pitch;
       src0 = first;
     }
-    const uint32_t dst = (uint32_t)((kt & 1) * kTileHalfs + 16 * wave * kHD) * 2u;
+    const uint32_t dst = (uint32_t)((kt & 1) * kTileHalfs + kRowsPerWave * wave * kHD) * 2u;
     auto load_rows = [&](uint32_t i, uint32_t ko, uint32_t vo) {
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                    :
@@ -306,19 +322,20 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
                    : "s"(v_lds + dst + 1024u * i), "v"(vo), "s"(vbase)
                    : "memory", "m0");
     };
-    if (row0 + 15 <= last_key) {
+    if (row0 + kRowsPerWave - 1 <= last_key) {
 #pragma unroll
-      for (int i = 0; i < kLoadsPerWave; ++i) load_rows(i, koff[i], voff[i]);
+      for (int i = 0; i < kLoads; ++i) load_rows(i, koff[i], voff[i]);
     } else {
       // Only in the last tile of a sequence. Rows past the last key re-read it: finite values
       // that zero probabilities multiply.
+      const int off0 = PAGED ? row0 - sub : row0;  // the key the offsets count from
 #pragma unroll
-      for (int i = 0; i < kLoadsPerWave; ++i) {
+      for (int i = 0; i < kLoads; ++i) {
         const int rip = kRowsPerLoad * i + r_loc;
         int tok = row0 + rip;
         tok = tok < last_key ? tok : last_key;
-        const uint32_t back = (uint32_t)(row0 + rip - tok) - (uint32_t)(row0 - src0);
-        // source row = rip - back: inside the page / at the clamped packed row
+        const uint32_t back = (uint32_t)(row0 + rip - tok) - (uint32_t)(off0 - src0);
+        // source row = offset row - back: inside the page / at the clamped packed row
         load_rows(i, koff[i] - back * k_pitch, voff[i] - back * v_pitch);
       }
     }
@@ -329,7 +346,8 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
   // the fragments are read back from there. Requested before tile 0: vmcnt counts in order.
   uint32_t q_lds = 0;
   if constexpr (!SHARED) {
-    q_lds = ((wave & 2) ? v_lds : k_lds) + (uint32_t)(kTileHalfs * 2 + (wave & 1) * (64 * kHD));
+    q_lds = wave < 4 ? ((wave & 2) ? v_lds : k_lds) + (uint32_t)(kTileHalfs * 2 + (wave & 1) * (64 * kHD))
+                     : x_lds + (uint32_t)((wave - 4) * (64 * kHD));
 #pragma unroll
     for (int u = 0; u < kColTiles; ++u) {
       const int t = wave * kColTiles + u;
@@ -394,7 +412,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
     if constexpr (FP8) {
       __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kRawVecs));
     } else {
-      __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kLoadsPerWave));
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kLoads));
     }
 #pragma unroll
     for (int u = 0; u < kColTiles; ++u) {
@@ -600,16 +618,16 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
   };
   int ids_ahead = 0;  // of the tile after the one being staged
   auto tile_bases = [&](int kt) {
-    const int row0 = (tile0 + kt) * kKvTile + 16 * wave;
+    const int row0 = (tile0 + kt) * kKvTile + kRowsPerWave * wave;
     if (PAGED) {
-      const int pid = __builtin_amdgcn_readlane(ids_ahead, wave);
+      const int pid = __builtin_amdgcn_readlane(ids_ahead, (kRowsPerWave * wave) / 16);
       next_kbase = (const char *)paged.kv + (int64_t)pid * ((int64_t)kPageSize * k_pitch);
       next_vbase = next_kbase;
     } else {
       next_kbase = (const char *)packed.k + (int64_t)(q_start + row0) * k_pitch;
       next_vbase = (const char *)packed.v + (int64_t)(q_start + row0) * v_pitch;
     }
-    next_dst = (uint32_t)((kt & 1) * kTileHalfs + 16 * wave * kHD) * 2u;
+    next_dst = (uint32_t)((kt & 1) * kTileHalfs + kRowsPerWave * wave * kHD) * 2u;
   };
   auto issue_rows = [&](int i) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -682,6 +700,7 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
   // exponentials and second products, so that in each basic block MFMAs of one half can run
   // beside the vector ALU work of the other. Returns like fast_tiles (a grown tile is redone
   // from its first half).
+  constexpr int kIssueEvery = kJTiles / kLoads;  // MFMA pairs between two row groups of the next tile
   auto fast_plain_tiles = [&](int kt_end) -> int {
     if constexpr (!FP8) {
       if (kt < kt_end) ids_ahead = page_ids_of_tile(kt + 1);
@@ -718,14 +737,14 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
         for (int u = 0; u < kColTiles; ++u) st[i & 1][u] = mfma_16x16x32(kf[i], qf[u][i >> 1], st[i & 1][u]);
         kf1[i] = load_kfrag(1, i);
         if constexpr (!FP8) {
-          if (i & 1) issue_rows(i >> 1);
+          if (i % kIssueEvery == kIssueEvery - 1) issue_rows(i / kIssueEvery);
         }
       }
 #pragma unroll
       for (int i = 0; i < kJTiles; ++i) {
         __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if (!FP8 && (i & 1)) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+        if (!FP8 && i % kIssueEvery == kIssueEvery - 1) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
       // Region 3: the second half's MFMAs beside the first half's exponentials; the first
@@ -807,7 +826,9 @@ __global__ __launch_bounds__(kTiledWaves *kWave, kHD == 64 ? 3 : 2) void varlen_
     // (the K/V tiles are done with) and leave as whole 256-byte rows, 4 rows per instruction.
     constexpr int kOutPitch = 2 * kHD + 16;  // bytes; at 128: 68 dwords, a half-wave's 8-byte writes hit 64 banks
     __syncthreads();                              // every wavefront is done reading the last tile
-    const uint32_t mine = ((wave & 2) ? v_lds : k_lds) + (uint32_t)((wave & 1) * kColTiles * 16 * kOutPitch);
+    const uint32_t mine = W == kWideWaves
+                              ? k_lds + (uint32_t)(wave * kColTiles * 16 * kOutPitch)
+                              : ((wave & 2) ? v_lds : k_lds) + (uint32_t)((wave & 1) * kColTiles * 16 * kOutPitch);
 #pragma unroll
     for (int u = 0; u < kColTiles; ++u) {
       const float inv = v_scale / dsum[u][0];
@@ -895,16 +916,17 @@ static int validate_prefill(const char *what, const void *q, int64_t q_stride, c
   return LITEKV_OK;
 }
 
-// How a GQA group of `group` heads is cut into workgroups of 8 column tiles.
+// How a GQA group of `group` heads is cut into workgroups of `col_tiles` column tiles (two per
+// wavefront).
 struct PrefillShape {
   int head_splits, heads_per_wg, row_tiles;
   unsigned row_blocks;
 };
-static PrefillShape prefill_shape(int group, int max_q_len) {
+static PrefillShape prefill_shape(int group, int max_q_len, int col_tiles = kWgColTiles) {
   PrefillShape s;
-  s.head_splits = (group + kWgColTiles - 1) / kWgColTiles;
+  s.head_splits = (group + col_tiles - 1) / col_tiles;
   s.heads_per_wg = (group + s.head_splits - 1) / s.head_splits;
-  s.row_tiles = kWgColTiles / s.heads_per_wg;
+  s.row_tiles = col_tiles / s.heads_per_wg;
   s.row_blocks = (unsigned)((max_q_len + 16 * s.row_tiles - 1) / (16 * s.row_tiles));
   return s;
 }
@@ -1031,11 +1053,12 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
                     num_kv_heads, (int32_t)num_pages, kv_scales, page_shift};
   PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
   const int group = num_q_heads / num_kv_heads;
-  const PrefillShape s = prefill_shape(group, max_q_len);
+  const int waves = (format == kKvF16 && LITEKV_PREFILL_WAVES == kWideWaves) ? kWideWaves : kTiledWaves;
+  const PrefillShape s = prefill_shape(group, max_q_len, kColTiles * waves);
   LITEKV_REQUIRE(s.row_blocks <= 65535u, "%s: max_q_len %d too large", what, max_q_len);
   const dim3 grid((unsigned)(num_kv_heads * s.head_splits), s.row_blocks, (unsigned)batch);
   auto launch = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, grid, dim3(kTiledWaves * kWave), 0, static_cast<hipStream_t>(stream),
+    hipLaunchKernelGGL(kernel, grid, dim3(waves * kWave), 0, static_cast<hipStream_t>(stream),
                        static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
                        out_token_stride, paged, packed, PrefixTask{}, cu_q_lens,
                        (const int32_t *)nullptr, context_lens, group, s.head_splits, s.heads_per_wg,
@@ -1045,6 +1068,8 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
     launch(varlen_prefill_tiled_kernel<kPagedPrefillInt8>);
   } else if (format == kKvFp8) {
     launch(varlen_prefill_tiled_kernel<kPagedPrefillFp8>);
+  } else if (waves == kWideWaves) {
+    launch(varlen_prefill_tiled_kernel<kPagedPrefill, kWideWaves>);
   } else {
     launch(varlen_prefill_tiled_kernel<kPagedPrefill>);
   }
@@ -1108,15 +1133,23 @@ static int launch_varlen_prefill(const void *q, int64_t q_token_stride, const vo
   PackedSource packed{static_cast<const half_t *>(k), static_cast<const half_t *>(v),
                       k_token_stride, v_token_stride, seq_starts};
   const int group = num_q_heads / num_kv_heads;
-  const PrefillShape s = prefill_shape(group, max_seq_len);
+  const int waves = LITEKV_PREFILL_WAVES == kWideWaves ? kWideWaves : kTiledWaves;
+  const PrefillShape s = prefill_shape(group, max_seq_len, kColTiles * waves);
   LITEKV_REQUIRE(s.row_blocks <= 65535u, "varlen_prefill: max_seq_len %d too large", max_seq_len);
-  hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kPackedPrefill>,
-                     dim3((unsigned)(num_kv_heads * s.head_splits), s.row_blocks, (unsigned)batch),
-                     dim3(kTiledWaves * kWave), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
-                     out_token_stride, paged, packed, PrefixTask{}, seq_starts, seq_lens,
-                     (const int32_t *)nullptr, group, s.head_splits, s.heads_per_wg, s.row_tiles,
-                     softmax_scale * kLog2eP);
+  auto launch = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel,
+                       dim3((unsigned)(num_kv_heads * s.head_splits), s.row_blocks, (unsigned)batch),
+                       dim3(waves * kWave), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
+                       out_token_stride, paged, packed, PrefixTask{}, seq_starts, seq_lens,
+                       (const int32_t *)nullptr, group, s.head_splits, s.heads_per_wg, s.row_tiles,
+                       softmax_scale * kLog2eP);
+  };
+  if (waves == kWideWaves) {
+    launch(varlen_prefill_tiled_kernel<kPackedPrefill, kWideWaves>);
+  } else {
+    launch(varlen_prefill_tiled_kernel<kPackedPrefill>);
+  }
   return check_launch("varlen_prefill");
 }
 }  // namespace LITEKV_HD_NS

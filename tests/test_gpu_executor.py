@@ -343,7 +343,8 @@ def test_static_batch_prefill_then_decode_equals_the_packed_flow():
         assert_attention_close(o_s, _oracle_decode(static, qd, 0), f"static batch decode step {step}")
 
 
-@pytest.mark.parametrize("page_size,head_dim", [(32, 128), (64, 64), (16, 64), (16, 256)])
+@pytest.mark.parametrize("page_size,head_dim", [(32, 128), (64, 64), (16, 64), (16, 256), (128, 128), (256, 128),
+                                                (256, 64), (128, 32)])
 def test_executor_flow_at_other_page_sizes_and_head_dims(page_size, head_dim):
     """The same host flow -- packed prefill, a chunk over cached history, fused decode steps --
     on pools with larger pages and other head dims."""
@@ -360,6 +361,8 @@ def test_executor_flow_at_other_page_sizes_and_head_dims(page_size, head_dim):
         return torch.randn((tokens, heads, head_dim), generator=g, device=DEV, dtype=torch.float16)
 
     lens = [37, 16, 90, 5]
+    if page_size > 64:
+        lens.append(page_size - 6)           # crosses into its second page during the decode steps
     ids = ex.reserve_paged_requests(lens, reserved_lengths=[n + 60 for n in lens])
     ex.activate_paged_packed_prefill_batch(ids, lens)
     info = ex.atten_info
