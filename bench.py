@@ -155,7 +155,9 @@ class DecodeLayerSet:
         bts = self.table.stride(0)
         if schedule == "balanced":
             self.shared_pages = shared_pages
-            self.chunks = c.extra.get("chunks") or lib.litekv_paged_decode_balanced_chunks(hkv)
+            self.chunks = c.extra.get("chunks") or (
+                lib.litekv_paged_decode_prefix_chunks(b, hq, hkv, 128, 16, shared_pages, 1 if kv_dtype == "f16" else 0)
+                if shared_pages > 0 else lib.litekv_paged_decode_balanced_chunks(hkv))
             self.plan_bytes = lib.litekv_decode_plan_bytes(b, bts, hkv, self.chunks)
             self.plan = torch.empty(self.plan_bytes // 4, dtype=torch.int32, device=device)
             ws_bytes = lib.litekv_paged_decode_prefix_workspace_bytes(b, hq, 128, self.chunks)

@@ -268,6 +268,17 @@ int litekv_paged_decode_static(const void *q, int64_t q_batch_stride, const void
  */
 int32_t litekv_paged_decode_balanced_chunks(int32_t num_kv_heads);
 
+/* The chunk count for a step behind `shared_pages` shared pages
+ * (litekv_paged_decode_prefix): the workgroups that attend the shared pages and
+ * those that stream the private pages are one launch and should all be
+ * resident at once, so the private pages get the compute units the others
+ * leave. pool_is_fp16: 0 for a pool of 8-bit codes. Falls back to
+ * litekv_paged_decode_balanced_chunks for arguments it cannot use. */
+int32_t litekv_paged_decode_prefix_chunks(int32_t batch, int32_t num_q_heads,
+                                          int32_t num_kv_heads, int32_t head_dim,
+                                          int32_t page_size, int32_t shared_pages,
+                                          int32_t pool_is_fp16);
+
 size_t litekv_paged_decode_balanced_workspace_bytes(int32_t batch, int32_t num_q_heads,
                                                     int32_t head_dim, int32_t chunks);
 

@@ -97,6 +97,7 @@ SIGNATURES = {
          c_int32, c_void_p],
     ),
     "litekv_paged_decode_balanced_chunks": (c_int32, [c_int32]),
+    "litekv_paged_decode_prefix_chunks": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32]),
     "litekv_paged_decode_balanced_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "litekv_decode_plan_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "litekv_decode_plan_bytes_paged": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32]),

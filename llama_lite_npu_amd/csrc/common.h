@@ -73,25 +73,6 @@ __host__ __device__ __forceinline__ HeadSlice head_slice(int hv, int slices, int
 // Most key slices the shared-prefix kernel may cut the prefix into (bounds its workspace).
 constexpr int kMaxPrefixSplits = 8;
 
-// Attention of every (sequence, query head) of a decode step over the first `shared_pages`
-// pages of block-table row 0 (which all sequences share), as normalised fp32 partial rows
-// part_o[split][batch][Hq][128] and log-sum-exps part_lse[split][batch][Hq]; *splits_out
-// receives the number of key slices written. `fp8_scales` (K heads, then V heads) marks an fp8 pool.
-// Defined beside the prefill kernel it reuses.
-int launch_shared_prefix(const void *q, int64_t q_batch_stride, const void *kv_pool,
-                         const float *fp8_scales,
-                         const int32_t *block_table, int32_t batch, int32_t num_q_heads,
-                         int32_t num_kv_heads, int64_t num_pages, int32_t shared_pages,
-                         int32_t page_shift, float *part_o, float *part_lse, float softmax_scale,
-                         hipStream_t stream, int *splits_out, int format);
-// The same for head dim 64 (defined in the head dim 64 build of paged_prefill.hip).
-int launch_shared_prefix_hd64(const void *q, int64_t q_batch_stride, const void *kv_pool,
-                              const float *fp8_scales, const int32_t *block_table, int32_t batch,
-                              int32_t num_q_heads, int32_t num_kv_heads, int64_t num_pages,
-                              int32_t shared_pages, int32_t page_shift, float *part_o,
-                              float *part_lse, float softmax_scale, hipStream_t stream,
-                              int *splits_out, int format);
-
 // ---- the plan of a balanced decode step (made by decode_plan_kernel in paged_decode.hip) -------
 // Plan buffer (int32 words): meta[kPlanMeta]; per sequence (first chunk, number of chunks it
 // spans); per sequence the position of its first 16-token page on the line; the chunk entries.

@@ -34,6 +34,7 @@
 
 #include "common.h"
 #include "kv_fp8.h"
+#include "prefill_tile.h"
 
 // This file is compiled once per head dim its kernels are tuned for: as itself for 128, and
 // through paged_decode_hd64.hip (which defines LITEKV_HD and includes it) for 64. Everything
@@ -43,17 +44,6 @@
 // At 64 the lane maps are those of 128 with half the MFMA k-steps and half the output column
 // tiles; lanes whose 16-byte column of a V row would lie past the row re-read the column of
 // their twin (n % 8) and stage it in a part of the LDS row nobody reads.
-#ifndef LITEKV_HD
-#define LITEKV_HD 128
-#endif
-#if LITEKV_HD == 128
-#define LITEKV_HD_NS hd128
-#elif LITEKV_HD == 64
-#define LITEKV_HD_NS hd64
-#else
-#error "paged_decode.hip is written for head dims 64 and 128"
-#endif
-
 namespace litekv {
 inline namespace LITEKV_HD_NS {
 
@@ -992,8 +982,17 @@ __global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merg
   }
 }
 
+// LDS of a workgroup of the balanced kernel: the V staging rows of its wavefronts, then their
+// parking areas.
+constexpr int kBalancedVstageBytes = kMaxWavesPerWg * kPageSize * kVPitch * (int)sizeof(half_t);
+constexpr int kBalancedLdsBytes = kBalancedVstageBytes + kMaxWavesPerWg * kParkFloats * (int)sizeof(float);
+
+// The body of the balanced kernel, run by the workgroup that stands at (block_x, block_y) of its
+// grid; `lds` is its kBalancedLdsBytes of LDS (16-byte aligned). A function, so that the decode
+// step with a shared prefix can run it as one role of a launch that also attends the prefix.
 template <int DEPTH, int KV>
-__global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_kernel(
+__device__ __forceinline__ void balanced_body(
+    char *lds, const int block_x, const int block_y,
     const half_t *__restrict__ q, int64_t q_batch_stride,
     typename KvStore<KV>::elem *__restrict__ kv, const float *__restrict__ scales,
     const int32_t *__restrict__ seq_lens, const int32_t *__restrict__ plan,
@@ -1002,8 +1001,8 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     float *__restrict__ part_lse, int32_t bt_stride, int32_t batch, int32_t num_q_heads,
     int32_t num_kv_heads, int32_t group_all, int32_t slices, int32_t heads_per_wg,
     int32_t replicas, int32_t chunks, int32_t skip, float scale_log2) {
-  __shared__ __attribute__((aligned(16))) half_t vstage_all[kMaxWavesPerWg][kPageSize * kVPitch];
-  __shared__ __attribute__((aligned(16))) float park_all[kMaxWavesPerWg][kParkFloats];
+  half_t(*vstage_all)[kPageSize * kVPitch] = reinterpret_cast<half_t(*)[kPageSize * kVPitch]>(lds);
+  float(*park_all)[kParkFloats] = reinterpret_cast<float(*)[kParkFloats]>(lds + kBalancedVstageBytes);
 
   // readfirstlane tells the compiler the wavefront index is uniform (scalar branches and loads)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1012,8 +1011,8 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   const int g = lane >> 4;
   // a wavefront per head slice: the kv head itself, or up to 16 of its query heads when it has
   // more than 16 (see head_slice)
-  const int hv = blockIdx.y * heads_per_wg + wave % heads_per_wg;
-  const int cidx = blockIdx.x * replicas + wave / heads_per_wg;
+  const int hv = block_y * heads_per_wg + wave % heads_per_wg;
+  const int cidx = block_x * replicas + wave / heads_per_wg;
   if (hv >= num_kv_heads * slices || cidx >= chunks) return;  // whole wavefront; no workgroup barriers below
   const HeadSlice hs = head_slice(hv, slices, group_all);
   const int h = hs.kv_head;
@@ -1338,6 +1337,80 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
   zero_empty_rows();
 }
 
+template <int DEPTH, int KV>
+__global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_kernel(
+    const half_t *__restrict__ q, int64_t q_batch_stride,
+    typename KvStore<KV>::elem *__restrict__ kv, const float *__restrict__ scales,
+    const int32_t *__restrict__ seq_lens, const int32_t *__restrict__ plan,
+    const half_t *__restrict__ k_new, const half_t *__restrict__ v_new, int64_t k_new_stride,
+    int64_t v_new_stride, half_t *__restrict__ out, float *__restrict__ part_o,
+    float *__restrict__ part_lse, int32_t bt_stride, int32_t batch, int32_t num_q_heads,
+    int32_t num_kv_heads, int32_t group_all, int32_t slices, int32_t heads_per_wg,
+    int32_t replicas, int32_t chunks, int32_t skip, float scale_log2) {
+  __shared__ __attribute__((aligned(16))) char lds[kBalancedLdsBytes];
+  balanced_body<DEPTH, KV>(lds, (int)blockIdx.x, (int)blockIdx.y, q, q_batch_stride, kv, scales, seq_lens,
+                           plan, k_new, v_new, k_new_stride, v_new_stride, out, part_o, part_lse,
+                           bt_stride, batch, num_q_heads, num_kv_heads, group_all, slices, heads_per_wg,
+                           replicas, chunks, skip, scale_log2);
+}
+
+// ---------------------------------------------------------------------------------------------
+// A decode step behind a shared prefix as ONE launch with two roles. The first `prefix_wgs`
+// workgroups attend the shared pages for the whole batch (prefill_tile.h in its shared-prefix
+// mode: columns = (sequence, query head) pairs, one key slice per workgroup, normalised fp32
+// partials out); the others are the workgroups of the balanced kernel over the pages behind the
+// prefix. The prefix role is bound by the matrix pipes of the few compute units it occupies, the
+// other by memory: as two launches they ran one after the other (17 + 20 us on 64 sequences
+// sharing 2048 tokens), each leaving half the device idle; two streams cost more in forks and
+// joins between hardware queues than they overlapped. Prefix workgroups come first in the grid:
+// they are the long ones, and x = kv head keeps a head's slices on one XCD. Registers are those
+// of the prefix role (two wavefronts per SIMD), so a compute unit holds one workgroup of either
+// role.
+// ---------------------------------------------------------------------------------------------
+template <int KV> struct PrefixMode { static constexpr int value = prefill_tile::kSharedPrefix; };
+template <> struct PrefixMode<kKvFp8> { static constexpr int value = prefill_tile::kSharedPrefixFp8; };
+template <> struct PrefixMode<kKvInt8> { static constexpr int value = prefill_tile::kSharedPrefixInt8; };
+
+template <int PW>
+constexpr int prefix_step_lds_bytes() {
+  return prefill_tile::tile_lds_bytes<PW>() > kBalancedLdsBytes ? prefill_tile::tile_lds_bytes<PW>()
+                                                                 : kBalancedLdsBytes;
+}
+
+template <int DEPTH, int KV, int PW>
+__global__ __launch_bounds__(kMaxWavesPerWg * kWave) void prefix_step_kernel(
+    prefill_tile::PagedSource shared, prefill_tile::PrefixTask task, int32_t prefix_wgs,
+    int32_t prefix_col_blocks, int32_t decode_wgs_x,
+    const half_t *__restrict__ q, int64_t q_batch_stride,
+    typename KvStore<KV>::elem *__restrict__ kv, const float *__restrict__ scales,
+    const int32_t *__restrict__ seq_lens, const int32_t *__restrict__ plan,
+    const half_t *__restrict__ k_new, const half_t *__restrict__ v_new, int64_t k_new_stride,
+    int64_t v_new_stride, half_t *__restrict__ out, float *__restrict__ part_o,
+    float *__restrict__ part_lse, int32_t bt_stride, int32_t batch, int32_t num_q_heads,
+    int32_t num_kv_heads, int32_t group_all, int32_t slices, int32_t heads_per_wg,
+    int32_t replicas, int32_t chunks, int32_t skip, float scale_log2) {
+  __shared__ __attribute__((aligned(1024))) char lds[prefix_step_lds_bytes<PW>()];
+  const int id = (int)blockIdx.x;
+  if (id < prefix_wgs) {
+    if ((int)threadIdx.x >= PW * kWave) return;  // the role has PW wavefronts; no barrier counts the others
+    const int h = id % num_kv_heads;
+    const int rest = id / num_kv_heads;
+    const int col_block = rest % prefix_col_blocks;
+    const int key_slice = rest / prefix_col_blocks;
+    prefill_tile::prefill_tile_body<PrefixMode<KV>::value, PW>(
+        (uint32_t)(uintptr_t)(prefill_tile::lds_half_t *)lds, h, col_block, key_slice, 1, q, (int64_t)0,
+        (half_t *)nullptr, (int64_t)0, shared, prefill_tile::PackedSource{nullptr, nullptr, 0, 0, nullptr},
+        task, (const int32_t *)nullptr, (const int32_t *)nullptr, (const int32_t *)nullptr, group_all, 1,
+        group_all, 1, scale_log2);
+    return;
+  }
+  const int d = id - prefix_wgs;
+  balanced_body<DEPTH, KV>(lds, d % decode_wgs_x, d / decode_wgs_x, q, q_batch_stride, kv, scales, seq_lens,
+                           plan, k_new, v_new, k_new_stride, v_new_stride, out, part_o, part_lse,
+                           bt_stride, batch, num_q_heads, num_kv_heads, group_all, slices, heads_per_wg,
+                           replicas, chunks, skip, scale_log2);
+}
+
 }  // namespace LITEKV_HD_NS
 }  // namespace litekv
 
@@ -1592,8 +1665,8 @@ static size_t plan_bytes_for(int64_t batch, int64_t bt_stride, int64_t hkv, int6
   return (size_t)words * sizeof(int32_t);
 }
 
-// Chunks per kv head that give every CU of the current device one workgroup.
-static int auto_chunks(int num_kv_heads) {
+// Compute units of the current device.
+static int device_cus() {
   static thread_local int cached_device = -1;
   static thread_local int cached_cus = 0;
   int dev = 0;
@@ -1607,8 +1680,13 @@ static int auto_chunks(int num_kv_heads) {
     cached_device = dev;
     cached_cus = cus;
   }
+  return cached_cus;
+}
+
+// Chunks per kv head that give every CU of the current device one workgroup.
+static int auto_chunks(int num_kv_heads) {
   const BalancedShape s = balanced_shape(num_kv_heads);
-  const int wgs = (cached_cus + s.head_groups - 1) / s.head_groups;
+  const int wgs = (device_cus() + s.head_groups - 1) / s.head_groups;
   return wgs * s.replicas;
 }
 
@@ -1622,6 +1700,60 @@ static int check_chunks(const char *what, int32_t batch, int32_t bt_stride, int3
   return LITEKV_OK;
 }
 
+// How the shared pages of a step are cut for the prefix role of prefix_step_kernel: `wide` says
+// that its workgroups have 8 wavefronts (256 columns) instead of 4 (128), `col_blocks` how many
+// of them cover the batch's (sequence, query head) pairs of one kv head, `splits` the key slices.
+struct PrefixShape {
+  bool wide;
+  int col_blocks, splits, keys_per_split, prefix_keys, wgs;
+};
+static PrefixShape prefix_shape(int batch, int group, int num_kv_heads, int shared_pages16,
+                                bool fp16_pool, int block_waves) {
+  // (fp16_pool: false for 8-bit codes, which eight wavefronts stage at head dim 128 only)
+  PrefixShape s;
+  s.prefix_keys = shared_pages16 * kPageSize;
+  const int cols = batch * group;
+  // Eight wavefronts share every staged K/V tile among twice the columns and leave twice the
+  // compute units to the other role; they take fp16 K/V and a batch that fills them.
+  s.wide = (fp16_pool || kHD == 128) && block_waves == prefill_tile::kWideWaves &&
+           cols > 16 * prefill_tile::kWgColTiles;
+  const int wg_cols = 16 * prefill_tile::kColTiles * (s.wide ? prefill_tile::kWideWaves : prefill_tile::kTiledWaves);
+  s.col_blocks = (cols + wg_cols - 1) / wg_cols;
+  // Enough key slices for 512 wavefronts of this role (a quarter of the device's slots), at
+  // least 128 keys each: every slice is one more partial row per (sequence, head) to write here
+  // and to read in the merge (64 sequences sharing 2048 tokens, per layer, as separate launches:
+  // 8 slices 47.1 us, 4 slices 44.3 us, 2 slices 49.3 us).
+  const int target_wgs = s.wide ? 64 : 128;
+  int splits = target_wgs / (num_kv_heads * s.col_blocks);
+  splits = splits < 1 ? 1 : (splits > kMaxPrefixSplits ? kMaxPrefixSplits : splits);
+  const int max_by_keys = (s.prefix_keys + 127) / 128;
+  splits = splits < max_by_keys ? splits : max_by_keys;
+  int keys_per_split = (s.prefix_keys + splits - 1) / splits;
+  keys_per_split = (keys_per_split + prefill_tile::kKvTile - 1) / prefill_tile::kKvTile * prefill_tile::kKvTile;
+  s.keys_per_split = keys_per_split;
+  s.splits = (s.prefix_keys + keys_per_split - 1) / keys_per_split;
+  s.wgs = num_kv_heads * s.col_blocks * s.splits;
+  return s;
+}
+
+// Chunks per kv head for a step behind a shared prefix: the workgroups of both roles of
+// prefix_step_kernel should be resident at once (a compute unit holds one of either), so the
+// private pages get the compute units the prefix role leaves, less a sixteenth of the device
+// (64 sequences sharing 2048 tokens, 64 prefix workgroups, per layer: 256 chunks 39.7 us, 192
+// 33.6 us, 176 33.1 us).
+static int auto_prefix_chunks(int batch, int num_q_heads, int num_kv_heads, int shared_pages16,
+                              bool fp16_pool) {
+  const int group = num_q_heads / num_kv_heads;
+  const BalancedShape s = balanced_shape(num_kv_heads * head_slices(group));
+  const PrefixShape ps = prefix_shape(batch, group, num_kv_heads, shared_pages16, fp16_pool,
+                                      s.heads_per_wg * s.replicas);
+  const int cus = device_cus();
+  int wgs = cus - ps.wgs - cus / 16;
+  wgs = wgs > cus / 4 ? wgs : cus / 4;
+  wgs = (wgs + s.head_groups - 1) / s.head_groups;
+  return wgs * s.replicas;
+}
+
 // Optional HIP events bracketing the next balanced decode launch of this thread (profiling).
 static thread_local hipEvent_t g_profile_start = nullptr;
 static thread_local hipEvent_t g_profile_stop = nullptr;
@@ -1632,6 +1764,21 @@ static thread_local hipEvent_t g_profile_stop = nullptr;
 #if LITEKV_HD == 128  // the C ABI lives in the head dim 128 build of this file
 extern "C" int32_t litekv_paged_decode_balanced_chunks(int32_t num_kv_heads) {
   return num_kv_heads > 0 ? litekv::auto_chunks(num_kv_heads) : 0;
+}
+
+extern "C" int32_t litekv_paged_decode_prefix_chunks(int32_t batch, int32_t num_q_heads,
+                                                     int32_t num_kv_heads, int32_t head_dim,
+                                                     int32_t page_size, int32_t shared_pages,
+                                                     int32_t pool_is_fp16) {
+  const int shift = litekv::page_shift_of(page_size);
+  if (batch <= 0 || num_kv_heads <= 0 || num_q_heads <= 0 || num_q_heads % num_kv_heads != 0 ||
+      num_q_heads / num_kv_heads > litekv::kMaxGroup || shift < 0 || shared_pages <= 0 ||
+      shared_pages > (1 << 20)) {
+    return num_kv_heads > 0 ? litekv::auto_chunks(num_kv_heads) : 0;
+  }
+  (void)head_dim;  // both tuned builds cut the prefix alike; other head dims ignore the chunk count
+  return litekv::auto_prefix_chunks(batch, num_q_heads, num_kv_heads, shared_pages << shift,
+                                    pool_is_fp16 != 0);
 }
 
 extern "C" size_t litekv_paged_decode_balanced_workspace_bytes(int32_t batch, int32_t num_q_heads,
@@ -1803,39 +1950,76 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
   float *pre_o = part_lse + (size_t)(chunks + batch) * num_q_heads;
   float *pre_lse = pre_o + (size_t)kMaxPrefixSplits * batch * num_q_heads * head_dim;
   int pre_splits = 0;
-  if (shared_pages > 0) {
-    LITEKV_REQUIRE(block_table != nullptr, "%s: block_table is null", what);
-#if LITEKV_HD == 64
-    rc = launch_shared_prefix_hd64(
-#else
-    rc = launch_shared_prefix(
-#endif
-                              q, q_batch_stride, kv_pool, fp8_scales, block_table, batch, num_q_heads,
-                              num_kv_heads, num_pages, shared_pages, shift, pre_o, pre_lse,
-                              softmax_scale, static_cast<hipStream_t>(stream), &pre_splits, format);
-    if (rc != LITEKV_OK) return rc;
-  }
   const unsigned wgs = (unsigned)((chunks + s.replicas - 1) / s.replicas);
   hipEvent_t ev0 = g_profile_start, ev1 = g_profile_stop;
   g_profile_start = g_profile_stop = nullptr;
-  const dim3 grid(wgs, (unsigned)s.head_groups);
   const dim3 block((unsigned)(kWave * s.heads_per_wg * s.replicas));
-  auto launch = [&](auto kernel, auto *kv) {
-    hipExtLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), ev0, ev1, 0,
-                          static_cast<const half_t *>(q), q_batch_stride, kv, fp8_scales, seq_lens,
-                          static_cast<const int32_t *>(plan), static_cast<const half_t *>(k_new),
-                          static_cast<const half_t *>(v_new), k_new_stride, v_new_stride,
-                          static_cast<half_t *>(out), part_o, part_lse, sub_stride, batch,
-                          num_q_heads, num_kv_heads, num_q_heads / num_kv_heads, slices,
-                          s.heads_per_wg, s.replicas, chunks, shared_pages << shift,
-                          softmax_scale * kLog2e);
-  };
-  if (fp8_scales != nullptr && format == kKvInt8) {
-    launch(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, kKvInt8>, static_cast<uint8_t *>(kv_pool));
-  } else if (fp8_scales != nullptr) {
-    launch(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, kKvFp8>, static_cast<uint8_t *>(kv_pool));
+  const int group = num_q_heads / num_kv_heads;
+  if (shared_pages > 0) {
+    // one launch, two roles (see prefix_step_kernel)
+    LITEKV_REQUIRE(block_table != nullptr, "%s: block_table is null", what);
+    LITEKV_REQUIRE(num_kv_heads <= 1024, "%s: num_kv_heads %d > 1024", what, num_kv_heads);
+    LITEKV_REQUIRE(shared_pages <= (1 << 20), "%s: shared_pages %d out of range", what, shared_pages);
+    const PrefixShape ps = prefix_shape(batch, group, num_kv_heads, shared_pages << shift,
+                                        fp8_scales == nullptr, (int)(block.x / kWave));
+    const int64_t total_wgs = (int64_t)ps.wgs + (int64_t)wgs * s.head_groups;
+    LITEKV_REQUIRE(total_wgs <= 0x7fffffffLL, "%s: batch %d too large", what, batch);
+    pre_splits = ps.splits;
+    // only the first shared_pages entries of block-table row 0 are read
+    prefill_tile::PagedSource shared{static_cast<const half_t *>(kv_pool), block_table, shared_pages,
+                                     num_kv_heads, (int32_t)num_pages, fp8_scales, shift};
+    prefill_tile::PrefixTask task{pre_o, pre_lse, q_batch_stride, batch, num_q_heads, ps.prefix_keys,
+                                  ps.keys_per_split};
+    auto launch = [&](auto kernel, auto *kv) {
+      hipExtLaunchKernelGGL(kernel, dim3((unsigned)total_wgs), block, 0, static_cast<hipStream_t>(stream),
+                            ev0, ev1, 0, shared, task, ps.wgs, ps.col_blocks, (int32_t)wgs,
+                            static_cast<const half_t *>(q), q_batch_stride, kv, fp8_scales, seq_lens,
+                            static_cast<const int32_t *>(plan), static_cast<const half_t *>(k_new),
+                            static_cast<const half_t *>(v_new), k_new_stride, v_new_stride,
+                            static_cast<half_t *>(out), part_o, part_lse, sub_stride, batch,
+                            num_q_heads, num_kv_heads, group, slices, s.heads_per_wg, s.replicas, chunks,
+                            shared_pages << shift, softmax_scale * kLog2e);
+    };
+    constexpr int kWide8 = kHD == 128 ? prefill_tile::kWideWaves : prefill_tile::kTiledWaves;
+    if (fp8_scales != nullptr && format == kKvInt8) {
+      if (ps.wide) {
+        launch(prefix_step_kernel<LITEKV_DECODE_DEPTH, kKvInt8, kWide8>, static_cast<uint8_t *>(kv_pool));
+      } else {
+        launch(prefix_step_kernel<LITEKV_DECODE_DEPTH, kKvInt8, prefill_tile::kTiledWaves>,
+               static_cast<uint8_t *>(kv_pool));
+      }
+    } else if (fp8_scales != nullptr) {
+      if (ps.wide) {
+        launch(prefix_step_kernel<LITEKV_DECODE_DEPTH, kKvFp8, kWide8>, static_cast<uint8_t *>(kv_pool));
+      } else {
+        launch(prefix_step_kernel<LITEKV_DECODE_DEPTH, kKvFp8, prefill_tile::kTiledWaves>,
+               static_cast<uint8_t *>(kv_pool));
+      }
+    } else if (ps.wide) {
+      launch(prefix_step_kernel<LITEKV_DECODE_DEPTH, kKvF16, prefill_tile::kWideWaves>,
+             static_cast<half_t *>(kv_pool));
+    } else {
+      launch(prefix_step_kernel<LITEKV_DECODE_DEPTH, kKvF16, prefill_tile::kTiledWaves>,
+             static_cast<half_t *>(kv_pool));
+    }
   } else {
-    launch(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, kKvF16>, static_cast<half_t *>(kv_pool));
+    const dim3 grid(wgs, (unsigned)s.head_groups);
+    auto launch = [&](auto kernel, auto *kv) {
+      hipExtLaunchKernelGGL(kernel, grid, block, 0, static_cast<hipStream_t>(stream), ev0, ev1, 0,
+                            static_cast<const half_t *>(q), q_batch_stride, kv, fp8_scales, seq_lens,
+                            static_cast<const int32_t *>(plan), static_cast<const half_t *>(k_new),
+                            static_cast<const half_t *>(v_new), k_new_stride, v_new_stride,
+                            static_cast<half_t *>(out), part_o, part_lse, sub_stride, batch,
+                            num_q_heads, num_kv_heads, group, slices, s.heads_per_wg, s.replicas,
+                            chunks, 0, softmax_scale * kLog2e);
+    };
+    if (fp8_scales != nullptr && format == kKvInt8) {
+      launch(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, kKvInt8>, static_cast<uint8_t *>(kv_pool));
+    } else if (fp8_scales != nullptr) {
+      launch(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, kKvFp8>, static_cast<uint8_t *>(kv_pool));
+    } else {
+      launch(paged_decode_balanced_kernel<LITEKV_DECODE_DEPTH, kKvF16>, static_cast<half_t *>(kv_pool));
+    }
   }
   rc = check_launch(what);
   if (rc != LITEKV_OK) return rc;

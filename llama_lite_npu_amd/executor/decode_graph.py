@@ -88,7 +88,8 @@ class DeviceDecodeBatch:
         self.decode_plan = ops.DecodePlan(self.block_table, self.seq_lens_i32, executor.local_q_heads,
                                           executor.local_kv_heads, executor.kv_mem_manager.num_pages,
                                           page_size=executor.page_size, shared_pages=self.shared_pages,
-                                          token_bytes=getattr(executor, "kv_token_bytes", None))
+                                          token_bytes=getattr(executor, "kv_token_bytes", None),
+                                          kv_dtype=executor.kv_mem_manager.gpu_kv_buffer[0].dtype)
         self.load(request_ids, reserve_tokens, host_ahead)
 
     # ---- host side -------------------------------------------------------------------------
@@ -353,7 +354,8 @@ class DecodeGraphRunner:
 
             info.decode_plan = ops.DecodePlan(info.block_table, info.seq_lens_i32, plan.num_q_heads,
                                               plan.num_kv_heads, plan.num_pages, plan.chunks, plan.page_size,
-                                              plan.shared_pages, token_bytes=plan.token_bytes)
+                                              plan.shared_pages, token_bytes=plan.token_bytes,
+                                              kv_dtype=getattr(plan, "kv_dtype", None))
             info.decode_plan.per_sequence = bool(plan.per_sequence)
         return info
 

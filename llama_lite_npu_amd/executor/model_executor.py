@@ -315,7 +315,8 @@ class ModelExecutor:
                                               page_size=self.page_size,
                                               shared_pages=self.shared_prefix_pages(ids),
                                               host_seq_lens=[mgr.req_token_count[r] for r in ids],
-                                              token_bytes=self.kv_token_bytes)
+                                              token_bytes=self.kv_token_bytes,
+                                              kv_dtype=self.kv_mem_manager.gpu_kv_buffer[0].dtype)
         self._decode_meta_sig = sig
 
     def common_leading_pages(self, request_ids: Sequence[int], upcoming_tokens: int = 0) -> int:

@@ -258,6 +258,15 @@ def balanced_chunks(num_kv_heads: int) -> int:
     return int(_lib.load().litekv_paged_decode_balanced_chunks(int(num_kv_heads)))
 
 
+def prefix_chunks(batch: int, num_q_heads: int, num_kv_heads: int, shared_pages: int,
+                  page_size: int = PAGE_SIZE, head_dim: int = HEAD_DIM, fp16_pool: bool = True) -> int:
+    """Chunks per kv head for a step behind ``shared_pages`` shared pages: the private pages get the
+    compute units that the workgroups attending the shared pages (same launch) leave free."""
+    return int(_lib.load().litekv_paged_decode_prefix_chunks(int(batch), int(num_q_heads), int(num_kv_heads),
+                                                             int(head_dim), int(page_size), int(shared_pages),
+                                                             1 if fp16_pool else 0))
+
+
 def per_sequence_decode_is_faster(batch: int, num_kv_heads: int, max_pages: int, total_pages: int,
                                   token_bytes: int, page_size: int = PAGE_SIZE, margin: float = 1.1,
                                   heads_per_kv_head: int = 8) -> bool:
@@ -298,14 +307,17 @@ class DecodePlan:
     def __init__(self, block_table: torch.Tensor, seq_lens: torch.Tensor, num_q_heads: int,
                  num_kv_heads: int, num_pages: int, chunks: Optional[int] = None,
                  page_size: int = PAGE_SIZE, shared_pages: int = 0,
-                 host_seq_lens: Optional[Sequence[int]] = None, token_bytes: Optional[int] = None):
+                 host_seq_lens: Optional[Sequence[int]] = None, token_bytes: Optional[int] = None,
+                 kv_dtype: Optional[torch.dtype] = None):
         """``shared_pages``: leading block-table entries that are the same physical pages in every
         row (a shared cached prefix); they are then attended once for the whole batch.
         ``host_seq_lens``: the lengths as the host knows them; with them the plan picks the
         per-sequence schedule where ``per_sequence_decode_is_faster`` says so. ``token_bytes``:
-        K + V bytes of one token in the pool (default: fp16)."""
+        K + V bytes of one token in the pool (default: fp16). ``kv_dtype``: the pool's element type
+        (default fp16); with a shared prefix it decides how the default chunk count is chosen."""
         lib = _lib.load()
         self.shared_pages = int(shared_pages)
+        self.kv_dtype = kv_dtype
         self.per_sequence = False
         self.token_bytes = int(token_bytes) if token_bytes is not None else 2 * int(num_kv_heads) * HEAD_DIM * 2
         _need(0 <= self.shared_pages <= block_table.shape[1], "shared_pages out of range")
@@ -317,7 +329,13 @@ class DecodePlan:
         self.num_q_heads, self.num_kv_heads = int(num_q_heads), int(num_kv_heads)
         self.num_pages, self.page_size = int(num_pages), int(page_size)
         self.bt_stride = int(self.block_table.stride(0))
-        self.chunks = int(chunks) if chunks is not None else balanced_chunks(num_kv_heads)
+        if chunks is not None:
+            self.chunks = int(chunks)
+        elif self.shared_pages > 0 and block_table.shape[0] > 0:
+            self.chunks = prefix_chunks(block_table.shape[0], num_q_heads, num_kv_heads, self.shared_pages, page_size,
+                                        fp16_pool=kv_dtype in (None, torch.float16))
+        else:
+            self.chunks = balanced_chunks(num_kv_heads)
         dev = self.block_table.device
         self.plan_bytes = int(lib.litekv_decode_plan_bytes_paged(self.batch, self.bt_stride, self.num_kv_heads,
                                                                  self.chunks, self.page_size))
@@ -515,7 +533,8 @@ def paged_decode(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Tens
         _need(stage == "both", "the balanced schedule is a single launch")
         _need(k_new is None, "the balanced schedule appends through decode_step")
         if plan is None:
-            plan = DecodePlan(block_table, seq_lens, hq, hkv, n_pages, chunks, page_size, shared_pages)
+            plan = DecodePlan(block_table, seq_lens, hq, hkv, n_pages, chunks, page_size, shared_pages,
+                              kv_dtype=kv_pool.dtype)
         return decode_step(q, kv_pool, plan, None, None, softmax_scale, out, kv_scales)
 
     fp8 = is_quantised_pool(kv_pool)
