@@ -69,7 +69,7 @@ def _hipcc() -> str:
 
 
 def _headers() -> list[Path]:
-    return sorted(CSRC.glob("*.h")) + sorted((CSRC.parents[1] / "include").glob("*.h"))
+    return sorted(CSRC.glob("*.h")) + sorted(CSRC.glob("*.inc")) + sorted((CSRC.parents[1] / "include").glob("*.h"))
 
 
 def is_stale() -> bool:

@@ -64,6 +64,7 @@ struct HeadSlice {
 };
 // Slice `hv` of the launch's kv_heads * slices slices (slices of one kv head are neighbours).
 __host__ __device__ __forceinline__ HeadSlice head_slice(int hv, int slices, int group) {
+  if (slices == 1) return HeadSlice{hv, hv * group, group};  // the usual case, without the divisions
   const int kv = hv / slices, sub = hv - kv * slices;
   const int per = (group + slices - 1) / slices;
   const int left = group - sub * per;

@@ -987,12 +987,14 @@ __global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merg
 constexpr int kBalancedVstageBytes = kMaxWavesPerWg * kPageSize * kVPitch * (int)sizeof(half_t);
 constexpr int kBalancedLdsBytes = kBalancedVstageBytes + kMaxWavesPerWg * kParkFloats * (int)sizeof(float);
 
-// The body of the balanced kernel, run by the workgroup that stands at (block_x, block_y) of its
-// grid; `lds` is its kBalancedLdsBytes of LDS (16-byte aligned). A function, so that the decode
-// step with a shared prefix can run it as one role of a launch that also attends the prefix.
+// What a workgroup of the balanced kernel does is in balanced_body.inc. It is compiled into the
+// kernel below and into this function, which the kernel of a step behind a shared prefix
+// (prefix_step_kernel) runs as one of its two roles, on the workgroup standing at (block_x,
+// block_y) of the balanced grid and with its two LDS areas.
 template <int DEPTH, int KV>
 __device__ __forceinline__ void balanced_body(
-    char *lds, const int block_x, const int block_y,
+    half_t (*vstage_all)[kPageSize * kVPitch], float (*park_all)[kParkFloats], const int block_x,
+    const int block_y,
     const half_t *__restrict__ q, int64_t q_batch_stride,
     typename KvStore<KV>::elem *__restrict__ kv, const float *__restrict__ scales,
     const int32_t *__restrict__ seq_lens, const int32_t *__restrict__ plan,
@@ -1001,340 +1003,7 @@ __device__ __forceinline__ void balanced_body(
     float *__restrict__ part_lse, int32_t bt_stride, int32_t batch, int32_t num_q_heads,
     int32_t num_kv_heads, int32_t group_all, int32_t slices, int32_t heads_per_wg,
     int32_t replicas, int32_t chunks, int32_t skip, float scale_log2) {
-  half_t(*vstage_all)[kPageSize * kVPitch] = reinterpret_cast<half_t(*)[kPageSize * kVPitch]>(lds);
-  float(*park_all)[kParkFloats] = reinterpret_cast<float(*)[kParkFloats]>(lds + kBalancedVstageBytes);
-
-  // readfirstlane tells the compiler the wavefront index is uniform (scalar branches and loads)
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int lane = threadIdx.x & 63;
-  const int n = lane & 15;
-  const int g = lane >> 4;
-  // a wavefront per head slice: the kv head itself, or up to 16 of its query heads when it has
-  // more than 16 (see head_slice)
-  const int hv = block_y * heads_per_wg + wave % heads_per_wg;
-  const int cidx = block_x * replicas + wave / heads_per_wg;
-  if (hv >= num_kv_heads * slices || cidx >= chunks) return;  // whole wavefront; no workgroup barriers below
-  const HeadSlice hs = head_slice(hv, slices, group_all);
-  const int h = hs.kv_head;
-  const int group = hs.q_heads;
-  half_t *vstage = vstage_all[wave];
-
-  // Empty sequences are on no chunk's line: chunk c zeroes the rows of sequences c, c + chunks, ...
-  // Like every store of this kernel it comes after the page loop (see park_state).
-  auto zero_empty_rows = [&]() {
-    for (int bz = cidx; bz < batch; bz += chunks) {
-      if (seq_lens[bz] <= 0 && n < group) {
-        half_t *o = out + ((int64_t)bz * num_q_heads + hs.q_head0 + n) * kHD + 4 * g;
-#pragma unroll
-        for (int j = 0; j < kJTiles; ++j) *(half4_t *)(o + 16 * j) = half4_t{0, 0, 0, 0};
-      }
-    }
-  };
-
-  const int entry_stride = plan_entry_stride(batch, bt_stride, chunks);
-  const uniform_i32_ptr lens = as_uniform(seq_lens);
-  const uniform_i32_ptr entry =
-      as_uniform(plan) + plan_entries_offset(batch) + (int64_t)cidx * entry_stride;
-  const int f0 = entry[0];
-  const int f1 = entry[1];
-  if (f1 <= f0) {
-    zero_empty_rows();
-    return;
-  }
-  const int seq_word = entry[2];
-  int cur_b = seq_word & 0xffff;
-  const int ahead_b = (int)((uint32_t)seq_word >> 16);  // the next sequence with pages, or batch
-  int cu_lo = entry[3];  // current sequence: [first, last) page on the line
-  int cu_hi = entry[4];
-  int len_b = entry[7];
-  const uniform_i32_ptr page_ids = entry + kEntryHeader;
-  // The first DEPTH ids are read at fixed offsets (an entry always has room for them), in the
-  // same round trip as the header, and clamped afterwards: one dependent hop less before the
-  // first K/V request.
-  static_assert(DEPTH <= 4, "an entry is only guaranteed to hold kEntryHeader + 4 words");
-  int first_ids[DEPTH];
-#pragma unroll
-  for (int dd = 0; dd < DEPTH; ++dd) first_ids[dd] = page_ids[dd];
-#pragma unroll
-  for (int dd = 1; dd < DEPTH; ++dd) first_ids[dd] = dd < f1 - f0 ? first_ids[dd] : first_ids[dd - 1];
-
-  // Read ahead for the crossing. Everything the first requests need came with the entry: this
-  // second hop is under way while they are issued.
-  // (the lengths of the next kLensAhead sequences: a scalar load issued at a crossing is waited
-  // for by the next LDS wait of the page loop, its whole latency exposed)
-  constexpr int kLensAhead = 2;
-  int lens_ahead[kLensAhead];
-  auto fetch_lens_ahead = [&]() {
-#pragma unroll
-    for (int i = 0; i < kLensAhead; ++i) {
-      lens_ahead[i] = lens[cur_b + 1 + i < batch ? cur_b + 1 + i : batch - 1];
-    }
-#pragma unroll
-    for (int i = 0; i < kLensAhead; ++i) lens_ahead[i] = cur_b + 1 + i < batch ? lens_ahead[i] : 0;
-  };
-  fetch_lens_ahead();
-  int lens_left = kLensAhead;
-
-  constexpr bool FP8 = KV != kKvF16;  // 8-bit codes (either format): the layout they share
-  typedef typename KvStore<KV>::elem Elem;
-  typedef typename KvStore<KV>::page Page;
-  // fp8 pool: the K scale joins the softmax scale, the V scale the final normalisation, and the
-  // step's new rows are quantised with the reciprocals
-  float k_inv = 1.0f, v_inv = 1.0f, v_scale = 1.0f;
-  if constexpr (FP8) {
-    const float ks = scales[h];
-    v_scale = scales[num_kv_heads + h];
-    scale_log2 *= ks;
-    k_inv = 1.0f / ks;
-    v_inv = 1.0f / v_scale;
-  }
-
-  const int hq0 = hs.q_head0;
-  const int64_t row_stride = (int64_t)2 * num_kv_heads * kHD;
-  // this lane's row and column inside page 0 (see PageRegs / PageRegsFp8)
-  Elem *k_lane = kv + (int64_t)h * kHD + (FP8 ? 16 : 8) * g + n * row_stride;
-  Elem *v_lane = FP8 ? kv + (int64_t)(num_kv_heads + h) * kHD + 16 * (n & (kHD / 16 - 1)) +
-                           (2 * g + (n >> 3)) * row_stride
-                     : kv + (int64_t)(num_kv_heads + h) * kHD + 8 * (n & (kVCols - 1)) + g * row_stride;
-  const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
-  half8_t qf[4];
-  auto fetch_q_into = [&](half8_t (&dst)[4], int b) {
-    const half_t *row0 = q + (int64_t)b * q_batch_stride + (int64_t)hq0 * kHD;
-    if constexpr (FP8) {
-      load_q_fp8_order(dst, row0, n, g, group);
-    } else {
-      load_q(dst, row0, n, g, group);
-    }
-  };
-  // This lane's parts of the step's new K and V rows of sequence b (see the fused append below).
-  auto fetch_new_rows = [&](uint4_t (&kr)[4], uint4_t (&vr)[2], int b) {
-    const half_t *kn = k_new + (int64_t)b * k_new_stride + (int64_t)h * kHD;
-    const half_t *vn = v_new + (int64_t)b * v_new_stride + (int64_t)h * kHD;
-    if constexpr (FP8) {
-#pragma unroll
-      for (int j = 0; j < kHD / 64; ++j) {
-        kr[2 * j] = *(const uint4_t *)(kn + 64 * j + 16 * g);
-        kr[2 * j + 1] = *(const uint4_t *)(kn + 64 * j + 16 * g + 8);
-      }
-      vr[0] = *(const uint4_t *)(vn + 16 * (n & (kHD / 16 - 1)));
-      vr[1] = *(const uint4_t *)(vn + 16 * (n & (kHD / 16 - 1)) + 8);
-    } else {
-#pragma unroll
-      for (int kk = 0; kk < kKSteps; ++kk) kr[kk] = *(const uint4_t *)(kn + 32 * kk + 8 * g);
-      vr[0] = *(const uint4_t *)(vn + 8 * (n & (kVCols - 1)));
-      vr[1] = uint4_t{0, 0, 0, 0};  // fp8 only
-    }
-  };
-
-  // Page ids travel through scalar loads, one request ahead of their use.
-  int pid_next = 0;
-  int pid_held[DEPTH];  // the ids of the pages in flight, by buffer (the fused append needs one)
-  auto request = [&](int i, Page &r, int &held) {  // i = page index inside the chunk
-    held = pid_next;
-    const int64_t page_off = (int64_t)pid_next * kPageSize * row_stride;
-    const int nx = i + 1 < f1 - f0 ? i + 1 : f1 - f0 - 1;
-    pid_next = page_ids[nx];
-    request_page(r, k_lane, v_lane, page_off, row_stride);
-  };
-
-  HeadState st;
-  st.reset();
-  fetch_q_into(qf, cur_b);
-  // What the first sequence crossing and the first fused append of the chunk need is requested
-  // here, unconditionally and before the pages (loads return in order: by the time a page has
-  // arrived these have too), so neither waits for a load it has just issued. Later crossings and
-  // appends of the same chunk (sequences shorter than a chunk) load and wait. The registers are
-  // written once, outside the loop: written in a rarely taken branch of it they become
-  // two-versioned at the loop's join and the compiler copies them on every page.
-  uint4_t q_ahead[4];  // raw dwords: as fp16 vectors the compiler splits them into halves up here
-  uint4_t k_ahead[4];
-  uint4_t v_ahead[2];
-  {
-    // Every lane loads, lanes past the group the group's last head: their columns are computed
-    // and never stored. A load under a lane condition is merged with its zero default through
-    // register copies that wait for it, here in front of the first page requests.
-    const int nn = n < group ? n : group - 1;
-    const half_t *row = q + (int64_t)(ahead_b < batch ? ahead_b : cur_b) * q_batch_stride +
-                        (int64_t)(hq0 + nn) * kHD + (FP8 ? 16 : 8) * g;
-#pragma unroll
-    for (int kk = 0; kk < kKSteps; ++kk) {  // the d order of load_q / load_q_fp8_order
-      q_ahead[kk] = *(const uint4_t *)(row + (FP8 ? 64 * (kk >> 1) + 8 * (kk & 1) : 32 * kk));
-    }
-  }
-  const int rows_b = k_new != nullptr ? cur_b : -1;
-  if (k_new != nullptr) fetch_new_rows(k_ahead, v_ahead, cur_b);
-
-  auto flush = [&]() {
-    // the sequence lies inside this chunk and has no shared-prefix partials to merge with
-    const bool whole = cu_lo >= f0 && cu_hi <= f1 && skip == 0;
-    const int64_t cell = (int64_t)(cidx + cur_b) * num_q_heads + hq0;
-    half_t *out_row = out + ((int64_t)cur_b * num_q_heads + hq0) * kHD;
-    store_state(st, whole, out_row, part_o + cell * kHD, kHD, part_lse + cell, 1, n, g,
-                group, v_scale);
-  };
-  // A sequence that ends inside the chunk is parked (see park_state) and written with the
-  // chunk's last one; a second one ending in the same chunk first sends the parked one off.
-  float *park = park_all[wave];
-  int parked_b = -1;
-  bool parked_whole = false;
-  auto unpark = [&]() {
-    const int64_t cell = (int64_t)(cidx + parked_b) * num_q_heads + hq0;
-    half_t *out_row = out + ((int64_t)parked_b * num_q_heads + hq0) * kHD;
-    unpark_state(park, parked_whole, out_row, part_o + cell * kHD, part_lse + cell, n, g, group);
-    parked_b = -1;
-  };
-  auto flush_at_crossing = [&]() {
-    if (group > kParkHeads) {
-      flush();
-      return;
-    }
-    if (parked_b >= 0) unpark();
-    park_state(st, park, n, g, group, v_scale);
-    parked_b = cur_b;
-    parked_whole = cu_lo >= f0 && cu_hi <= f1 && skip == 0;
-  };
-
-  // Stores the step's new fp16 rows (the lanes that own them in a page's registers).
-  auto store_new_rows = [&](const uint4_t (&k_row)[4], const uint4_t (&v_row)[2], int64_t slot_off,
-                            int t_new) {
-    if constexpr (!FP8) {
-      if (n == t_new) {
-        half_t *dst = kv + slot_off + (int64_t)h * kHD + 8 * g;
-#pragma unroll
-        for (int kk = 0; kk < kKSteps; ++kk) *(uint4_t *)(dst + 32 * kk) = k_row[kk];
-      }
-      if (g == (t_new & 3)) {
-        *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHD + 8 * (n & (kVCols - 1))) = v_row[0];
-      }
-    }
-  };
-  // In an fp16 pool the rows requested ahead (the chunk's first sequence) are stored after the
-  // page loop, for the reason a finished state is parked: a store in the middle of the chunk
-  // delays every later counted wait by its acknowledgement (C2: -0.25 us per layer). The page's
-  // registers are patched where it is attended. With 8-bit codes the rows kept for the end cost
-  // 30 registers and the step is 0.3 to 1.5 us slower: those are stored where they are appended.
-  int late_row = -1;  // the pool row (page * 16 + token) they go to
-
-  Page buf[DEPTH];
-#pragma unroll
-  for (int dd = 0; dd < DEPTH; ++dd) {
-    pid_next = first_ids[dd];
-    pid_held[dd] = 0;
-    if (dd < f1 - f0) request(dd, buf[dd], pid_held[dd]);
-  }
-  // after the prologue pid_next holds the id of page DEPTH (clamped), as the loop expects
-  for (int f = f0; f < f1; f += DEPTH) {
-    // Keep the wavefronts of the workgroup (the kv heads of one chunk) in step: the hardware
-    // favours the older wavefront of each SIMD, the favoured half would finish a third earlier
-    // and leave the memory system half loaded for the rest of the launch. A wavefront that has
-    // left the kernel no longer counts at the barrier, so unequal chunk lengths are harmless.
-    __builtin_amdgcn_s_barrier();
-#pragma unroll
-    for (int dd = 0; dd < DEPTH; ++dd) {
-      const int ff = f + dd;
-      if (ff < f1) {
-        if (ff >= cu_hi) {  // the line enters the next non-empty sequence
-          flush_at_crossing();
-          do {
-            if (lens_left == 0) {
-              fetch_lens_ahead();
-              lens_left = kLensAhead;
-            }
-            ++cur_b;
-            --lens_left;
-            len_b = lens_ahead[0];
-#pragma unroll
-            for (int i = 0; i + 1 < kLensAhead; ++i) lens_ahead[i] = lens_ahead[i + 1];
-            int pg = pages_of(len_b);
-            pg = (pg < bt_stride ? pg : bt_stride) - skip;
-            pg = pg > 0 ? pg : 0;
-            cu_lo = cu_hi;
-            cu_hi += pg;
-          } while (ff >= cu_hi);
-          st.reset();
-          if (cur_b == ahead_b) {
-#pragma unroll
-            for (int kk = 0; kk < kKSteps; ++kk) qf[kk] = __builtin_bit_cast(half8_t, q_ahead[kk]);
-          } else {
-            fetch_q_into(qf, cur_b);
-            wait_vector_loads();
-          }
-        }
-        const int p = ff - cu_lo + skip;  // page index inside the sequence
-        if (k_new != nullptr && (p + 1) * kPageSize >= len_b) {
-          // Last page of the sequence: the step's new token (logical position len_b - 1) is
-          // appended here. Its K and V rows go to the pool and replace the stale values this
-          // wavefront requested before the write.
-          const int t_new = (len_b - 1) & (kPageSize - 1);
-          uint4_t k_row[4];
-          uint4_t v_row[2];
-          if (cur_b == rows_b) {
-#pragma unroll
-            for (int kk = 0; kk < kKSteps; ++kk) k_row[kk] = k_ahead[kk];
-            v_row[0] = v_ahead[0];
-            v_row[1] = v_ahead[1];
-          } else {
-            fetch_new_rows(k_row, v_row, cur_b);
-            wait_vector_loads();
-          }
-          const int64_t slot_off = ((int64_t)pid_held[dd] * kPageSize + t_new) * row_stride;
-          if constexpr (FP8) {
-            // the rows are quantised as the append kernel would, stored, and attended as stored
-            if (n == t_new) {
-              uint8_t *dst = kv + slot_off + (int64_t)h * kHD + 16 * g;
-#pragma unroll
-              for (int j = 0; j < kHD / 64; ++j) {
-                const uint2_t lo = half_to_codes<KV>(__builtin_bit_cast(half8_t, k_row[2 * j]), k_inv);
-                const uint2_t hi = half_to_codes<KV>(__builtin_bit_cast(half8_t, k_row[2 * j + 1]), k_inv);
-                const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
-                buf[dd].k[j] = x;
-                *(uint4_t *)(dst + 64 * j) = x;
-              }
-            }
-            if (2 * g + (n >> 3) == (t_new & 7)) {
-              const uint2_t lo = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[0]), v_inv);
-              const uint2_t hi = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[1]), v_inv);
-              const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
-              *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHD + 16 * (n & (kHD / 16 - 1))) = x;
-#pragma unroll
-              for (int i = 0; i < 2; ++i) {
-                if (i == (t_new >> 3)) buf[dd].v[i] = x;
-              }
-            }
-          } else {
-            if (n == t_new) {
-#pragma unroll
-              for (int kk = 0; kk < kKSteps; ++kk) buf[dd].k[kk] = __builtin_bit_cast(half8_t, k_row[kk]);
-            }
-            if (g == (t_new & 3)) {
-              const half8_t x = __builtin_bit_cast(half8_t, v_row[0]);
-#pragma unroll
-              for (int i = 0; i < 4; ++i) {
-                if (i == (t_new >> 2)) buf[dd].v[i] = x;
-              }
-            }
-            if (cur_b == rows_b) {  // from k_ahead / v_ahead, after the page loop
-              late_row = pid_held[dd] * kPageSize + t_new;
-            } else {
-              store_new_rows(k_row, v_row, slot_off, t_new);
-            }
-          }
-        }
-        attend_page(st, buf[dd], qf, vstage, vt_lane, p, len_b, n, g, scale_log2);
-      }
-      // Only pages of the chunk are requested. (Requests past its end used to be issued as loads
-      // of 16 bytes, so that the number of loads in flight was a compile-time constant and every
-      // wait named exactly the page it needed; with the condition the compiler's waits also
-      // cover part of the next page's loads, and the launch is still faster: C2 0.65 us per layer.)
-      if (ff + DEPTH < f1) request(ff - f0 + DEPTH, buf[dd], pid_held[dd]);
-    }
-  }
-  if (late_row >= 0) {
-    store_new_rows(k_ahead, v_ahead, (int64_t)late_row * row_stride, late_row & (kPageSize - 1));
-  }
-  flush();
-  if (parked_b >= 0) unpark();
-  zero_empty_rows();
+#include "balanced_body.inc"
 }
 
 template <int DEPTH, int KV>
@@ -1347,11 +1016,10 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void paged_decode_balanced_
     float *__restrict__ part_lse, int32_t bt_stride, int32_t batch, int32_t num_q_heads,
     int32_t num_kv_heads, int32_t group_all, int32_t slices, int32_t heads_per_wg,
     int32_t replicas, int32_t chunks, int32_t skip, float scale_log2) {
-  __shared__ __attribute__((aligned(16))) char lds[kBalancedLdsBytes];
-  balanced_body<DEPTH, KV>(lds, (int)blockIdx.x, (int)blockIdx.y, q, q_batch_stride, kv, scales, seq_lens,
-                           plan, k_new, v_new, k_new_stride, v_new_stride, out, part_o, part_lse,
-                           bt_stride, batch, num_q_heads, num_kv_heads, group_all, slices, heads_per_wg,
-                           replicas, chunks, skip, scale_log2);
+  __shared__ __attribute__((aligned(16))) half_t vstage_all[kMaxWavesPerWg][kPageSize * kVPitch];
+  __shared__ __attribute__((aligned(16))) float park_all[kMaxWavesPerWg][kParkFloats];
+  const int block_x = (int)blockIdx.x, block_y = (int)blockIdx.y;
+#include "balanced_body.inc"
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1405,7 +1073,9 @@ __global__ __launch_bounds__(kMaxWavesPerWg * kWave) void prefix_step_kernel(
     return;
   }
   const int d = id - prefix_wgs;
-  balanced_body<DEPTH, KV>(lds, d % decode_wgs_x, d / decode_wgs_x, q, q_batch_stride, kv, scales, seq_lens,
+  balanced_body<DEPTH, KV>(reinterpret_cast<half_t(*)[kPageSize * kVPitch]>(lds),
+                           reinterpret_cast<float(*)[kParkFloats]>(lds + kBalancedVstageBytes),
+                           d % decode_wgs_x, d / decode_wgs_x, q, q_batch_stride, kv, scales, seq_lens,
                            plan, k_new, v_new, k_new_stride, v_new_stride, out, part_o, part_lse,
                            bt_stride, batch, num_q_heads, num_kv_heads, group_all, slices, heads_per_wg,
                            replicas, chunks, skip, scale_log2);
