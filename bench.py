@@ -339,10 +339,12 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
         },
     }
     if shared_pages > 0:
-        # three launches share the work (prefix kernel, decode kernel, merge): the rate is taken over
-        # the layer's wall-clock share of the step instead of one kernel's duration
+        # two launches share the work (the two-role kernel that attends the shared pages and streams
+        # the private ones, then the merge): the rate is taken over the layer's wall-clock share of
+        # the step instead of one kernel's duration
+        res["prefix_step_kernel_us_mean"] = k_mean * 1e3
         k_mean = ms_per_step / layers
-        res["roofline"]["kernel"] = "shared prefix (varlen_prefill_tiled_kernel<2>) + paged_decode_balanced_kernel + merge"
+        res["roofline"]["kernel"] = "prefix_step_kernel (shared-prefix role + balanced role) + merge"
         res["roofline"]["duration_us"] = k_mean * 1e3
     unique = case.unique_decode_bytes() + (append_bytes if balanced else 0)
     if kv_dtype in ("fp8", "int8"):
@@ -574,14 +576,17 @@ def run_prefill(case, steps: int, warmup: int, device: str, label: str) -> dict:
     }
 
 
-def cpu_baseline_decode(case, budget_s: float = 10.0, max_sequences=None) -> dict:
+def cpu_baseline_decode(case, budget_s: float = 10.0, max_sequences=None, kv_dtype: str = "f16") -> dict:
     """The reference's torch CPU path (append + gathered fp32 attention) for ONE layer of `case`,
     on the host cores: 1 warm-up, then repetitions for about `budget_s` seconds, min taken.
     `max_sequences`: time only the first that many sequences and scale the rate as measured (the
     result is then flagged as extrapolated; the pool stays on the GPU side, only those sequences'
-    pages are brought to the host)."""
+    pages are brought to the host). `kv_dtype` fp8 / int8: the pool holds 8-bit codes, the CPU
+    path quantises the appended rows, decodes the pool's codes (oracle/fp8.py, oracle/int8.py) and
+    attends the decoded values; the rate is over the 8-bit algorithmic bytes."""
+    import numpy as np
     import torch
-    from oracle import cpu_ref
+    from oracle import cpu_ref, fp8 as fp8_codec, int8 as int8_codec
 
     cores = _host_threads()
     torch.set_num_threads(cores)
@@ -592,11 +597,26 @@ def cpu_baseline_decode(case, budget_s: float = 10.0, max_sequences=None) -> dic
         c = case.to("cpu")
     kv = torch.cat([c.k_new, c.v_new], dim=1)
     pool = c.kv_pool
+    q8 = kv_dtype in ("fp8", "int8")
+    if q8:
+        codec = fp8_codec if kv_dtype == "fp8" else int8_codec
+        scales = np.full(2 * c.num_kv_heads, 0.02, dtype=np.float32)
+        rng = np.random.default_rng(4242)     # random codes, as the GPU leg's pools hold (no NaN codes, no -128)
+        if kv_dtype == "fp8":
+            codes = rng.integers(0, 0x7F, size=tuple(pool.shape), dtype=np.uint8)
+        else:
+            codes = rng.integers(-127, 128, size=tuple(pool.shape), dtype=np.int8)
+        k_new, v_new, slots = c.k_new.numpy(), c.v_new.numpy(), c.slot_mapping.numpy()
 
     def one():
         t0 = time.perf_counter()
-        cpu_ref.kv_append_ref(kv, c.slot_mapping, pool)
-        cpu_ref.paged_decode_ref(c.q, pool, c.block_table, c.seq_lens, c.softmax_scale)
+        if q8:
+            codec.kv_append(k_new, v_new, slots, codes, scales)
+            values = torch.from_numpy(codec.dequantize_pool(codes, scales))
+            cpu_ref.paged_decode_ref(c.q, values, c.block_table, c.seq_lens, c.softmax_scale)
+        else:
+            cpu_ref.kv_append_ref(kv, c.slot_mapping, pool)
+            cpu_ref.paged_decode_ref(c.q, pool, c.block_table, c.seq_lens, c.softmax_scale)
         return time.perf_counter() - t0
 
     first = one()
@@ -610,6 +630,10 @@ def cpu_baseline_decode(case, budget_s: float = 10.0, max_sequences=None) -> dic
         t_used += dt
     best = min(times) if times else first
     nbytes = c.decode_bytes() + c.append_bytes()
+    whole = case.decode_bytes() + case.append_bytes()
+    if q8:   # one byte per cached element (see run_decode)
+        nbytes -= int(c.seq_lens.sum()) * c.tok_bytes // 2 + c.batch * c.tok_bytes // 2
+        whole -= int(case.seq_lens.sum()) * case.tok_bytes // 2 + case.batch * case.tok_bytes // 2
     return {
         "value": nbytes / best / 1e9,
         "unit": "GB/s",
@@ -618,10 +642,11 @@ def cpu_baseline_decode(case, budget_s: float = 10.0, max_sequences=None) -> dic
         "cpu_model": _cpu_model(),
         "sample": (f"the first {c.batch} of {case.batch} sequences of one layer (rate extrapolated to the "
                    f"whole layer), " if extrapolated else "1 of the layers of the same workload, ")
-                  + f"append + decode, {nbytes / 1e6:.1f} MB algorithmic, torch CPU restatement, "
+                  + (f"quantising append + decoding the {kv_dtype} pool + decode, " if q8 else "append + decode, ")
+                  + f"{nbytes / 1e6:.1f} MB algorithmic, torch CPU restatement, "
                     f"min of {max(1, len(times))} reps after 1 warm-up, {best:.3f} s",
         "extrapolated": extrapolated,
-        "seconds_per_layer": best * (case.decode_bytes() + case.append_bytes()) / nbytes,
+        "seconds_per_layer": best * whole / nbytes,
     }
 
 
@@ -654,7 +679,8 @@ def _first_sequences(case, n: int):
 CONFIGS = ("c1", "c2", "c3", "c4", "c5")
 
 
-def measure(name: str, args, device: str, cpu_budget_s: float, schedule=None) -> dict:
+def measure(name: str, args, device: str, cpu_budget_s: float, schedule=None, kv_dtype=None,
+            cpu: bool = True) -> dict:
     """One configuration measured in full: the step (value, ms_per_step), the roofline of its
     dominant kernel(s), the launches beside it, and the CPU baseline, in the schema of the
     headline line."""
@@ -677,7 +703,7 @@ def measure(name: str, args, device: str, cpu_budget_s: float, schedule=None) ->
         shared = 0
         if schedule == "balanced" and not args.no_shared_prefix and not case.extra.get("private_prefix"):
             shared = int(case.extra.get("n_shared", 0))
-        kv_dtype = args.kv_dtype if schedule == "balanced" else "f16"
+        kv_dtype = (kv_dtype or args.kv_dtype) if schedule == "balanced" else "f16"
         res = run_decode(case, layers, steps, warmup, device, case.name, schedule, shared,
                          graph=not args.no_graph, kv_dtype=kv_dtype)
     traffic, stamp = measured_traffic(name, schedule, kv_dtype)
@@ -718,8 +744,9 @@ def measure(name: str, args, device: str, cpu_budget_s: float, schedule=None) ->
             row["detail"].update(cow_step(case))
         if name == "c5" and schedule == "balanced":
             row["detail"].update(compaction_step(case))
-        if not args.no_cpu_baseline:
-            row["cpu_baseline"] = cpu_baseline_decode(case, cpu_budget_s, max_sequences=8 if name == "c5" else None)
+        if cpu and not args.no_cpu_baseline:
+            row["cpu_baseline"] = cpu_baseline_decode(case, cpu_budget_s, max_sequences=8 if name == "c5" else None,
+                                                      kv_dtype=kv_dtype)
     else:
         row["pct_of_mfma_peak"] = 100.0 * res["roofline"]["frac"]
         row["detail"].update(time_qk_epilogue(int(case.seq_lens.sum()), case.num_q_heads, case.num_kv_heads,
@@ -818,8 +845,13 @@ def main() -> int:
                 continue
             others[name] = measure(name, args, device, cpu_budget_s=3.0)
             if name == "c5":
-                others["c5_16_splits"] = measure("c5", args, device, cpu_budget_s=0.0, schedule="splits")
-                others["c5_16_splits"].pop("cpu_baseline", None)   # the same CPU work as c5
+                others["c5_16_splits"] = measure("c5", args, device, cpu_budget_s=0.0, schedule="splits", cpu=False)
+                if "cpu_baseline" in others["c5"]:   # the CPU path has one schedule: the same work, timed once
+                    others["c5_16_splits"]["cpu_baseline"] = dict(others["c5"]["cpu_baseline"])
+        if args.config == "c2" and args.kv_dtype == "f16":
+            # the headline workload over pools of 8-bit codes (half the K/V bytes per token)
+            for q8 in ("fp8", "int8"):
+                others[f"c2_{q8}"] = measure("c2", args, device, cpu_budget_s=3.0, kv_dtype=q8)
         rows.update(others)
         line["detail"]["configs"] = others
     print(json.dumps(line), flush=True)
