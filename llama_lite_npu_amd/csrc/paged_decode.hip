@@ -1630,6 +1630,9 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
     LITEKV_REQUIRE(block_table != nullptr, "%s: block_table is null", what);
     LITEKV_REQUIRE(num_kv_heads <= 1024, "%s: num_kv_heads %d > 1024", what, num_kv_heads);
     LITEKV_REQUIRE(shared_pages <= (1 << 20), "%s: shared_pages %d out of range", what, shared_pages);
+    // the prefix role numbers its partial rows (slice, sequence, head) in 32 bits
+    LITEKV_REQUIRE((int64_t)kMaxPrefixSplits * batch * num_q_heads < 0x7fffffffLL,
+                   "%s: batch %d x %d query heads too large for a shared prefix", what, batch, num_q_heads);
     const PrefixShape ps = prefix_shape(batch, group, num_kv_heads, shared_pages << shift,
                                         fp8_scales == nullptr, (int)(block.x / kWave));
     const int64_t total_wgs = (int64_t)ps.wgs + (int64_t)wgs * s.head_groups;

@@ -862,28 +862,56 @@ __device__ __forceinline__ void prefill_tile_body(
     }
     return;
   }
+  if constexpr (SHARED) {
+    // The partial rows (fp32, normalised) leave as whole rows like the output of a prefill block:
+    // a lane holds 4 consecutive elements of each of its column's 16-element groups, so stored
+    // straight from registers one instruction would touch 16 rows with 64 bytes each. One column
+    // tile at a time goes through this wavefront's part of the K/V staging area (the tiles are
+    // done with) and leaves 1 KiB per instruction.
+    constexpr int kPartPitch = 4 * kHD + 16;           // bytes; rows 4 banks apart: a 16-lane group's writes hit 64 banks
+    constexpr int kRowLanes = kHD / 4;                 // lanes that carry one row (16 bytes each)
+    constexpr int kRowsPerStore = kWave / kRowLanes;   // rows one store instruction writes
+    __syncthreads();                                   // every wavefront is done reading the last tile
+    const uint32_t mine = k_lds + (uint32_t)(wave * 16 * kPartPitch);
+    typedef __attribute__((address_space(3))) float4_t lds_float4_t;
+#pragma unroll
+    for (int u = 0; u < kColTiles; ++u) {
+      const float inv = v_scale / dsum[u][0];
+      // the partial row of this lane's column (the same in its four lane groups), or -1
+      const int cell = out_row[u] >= 0
+                           ? (block_z * prefix.batch + out_row[u]) * prefix.num_q_heads + out_head[u]
+                           : -1;
+      if (g == 0 && cell >= 0) {
+        // read once, by the merge launch: streaming stores (see store_state in paged_decode.hip)
+        __builtin_nontemporal_store((m_run[u] + fast_log2(dsum[u][0])) * 0.6931471805599453f,
+                                    prefix.part_lse + cell);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the reads of the tile before are done
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int j = 0; j < kJTiles; ++j) {
+        *(lds_float4_t *)(uintptr_t)(mine + (uint32_t)(n * kPartPitch + 4 * (16 * j + 4 * g))) =
+            float4_t{acc[j][u][0] * inv, acc[j][u][1] * inv, acc[j][u][2] * inv, acc[j][u][3] * inv};
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int step = 0; step < 16 / kRowsPerStore; ++step) {
+        const int r = kRowsPerStore * step + lane / kRowLanes;      // column of the tile = row staged
+        const int c = lane % kRowLanes;
+        const int row_cell = __shfl(cell, r, kWave);
+        const float4_t x = *(const lds_float4_t *)(uintptr_t)(mine + (uint32_t)(r * kPartPitch + 16 * c));
+        if (row_cell >= 0) {
+          __builtin_nontemporal_store(x, (float4_t *)(prefix.part_o + (int64_t)row_cell * kHD + 4 * c));
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int u = 0; u < kColTiles; ++u) {
     const float inv = v_scale / dsum[u][0];
-    if constexpr (SHARED) {
-      if (out_row[u] >= 0) {
-        const int64_t cell =
-            ((int64_t)block_z * prefix.batch + out_row[u]) * prefix.num_q_heads + out_head[u];
-        float *po = prefix.part_o + cell * kHD + 4 * g;
-#pragma unroll
-        for (int j = 0; j < kJTiles; ++j) {
-          // read once, by the merge launch: streaming stores (see store_state in paged_decode.hip)
-          __builtin_nontemporal_store(float4_t{acc[j][u][0] * inv, acc[j][u][1] * inv,
-                                               acc[j][u][2] * inv, acc[j][u][3] * inv},
-                                      (float4_t *)(po + 16 * j));
-        }
-        if (g == 0) {
-          __builtin_nontemporal_store((m_run[u] + fast_log2(dsum[u][0])) * 0.6931471805599453f,
-                                      prefix.part_lse + cell);
-        }
-      }
-      continue;
-    }
     if (out_row[u] >= 0) {
       half_t *o = out + (int64_t)out_row[u] * out_stride + (int64_t)out_head[u] * kHD + 4 * g;
 #pragma unroll
