@@ -5,13 +5,17 @@
 // (lite_llama/models/model_config.py:200); this is that generality, with plain fp32 arithmetic
 // instead of MFMA tiles.
 //
-// One wavefront per (kv head, query row): decode has one query row per sequence, prefill one per
-// prompt token (row i of a sequence sees its history and keys 0..i of the prompt). The wavefront
-// walks the row's keys 64 at a time. Scores: lane l holds key l of the tile, reads that key's K
-// row once and takes its dot product with the (up to 16) query heads of the kv head, whose rows
+// One wavefront per (kv head, block of query rows). It works on 16 columns, a column being one
+// (query row, query head of the kv head) pair: a decode step has one query row per sequence, so
+// its columns are the (up to 16) query heads of the kv head; a prefill block takes
+// 16 / (query heads per kv head) neighbouring prompt rows, so that the K and V rows they share
+// are read once for all of them (row i of a sequence sees its history and keys 0..i of the
+// prompt: each column has its own number of keys). The wavefront walks the keys of the block's
+// last row 64 at a time. Scores: lane l holds key l of the tile, reads that key's K
+// row once and takes its dot product with the columns' query rows, which
 // sit in LDS as fp32, already multiplied by softmax_scale * log2(e). Softmax state (running
-// maximum and denominator per head) is kept by every lane alike. Values: the probabilities of
-// the tile go through LDS, lane l then holds output elements l, l + 64, ... of every head and
+// maximum and denominator per column) is kept by every lane alike. Values: the probabilities of
+// the tile go through LDS, lane l then holds output elements l, l + 64, ... of every column and
 // adds the tile's V rows, read one row per step by all lanes together.
 //
 // Pools of 8-bit codes are read as in the tuned kernels: codes become fp16 exactly, the K scale
@@ -52,6 +56,7 @@ struct GenericTask {
   const half_t *k_new, *v_new; // [B][Hkv][D]
   int64_t k_new_stride, v_new_stride;
   int32_t num_q_heads, num_kv_heads, group, head_dim;
+  int32_t rows_per_wave;       // query rows of one sequence a wavefront takes (1 for a decode step)
   float scale_log2;
 };
 
@@ -84,8 +89,9 @@ __device__ __forceinline__ void store8(void *row, int d8, half8_t x, float inv_s
   }
 }
 
-// grid (head slices, query rows per sequence, sequences), one wavefront each; a head slice is a
-// kv head, or up to 16 of its query heads when it has more than 16 (see head_slice)
+// grid (head slices, blocks of rows_per_wave query rows per sequence, sequences), one wavefront
+// each; a head slice is a kv head, or up to 16 of its query heads when it has more than 16 (see
+// head_slice)
 template <int KV>
 __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t) {
   __shared__ float qs[kGenericMaxGroup][kGenericMaxDim];
@@ -93,35 +99,56 @@ __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t)
   const int lane = threadIdx.x;
   const HeadSlice hs = head_slice((int)blockIdx.x, head_slices(t.group), t.group);
   const int h = hs.kv_head;
-  const int row_in_seq = blockIdx.y;
+  const int row0 = blockIdx.y * t.rows_per_wave;  // first query row of the block in its sequence
   const int b = blockIdx.z;
   const int D = t.head_dim;
-  const int group = hs.q_heads;
   const bool paged = t.kv_pool != nullptr;
 
-  // the query row, the number of keys it sees, and where its sequence's packed keys start
-  int64_t q_row;
-  int n_keys;
+  // the block's first query row, the keys that row sees, how many rows the block holds, and
+  // where its sequence's packed keys start
+  int64_t q_row0;
+  int keys0;
+  int rows_here = 1;
   int64_t packed0 = 0;
   if (t.cu_q_lens != nullptr) {
     const int q_start = t.cu_q_lens[b];
-    if (row_in_seq >= t.cu_q_lens[b + 1] - q_start) return;
-    q_row = q_start + row_in_seq;
-    n_keys = (t.context_lens ? t.context_lens[b] : 0) + row_in_seq + 1;
+    const int q_len = t.cu_q_lens[b + 1] - q_start;
+    if (row0 >= q_len) return;
+    rows_here = q_len - row0 < t.rows_per_wave ? q_len - row0 : t.rows_per_wave;
+    q_row0 = q_start + row0;
+    keys0 = (t.context_lens ? t.context_lens[b] : 0) + row0 + 1;
   } else if (t.q_lens != nullptr) {
-    if (row_in_seq >= t.q_lens[b]) return;
+    if (row0 >= t.q_lens[b]) return;
+    rows_here = t.q_lens[b] - row0 < t.rows_per_wave ? t.q_lens[b] - row0 : t.rows_per_wave;
     packed0 = t.seq_starts[b];
-    q_row = packed0 + row_in_seq;
-    n_keys = row_in_seq + 1;
+    q_row0 = packed0 + row0;
+    keys0 = row0 + 1;
   } else {
-    q_row = b;
-    n_keys = t.seq_lens[b];
+    q_row0 = b;
+    keys0 = t.seq_lens[b];
   }
   const int hq0 = hs.q_head0;
-  half_t *out_row = t.out + q_row * t.out_row_stride + (int64_t)hq0 * D;
-  if (n_keys <= 0) {  // an empty sequence of a decode step
-    for (int i = lane; i < group * D; i += kWave) out_row[i] = (half_t)0.f;
+  if (keys0 <= 0) {  // an empty sequence of a decode step
+    half_t *out_row = t.out + q_row0 * t.out_row_stride + (int64_t)hq0 * D;
+    for (int i = lane; i < hs.q_heads * D; i += kWave) out_row[i] = (half_t)0.f;
     return;
+  }
+  const int n_keys = keys0 + rows_here - 1;  // of the block's last row: the keys the wavefront walks
+
+  // Column g is query head g % heads_per_row of row g / heads_per_row of the block. A column
+  // past the block's rows or the slice's heads repeats column 0 and is not written.
+  const int heads_per_row = t.rows_per_wave > 1 ? kGenericMaxGroup / t.rows_per_wave : hs.q_heads;
+  const int cols = t.rows_per_wave > 1 ? kGenericMaxGroup : hs.q_heads;
+  int col_keys[kGenericMaxGroup];
+  bool col_written[kGenericMaxGroup];
+  int col_row[kGenericMaxGroup], col_head[kGenericMaxGroup];
+#pragma unroll
+  for (int g = 0; g < kGenericMaxGroup; ++g) {
+    const int r = g / heads_per_row, hd = g - r * heads_per_row;
+    col_written[g] = g < cols && r < rows_here && hd < hs.q_heads;
+    col_row[g] = col_written[g] ? r : 0;
+    col_head[g] = col_written[g] ? hd : 0;
+    col_keys[g] = keys0 + col_row[g];
   }
 
   float k_scale = 1.0f, v_scale = 1.0f;
@@ -131,8 +158,13 @@ __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t)
   }
   const float k_inv = 1.0f / k_scale, v_inv = 1.0f / v_scale;
 
-  const half_t *q_heads = t.q + q_row * t.q_row_stride + (int64_t)hq0 * D;
-  for (int i = lane; i < group * D; i += kWave) qs[i / D][i % D] = (float)q_heads[i] * t.scale_log2;
+#pragma unroll
+  for (int g = 0; g < kGenericMaxGroup; ++g) {
+    if (g < cols) {
+      const half_t *q_col = t.q + (q_row0 + col_row[g]) * t.q_row_stride + (int64_t)(hq0 + col_head[g]) * D;
+      for (int i = lane; i < D; i += kWave) qs[g][i] = (float)q_col[i] * t.scale_log2;
+    }
+  }
   __syncthreads();
 
   const int elem = KV == kKvF16 ? 2 : 1;  // bytes per stored element
@@ -211,7 +243,7 @@ __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t)
       }
 #pragma unroll
       for (int g = 0; g < kGenericMaxGroup; ++g) {
-        if (g < group) {
+        if (g < cols) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) s[g] += qs[g][8 * d8 + e] * (float)kv8[e];
         }
@@ -220,12 +252,14 @@ __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t)
     // softmax of the tile against the running state; probabilities to LDS
 #pragma unroll
     for (int g = 0; g < kGenericMaxGroup; ++g) {
-      if (g < group) {
-        const float sv = live ? s[g] * k_scale : -INFINITY;
+      if (g < cols) {
+        // a key past the column's own row is masked; key 0 is in every column's first tile, so
+        // the running maximum is finite from then on
+        const float sv = tok < col_keys[g] ? s[g] * k_scale : -INFINITY;
         float mx = sv;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
-        const float m_new = fmaxf(m[g], mx);  // finite: the tile holds at least one key
+        const float m_new = fmaxf(m[g], mx);
         const float alpha = fast_exp2(m[g] - m_new);
         const float p = fast_exp2(sv - m_new);
         float sum = p;
@@ -257,7 +291,7 @@ __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t)
           }
 #pragma unroll
           for (int g = 0; g < kGenericMaxGroup; ++g) {
-            if (g < group) acc[g][c] += ps[j][g] * val;
+            if (g < cols) acc[g][c] += ps[j][g] * val;
           }
         }
       }
@@ -267,12 +301,13 @@ __global__ __launch_bounds__(kWave) void generic_attention_kernel(GenericTask t)
 
 #pragma unroll
   for (int g = 0; g < kGenericMaxGroup; ++g) {
-    if (g < group) {
+    if (col_written[g]) {
       const float inv = v_scale / den[g];
+      half_t *out_col = t.out + (q_row0 + col_row[g]) * t.out_row_stride + (int64_t)(hq0 + col_head[g]) * D;
 #pragma unroll
       for (int c = 0; c < kGenericMaxDim / kWave; ++c) {
         const int d = lane + kWave * c;
-        if (d < D) out_row[(int64_t)g * D + d] = (half_t)(acc[g][c] * inv);
+        if (d < D) out_col[d] = (half_t)(acc[g][c] * inv);
       }
     }
   }
@@ -359,10 +394,20 @@ int launch_generic_attention(const char *what, const GenericLaunch &a) {
   t.num_kv_heads = a.num_kv_heads;
   t.group = group;
   t.head_dim = a.head_dim;
+  // a decode step has one query row per sequence; a prefill block takes as many rows as fit the
+  // 16 columns beside the (at most 16) query heads of a slice
+  const int slices = head_slices(group);
+  const int heads_per_slice = (group + slices - 1) / slices;
+  int rows_per_wave = 1;
+  if (a.cu_q_lens != nullptr || a.q_lens != nullptr) {
+    while (rows_per_wave * 2 * heads_per_slice <= kGenericMaxGroup) rows_per_wave *= 2;
+  }
+  t.rows_per_wave = rows_per_wave;
   t.scale_log2 = a.softmax_scale * 1.4426950408889634f;
   const int slice_heads = a.num_kv_heads * head_slices(group);
   LITEKV_REQUIRE(slice_heads <= 65535, "%s: num_q_heads %d too large", what, a.num_q_heads);
-  const dim3 grid((unsigned)slice_heads, (unsigned)a.rows_per_seq, (unsigned)a.batch);
+  const dim3 grid((unsigned)slice_heads, (unsigned)((a.rows_per_seq + rows_per_wave - 1) / rows_per_wave),
+                  (unsigned)a.batch);
   const hipStream_t stream = static_cast<hipStream_t>(a.stream);
   const int format = a.kv_pool != nullptr ? a.format : kKvF16;
   if (format == kKvInt8) {

@@ -184,6 +184,9 @@ def test_paged_prefill_page_sizes(page_size, hq, hkv, lens, ctx):
     (14, 2, [128, 77], None, 16),
     (32, 4, [100, 5, 96], [100, 31, 64], 32),       # chunks over cached history
     (16, 1, [70, 40], [17, 200], 64),
+    (8, 8, [45, 1, 18], [3, 70, 0], 16),            # no grouping: 16 query rows per wavefront at 32 / 256
+    (12, 3, [33, 64, 7], None, 32),                 # 4 heads per kv head: 4 rows per wavefront, ragged last blocks
+    (40, 2, [20, 9], [5, 0], 16),                   # 20 heads per kv head: two slices of 10, one row each
 ])
 def test_prefill_head_dims(head_dim, hq, hkv, lens, ctx, page_size):
     """Prefill at head dims 32, 64 and 256: prompts (paged and packed entry points agree bit for
