@@ -87,7 +87,11 @@ struct PageRegs {
 // dot product may run in any order as long as K and q agree, so a lane takes 16 consecutive
 // codes per load and MFMA step kk uses its lower or upper 8:
 //   k[j]: token n, d = 16*(g + 4*j) .. +15      step kk = 2*j + (0: lower, 1: upper 8 codes)
-//   v[i]: V row 8*i + 2*g + n/8, d = 16*(n%8) .. +15
+//   v[i]: V row 8*i + 2*g + n%2, d = 16*(n/2) .. +15
+// Neighbouring lanes hold the same column of two neighbouring rows: the 32 bytes a lane stages per
+// row (16 codes as fp16) then fall on different LDS banks for the eight lanes a 16-byte store
+// serves per cycle. (With eight neighbouring lanes on one row, 32 bytes apart, every such store
+// took two cycles: half of the kernel's LDS cycles were bank conflicts.)
 template <int KV>
 struct PageRegsQ8 {
   uint4_t k[2];
@@ -95,6 +99,8 @@ struct PageRegsQ8 {
 };
 
 // Storage of the pool a kernel reads: fp16, or the codes of format KV (kKvFp8, kKvInt8).
+__device__ __forceinline__ int q8_v_row(int n, int g) { return 2 * g + (n & 1); }  // inside its block of 8 rows
+__device__ __forceinline__ int q8_v_col(int n) { return n >> 1; }                 // in units of 16 codes
 template <int KV> struct KvStore { typedef uint8_t elem; typedef PageRegsQ8<KV> page; };
 template <> struct KvStore<kKvF16> { typedef half_t elem; typedef PageRegs page; };
 
@@ -162,7 +168,7 @@ __device__ __forceinline__ void request_page(PageRegs &r, const half_t *k_lane,
   for (int i = 0; i < 4; ++i) r.v[i] = __builtin_nontemporal_load((const half8_t *)(vr + i * v_step));
 }
 
-// fp8 pool: k_lane points at token n, code 16*g; v_lane at row 2*g + n/8, code 16*(n%8).
+// 8-bit pool: k_lane points at token n, code 16*g; v_lane at row q8_v_row, code 16*q8_v_col.
 template <int KV>
 __device__ __forceinline__ void request_page(PageRegsQ8<KV> &r, const uint8_t *k_lane,
                                              const uint8_t *v_lane, int64_t page_off,
@@ -270,14 +276,14 @@ __device__ __forceinline__ void attend_page(HeadState &st, const PageRegsQ8<KV> 
   attend_core(st, kf, qf, vt_lane, p, len, n, g, scale_log2, [&](bool tail) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int row = 8 * i + 2 * g + (n >> 3);
+      const int row = 8 * i + q8_v_row(n, g);
       half8_t lo = codes_to_half<KV>(uint2_t{r.v[i][0], r.v[i][1]});
       half8_t hi = codes_to_half<KV>(uint2_t{r.v[i][2], r.v[i][3]});
       if (tail && p * kPageSize + row >= len) {
         lo = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
         hi = lo;
       }
-      half_t *dst = &vstage[row * kVPitch + 16 * (n & 7)];
+      half_t *dst = &vstage[row * kVPitch + 16 * q8_v_col(n)];
       *(half8_t *)dst = lo;
       *(half8_t *)(dst + 8) = hi;
     }
@@ -401,8 +407,8 @@ __device__ __forceinline__ void load_new_rows(uint4_t (&kr)[4], uint4_t (&vr)[2]
       kr[2 * j] = *(const uint4_t *)(kn + 64 * j + 16 * g);
       kr[2 * j + 1] = *(const uint4_t *)(kn + 64 * j + 16 * g + 8);
     }
-    vr[0] = *(const uint4_t *)(vn + 16 * (n & (kHD / 16 - 1)));
-    vr[1] = *(const uint4_t *)(vn + 16 * (n & (kHD / 16 - 1)) + 8);
+    vr[0] = *(const uint4_t *)(vn + 16 * (q8_v_col(n) & (kHD / 16 - 1)));
+    vr[1] = *(const uint4_t *)(vn + 16 * (q8_v_col(n) & (kHD / 16 - 1)) + 8);
   } else {
 #pragma unroll
     for (int kk = 0; kk < kKSteps; ++kk) kr[kk] = *(const uint4_t *)(kn + 32 * kk + 8 * g);
@@ -488,8 +494,8 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
   const int64_t row_stride = (int64_t)2 * num_kv_heads * kHD;  // elements per slot
   // this lane's row and column inside page 0 (see PageRegs / PageRegsFp8)
   Elem *k_lane = kv + (int64_t)h * kHD + (FP8 ? 16 : 8) * g + n * row_stride;
-  Elem *v_lane = FP8 ? kv + (int64_t)(num_kv_heads + h) * kHD + 16 * (n & (kHD / 16 - 1)) +
-                           (2 * g + (n >> 3)) * row_stride
+  Elem *v_lane = FP8 ? kv + (int64_t)(num_kv_heads + h) * kHD + 16 * (q8_v_col(n) & (kHD / 16 - 1)) +
+                           q8_v_row(n, g) * row_stride
                      : kv + (int64_t)(num_kv_heads + h) * kHD + 8 * (n & (kVCols - 1)) + g * row_stride;
   const half_t *vt_lane = &vstage[(4 * g + (n >> 2)) * kVPitch + 4 * (n & 3)];
   const int32_t *table = block_table + (int64_t)b * bt_stride;
@@ -545,11 +551,11 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
                 *(uint4_t *)(dst + 64 * j) = x;
               }
             }
-            if (2 * g + (n >> 3) == (t_new & 7)) {
+            if (q8_v_row(n, g) == (t_new & 7)) {
               const uint2_t lo = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[0]), v_inv);
               const uint2_t hi = half_to_codes<KV>(__builtin_bit_cast(half8_t, v_row[1]), v_inv);
               const uint4_t x = uint4_t{lo[0], lo[1], hi[0], hi[1]};
-              *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHD + 16 * (n & (kHD / 16 - 1))) = x;
+              *(uint4_t *)(kv + slot_off + (int64_t)(num_kv_heads + h) * kHD + 16 * (q8_v_col(n) & (kHD / 16 - 1))) = x;
 #pragma unroll
               for (int i = 0; i < 2; ++i) {
                 if (i == (t_new >> 3)) r.v[i] = x;
