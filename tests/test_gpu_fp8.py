@@ -343,9 +343,11 @@ def test_fp8_decode_steps_replay_as_graphs():
         assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
 
 
-def test_fused_epilogue_into_an_fp8_pool_equals_epilogue_then_quantising_append():
-    print("fp8: fused QK-norm + RoPE + quantising append", flush=True)
-    t, hq, hkv = 77, 16, 4
+@pytest.mark.parametrize("t", [77, 8197])          # one token per lane, and four (prefill-sized launches)
+def test_fused_epilogue_into_an_fp8_pool_equals_epilogue_then_quantising_append(t):
+    print(f"fp8: fused QK-norm + RoPE + quantising append, {t} tokens", flush=True)
+    hq, hkv = 16, 4
+    n_slots = max(256, 2 * t)
     g = torch.Generator(device=DEV).manual_seed(61)
     qkv = torch.randn((t, hq + 2 * hkv, D), generator=g, device=DEV, dtype=torch.float16) * 1.5
     q, k, v = qkv[:, :hq], qkv[:, hq:hq + hkv], qkv[:, hq + hkv:]
@@ -355,18 +357,18 @@ def test_fused_epilogue_into_an_fp8_pool_equals_epilogue_then_quantising_append(
     inv = 10000.0 ** (-torch.arange(0, D, 2, device=DEV, dtype=torch.float64) / D)
     emb = torch.cat([pos[:, None] * inv[None, :]] * 2, dim=1)
     cos, sin = emb.cos().half(), emb.sin().half()
-    slots = torch.randperm(256, generator=torch.Generator().manual_seed(3))[:t].to(torch.int32).to(DEV)
+    slots = torch.randperm(n_slots, generator=torch.Generator().manual_seed(3))[:t].to(torch.int32).to(DEV)
     slots[7] = -1
     scales = torch.tensor([0.02, 0.03, 0.025, 0.04, 0.015, 0.02, 0.01, 0.03], device=DEV)
     # two launches: epilogue into fp16 rows, then the quantising append
     q_a = q.clone()
     rows = torch.empty((t, 2 * hkv, D), dtype=torch.float16, device=DEV)
     ops.qk_norm_rope_append(q_a, k, v, torch.arange(t, dtype=torch.int32, device=DEV), rows, wq, wk, cos, sin)
-    pool_a = torch.full((256, 2 * hkv, D), 0x55, dtype=torch.uint8, device=DEV)
+    pool_a = torch.full((n_slots, 2 * hkv, D), 0x55, dtype=torch.uint8, device=DEV)
     ops.kv_append_fp8(rows[:, :hkv], rows[:, hkv:], slots, pool_a, scales)
     # one launch
     q_b = q.clone()
-    pool_b = torch.full((256, 2 * hkv, D), 0x55, dtype=torch.uint8, device=DEV)
+    pool_b = torch.full((n_slots, 2 * hkv, D), 0x55, dtype=torch.uint8, device=DEV)
     ops.qk_norm_rope_append(q_b, k, v, slots, pool_b, wq, wk, cos, sin, kv_scales=scales)
     torch.cuda.synchronize()
     assert torch.equal(q_a, q_b)

@@ -206,9 +206,11 @@ def test_argument_checks():
         ops.paged_decode(q, pool, table, seq_lens, SCALE, kv_scales=scales[:3])
 
 
-def test_fused_epilogue_into_an_int8_pool_equals_epilogue_then_quantising_append():
-    print("int8: fused QK-norm + RoPE + quantising append", flush=True)
-    t, hq, hkv = 77, 16, 4
+@pytest.mark.parametrize("t", [77, 8197])          # one token per lane, and four (prefill-sized launches)
+def test_fused_epilogue_into_an_int8_pool_equals_epilogue_then_quantising_append(t):
+    print(f"int8: fused QK-norm + RoPE + quantising append, {t} tokens", flush=True)
+    hq, hkv = 16, 4
+    n_slots = max(256, 2 * t)
     g = torch.Generator(device=DEV).manual_seed(61)
     qkv = torch.randn((t, hq + 2 * hkv, D), generator=g, device=DEV, dtype=torch.float16) * 1.5
     q, k, v = qkv[:, :hq], qkv[:, hq:hq + hkv], qkv[:, hq + hkv:]
@@ -218,16 +220,16 @@ def test_fused_epilogue_into_an_int8_pool_equals_epilogue_then_quantising_append
     inv = 10000.0 ** (-torch.arange(0, D, 2, device=DEV, dtype=torch.float64) / D)
     emb = torch.cat([pos[:, None] * inv[None, :]] * 2, dim=1)
     cos, sin = emb.cos().half(), emb.sin().half()
-    slots = torch.randperm(256, generator=torch.Generator().manual_seed(3))[:t].to(torch.int32).to(DEV)
+    slots = torch.randperm(n_slots, generator=torch.Generator().manual_seed(3))[:t].to(torch.int32).to(DEV)
     slots[7] = -1
     scales = torch.tensor([0.02, 0.03, 0.025, 0.04, 0.015, 0.02, 0.01, 0.03], device=DEV)
     q_a = q.clone()
     rows = torch.empty((t, 2 * hkv, D), dtype=torch.float16, device=DEV)
     ops.qk_norm_rope_append(q_a, k, v, torch.arange(t, dtype=torch.int32, device=DEV), rows, wq, wk, cos, sin)
-    pool_a = torch.full((256, 2 * hkv, D), 0x55, dtype=torch.int8, device=DEV)
+    pool_a = torch.full((n_slots, 2 * hkv, D), 0x55, dtype=torch.int8, device=DEV)
     ops.kv_append_quantised(rows[:, :hkv], rows[:, hkv:], slots, pool_a, scales)
     q_b = q.clone()
-    pool_b = torch.full((256, 2 * hkv, D), 0x55, dtype=torch.int8, device=DEV)
+    pool_b = torch.full((n_slots, 2 * hkv, D), 0x55, dtype=torch.int8, device=DEV)
     ops.qk_norm_rope_append(q_b, k, v, slots, pool_b, wq, wk, cos, sin, kv_scales=scales)
     torch.cuda.synchronize()
     assert torch.equal(q_a, q_b)

@@ -59,6 +59,13 @@ def test_fused_epilogue_other_head_dims(head_dim, t, hq, hkv, norm, rope):
     _epilogue_case(t, hq, hkv, norm, rope, head_dim)
 
 
+@pytest.mark.parametrize("head_dim,t,hq,hkv", [(128, 3301, 64, 8), (256, 4101, 16, 8), (64, 5465, 64, 8), (32, 8197, 64, 8)])
+def test_fused_epilogue_prefill_sized(head_dim, t, hq, hkv):
+    """Launches large enough for the kernel's other shape (four tokens per lane instead of one),
+    with a token count that leaves the last group partly filled."""
+    _epilogue_case(t, hq, hkv, True, True, head_dim)
+
+
 def _epilogue_case(t, hq, hkv, norm, rope, head_dim):
     print(f"qk epilogue T={t} {hq}/{hkv} norm={norm} rope={rope} head_dim={head_dim}", flush=True)
     q, k, v, wq, wk, cos, sin, pool, slots = _inputs(900 + t, t, hq, hkv, head_dim)
