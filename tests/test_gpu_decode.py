@@ -508,7 +508,7 @@ def test_head_dim_64_long_shared_prefix(page_size, shared_tokens):
 # flashdecoding.py:44, 170-175: no bound on the group) ----
 
 @pytest.mark.parametrize("head_dim", [128, 64, 32])
-@pytest.mark.parametrize("hq,hkv", [(32, 1), (64, 2), (96, 4), (20, 1), (51, 3)])
+@pytest.mark.parametrize("hq,hkv", [(32, 1), (64, 2), (96, 4), (20, 1), (51, 3), (64, 1)])
 def test_more_than_16_query_heads_per_kv_head(head_dim, hq, hkv):
     """Groups of 17 to 32 query heads run as two slices of their kv head (up to 16 columns each):
     both schedules, the fused append (written once per slice, the same bits), a shared prefix."""

@@ -239,6 +239,7 @@ def test_prefill_head_dim_64_on_the_tiled_kernel(hq, hkv, lens, ctx, page_size):
     (32, 1, [130, 40], None),                  # 32 heads per kv head: four workgroups per kv head
     (96, 4, [70, 200], None),                  # 24
     (40, 2, [260, 31], [100, 700]),            # 20, chunks over history
+    (64, 1, [90, 33], [0, 150]),               # 64: the most a kv head may carry
 ])
 def test_prefill_more_than_16_query_heads_per_kv_head(head_dim, hq, hkv, lens, ctx):
     """The reference's grid is per query head (flashattention2_nopad.py:195): no bound on the group."""
