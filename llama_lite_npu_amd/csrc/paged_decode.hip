@@ -417,6 +417,15 @@ __device__ __forceinline__ void load_new_rows(uint4_t (&kr)[4], uint4_t (&vr)[2]
   }
 }
 
+// Step metadata that no launch of the decode kernel modifies (plan entries, sequence lengths) is
+// read through the constant address space: with a wavefront-uniform address such a load is
+// always a scalar load, whatever fences and atomics surround it, so it never joins the in-order
+// queue of the vector loads that stream K/V.
+typedef const __attribute__((address_space(4))) int32_t *uniform_i32_ptr;
+__device__ __forceinline__ uniform_i32_ptr as_uniform(const int32_t *p) {
+  return (uniform_i32_ptr)(uintptr_t)p;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Schedule "splits": one wavefront per (kv head, split, sequence).
 // Partials: part_o[b][hq][split][D], part_lse[b][hq][split].
@@ -428,6 +437,33 @@ __device__ __forceinline__ void load_new_rows(uint4_t (&kr)[4], uint4_t (&vr)[2]
 // compute unit would hold one such workgroup and leave a third of its slots empty.
 // ---------------------------------------------------------------------------------------------
 constexpr int kSplitWaves = 4;
+
+// The sequence whose length is the r-th largest of the batch (ties by index). A grid whose
+// workgroups outnumber the device's slots is dispatched in index order; with the sequence as the
+// slowest index and ragged lengths, the launch then ends with the long pieces of whichever
+// sequences come last while most compute units idle (128 sequences of 8192 to 32768 tokens in 16
+// splits each on 512 slots: list scheduling in batch order ends at 1.25 times the mean load of a
+// slot, longest sequences first at 1.04 times). So blockIdx.z counts sequences from the longest
+// down. Every wavefront finds its sequence for itself (no barrier, no workspace): lane l ranks
+// sequences l, l + 64, ... against all lengths, which come through scalar loads.
+constexpr int kMaxOrderedBatch = 256;
+__device__ __forceinline__ int sequence_of_rank(const int32_t *seq_lens, int batch, int r, int lane) {
+  const uniform_i32_ptr lens = as_uniform(seq_lens);
+  int found = r;
+  for (int base = 0; base < batch; base += kWave) {
+    const int i = base + lane;
+    const int mine = i < batch ? seq_lens[i] : 0;
+    int rank = 0;
+    for (int j = 0; j < batch; ++j) {
+      const int other = lens[j];
+      rank += (other > mine || (other == mine && j < i)) ? 1 : 0;
+    }
+    const uint64_t hit = __builtin_amdgcn_ballot_w64(i < batch && rank == r);
+    if (hit != 0) found = base + (int)__builtin_ctzll(hit);
+  }
+  return found;
+}
+
 extern __shared__ __attribute__((aligned(16))) half_t split_vstage[];  // [waves][kPageSize * kVPitch]
 template <int DEPTH, int KV, bool APPEND>
 __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
@@ -438,7 +474,8 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
     const half_t *__restrict__ v_new, int64_t k_new_stride, int64_t v_new_stride,
     half_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_lse,
     int32_t num_q_heads, int32_t num_kv_heads, int32_t group_all, int32_t slices, int32_t max_splits,
-    int32_t min_pages_per_split, int32_t num_pages, int32_t page_shift, float scale_log2) {
+    int32_t min_pages_per_split, int32_t num_pages, int32_t page_shift, int32_t longest_first,
+    float scale_log2) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int n = lane & 15;   // query head inside the slice (column of S^T)
@@ -448,7 +485,9 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
   const int h = hs.kv_head;
   const int group = hs.q_heads;
   const int split = blockIdx.y;
-  const int b = blockIdx.z;
+  const int b = longest_first ? __builtin_amdgcn_readfirstlane(sequence_of_rank(
+                                    seq_lens, (int)gridDim.z, (int)blockIdx.z, lane))
+                              : (int)blockIdx.z;
   half_t *vstage = split_vstage + wave * (kPageSize * kVPitch);
 
   const int len = seq_lens[b];
@@ -737,15 +776,6 @@ __global__ __launch_bounds__(kWave) void paged_decode_merge_kernel(
 constexpr int kMaxWavesPerWg = 8;
 // (the layout of a plan buffer -- kPlanMeta, kEntryHeader, the meta words, plan_entries_offset,
 // LineCut -- is in common.h: the kernel for other head dims reads page ids from a plan too)
-
-// Step metadata that no launch of the decode kernel modifies (plan entries, sequence lengths) is
-// read through the constant address space: with a wavefront-uniform address such a load is
-// always a scalar load, whatever fences and atomics surround it, so it never joins the in-order
-// queue of the vector loads that stream K/V.
-typedef const __attribute__((address_space(4))) int32_t *uniform_i32_ptr;
-__device__ __forceinline__ uniform_i32_ptr as_uniform(const int32_t *p) {
-  return (uniform_i32_ptr)(uintptr_t)p;
-}
 
 // Entry stride (int32 words) that holds the largest possible chunk: no sequence has more than
 // `bt_stride` pages, so total <= batch * bt_stride.
@@ -1198,6 +1228,24 @@ static int check_split_plan(const char *what, int32_t max_splits, int32_t min_pa
   return LITEKV_OK;
 }
 
+// Compute units of the current device.
+static int device_cus() {
+  static thread_local int cached_device = -1;
+  static thread_local int cached_cus = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 256;
+  if (dev != cached_device) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus <= 0) {
+      cus = 256;
+    }
+    cached_device = dev;
+    cached_cus = cus;
+  }
+  return cached_cus;
+}
+
 // fp8_scales: the scales of a pool of 8-bit codes of format `format` (kKvFp8, kKvInt8), or null.
 static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split,
                         const float *fp8_scales = nullptr, int format = kKvFp8) {
@@ -1235,6 +1283,11 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   const dim3 grid((unsigned)(slice_heads / waves), (unsigned)max_splits, (unsigned)a.batch);
   const dim3 block((unsigned)(waves * kWave));
   const size_t lds = (size_t)waves * kPageSize * kVPitch * sizeof(half_t);
+  // Sequences from the longest down once the launch has more workgroups than the device holds at
+  // a time (see sequence_of_rank; a launch that is resident at once ends with its longest piece
+  // in any order). Ranking costs every wavefront batch^2 / 64 comparisons: small batches only.
+  const int32_t longest_first =
+      max_splits > 1 && a.batch <= kMaxOrderedBatch && units / waves > 3 * (int64_t)device_cus();
   LITEKV_REQUIRE((a.k_new == nullptr) == (a.v_new == nullptr), "%s: k_new and v_new go together", what);
   if (a.k_new != nullptr) {
     const int64_t row = (int64_t)a.num_kv_heads * a.head_dim;
@@ -1255,7 +1308,7 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
                        a.k_new_stride, a.v_new_stride, static_cast<half_t *>(a.out), part_o, part_lse,
                        a.num_q_heads, a.num_kv_heads, group, slices, max_splits,
                        min_16_token_pages(min_pages_per_split, a.page_size), (int32_t)a.num_pages,
-                       page_shift_of(a.page_size), a.softmax_scale * kLog2e);
+                       page_shift_of(a.page_size), longest_first, a.softmax_scale * kLog2e);
   };
   if (fp8_scales != nullptr && format == kKvInt8) {
     if (a.k_new != nullptr) {
@@ -1339,24 +1392,6 @@ static size_t plan_bytes_for(int64_t batch, int64_t bt_stride, int64_t hkv, int6
   const int64_t words = plan_entries_offset((int)batch) +
                         chunks * plan_entry_stride((int)batch, (int)bt_stride, (int)chunks);
   return (size_t)words * sizeof(int32_t);
-}
-
-// Compute units of the current device.
-static int device_cus() {
-  static thread_local int cached_device = -1;
-  static thread_local int cached_cus = 0;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return 256;
-  if (dev != cached_device) {
-    int cus = 0;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-        cus <= 0) {
-      cus = 256;
-    }
-    cached_device = dev;
-    cached_cus = cus;
-  }
-  return cached_cus;
 }
 
 // Chunks per kv head that give every CU of the current device one workgroup.

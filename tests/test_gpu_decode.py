@@ -598,3 +598,40 @@ def test_length_beyond_the_block_table_row_touches_no_other_page(head_dim):
     torch.cuda.synchronize()
     assert torch.equal(pool.view(torch.int16), pool_ref.view(torch.int16)), "pool changed elsewhere (balanced)"
     assert_attention_close(out[good], ref[good], "length beyond the table, balanced")
+
+
+@pytest.mark.parametrize("hq,hkv,fused", [(64, 8, False), (32, 4, True), (16, 8, False)])
+def test_split_schedule_dispatched_longest_first(hq, hkv, fused):
+    """A split launch with more workgroups than the device holds at once walks the sequences from
+    the longest down. Which workgroup attends which sequence must not show in the result: every
+    row equals, bit for bit, the row of the same sequence decoded in a batch of one (no ordering,
+    the same split boundaries); lengths with ties, empty rows and one-token rows among them."""
+    print(f"decode splits, longest first {hq}/{hkv} fused={fused}", flush=True)
+    lens = [(37 * i * i + 11 * i) % 900 for i in range(96)]
+    for i in (3, 40, 41, 77):
+        lens[i] = 0                                  # empty rows
+    lens[10] = lens[11] = lens[60] = 512             # ties
+    lens[20] = 1
+    case = workloads.make_decode_case("lpt", 4100 + hq, lens, hq, hkv, device=DEV)
+    pool0 = case.kv_pool.clone()
+    ops.kv_append(case.k_new, case.v_new, case.slot_mapping, case.kv_pool)
+    for i in (3, 40, 41, 77):
+        case.seq_lens[i] = 0
+    ref = _oracle(case)
+    kw = dict(max_splits=16, min_pages_per_split=1)
+    if fused:
+        pool = pool0.clone()
+        out = ops.paged_decode(case.q, pool, case.block_table, case.seq_lens, case.softmax_scale,
+                               k_new=case.k_new, v_new=case.v_new, **kw)
+        torch.cuda.synchronize()
+        live = case.seq_lens > 0
+        slots = case.slot_mapping[live].long()
+        assert torch.equal(pool[slots].view(torch.int16), case.kv_pool[slots].view(torch.int16))
+    else:
+        out = _run(case, **kw)
+    assert_attention_close(out, ref, "splits, longest first")
+    for b in (0, 10, 11, 20, 41, 60, 95, max(range(96), key=lambda i: lens[i])):
+        alone = ops.paged_decode(case.q[b:b + 1].contiguous(), case.kv_pool, case.block_table[b:b + 1].contiguous(),
+                                 case.seq_lens[b:b + 1].contiguous(), case.softmax_scale, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(alone[0], out[b]), f"sequence {b} of length {int(case.seq_lens[b])}"
