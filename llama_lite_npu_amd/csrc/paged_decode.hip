@@ -31,6 +31,7 @@
 // scalars, and the merge adds the fp32 partials in index order: results do not
 // depend on timing.
 #include <atomic>
+#include <type_traits>
 
 #include "common.h"
 #include "kv_fp8.h"
@@ -444,28 +445,60 @@ constexpr int kSplitWaves = 4;
 // sequences come last while most compute units idle (128 sequences of 8192 to 32768 tokens in 16
 // splits each on 512 slots: list scheduling in batch order ends at 1.25 times the mean load of a
 // slot, longest sequences first at 1.04 times). So blockIdx.z counts sequences from the longest
-// down. Every wavefront finds its sequence for itself (no barrier, no workspace): lane l ranks
-// sequences l, l + 64, ... against all lengths, which come through scalar loads.
+// down. Every wavefront finds its sequence for itself (no barrier, no workspace): lane l holds
+// the lengths of sequences l, l + 64, ...; the r-th largest length is found bit by bit from the
+// top (31 rounds of one comparison and one population count per 64 sequences), then the tie is
+// resolved by index. A few hundred instructions for a batch of 256.
 constexpr int kMaxOrderedBatch = 256;
-__device__ __forceinline__ int sequence_of_rank(const int32_t *seq_lens, int batch, int r, int lane) {
-  const uniform_i32_ptr lens = as_uniform(seq_lens);
-  int found = r;
-  for (int base = 0; base < batch; base += kWave) {
-    const int i = base + lane;
-    const int mine = i < batch ? seq_lens[i] : 0;
-    int rank = 0;
-    for (int j = 0; j < batch; ++j) {
-      const int other = lens[j];
-      rank += (other > mine || (other == mine && j < i)) ? 1 : 0;
-    }
-    const uint64_t hit = __builtin_amdgcn_ballot_w64(i < batch && rank == r);
-    if (hit != 0) found = base + (int)__builtin_ctzll(hit);
+// `capacity`: the most tokens a block-table row can name; lengths count up to it (the kernel reads
+// no page beyond the row either). *length_out: the sequence's length as it was ranked, at least 0.
+__device__ __forceinline__ int sequence_of_rank(const int32_t *seq_lens, int batch, int r, int lane,
+                                                int capacity, int *length_out) {
+  constexpr int kRegs = kMaxOrderedBatch / kWave;
+  const int regs = (batch + kWave - 1) / kWave;  // wavefront-uniform
+  int len[kRegs];
+#pragma unroll
+  for (int p = 0; p < kRegs; ++p) {
+    const int i = kWave * p + lane;
+    int v = (p < regs && i < batch) ? seq_lens[i] : -1;
+    v = v < capacity ? v : capacity;
+    len[p] = i < batch ? (v > 0 ? v : 0) : -1;  // lanes past the batch never count
   }
-  return found;
+  auto at_least = [&](int t) {  // sequences whose length is >= t
+    int c = 0;
+#pragma unroll
+    for (int p = 0; p < kRegs; ++p) {
+      if (p < regs) c += __builtin_popcountll(__builtin_amdgcn_ballot_w64(len[p] >= t));
+    }
+    return c;
+  };
+  int v = 0;  // the largest t with more than r sequences of length >= t: the length of rank r
+  for (int bit = 31 - __builtin_clz(capacity | 1); bit >= 0; --bit) {
+    const int t = v | (1 << bit);
+    if (at_least(t) > r) v = t;
+  }
+  *length_out = v;
+  int k = r - at_least(v + 1);  // its place among the sequences of exactly that length
+#pragma unroll
+  for (int p = 0; p < kRegs; ++p) {
+    if (p < regs) {
+      uint64_t same = __builtin_amdgcn_ballot_w64(len[p] == v);
+      const int n = __builtin_popcountll(same);
+      if (k >= 0 && k < n) {
+        for (int skip = 0; skip < k; ++skip) same &= same - 1;  // drop the k lowest lanes
+        return kWave * p + (int)__builtin_ctzll(same);
+      }
+      k -= n;
+    }
+  }
+  return r;  // not reached for r < batch
 }
 
 extern __shared__ __attribute__((aligned(16))) half_t split_vstage[];  // [waves][kPageSize * kVPitch]
-template <int DEPTH, int KV, bool APPEND>
+// ORDERED: blockIdx.z is a rank by length instead of the sequence (see sequence_of_rank); an
+// instantiation of its own, so that launches bound by the dispatch of many short workgroups keep
+// the short prologue.
+template <int DEPTH, int KV, bool APPEND, bool ORDERED = false>
 __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
     const half_t *__restrict__ q, int64_t q_batch_stride,
     typename KvStore<KV>::elem *__restrict__ kv, const float *__restrict__ scales,
@@ -474,8 +507,7 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
     const half_t *__restrict__ v_new, int64_t k_new_stride, int64_t v_new_stride,
     half_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_lse,
     int32_t num_q_heads, int32_t num_kv_heads, int32_t group_all, int32_t slices, int32_t max_splits,
-    int32_t min_pages_per_split, int32_t num_pages, int32_t page_shift, int32_t longest_first,
-    float scale_log2) {
+    int32_t min_pages_per_split, int32_t num_pages, int32_t page_shift, float scale_log2) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int n = lane & 15;   // query head inside the slice (column of S^T)
@@ -485,12 +517,19 @@ __global__ __launch_bounds__(kSplitWaves *kWave) void paged_decode_split_kernel(
   const int h = hs.kv_head;
   const int group = hs.q_heads;
   const int split = blockIdx.y;
-  const int b = longest_first ? __builtin_amdgcn_readfirstlane(sequence_of_rank(
-                                    seq_lens, (int)gridDim.z, (int)blockIdx.z, lane))
-                              : (int)blockIdx.z;
   half_t *vstage = split_vstage + wave * (kPageSize * kVPitch);
-
-  const int len = seq_lens[b];
+  int b = blockIdx.z, len;
+  if constexpr (ORDERED) {
+    const int64_t capacity = (int64_t)bt_stride << (page_shift + 4);
+    b = sequence_of_rank(seq_lens, (int)gridDim.z, (int)blockIdx.z, lane,
+                         capacity < 0x40000000 ? (int)capacity : 0x40000000, &len);
+    b = __builtin_amdgcn_readfirstlane(b);
+    len = __builtin_amdgcn_readfirstlane(len);
+    // a length beyond the row keeps its own value for the masks below
+    if (len >= capacity) len = seq_lens[b];
+  } else {
+    len = seq_lens[b];
+  }
   const int hq0 = hs.q_head0;
   half_t *out_row = out + ((int64_t)b * num_q_heads + hq0) * kHD;
   if (len <= 0) {
@@ -1285,9 +1324,14 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   const size_t lds = (size_t)waves * kPageSize * kVPitch * sizeof(half_t);
   // Sequences from the longest down once the launch has more workgroups than the device holds at
   // a time (see sequence_of_rank; a launch that is resident at once ends with its longest piece
-  // in any order). Ranking costs every wavefront batch^2 / 64 comparisons: small batches only.
-  const int32_t longest_first =
-      max_splits > 1 && a.batch <= kMaxOrderedBatch && units / waves > 3 * (int64_t)device_cus();
+  // in any order), for block tables wide enough that a split can be 16 pages long: finding its
+  // sequence costs a wavefront about a microsecond, which pieces of a page or two would not
+  // return (200 sequences of 64 to 256 tokens in 16 splits: 82 us in batch order, 120 us ranked;
+  // 256 sequences of 128 to 1024 tokens in 4 splits: 150 against 134 us).
+  const int64_t row_pages = (int64_t)a.block_table_stride << page_shift_of(a.page_size);
+  const bool longest_first = max_splits > 1 && a.k_new == nullptr && a.batch <= kMaxOrderedBatch &&
+                             units / waves > 3 * (int64_t)device_cus() &&
+                             row_pages >= 16 * (int64_t)max_splits;
   LITEKV_REQUIRE((a.k_new == nullptr) == (a.v_new == nullptr), "%s: k_new and v_new go together", what);
   if (a.k_new != nullptr) {
     const int64_t row = (int64_t)a.num_kv_heads * a.head_dim;
@@ -1308,24 +1352,24 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
                        a.k_new_stride, a.v_new_stride, static_cast<half_t *>(a.out), part_o, part_lse,
                        a.num_q_heads, a.num_kv_heads, group, slices, max_splits,
                        min_16_token_pages(min_pages_per_split, a.page_size), (int32_t)a.num_pages,
-                       page_shift_of(a.page_size), longest_first, a.softmax_scale * kLog2e);
+                       page_shift_of(a.page_size), a.softmax_scale * kLog2e);
+  };
+  auto by_append = [&](auto kv_tag, auto *kv) {
+    constexpr int KV = decltype(kv_tag)::value;
+    if (a.k_new != nullptr) {
+      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, KV, true>, kv);
+    } else if (longest_first) {
+      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, KV, false, true>, kv);
+    } else {
+      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, KV, false>, kv);
+    }
   };
   if (fp8_scales != nullptr && format == kKvInt8) {
-    if (a.k_new != nullptr) {
-      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvInt8, true>, static_cast<uint8_t *>(pool));
-    } else {
-      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvInt8, false>, static_cast<uint8_t *>(pool));
-    }
+    by_append(std::integral_constant<int, kKvInt8>{}, static_cast<uint8_t *>(pool));
   } else if (fp8_scales != nullptr) {
-    if (a.k_new != nullptr) {
-      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvFp8, true>, static_cast<uint8_t *>(pool));
-    } else {
-      launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvFp8, false>, static_cast<uint8_t *>(pool));
-    }
-  } else if (a.k_new != nullptr) {
-    launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvF16, true>, static_cast<half_t *>(pool));
+    by_append(std::integral_constant<int, kKvFp8>{}, static_cast<uint8_t *>(pool));
   } else {
-    launch(paged_decode_split_kernel<LITEKV_DECODE_DEPTH, kKvF16, false>, static_cast<half_t *>(pool));
+    by_append(std::integral_constant<int, kKvF16>{}, static_cast<half_t *>(pool));
   }
   return check_launch(what);
 }
