@@ -635,3 +635,25 @@ def test_split_schedule_dispatched_longest_first(hq, hkv, fused):
                                  case.seq_lens[b:b + 1].contiguous(), case.softmax_scale, **kw)
         torch.cuda.synchronize()
         assert torch.equal(alone[0], out[b]), f"sequence {b} of length {int(case.seq_lens[b])}"
+
+
+def test_prefix_chunk_count_leaves_room_for_the_prefix_role():
+    """The chunk count a plan takes for a step behind a shared prefix: the compute units the
+    prefix workgroups leave, less a sixteenth of the device, never under a quarter of it; shapes
+    the helper cannot judge get the plain balanced count."""
+    print("decode prefix chunk count", flush=True)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    plain = ops.balanced_chunks(8)
+    c4 = ops.prefix_chunks(64, 64, 8, 128)
+    assert c4 == cus - 64 - cus // 16                     # 64 prefix workgroups of 8 wavefronts on this shape
+    small = ops.prefix_chunks(2, 8, 8, 128)               # too few columns for wide workgroups
+    assert cus // 4 <= small <= cus
+    assert ops.prefix_chunks(64, 64, 8, 8, page_size=256) == c4      # 8 pages of 256 tokens are the same 2048 keys
+    eight_bit = ops.prefix_chunks(64, 64, 8, 128, fp16_pool=False)
+    assert cus // 4 <= eight_bit <= cus
+    assert ops.prefix_chunks(64, 64, 8, 0) == plain       # no shared pages: the plain count
+    assert ops.prefix_chunks(64, 64, 8, 128, page_size=48) == plain
+    plan = ops.DecodePlan(torch.zeros((64, 160), dtype=torch.int32, device=DEV),
+                          torch.full((64,), 2100, dtype=torch.int32, device=DEV), 64, 8, 4096,
+                          shared_pages=128, kv_dtype=torch.float16)
+    assert plan.chunks == c4
