@@ -538,6 +538,47 @@ int litekv_paged_prefill(const void *q, int64_t q_token_stride,
                          int32_t max_q_len, float softmax_scale, void *stream);
 
 /*
+ * The same for launches with too few query rows to fill the device: one
+ * request's chunk over a long history, the case of the reference's chunked
+ * prefill (`prefill_chunk_size`, lite_llama/continuous_batching.py:194-611
+ * calls paged_chunk_flash_attention once per chunk). Every block of query rows
+ * is cut along its keys into `key_slices` runs of key tiles, one workgroup
+ * each; the slices leave fp32 partial rows + log-sum-exps in `workspace`, and
+ * a second launch folds them in slice order (results do not depend on timing;
+ * they differ from litekv_paged_prefill's within fp32 rounding of the merge).
+ * fp16 pools, head_dim 64 or 128, 2 <= key_slices <= 8.
+ *
+ *   litekv_paged_prefill_key_slices  the count that brings the launch's
+ *       workgroups to the device's resident slots with at least 32 key tiles
+ *       (2048 keys) per slice when the longest row sees max_kv_len keys;
+ *       1: do not split
+ *       (call litekv_paged_prefill)
+ *   num_tokens    T, the query rows of the launch (= cu_q_lens[batch])
+ *   workspace     litekv_paged_prefill_split_workspace_bytes(T, Hq, D,
+ *                 key_slices) bytes, 16-byte aligned; launches that share it
+ *                 must be ordered on one stream
+ */
+size_t litekv_paged_prefill_split_workspace_bytes(int64_t num_tokens,
+                                                  int32_t num_q_heads,
+                                                  int32_t head_dim,
+                                                  int32_t key_slices);
+int32_t litekv_paged_prefill_key_slices(int32_t batch, int32_t num_q_heads,
+                                        int32_t num_kv_heads, int32_t head_dim,
+                                        int32_t max_q_len, int64_t max_kv_len);
+int litekv_paged_prefill_split(const void *q, int64_t q_token_stride,
+                               const void *kv_pool, const int32_t *block_table,
+                               int32_t block_table_stride,
+                               const int32_t *cu_q_lens,
+                               const int32_t *context_lens, void *out,
+                               int64_t out_token_stride, int32_t batch,
+                               int32_t num_q_heads, int32_t num_kv_heads,
+                               int32_t head_dim, int32_t page_size,
+                               int64_t num_pages, int32_t max_q_len,
+                               int64_t num_tokens, int32_t key_slices,
+                               void *workspace, size_t workspace_bytes,
+                               float softmax_scale, void *stream);
+
+/*
  * The same over an fp8 (E4M3) pool with per-head scales (kv_scales: float32
  * [2 * Hkv], K heads then V heads, value = code * scale), as written by
  * litekv_kv_append_fp8: the chunk rows of a chunked prefill or of a

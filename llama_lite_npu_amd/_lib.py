@@ -189,6 +189,14 @@ SIGNATURES = {
         [c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
          c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_float, c_void_p],
     ),
+    "litekv_paged_prefill_split_workspace_bytes": (c_size_t, [c_int64, c_int32, c_int32, c_int32]),
+    "litekv_paged_prefill_key_slices": (c_int32, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int64]),
+    "litekv_paged_prefill_split": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
+         c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int64, c_int32, c_void_p, c_size_t,
+         c_float, c_void_p],
+    ),
     "litekv_paged_prefill_fp8": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,

@@ -64,12 +64,16 @@ class Attention:
             return self._context_forward_fp8(xq, xk, xv, atten_info, pool, atten_info.kv_scales[layer_index], scale)
         if xk is not None:
             ops.kv_append(xk, xv, atten_info.cur_select_index, pool)
+        # max_kv_len: the longest history + chunk of the batch, which the executor knows on the host;
+        # a lone chunk over a long history is then cut along its keys as well (ops.paged_prefill)
         if getattr(atten_info, "is_paged_chunk_prefill", False):
             return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens,
                                      atten_info.context_lens_i32, int(atten_info.max_actual_q_seq_len), scale,
-                                     page_size=_page_size(atten_info))
+                                     page_size=_page_size(atten_info),
+                                     max_kv_len=int(atten_info.max_actual_seq_len))
         return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens, None,
-                                 int(atten_info.max_actual_seq_len), scale, page_size=_page_size(atten_info))
+                                 int(atten_info.max_actual_seq_len), scale, page_size=_page_size(atten_info),
+                                 max_kv_len=int(atten_info.max_actual_seq_len))
 
     def _context_forward_fp8(self, xq, xk, xv, atten_info, pool, scales, scale) -> torch.Tensor:
         chunked = getattr(atten_info, "is_paged_chunk_prefill", False)

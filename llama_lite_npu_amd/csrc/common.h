@@ -128,6 +128,16 @@ struct DecodeArgs {
   int64_t k_new_stride = 0, v_new_stride = 0;
 };
 
+// A paged prefill whose blocks are cut into key slices (see kPagedPrefillSplit in prefill_tile.h):
+// how many, the workspace for the slices' partial rows, and the query rows of the launch.
+struct PrefillKeySplit {
+  int32_t key_slices = 1;   // 1: no split, nothing else is read
+  void *workspace = nullptr;
+  size_t workspace_bytes = 0;
+  int64_t num_tokens = 0;   // query rows of the launch (cu_q_lens[batch])
+};
+constexpr int kMaxPrefillKeySlices = 8;
+
 // The launchers of the head dim 64 build of paged_prefill.hip (paged_prefill_hd64.hip).
 int hd64_paged_prefill(const char *what, const void *q, int64_t q_token_stride, const void *kv_pool,
                        const float *kv_scales, int format, const int32_t *block_table,
@@ -135,7 +145,10 @@ int hd64_paged_prefill(const char *what, const void *q, int64_t q_token_stride, 
                        const int32_t *cu_q_lens, const int32_t *context_lens, void *out,
                        int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
                        int32_t num_kv_heads, int32_t page_size, int64_t num_pages,
-                       int32_t max_q_len, float softmax_scale, void *stream);
+                       int32_t max_q_len, float softmax_scale, void *stream,
+                       const PrefillKeySplit &split);
+int32_t hd64_prefill_key_slices(int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                                int32_t max_q_len, int64_t max_kv_len);
 int hd64_varlen_prefill(const void *q, int64_t q_token_stride, const void *k, int64_t k_token_stride,
                         const void *v, int64_t v_token_stride, const int32_t *seq_starts,
                         const int32_t *seq_lens, void *out, int64_t out_token_stride, int32_t batch,

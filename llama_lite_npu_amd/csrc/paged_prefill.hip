@@ -44,6 +44,81 @@ static PrefillShape prefill_shape(int group, int max_q_len, int col_tiles = kWgC
   return s;
 }
 
+// Folds the key slices of a split prefill: one wavefront per (query row, head) reads the row's
+// `slices` log-sum-exps and partial rows (fp32, normalised per slice) and writes the fp16 row.
+// A slice without keys has log-sum-exp -inf and weight 0; the last slice always has keys.
+__global__ __launch_bounds__(4 * kWave) void prefill_split_merge_kernel(
+    const float *__restrict__ part_o, const float *__restrict__ part_lse, half_t *__restrict__ out,
+    int64_t out_stride, int64_t num_tokens, int32_t num_q_heads, int32_t slices) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t id = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (id >= num_tokens * num_q_heads) return;  // whole wavefronts
+  const int64_t token = id / num_q_heads;
+  const int head = (int)(id - token * num_q_heads);
+  const int64_t piece_stride = num_tokens * num_q_heads;  // cells between the slices of a row
+  const float l = lane < slices ? part_lse[lane * piece_stride + id] : -INFINITY;
+  float mx = l;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, xor_lane(mx, off));
+  const float w = lane < slices ? fast_exp2((l - mx) * 1.4426950408889634f) : 0.f;
+  float den = w;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) den += xor_lane(den, off);
+  if (2 * lane >= kHD) return;
+  float o0 = 0.f, o1 = 0.f;
+  for (int sidx = 0; sidx < slices; ++sidx) {  // in slice order: the sum does not depend on timing
+    const float ws = __shfl(w, sidx, kWave);
+    const float2 r = *(const float2 *)(part_o + (sidx * piece_stride + id) * kHD + 2 * lane);
+    o0 += ws * r.x;
+    o1 += ws * r.y;
+  }
+  const float inv = 1.0f / den;
+  typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+  *(half2_t *)(out + token * out_stride + (int64_t)head * kHD + 2 * lane) =
+      half2_t{(half_t)(o0 * inv), (half_t)(o1 * inv)};
+}
+
+static size_t prefill_split_workspace_bytes(int64_t num_tokens, int32_t num_q_heads, int32_t key_slices) {
+  if (num_tokens <= 0 || num_q_heads <= 0 || key_slices <= 1) return 0;
+  return (size_t)key_slices * (size_t)num_tokens * (size_t)num_q_heads * (kHD + 1) * sizeof(float);
+}
+
+// Key slices that fill the device for a paged prefill whose row blocks alone would not: as many as
+// bring its workgroups to the device's resident slots, at most kMaxPrefillKeySlices, each with at
+// least 32 key tiles (2048 keys) if the longest row sees `max_kv_len` keys: a slice costs a partial
+// row (fp32) written and read back per query row and head, and the launch a merge. 1 means: do
+// not split. (64 query / 8 kv heads, one request's chunk over 32k cached tokens, plain against
+// sliced: 128 rows 527 -> 176 us, 256 rows 533 -> 298 us, 512 rows 609 -> 551 us; 512 rows over
+// 2048 tokens in two slices 77 -> 90 us, which the 32 tiles rule out.)
+static int32_t prefill_key_slices(int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                                  int32_t max_q_len, int64_t max_kv_len) {
+  if (batch <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0 ||
+      max_q_len <= 0 || num_q_heads / num_kv_heads > kMaxGroup) {
+    return 1;
+  }
+  const PrefillShape s = prefill_shape(num_q_heads / num_kv_heads, max_q_len, kColTiles * kTiledWaves);
+  const int64_t wgs = (int64_t)num_kv_heads * s.head_splits * s.row_blocks * batch;
+  static thread_local int cached_device = -1, cached_cus = 0;  // compute units of the current device
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = -2;
+  if (dev != cached_device) {
+    int cus = 0;
+    if (dev < 0 || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        cus <= 0) {
+      cus = 256;
+    }
+    cached_device = dev;
+    cached_cus = cus;
+  }
+  const int64_t slots = (int64_t)cached_cus * (kHD == 64 ? 3 : 2);
+  if (2 * wgs > slots) return 1;
+  int64_t n = slots / wgs;
+  n = n < kMaxPrefillKeySlices ? n : kMaxPrefillKeySlices;
+  const int64_t tiles = max_kv_len / kKvTile;
+  while (n > 1 && tiles / n < 32) --n;
+  return (int32_t)n;
+}
+
 // Causal chunk attention over paged KV; `kv_scales` selects the fp8 pool.
 static int launch_paged_prefill(const char *what, const void *q, int64_t q_token_stride,
                                 const void *kv_pool, const float *kv_scales,
@@ -52,13 +127,18 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
                                 int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
                                 int32_t num_kv_heads, int32_t head_dim, int32_t page_size,
                                 int64_t num_pages, int32_t max_q_len, float softmax_scale,
-                                void *stream, int format) {
+                                void *stream, int format,
+                                const PrefillKeySplit &split = PrefillKeySplit{}) {
   const bool fp8 = format != kKvF16;  // a pool of 8-bit codes
+  LITEKV_REQUIRE(split.key_slices >= 1 && split.key_slices <= kMaxPrefillKeySlices,
+                 "%s: key_slices %d out of [1, %d]", what, split.key_slices, kMaxPrefillKeySlices);
+  LITEKV_REQUIRE(split.key_slices == 1 || (!fp8 && (head_dim == 128 || head_dim == 64)),
+                 "%s: key slices take an fp16 pool and head_dim 64 or 128", what);
 #if LITEKV_HD == 128
   if (head_dim == 64) {  // the head dim 64 build of this file
     return hd64_paged_prefill(what, q, q_token_stride, kv_pool, kv_scales, format, block_table, block_table_stride,
                               cu_q_lens, context_lens, out, out_token_stride, batch, num_q_heads,
-                              num_kv_heads, page_size, num_pages, max_q_len, softmax_scale, stream);
+                              num_kv_heads, page_size, num_pages, max_q_len, softmax_scale, stream, split);
   }
 #endif
   if (head_dim != kHD && generic_head_dim(head_dim)) {  // see generic_attention.hip
@@ -109,6 +189,36 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
                     num_kv_heads, (int32_t)num_pages, kv_scales, page_shift};
   PackedSource packed{nullptr, nullptr, 0, 0, nullptr};
   const int group = num_q_heads / num_kv_heads;
+  if (split.key_slices > 1) {
+    // every block's keys in key_slices runs of tiles, one workgroup each, then the merge
+    const int slices = split.key_slices;
+    const int64_t rows = split.num_tokens;
+    LITEKV_REQUIRE(rows >= 1 && rows * num_q_heads * slices <= 0x7fffffffLL,
+                   "%s: num_tokens %lld out of range for %d key slices", what, (long long)rows, slices);
+    const size_t need = prefill_split_workspace_bytes(rows, num_q_heads, slices);
+    LITEKV_REQUIRE(split.workspace != nullptr && aligned16(split.workspace) && split.workspace_bytes >= need,
+                   "%s: workspace of %zu bytes needed for %d key slices, got %zu", what, need, slices,
+                   split.workspace_bytes);
+    const PrefillShape s = prefill_shape(group, max_q_len, kColTiles * kTiledWaves);
+    LITEKV_REQUIRE((uint64_t)s.row_blocks * slices <= 65535u, "%s: max_q_len %d too large for %d key slices",
+                   what, max_q_len, slices);
+    float *part_o = static_cast<float *>(split.workspace);
+    float *part_lse = part_o + (size_t)slices * rows * num_q_heads * kHD;
+    const PrefixTask task{part_o, part_lse, 0, (int32_t)rows, num_q_heads, 0, 0};
+    const dim3 grid((unsigned)(num_kv_heads * s.head_splits), s.row_blocks * (unsigned)slices, (unsigned)batch);
+    hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kPagedPrefillSplit>, grid, dim3(kTiledWaves * kWave), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const half_t *>(q), q_token_stride,
+                       static_cast<half_t *>(out), out_token_stride, paged, packed, task, cu_q_lens,
+                       (const int32_t *)nullptr, context_lens, group, s.head_splits, s.heads_per_wg,
+                       s.row_tiles, softmax_scale * kLog2eP, slices);
+    int rc2 = check_launch(what);
+    if (rc2 != LITEKV_OK) return rc2;
+    const int64_t merge_rows = rows * num_q_heads;
+    hipLaunchKernelGGL(prefill_split_merge_kernel, dim3((unsigned)((merge_rows + 3) / 4)), dim3(4 * kWave), 0,
+                       static_cast<hipStream_t>(stream), part_o, part_lse, static_cast<half_t *>(out),
+                       out_token_stride, rows, num_q_heads, slices);
+    return check_launch(what);
+  }
   const int waves = (format == kKvF16 && LITEKV_PREFILL_WAVES == kWideWaves) ? kWideWaves : kTiledWaves;
   const PrefillShape s = prefill_shape(group, max_q_len, kColTiles * waves);
   LITEKV_REQUIRE(s.row_blocks <= 65535u, "%s: max_q_len %d too large", what, max_q_len);
@@ -118,7 +228,7 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
                        static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
                        out_token_stride, paged, packed, PrefixTask{}, cu_q_lens,
                        (const int32_t *)nullptr, context_lens, group, s.head_splits, s.heads_per_wg,
-                       s.row_tiles, softmax_scale * kLog2eP);
+                       s.row_tiles, softmax_scale * kLog2eP, 1);
   };
   if (format == kKvInt8) {
     launch(varlen_prefill_tiled_kernel<kPagedPrefillInt8>);
@@ -199,7 +309,7 @@ static int launch_varlen_prefill(const void *q, int64_t q_token_stride, const vo
                        static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
                        out_token_stride, paged, packed, PrefixTask{}, seq_starts, seq_lens,
                        (const int32_t *)nullptr, group, s.head_splits, s.heads_per_wg, s.row_tiles,
-                       softmax_scale * kLog2eP);
+                       softmax_scale * kLog2eP, 1);
   };
   if (waves == kWideWaves) {
     launch(varlen_prefill_tiled_kernel<kPackedPrefill, kWideWaves>);
@@ -217,11 +327,16 @@ int hd64_paged_prefill(const char *what, const void *q, int64_t q_token_stride, 
                        const int32_t *cu_q_lens, const int32_t *context_lens, void *out,
                        int64_t out_token_stride, int32_t batch, int32_t num_q_heads,
                        int32_t num_kv_heads, int32_t page_size, int64_t num_pages,
-                       int32_t max_q_len, float softmax_scale, void *stream) {
+                       int32_t max_q_len, float softmax_scale, void *stream,
+                       const PrefillKeySplit &split) {
   return launch_paged_prefill(what, q, q_token_stride, kv_pool, kv_scales, block_table,
                               block_table_stride, cu_q_lens, context_lens, out, out_token_stride,
                               batch, num_q_heads, num_kv_heads, 64, page_size, num_pages, max_q_len,
-                              softmax_scale, stream, format);
+                              softmax_scale, stream, format, split);
+}
+int32_t hd64_prefill_key_slices(int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                                int32_t max_q_len, int64_t max_kv_len) {
+  return prefill_key_slices(batch, num_q_heads, num_kv_heads, max_q_len, max_kv_len);
 }
 int hd64_varlen_prefill(const void *q, int64_t q_token_stride, const void *k, int64_t k_token_stride,
                         const void *v, int64_t v_token_stride, const int32_t *seq_starts,
@@ -249,6 +364,43 @@ extern "C" int litekv_paged_prefill(const void *q, int64_t q_token_stride, const
                                       out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
                                       page_size, num_pages, max_q_len, softmax_scale, stream,
                                       litekv::kKvF16);
+}
+
+extern "C" size_t litekv_paged_prefill_split_workspace_bytes(int64_t num_tokens, int32_t num_q_heads,
+                                                             int32_t head_dim, int32_t key_slices) {
+  if (head_dim != 128 && head_dim != 64) return 0;
+  if (num_tokens <= 0 || num_q_heads <= 0 || key_slices <= 1) return 0;
+  return (size_t)key_slices * (size_t)num_tokens * (size_t)num_q_heads * (size_t)(head_dim + 1) * sizeof(float);
+}
+
+extern "C" int32_t litekv_paged_prefill_key_slices(int32_t batch, int32_t num_q_heads,
+                                                   int32_t num_kv_heads, int32_t head_dim,
+                                                   int32_t max_q_len, int64_t max_kv_len) {
+  if (head_dim == 64) {
+    return litekv::hd64_prefill_key_slices(batch, num_q_heads, num_kv_heads, max_q_len, max_kv_len);
+  }
+  if (head_dim != 128) return 1;
+  return litekv::prefill_key_slices(batch, num_q_heads, num_kv_heads, max_q_len, max_kv_len);
+}
+
+extern "C" int litekv_paged_prefill_split(const void *q, int64_t q_token_stride, const void *kv_pool,
+                                          const int32_t *block_table, int32_t block_table_stride,
+                                          const int32_t *cu_q_lens, const int32_t *context_lens,
+                                          void *out, int64_t out_token_stride, int32_t batch,
+                                          int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                          int32_t page_size, int64_t num_pages, int32_t max_q_len,
+                                          int64_t num_tokens, int32_t key_slices, void *workspace,
+                                          size_t workspace_bytes, float softmax_scale, void *stream) {
+  litekv::PrefillKeySplit split;
+  split.key_slices = key_slices;
+  split.workspace = workspace;
+  split.workspace_bytes = workspace_bytes;
+  split.num_tokens = num_tokens;
+  return litekv::launch_paged_prefill("paged_prefill_split", q, q_token_stride, kv_pool, nullptr,
+                                      block_table, block_table_stride, cu_q_lens, context_lens, out,
+                                      out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
+                                      page_size, num_pages, max_q_len, softmax_scale, stream,
+                                      litekv::kKvF16, split);
 }
 
 extern "C" int litekv_paged_prefill_fp8(const void *q, int64_t q_token_stride, const void *kv_pool,

@@ -102,6 +102,8 @@ struct PagedSource {
 // Shared-prefix decode (mode kSharedPrefix): the columns are (sequence, query head) pairs of one
 // decode step, the keys are a slice of the pages every sequence starts with, and the result is
 // a normalised fp32 partial row + log-sum-exp per column, for the decode merge.
+// Prefill over key slices (mode kPagedPrefillSplit) writes the same kind of partial rows, one
+// per (key slice, query row, head): `batch` then counts the query rows of the launch.
 struct PrefixTask {
   float *part_o;            // [splits][batch][Hq][128]
   float *part_lse;          // [splits][batch][Hq]
@@ -139,7 +141,12 @@ __device__ __forceinline__ float vmax3(float a, float b, float c) {
 }
 __device__ __forceinline__ float vmax2(float a, float b) { return __builtin_fmaxf(a, b); }
 constexpr int kPagedPrefill = 0, kPackedPrefill = 1, kSharedPrefix = 2, kPagedPrefillFp8 = 3,
-              kSharedPrefixFp8 = 4, kPagedPrefillInt8 = 5, kSharedPrefixInt8 = 6;
+              kSharedPrefixFp8 = 4, kPagedPrefillInt8 = 5, kSharedPrefixInt8 = 6,
+              kPagedPrefillSplit = 7;
+// kPagedPrefillSplit: a launch with too few row blocks to fill the device (one request's chunk
+// over a long history) cuts every block's keys into `key_slices` runs of tiles, one workgroup
+// each; a slice leaves a normalised fp32 partial row + log-sum-exp per (query row, head), and a
+// merge launch folds the slices of a row (prefill_split_merge_kernel in paged_prefill.hip).
 
 // The body of the kernel, run by a workgroup of W wavefronts that stands at (block_x, block_y,
 // block_z) of a grid block_y runs over grid_y values of; k_lds is the LDS byte address of its
@@ -155,8 +162,10 @@ __device__ __forceinline__ void prefill_tile_body(
     const PagedSource &paged, const PackedSource &packed, const PrefixTask &prefix,
     const int32_t *__restrict__ q_starts_or_cu, const int32_t *__restrict__ q_lens_or_null,
     const int32_t *__restrict__ context_lens, int32_t group, int32_t head_splits,
-    int32_t heads_per_wg, int32_t row_tiles, float scale_log2) {
+    int32_t heads_per_wg, int32_t row_tiles, float scale_log2, const int key_slice = 0,
+    const int key_slices = 1) {
   constexpr bool PAGED = MODE != kPackedPrefill;
+  constexpr bool KSPLIT = MODE == kPagedPrefillSplit;  // causal prefill over one slice of the block's keys
   // An fp8 pool cannot take the direct HBM -> LDS load: its codes go through registers, are
   // converted to fp16 (exactly) and written to LDS in the same swizzled layout, so everything
   // after the staging is shared. The K scale joins the softmax scale, the V scale the final
@@ -230,6 +239,37 @@ __device__ __forceinline__ void prefill_tile_body(
     kv_end = ctx + m0 + rows;
     diag = ctx + m0;
     last_key = ctx + q_len - 1;
+    if constexpr (KSPLIT) {
+      // The tiles every row of the block sees in full (`plain` of them) are shared out among the
+      // slices; the last slice also takes the tiles at the diagonal, and starts no later than
+      // the last plain tile, so that each of its rows sees at least one key.
+      const int total = (kv_end + kKvTile - 1) / kKvTile;
+      const int plain = (diag + 1) / kKvTile;
+      const int last_start = plain > 0 ? plain - 1 : 0;
+      const int per = (plain + key_slices - 1) / key_slices;
+      int t_begin = key_slice * per;
+      t_begin = t_begin < last_start ? t_begin : last_start;
+      int t_end = (key_slice + 1) * per;
+      t_end = key_slice == key_slices - 1 ? total : (t_end < last_start ? t_end : last_start);
+      if (t_end <= t_begin) {
+        // Nothing for this slice: its partial rows say so (log-sum-exp -inf, a row of zeros).
+        for (int t = wave * kColTiles; t < wave * kColTiles + kColTiles; ++t) {
+          const int head = t / row_tiles;
+          const int row = m0 + (t - head * row_tiles) * 16 + n;
+          if (head < heads_here && row < q_len) {
+            const int64_t cell = ((int64_t)key_slice * prefix.batch + q_start + row) * prefix.num_q_heads +
+                                 h * group + head0 + head;
+            if (g == 0) prefix.part_lse[cell] = -INFINITY;
+            float4_t *dst = (float4_t *)(prefix.part_o + cell * kHD) + g * (kHD / 16);
+#pragma unroll
+            for (int i = 0; i < kHD / 16; ++i) dst[i] = float4_t{0.f, 0.f, 0.f, 0.f};
+          }
+        }
+        return;
+      }
+      tile0 = t_begin;
+      kv_end = kv_end < t_end * kKvTile ? kv_end : t_end * kKvTile;
+    }
   }
   const int n_tiles = (kv_end + kKvTile - 1) / kKvTile - tile0;
 
@@ -823,7 +863,7 @@ __device__ __forceinline__ void prefill_tile_body(
     }
   }
 
-  if constexpr (!SHARED) {
+  if constexpr (!SHARED && !KSPLIT) {
     // The accumulators hold O^T: a lane has 4 consecutive d of one row, so stored directly every
     // store instruction would touch 16 rows with 32 bytes each. The rows go through LDS instead
     // (the K/V tiles are done with) and leave as whole 256-byte rows, 4 rows per instruction.
@@ -862,7 +902,7 @@ __device__ __forceinline__ void prefill_tile_body(
     }
     return;
   }
-  if constexpr (SHARED) {
+  if constexpr (SHARED || KSPLIT) {
     // The partial rows (fp32, normalised) leave as whole rows like the output of a prefill block:
     // a lane holds 4 consecutive elements of each of its column's 16-element groups, so stored
     // straight from registers one instruction would touch 16 rows with 64 bytes each. One column
@@ -878,8 +918,9 @@ __device__ __forceinline__ void prefill_tile_body(
     for (int u = 0; u < kColTiles; ++u) {
       const float inv = v_scale / dsum[u][0];
       // the partial row of this lane's column (the same in its four lane groups), or -1
+      const int piece = SHARED ? block_z : key_slice;  // which partial of the row this block writes
       const int cell = out_row[u] >= 0
-                           ? (block_z * prefix.batch + out_row[u]) * prefix.num_q_heads + out_head[u]
+                           ? (piece * prefix.batch + out_row[u]) * prefix.num_q_heads + out_head[u]
                            : -1;
       if (g == 0 && cell >= 0) {
         // read once, by the merge launch: streaming stores (see store_state in paged_decode.hip)
@@ -930,12 +971,22 @@ __global__ __launch_bounds__(W *kWave, W == kWideWaves ? 1 : (kHD == 64 ? 3 : 2)
     PagedSource paged, PackedSource packed, PrefixTask prefix,
     const int32_t *__restrict__ q_starts_or_cu, const int32_t *__restrict__ q_lens_or_null,
     const int32_t *__restrict__ context_lens, int32_t group, int32_t head_splits,
-    int32_t heads_per_wg, int32_t row_tiles, float scale_log2) {
+    int32_t heads_per_wg, int32_t row_tiles, float scale_log2, int32_t key_slices) {
   __shared__ __attribute__((aligned(1024))) half_t lds_all[tile_lds_bytes<W>() / 2];
-  prefill_tile_body<MODE, W>((uint32_t)(uintptr_t)(lds_half_t *)lds_all, (int)blockIdx.x, (int)blockIdx.y,
-                             (int)blockIdx.z, (int)gridDim.y, q, q_stride, out, out_stride, paged, packed,
-                             prefix, q_starts_or_cu, q_lens_or_null, context_lens, group, head_splits,
-                             heads_per_wg, row_tiles, scale_log2);
+  if constexpr (MODE == kPagedPrefillSplit) {
+    // blockIdx.y = row block * key_slices + slice: the slices of a block are neighbours
+    const int by = (int)blockIdx.y / key_slices;
+    prefill_tile_body<MODE, W>((uint32_t)(uintptr_t)(lds_half_t *)lds_all, (int)blockIdx.x, by,
+                               (int)blockIdx.z, (int)gridDim.y / key_slices, q, q_stride, out, out_stride,
+                               paged, packed, prefix, q_starts_or_cu, q_lens_or_null, context_lens, group,
+                               head_splits, heads_per_wg, row_tiles, scale_log2,
+                               (int)blockIdx.y - by * key_slices, key_slices);
+  } else {
+    prefill_tile_body<MODE, W>((uint32_t)(uintptr_t)(lds_half_t *)lds_all, (int)blockIdx.x, (int)blockIdx.y,
+                               (int)blockIdx.z, (int)gridDim.y, q, q_stride, out, out_stride, paged, packed,
+                               prefix, q_starts_or_cu, q_lens_or_null, context_lens, group, head_splits,
+                               heads_per_wg, row_tiles, scale_log2);
+  }
 }
 
 }  // namespace prefill_tile

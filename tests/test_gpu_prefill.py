@@ -274,3 +274,85 @@ def test_prefill_length_beyond_the_block_table_row():
     assert bool(torch.isfinite(out).all())
     rows = torch.cat([torch.arange(0, 20), torch.arange(50, 67)])
     assert_attention_close(out[rows.to(DEV)], ref[rows.numpy()], "rows of the other sequences")
+
+
+@pytest.mark.parametrize("head_dim", [128, 64])
+@pytest.mark.parametrize("hq,hkv,lens,ctx,slices,page_size", [
+    (64, 8, [512], [4096], 2, 16),              # one request's chunk over a long history
+    (64, 8, [200], [3000], 4, 16),              # ragged last row block
+    (32, 4, [77, 130], [1000, 17], 3, 32),      # a sequence whose slices are mostly empty beside a long one
+    (16, 8, [16], [2049], 8, 16),               # a single row block, eight slices
+    (8, 8, [300], [0], 2, 16),                  # no history: 128 rows per block, the diagonal in the last slice only
+    (14, 2, [64], [63], 5, 64),                 # fewer plain tiles than slices
+    (32, 1, [40], [900], 2, 16),                # 32 heads per kv head: four workgroups per kv head
+    (64, 8, [1, 3], [640, 5000], 4, 128),       # one and three rows
+])
+def test_paged_prefill_over_key_slices(head_dim, hq, hkv, lens, ctx, slices, page_size):
+    """A chunk whose row blocks are cut along their keys (key_slices workgroups per block and a merge
+    launch): within tolerance of the oracle and of the unsplit launch, the same bits on a second
+    launch, and with one slice the plain kernel itself."""
+    print(f"prefill over {slices} key slices d={head_dim} {hq}/{hkv} {lens} ctx {ctx} page_size {page_size}", flush=True)
+    case = workloads.make_prefill_case("ks", 7300 + hq + slices, lens, hq, hkv, context_lens=ctx, device=DEV,
+                                       page_size=page_size, head_dim=head_dim)
+    _append(case)
+    args = (case.q, case.kv_pool, case.block_table, case.cu_q_lens, case.context_lens, case.max_q_len,
+            case.softmax_scale)
+    plain = ops.paged_prefill(*args, page_size=page_size, key_slices=1)
+    split = ops.paged_prefill(*args, page_size=page_size, key_slices=slices)
+    again = ops.paged_prefill(*args, page_size=page_size, key_slices=slices)
+    torch.cuda.synchronize()
+    ref = _oracle_paged(case)
+    assert_attention_close(split, ref, f"{slices} key slices")
+    assert_attention_close(plain, ref, "one slice")
+    assert torch.equal(split, again)
+    assert float((split.float() - plain.float()).abs().max()) <= 1e-3
+    # the workspace may be the caller's, and larger than needed
+    need = ops.paged_prefill_workspace_floats(case.q.shape[0], hq, head_dim, slices)
+    ws = torch.full((need + 64,), float("nan"), dtype=torch.float32, device=DEV)
+    mine = ops.paged_prefill(*args, page_size=page_size, key_slices=slices, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(mine, split)
+
+
+def test_key_slices_are_chosen_for_launches_that_leave_the_device_idle():
+    print("prefill key slice rule", flush=True)
+    lib = ops._lib.load()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    rule = lambda *a: int(lib.litekv_paged_prefill_key_slices(*a))
+    # 512 rows x 64/8 heads = 32 row blocks x 8 kv heads = 256 workgroups on 2 per compute unit
+    assert rule(1, 64, 8, 128, 512, 32768 + 512) == (2 * cus) // 256
+    assert rule(1, 64, 8, 128, 128, 32768) == min(8, (2 * cus) // 64)
+    assert rule(4, 64, 8, 128, 512, 32768) == 1                    # four such chunks fill it
+    assert rule(1, 64, 8, 128, 512, 700) == 1                      # too few keys to share out
+    assert rule(1, 64, 8, 128, 128, 64 * 32 * 3) == 3              # 32 key tiles per slice at least
+    assert rule(1, 64, 8, 128, 512, 2048 + 512) == 1               # two slices of 20 tiles would not pay
+    assert rule(1, 64, 8, 256, 128, 32768) == 1 and rule(1, 64, 8, 32, 128, 32768) == 1
+    assert rule(1, 32, 8, 64, 256, 16384) >= 2                     # head dim 64 has its own build
+    # chosen by default from what the block table can name
+    case = workloads.make_prefill_case("ksr", 7400, [256], 64, 8, context_lens=[6000], device=DEV)
+    _append(case)
+    auto = ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, case.context_lens,
+                             case.max_q_len, case.softmax_scale)
+    forced = ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, case.context_lens,
+                               case.max_q_len, case.softmax_scale,
+                               key_slices=rule(1, 64, 8, 128, 256, case.block_table.shape[1] * 16))
+    torch.cuda.synchronize()
+    assert torch.equal(auto, forced)
+    assert_attention_close(auto, _oracle_paged(case), "key slices by default")
+
+
+def test_key_slices_argument_errors():
+    print("prefill key slice errors", flush=True)
+    case = workloads.make_prefill_case("kse", 7500, [64], 16, 8, context_lens=[1024], device=DEV)
+    _append(case)
+    args = (case.q, case.kv_pool, case.block_table, case.cu_q_lens, case.context_lens, case.max_q_len,
+            case.softmax_scale)
+    with pytest.raises(ops._lib.LiteKVError, match="key_slices"):
+        ops.paged_prefill(*args, key_slices=9)
+    with pytest.raises(ValueError, match="workspace"):
+        ops.paged_prefill(*args, key_slices=2, workspace=torch.empty(16, dtype=torch.float32, device=DEV))
+    pool8 = torch.zeros(case.kv_pool.shape, dtype=torch.uint8, device=DEV)
+    scales = torch.ones(16, dtype=torch.float32, device=DEV)
+    with pytest.raises(ValueError, match="fp16 pool"):
+        ops.paged_prefill(case.q, pool8, case.block_table, case.cu_q_lens, case.context_lens, case.max_q_len,
+                          case.softmax_scale, kv_scales=scales, key_slices=2)
