@@ -50,7 +50,7 @@ extern "C" {
 #define LITEKV_ERR_INVALID_ARGUMENT 1
 #define LITEKV_ERR_LAUNCH 2
 
-#define LITEKV_ABI_VERSION 2
+#define LITEKV_ABI_VERSION 3
 
 /* ABI version of the loaded library (LITEKV_ABI_VERSION at build time). */
 int litekv_abi_version(void);
@@ -579,7 +579,7 @@ int litekv_paged_prefill_split(const void *q, int64_t q_token_stride,
                                float softmax_scale, void *stream);
 
 /*
- * The same over an fp8 (E4M3) pool with per-head scales (kv_scales: float32
+ * litekv_paged_prefill over an fp8 (E4M3) pool with per-head scales (kv_scales: float32
  * [2 * Hkv], K heads then V heads, value = code * scale), as written by
  * litekv_kv_append_fp8: the chunk rows of a chunked prefill or of a
  * prefix-cache hit attend to their history without the pages being

@@ -18,7 +18,7 @@ import torch  # noqa: F401
 
 LIB_PATH = Path(__file__).resolve().parent / "csrc" / "liblitekv.so"
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # name -> (restype, argtypes); mirrors include/litekv.h declaration by declaration.
 SIGNATURES = {

@@ -110,6 +110,34 @@ def test_chunked_prefill_matches_one_shot_prefill():
     assert_attention_close(got, ref, "chunked prefill")
 
 
+def test_lone_chunk_over_a_long_history_is_cut_along_its_keys():
+    """One request prefilled 128 rows at a time: from 4224 cached tokens on, the chunk's launch has
+    too few row blocks for the device and the attention layer's prefill call cuts it along its
+    keys (the executor's host-side lengths say how far the rows see). Every chunk against the
+    oracle on the whole prompt."""
+    print("executor: chunked prefill over a long history", flush=True)
+    attn = Attention(HQ, HKV, D)
+    n, chunk = 4608, 128
+    q, k, v = _qkv(n, 17)
+    ex = _executor(num_pages=320, layers=1, max_requests=2, max_seq_len=5120)
+    (rid,) = ex.reserve_paged_requests([chunk], reserved_lengths=[n])
+    ex.activate_paged_packed_prefill_batch((rid,), [chunk])
+    outs = [attn.context_forward(q[:chunk], k[:chunk], v[:chunk], ex.atten_info, 0, SCALE * LOG2E)]
+    sliced = 0
+    for done in range(chunk, n, chunk):
+        ex.activate_paged_chunk_prefill_batch((rid,), [done], [chunk])
+        info = ex.atten_info
+        sliced += int(ops._lib.load().litekv_paged_prefill_key_slices(1, HQ, HKV, D, chunk, int(info.max_actual_seq_len))) > 1
+        sl = slice(done, done + chunk)
+        outs.append(attn.context_forward(q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous(), info, 0,
+                                         SCALE * LOG2E))
+    torch.cuda.synchronize()
+    assert sliced >= 3                      # the last chunks see 4224 keys and more: two slices of 2048 at least
+    ref = c_oracle.varlen_prefill(to_np16(q), to_np16(k), to_np16(v), np.array([0], dtype=np.int32),
+                                  np.array([n], dtype=np.int32), SCALE)
+    assert_attention_close(torch.cat(outs), ref, "chunks over a growing history")
+
+
 def test_prefix_sharing_with_copy_on_write():
     print("executor: prefix sharing + COW", flush=True)
     ex = _executor(layers=1)
