@@ -546,7 +546,7 @@ int litekv_paged_prefill(const void *q, int64_t q_token_stride,
  * each; the slices leave fp32 partial rows + log-sum-exps in `workspace`, and
  * a second launch folds them in slice order (results do not depend on timing;
  * they differ from litekv_paged_prefill's within fp32 rounding of the merge).
- * fp16 pools, head_dim 64 or 128, 2 <= key_slices <= 8.
+ * head_dim 64 or 128, 2 <= key_slices <= 8.
  *
  *   litekv_paged_prefill_key_slices  the count that brings the launch's
  *       workgroups to the device's resident slots with at least 32 key tiles
@@ -577,6 +577,24 @@ int litekv_paged_prefill_split(const void *q, int64_t q_token_stride,
                                int64_t num_tokens, int32_t key_slices,
                                void *workspace, size_t workspace_bytes,
                                float softmax_scale, void *stream);
+
+/* litekv_paged_prefill_split over a pool of 8-bit codes with per-head scales
+ * (fp8 E4M3, or int8 when pool_is_int8 is not 0): see litekv_paged_prefill_fp8
+ * / _int8 below for the pool, litekv_paged_prefill_split for the rest. */
+int litekv_paged_prefill_split_q8(const void *q, int64_t q_token_stride,
+                                  const void *kv_pool, const float *kv_scales,
+                                  int32_t pool_is_int8,
+                                  const int32_t *block_table,
+                                  int32_t block_table_stride,
+                                  const int32_t *cu_q_lens,
+                                  const int32_t *context_lens, void *out,
+                                  int64_t out_token_stride, int32_t batch,
+                                  int32_t num_q_heads, int32_t num_kv_heads,
+                                  int32_t head_dim, int32_t page_size,
+                                  int64_t num_pages, int32_t max_q_len,
+                                  int64_t num_tokens, int32_t key_slices,
+                                  void *workspace, size_t workspace_bytes,
+                                  float softmax_scale, void *stream);
 
 /*
  * litekv_paged_prefill over an fp8 (E4M3) pool with per-head scales (kv_scales: float32

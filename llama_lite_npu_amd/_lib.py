@@ -197,6 +197,12 @@ SIGNATURES = {
          c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int64, c_int32, c_void_p, c_size_t,
          c_float, c_void_p],
     ),
+    "litekv_paged_prefill_split_q8": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
+         c_int32, c_int32, c_int32, c_int32, c_int32, c_int64, c_int32, c_int64, c_int32, c_void_p, c_size_t,
+         c_float, c_void_p],
+    ),
     "litekv_paged_prefill_fp8": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64,

@@ -87,10 +87,11 @@ class Attention:
         if chunked:
             return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens,
                                      atten_info.context_lens_i32, int(atten_info.max_actual_q_seq_len), scale,
-                                     kv_scales=scales, page_size=_page_size(atten_info))
+                                     kv_scales=scales, page_size=_page_size(atten_info),
+                                     max_kv_len=int(atten_info.max_actual_seq_len))
         return ops.paged_prefill(xq, pool, atten_info.block_table, atten_info.cu_q_lens, None,
                                  int(atten_info.max_actual_seq_len), scale, kv_scales=scales,
-                                 page_size=_page_size(atten_info))
+                                 page_size=_page_size(atten_info), max_kv_len=int(atten_info.max_actual_seq_len))
 
     def token_forward(self, xq, xk, xv, atten_info, layer_index: int, qk_scale=None) -> torch.Tensor:
         """Decode: xq [B, Hq, D], xk / xv [B, Hkv, D], one new token per sequence (None when

@@ -132,8 +132,8 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
   const bool fp8 = format != kKvF16;  // a pool of 8-bit codes
   LITEKV_REQUIRE(split.key_slices >= 1 && split.key_slices <= kMaxPrefillKeySlices,
                  "%s: key_slices %d out of [1, %d]", what, split.key_slices, kMaxPrefillKeySlices);
-  LITEKV_REQUIRE(split.key_slices == 1 || (!fp8 && (head_dim == 128 || head_dim == 64)),
-                 "%s: key slices take an fp16 pool and head_dim 64 or 128", what);
+  LITEKV_REQUIRE(split.key_slices == 1 || head_dim == 128 || head_dim == 64,
+                 "%s: key slices take head_dim 64 or 128", what);
 #if LITEKV_HD == 128
   if (head_dim == 64) {  // the head dim 64 build of this file
     return hd64_paged_prefill(what, q, q_token_stride, kv_pool, kv_scales, format, block_table, block_table_stride,
@@ -206,11 +206,20 @@ static int launch_paged_prefill(const char *what, const void *q, int64_t q_token
     float *part_lse = part_o + (size_t)slices * rows * num_q_heads * kHD;
     const PrefixTask task{part_o, part_lse, 0, (int32_t)rows, num_q_heads, 0, 0};
     const dim3 grid((unsigned)(num_kv_heads * s.head_splits), s.row_blocks * (unsigned)slices, (unsigned)batch);
-    hipLaunchKernelGGL(varlen_prefill_tiled_kernel<kPagedPrefillSplit>, grid, dim3(kTiledWaves * kWave), 0,
-                       static_cast<hipStream_t>(stream), static_cast<const half_t *>(q), q_token_stride,
-                       static_cast<half_t *>(out), out_token_stride, paged, packed, task, cu_q_lens,
-                       (const int32_t *)nullptr, context_lens, group, s.head_splits, s.heads_per_wg,
-                       s.row_tiles, softmax_scale * kLog2eP, slices);
+    auto launch_slices = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, grid, dim3(kTiledWaves * kWave), 0, static_cast<hipStream_t>(stream),
+                         static_cast<const half_t *>(q), q_token_stride, static_cast<half_t *>(out),
+                         out_token_stride, paged, packed, task, cu_q_lens, (const int32_t *)nullptr,
+                         context_lens, group, s.head_splits, s.heads_per_wg, s.row_tiles,
+                         softmax_scale * kLog2eP, slices);
+    };
+    if (format == kKvInt8) {
+      launch_slices(varlen_prefill_tiled_kernel<kPagedPrefillSplitInt8>);
+    } else if (format == kKvFp8) {
+      launch_slices(varlen_prefill_tiled_kernel<kPagedPrefillSplitFp8>);
+    } else {
+      launch_slices(varlen_prefill_tiled_kernel<kPagedPrefillSplit>);
+    }
     int rc2 = check_launch(what);
     if (rc2 != LITEKV_OK) return rc2;
     const int64_t merge_rows = rows * num_q_heads;
@@ -401,6 +410,28 @@ extern "C" int litekv_paged_prefill_split(const void *q, int64_t q_token_stride,
                                       out_token_stride, batch, num_q_heads, num_kv_heads, head_dim,
                                       page_size, num_pages, max_q_len, softmax_scale, stream,
                                       litekv::kKvF16, split);
+}
+
+extern "C" int litekv_paged_prefill_split_q8(const void *q, int64_t q_token_stride, const void *kv_pool,
+                                             const float *kv_scales, int32_t pool_is_int8,
+                                             const int32_t *block_table, int32_t block_table_stride,
+                                             const int32_t *cu_q_lens, const int32_t *context_lens,
+                                             void *out, int64_t out_token_stride, int32_t batch,
+                                             int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                             int32_t page_size, int64_t num_pages, int32_t max_q_len,
+                                             int64_t num_tokens, int32_t key_slices, void *workspace,
+                                             size_t workspace_bytes, float softmax_scale, void *stream) {
+  litekv::PrefillKeySplit split;
+  split.key_slices = key_slices;
+  split.workspace = workspace;
+  split.workspace_bytes = workspace_bytes;
+  split.num_tokens = num_tokens;
+  return litekv::launch_paged_prefill(pool_is_int8 ? "paged_prefill_split_int8" : "paged_prefill_split_fp8", q,
+                                      q_token_stride, kv_pool, kv_scales, block_table, block_table_stride,
+                                      cu_q_lens, context_lens, out, out_token_stride, batch, num_q_heads,
+                                      num_kv_heads, head_dim, page_size, num_pages, max_q_len,
+                                      softmax_scale, stream, pool_is_int8 ? litekv::kKvInt8 : litekv::kKvFp8,
+                                      split);
 }
 
 extern "C" int litekv_paged_prefill_fp8(const void *q, int64_t q_token_stride, const void *kv_pool,

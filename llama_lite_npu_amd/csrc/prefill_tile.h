@@ -142,7 +142,7 @@ __device__ __forceinline__ float vmax3(float a, float b, float c) {
 __device__ __forceinline__ float vmax2(float a, float b) { return __builtin_fmaxf(a, b); }
 constexpr int kPagedPrefill = 0, kPackedPrefill = 1, kSharedPrefix = 2, kPagedPrefillFp8 = 3,
               kSharedPrefixFp8 = 4, kPagedPrefillInt8 = 5, kSharedPrefixInt8 = 6,
-              kPagedPrefillSplit = 7;
+              kPagedPrefillSplit = 7, kPagedPrefillSplitFp8 = 8, kPagedPrefillSplitInt8 = 9;
 // kPagedPrefillSplit: a launch with too few row blocks to fill the device (one request's chunk
 // over a long history) cuts every block's keys into `key_slices` runs of tiles, one workgroup
 // each; a slice leaves a normalised fp32 partial row + log-sum-exp per (query row, head), and a
@@ -165,14 +165,18 @@ __device__ __forceinline__ void prefill_tile_body(
     int32_t heads_per_wg, int32_t row_tiles, float scale_log2, const int key_slice = 0,
     const int key_slices = 1) {
   constexpr bool PAGED = MODE != kPackedPrefill;
-  constexpr bool KSPLIT = MODE == kPagedPrefillSplit;  // causal prefill over one slice of the block's keys
+  // causal prefill over one slice of the block's keys
+  constexpr bool KSPLIT = MODE == kPagedPrefillSplit || MODE == kPagedPrefillSplitFp8 ||
+                          MODE == kPagedPrefillSplitInt8;
   // An fp8 pool cannot take the direct HBM -> LDS load: its codes go through registers, are
   // converted to fp16 (exactly) and written to LDS in the same swizzled layout, so everything
   // after the staging is shared. The K scale joins the softmax scale, the V scale the final
   // normalisation, as in the decode kernel.
   constexpr bool FP8 = MODE == kPagedPrefillFp8 || MODE == kSharedPrefixFp8 ||
-                       MODE == kPagedPrefillInt8 || MODE == kSharedPrefixInt8;  // 8-bit codes
-  constexpr int KV = (MODE == kPagedPrefillInt8 || MODE == kSharedPrefixInt8) ? kKvInt8 : kKvFp8;
+                       MODE == kPagedPrefillInt8 || MODE == kSharedPrefixInt8 ||
+                       MODE == kPagedPrefillSplitFp8 || MODE == kPagedPrefillSplitInt8;  // 8-bit codes
+  constexpr int KV = (MODE == kPagedPrefillInt8 || MODE == kSharedPrefixInt8 ||
+                      MODE == kPagedPrefillSplitInt8) ? kKvInt8 : kKvFp8;
   constexpr bool SHARED = MODE == kSharedPrefix || MODE == kSharedPrefixFp8 || MODE == kSharedPrefixInt8;
   // (rows of 64 codes staged by 8 wavefronts would leave a lane 8 codes, half a 16-byte load)
   static_assert(W == kTiledWaves || (W == kWideWaves && (!FP8 || kHD == 128)),
@@ -973,7 +977,8 @@ __global__ __launch_bounds__(W *kWave, W == kWideWaves ? 1 : (kHD == 64 ? 3 : 2)
     const int32_t *__restrict__ context_lens, int32_t group, int32_t head_splits,
     int32_t heads_per_wg, int32_t row_tiles, float scale_log2, int32_t key_slices) {
   __shared__ __attribute__((aligned(1024))) half_t lds_all[tile_lds_bytes<W>() / 2];
-  if constexpr (MODE == kPagedPrefillSplit) {
+  if constexpr (MODE == kPagedPrefillSplit || MODE == kPagedPrefillSplitFp8 ||
+                MODE == kPagedPrefillSplitInt8) {
     // blockIdx.y = row block * key_slices + slice: the slices of a block are neighbours
     const int by = (int)blockIdx.y / key_slices;
     prefill_tile_body<MODE, W>((uint32_t)(uintptr_t)(lds_half_t *)lds_all, (int)blockIdx.x, by,

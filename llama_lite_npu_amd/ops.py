@@ -632,7 +632,7 @@ def paged_prefill(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Ten
 
     A launch with too few query rows to fill the device (one request's chunk over a long history)
     is cut along the keys as well: ``key_slices`` workgroups per row block and a merge launch
-    (fp16 pools, head_dim 64 / 128). None lets the library choose from the launch shape and
+    (head_dim 64 / 128, any pool format). None lets the library choose from the launch shape and
     ``max_kv_len`` (the most keys a row sees: history + chunk; default: what the block table can
     name); 1 switches it off. ``workspace`` (float32, see ``paged_prefill_workspace_floats``) is
     allocated when not given."""
@@ -659,29 +659,37 @@ def paged_prefill(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Ten
     if out is None:
         out = torch.empty((t, hq, d), dtype=torch.float16, device=q.device)
     lib = _lib.load()
-    if fp8:
-        _need(key_slices in (None, 1), "key slices take an fp16 pool")
-        _lib.check(_q8_entry(lib, "paged_prefill", kv_pool)(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(block_table),
-                                                block_table.stride(0), _ptr(cu_q_lens), _ptr(context_lens),
-                                                _ptr(out), _rows("out", out), b, hq, hkv, d, page_size, n_pages,
-                                                int(max_q_len), float(softmax_scale), _stream()))
-        return out
     if key_slices is None:
         if max_kv_len is None:
             max_kv_len = block_table.shape[1] * page_size
         # a workgroup takes 128 (row, head) columns: beyond 512 of them the device is full as it is
         few_rows = 0 < t * hq <= 128 * 512
         key_slices = int(lib.litekv_paged_prefill_key_slices(b, hq, hkv, d, int(max_q_len), int(max_kv_len))) if few_rows else 1
-    if int(key_slices) > 1:
-        need = paged_prefill_workspace_floats(t, hq, d, int(key_slices))
+    key_slices = int(key_slices)
+    if key_slices > 1:
+        need = paged_prefill_workspace_floats(t, hq, d, key_slices)
         if workspace is None:
             workspace = torch.empty(need, dtype=torch.float32, device=q.device)
         _need(workspace.is_cuda and workspace.dtype == torch.float32 and workspace.is_contiguous() and
               workspace.numel() >= need, f"workspace must be {need} contiguous float32 on the device")
+    if fp8:
+        if key_slices > 1:
+            _lib.check(lib.litekv_paged_prefill_split_q8(
+                _ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), 1 if is_int8_pool(kv_pool) else 0,
+                _ptr(block_table), block_table.stride(0), _ptr(cu_q_lens), _ptr(context_lens), _ptr(out),
+                _rows("out", out), b, hq, hkv, d, page_size, n_pages, int(max_q_len), t, key_slices,
+                _ptr(workspace), workspace.numel() * 4, float(softmax_scale), _stream()))
+            return out
+        _lib.check(_q8_entry(lib, "paged_prefill", kv_pool)(_ptr(q), q_stride, _ptr(kv_pool), _ptr(kv_scales), _ptr(block_table),
+                                                block_table.stride(0), _ptr(cu_q_lens), _ptr(context_lens),
+                                                _ptr(out), _rows("out", out), b, hq, hkv, d, page_size, n_pages,
+                                                int(max_q_len), float(softmax_scale), _stream()))
+        return out
+    if key_slices > 1:
         _lib.check(lib.litekv_paged_prefill_split(_ptr(q), q_stride, _ptr(kv_pool), _ptr(block_table),
                                                   block_table.stride(0), _ptr(cu_q_lens), _ptr(context_lens),
                                                   _ptr(out), _rows("out", out), b, hq, hkv, d, page_size, n_pages,
-                                                  int(max_q_len), t, int(key_slices), _ptr(workspace),
+                                                  int(max_q_len), t, key_slices, _ptr(workspace),
                                                   workspace.numel() * 4, float(softmax_scale), _stream()))
         return out
     _lib.check(lib.litekv_paged_prefill(_ptr(q), q_stride, _ptr(kv_pool), _ptr(block_table),

@@ -455,3 +455,37 @@ def test_codes_of_rows_that_are_not_finite(dtype):
                      k_new=case.k_new, v_new=case.v_new)
     torch.cuda.synchronize()
     assert same_codes(fused), "append fused into the per-sequence step"
+
+
+@pytest.mark.parametrize("dtype", [torch.int8, torch.uint8])
+@pytest.mark.parametrize("head_dim", [128, 64])
+@pytest.mark.parametrize("hq,hkv,lens,ctx,slices", [
+    (64, 8, [256], [4096], 3),
+    (16, 8, [77, 20], [2100, 130], 4),
+    (8, 8, [130], [1500], 2),
+])
+def test_chunk_prefill_over_key_slices_of_a_pool_of_codes(dtype, head_dim, hq, hkv, lens, ctx, slices):
+    """A lone chunk over a long 8-bit history, cut along its keys: the oracle on the decoded pool,
+    the unsplit launch within 1e-3, the same bits twice."""
+    from oracle import fp8
+    codec = int8 if dtype == torch.int8 else fp8
+    print(f"{dtype} chunk prefill over {slices} key slices d={head_dim} {hq}/{hkv} {lens} ctx {ctx}", flush=True)
+    case = workloads.make_prefill_case("q8ks", 8800 + hq + slices, lens, hq, hkv, context_lens=ctx, device=DEV,
+                                       head_dim=head_dim)
+    scale = 1.0 / math.sqrt(head_dim)
+    scales = _head_scales(hkv) if dtype == torch.int8 else _head_scales(hkv, 6.0 / 448, 5.0 / 448)
+    pool = torch.empty(case.kv_pool.shape, dtype=dtype, device=DEV)
+    every_slot = torch.arange(pool.shape[0], dtype=torch.int32, device=DEV)
+    ops.kv_append_quantised(case.kv_pool[:, :hkv], case.kv_pool[:, hkv:], every_slot, pool, scales)
+    ops.kv_append_quantised(case.k, case.v, case.slot_mapping, pool, scales)
+    args = (case.q, pool, case.block_table, case.cu_q_lens, case.context_lens, case.max_q_len, scale)
+    plain = ops.paged_prefill(*args, kv_scales=scales, key_slices=1)
+    split = ops.paged_prefill(*args, kv_scales=scales, key_slices=slices)
+    again = ops.paged_prefill(*args, kv_scales=scales, key_slices=slices)
+    torch.cuda.synchronize()
+    values = torch.from_numpy(codec.dequantize_pool(pool.cpu().numpy(), scales.cpu().numpy()))
+    ref = cpu_ref.paged_prefill_ref(case.q.cpu(), values, case.block_table.cpu(), case.cu_q_lens.cpu(),
+                                    case.context_lens.cpu(), scale).numpy()
+    assert_attention_close(split, ref, f"{dtype} {slices} key slices")
+    assert torch.equal(split, again)
+    assert float((split.float() - plain.float()).abs().max()) <= 1e-3

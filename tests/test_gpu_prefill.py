@@ -351,8 +351,9 @@ def test_key_slices_argument_errors():
         ops.paged_prefill(*args, key_slices=9)
     with pytest.raises(ValueError, match="workspace"):
         ops.paged_prefill(*args, key_slices=2, workspace=torch.empty(16, dtype=torch.float32, device=DEV))
-    pool8 = torch.zeros(case.kv_pool.shape, dtype=torch.uint8, device=DEV)
-    scales = torch.ones(16, dtype=torch.float32, device=DEV)
-    with pytest.raises(ValueError, match="fp16 pool"):
-        ops.paged_prefill(case.q, pool8, case.block_table, case.cu_q_lens, case.context_lens, case.max_q_len,
-                          case.softmax_scale, kv_scales=scales, key_slices=2)
+    case32 = workloads.make_prefill_case("kse32", 7501, [64], 16, 8, context_lens=[1024], device=DEV, head_dim=32)
+    ops.kv_append(case32.k, case32.v, case32.slot_mapping, case32.kv_pool)
+    with pytest.raises(ops._lib.LiteKVError, match="head_dim"):
+        ops.paged_prefill(case32.q, case32.kv_pool, case32.block_table, case32.cu_q_lens, case32.context_lens,
+                          case32.max_q_len, case32.softmax_scale, key_slices=2,
+                          workspace=torch.empty(1 << 20, dtype=torch.float32, device=DEV))
