@@ -113,7 +113,7 @@ class DecodeLayerSet:
     balanced decode call with the KV append fused in (decode kernel + merge kernel)."""
 
     def __init__(self, case, layers: int, device: str, schedule: str = "balanced", shared_pages: int = 0,
-                 kv_dtype: str = "f16"):
+                 kv_dtype: str = "f16", splits: int = 1):
         import torch
         from llama_lite_npu_amd import _lib, ops
 
@@ -130,8 +130,8 @@ class DecodeLayerSet:
         self.fp8 = kv_dtype in ("fp8", "int8")       # 8-bit codes with one scale per head
         self.q8 = kv_dtype
         if self.fp8:
-            if schedule != "balanced":
-                raise ValueError("8-bit pools are read by the balanced schedule in this benchmark")
+            if schedule == "splits":
+                raise ValueError("8-bit pools are read with the append fused in in this benchmark")
             # E4M3 codes (no NaN codes) or int8 codes (no -128), and one scale per head
             if kv_dtype == "fp8":
                 pools = torch.randint(0, 0x7F, (layers, slots, 2 * hkv, 128), generator=gen, device=device,
@@ -193,6 +193,31 @@ class DecodeLayerSet:
                 ]
             self.plan_info = {"schedule": "balanced", "chunks": self.chunks, "shared_pages": shared_pages,
                               "kv_dtype": kv_dtype}
+        elif schedule == "per_sequence":
+            # `splits` wavefronts per (sequence, kv head) with the append fused in, then (more than
+            # one split) the merge launch; per-step metadata on the device as on the balanced schedule
+            self.max_splits = int(splits)
+            self.ws = ops.decode_workspace(b, hq, self.max_splits, device)
+            ws_ptr = None if self.ws is None else self.ws.data_ptr()
+            ws_bytes = 0 if self.ws is None else self.ws.numel() * 4
+            self.req_ids = torch.arange(b, dtype=torch.int32, device=device)
+            self.batch_table = torch.zeros_like(self.table)
+            self.slot_out = torch.empty(b, dtype=torch.int32, device=device)
+            self.pos_out = torch.empty(b, dtype=torch.int64, device=device)
+            self.advance_args = (self.table.data_ptr(), bts, b, self.req_ids.data_ptr(), None,
+                                 self.seq_lens.data_ptr(), None, self.slot_out.data_ptr(), self.pos_out.data_ptr(),
+                                 self.batch_table.data_ptr(), bts, self.table.shape[1], None, b, 16, c.num_pages,
+                                 0, stream)
+            scales = (self.scales.data_ptr(),) if self.fp8 else ()
+            self.decode_args = [
+                (self.q.data_ptr(), hq * 128, pools[l].data_ptr(), *scales, self.batch_table.data_ptr(), bts,
+                 self.seq_lens.data_ptr(), c.k_new.data_ptr(), c.v_new.data_ptr(), hkv * 128, hkv * 128,
+                 self.out[l].data_ptr(), ws_ptr, ws_bytes, b, hq, hkv, 128, 16, c.num_pages, self.max_splits, 1,
+                 c.softmax_scale, stream)
+                for l in range(layers)
+            ]
+            self.plan_info = {"schedule": "per_sequence", "splits_per_sequence": self.max_splits,
+                              "kv_dtype": kv_dtype}
         else:
             self.max_splits, self.min_pps = ops.decode_split_plan(b, hkv, self.table.shape[1], c.num_splits)
             self.ws = ops.decode_workspace(b, hq, self.max_splits, device)
@@ -214,8 +239,8 @@ class DecodeLayerSet:
 
     def step(self, events=None, stream=None):
         """One pass over all layers. `events[l]`: (start, stop) raw HIP events for layer l's decode kernel
-        (balanced) or 3 torch events bracketing split and merge (splits). `stream`: launch there
-        instead of the stream the set was built on (balanced only; used under graph capture)."""
+        (balanced, per_sequence) or 3 torch events bracketing split and merge (splits). `stream`:
+        launch there instead of the stream the set was built on (used under graph capture)."""
         lib = self.lib
         rc = 0
         if self.schedule == "balanced":
@@ -224,6 +249,16 @@ class DecodeLayerSet:
             rc |= lib.litekv_decode_plan_prefix(*on(self.plan_args))
             dec = (getattr(lib, "litekv_paged_decode_prefix_" + self.q8) if self.fp8
                    else lib.litekv_paged_decode_prefix)
+            prof = lib.litekv_profile_next_decode
+            for l in range(self.layers):
+                if events is not None:
+                    prof(events[l][0], events[l][1])
+                rc |= dec(*on(self.decode_args[l]))
+        elif self.schedule == "per_sequence":
+            on = (lambda a: a) if stream is None else (lambda a: a[:-1] + (stream,))
+            rc |= lib.litekv_decode_advance(*on(self.advance_args))
+            dec = (getattr(lib, "litekv_paged_decode_append_" + self.q8) if self.fp8
+                   else lib.litekv_paged_decode_append)
             prof = lib.litekv_profile_next_decode
             for l in range(self.layers):
                 if events is not None:
@@ -259,14 +294,14 @@ class DecodeLayerSet:
 
 def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: str,
                schedule: str = "balanced", shared_pages: int = 0, graph: bool = True,
-               kv_dtype: str = "f16") -> dict:
+               kv_dtype: str = "f16", splits: int = 1) -> dict:
     import torch
 
-    ls = DecodeLayerSet(case, layers, device, schedule, shared_pages, kv_dtype)
+    ls = DecodeLayerSet(case, layers, device, schedule, shared_pages, kv_dtype, splits)
     for _ in range(max(1, warmup)):
         ls.step()
     torch.cuda.synchronize()
-    balanced = schedule == "balanced"
+    balanced = schedule in ("balanced", "per_sequence")      # one fused call per layer, timed by its own events
     if balanced:
         hip = HipEvents()
         events = [[(hip.create(), hip.create()) for _ in range(layers)] for _ in range(steps)]
@@ -329,7 +364,7 @@ def run_decode(case, layers: int, steps: int, warmup: int, device: str, label: s
         "append_bytes_per_layer": append_bytes,
         "layers": layers,
         "roofline": {
-            "kernel": "paged_decode_balanced_kernel" if balanced else "paged_decode_split_kernel",
+            "kernel": "paged_decode_balanced_kernel" if schedule == "balanced" else "paged_decode_split_kernel",
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
@@ -701,11 +736,22 @@ def measure(name: str, args, device: str, cpu_budget_s: float, schedule=None, kv
         if args.chunks:
             case.extra["chunks"] = args.chunks
         shared = 0
-        if schedule == "balanced" and not args.no_shared_prefix and not case.extra.get("private_prefix"):
+        if schedule in ("auto", "balanced") and not args.no_shared_prefix and not case.extra.get("private_prefix"):
             shared = int(case.extra.get("n_shared", 0))
-        kv_dtype = (kv_dtype or args.kv_dtype) if schedule == "balanced" else "f16"
+        kv_dtype = (kv_dtype or args.kv_dtype) if schedule != "splits" else "f16"
+        splits = args.splits
+        if schedule == "auto":
+            # what the library's host rule picks for this step from the lengths the host knows
+            # (ops.DecodePlan.choose_schedule): balanced, or so many splits per sequence
+            from llama_lite_npu_amd import ops
+
+            pages = [(int(n) + 15) // 16 for n in case.seq_lens.tolist() if n > 0]
+            splits = 0 if shared > 0 or args.chunks else ops.decode_schedule(
+                case.batch, case.num_kv_heads, max(pages), sum(pages),
+                case.tok_bytes // (1 if kv_dtype == "f16" else 2), heads_per_kv_head=case.num_q_heads // case.num_kv_heads)
+            schedule = "per_sequence" if splits > 0 else "balanced"
         res = run_decode(case, layers, steps, warmup, device, case.name, schedule, shared,
-                         graph=not args.no_graph, kv_dtype=kv_dtype)
+                         graph=not args.no_graph, kv_dtype=kv_dtype, splits=splits)
     traffic, stamp = measured_traffic(name, schedule, kv_dtype)
     res["roofline"]["traffic_source"] = stamp
     if traffic is not None and (name != "c4" or not args.no_shared_prefix):
@@ -769,8 +815,11 @@ def main() -> int:
                     help="measure --config alone (default: the other configurations follow in detail.configs)")
     ap.add_argument("--all", action="store_true",
                     help="also write one line per configuration, same schema, to bench_all.jsonl under --out-dir")
-    ap.add_argument("--schedule", default="balanced", choices=["balanced", "splits"],
-                    help="decode work decomposition (splits: separate append, split and merge launches)")
+    ap.add_argument("--schedule", default="auto", choices=["auto", "balanced", "per_sequence", "splits"],
+                    help="decode work decomposition (auto: what the library's host rule picks for the step; "
+                         "per_sequence: --splits wavefronts per sequence and kv head with the append fused in; "
+                         "splits: the workload's split count as separate append, split and merge launches)")
+    ap.add_argument("--splits", type=int, default=1, help="splits per sequence of --schedule per_sequence")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--chunks", type=int, default=None,
                     help="balanced schedule: pieces per kv head (default: one workgroup per compute unit)")

@@ -11,12 +11,14 @@ extern "C" {
 #endif
 
 /*
- * No counterpart in the reference. The next litekv_paged_decode_balanced /
- * litekv_paged_decode_prefix launch (fp16 or fp8 pool) made by the calling
- * thread carries the two hipEvent_t handles as the start and stop events of its
- * decode kernel's own dispatch, so its device-side duration can be read with
- * hipEventElapsedTime without extra packets in the stream. The request is held
- * per thread until that launch consumes it; pass NULLs to cancel.
+ * No counterpart in the reference. The next decode launch of head dim 128 made
+ * by the calling thread -- litekv_paged_decode_balanced / _prefix, or the split
+ * launch of litekv_paged_decode / _split / _append, any pool format -- carries
+ * the two hipEvent_t handles as the start and stop events of its decode
+ * kernel's own dispatch (not the merge launch that may follow), so its
+ * device-side duration can be read with hipEventElapsedTime without extra
+ * packets in the stream. The request is held per thread until that launch
+ * consumes it; pass NULLs to cancel.
  */
 int litekv_profile_next_decode(void *start_event, void *stop_event);
 

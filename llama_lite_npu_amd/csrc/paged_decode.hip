@@ -1286,6 +1286,11 @@ static int device_cus() {
 }
 
 // fp8_scales: the scales of a pool of 8-bit codes of format `format` (kKvFp8, kKvInt8), or null.
+// Optional HIP events bracketing the next decode launch of this thread (the balanced kernel or the
+// per-sequence split kernel, not their merge launches): profiling.
+static thread_local hipEvent_t g_profile_start = nullptr;
+static thread_local hipEvent_t g_profile_stop = nullptr;
+
 static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pages_per_split,
                         const float *fp8_scales = nullptr, int format = kKvFp8) {
   const char *what = !fp8_scales          ? "paged_decode_split"
@@ -1344,8 +1349,10 @@ static int launch_split(const DecodeArgs &a, int32_t max_splits, int32_t min_pag
   }
   // The pool is written only by the instantiations with the fused append.
   void *pool = const_cast<void *>(a.kv_pool);
+  hipEvent_t ev0 = g_profile_start, ev1 = g_profile_stop;
+  g_profile_start = g_profile_stop = nullptr;
   auto launch = [&](auto kernel, auto *kv) {
-    hipLaunchKernelGGL(kernel, grid, block, lds, static_cast<hipStream_t>(a.stream),
+    hipExtLaunchKernelGGL(kernel, grid, block, lds, static_cast<hipStream_t>(a.stream), ev0, ev1, 0,
                        static_cast<const half_t *>(a.q), a.q_batch_stride, kv, fp8_scales,
                        a.block_table, a.block_table_stride, a.seq_lens,
                        static_cast<const half_t *>(a.k_new), static_cast<const half_t *>(a.v_new),
@@ -1508,10 +1515,6 @@ static int auto_prefix_chunks(int batch, int num_q_heads, int num_kv_heads, int 
   wgs = (wgs + s.head_groups - 1) / s.head_groups;
   return wgs * s.replicas;
 }
-
-// Optional HIP events bracketing the next balanced decode launch of this thread (profiling).
-static thread_local hipEvent_t g_profile_start = nullptr;
-static thread_local hipEvent_t g_profile_stop = nullptr;
 
 }  // namespace LITEKV_HD_NS
 }  // namespace litekv

@@ -167,12 +167,12 @@ class DeviceDecodeBatch:
             self._choose_schedule()
 
     def _choose_schedule(self) -> None:
-        """Balanced or per-sequence decode for the coming steps, from the host's lengths. The
-        schedule in use keeps a 10 % advantage so that a batch near the boundary does not flip
-        (a graph runner holds one graph per schedule)."""
+        """Balanced or per-sequence decode (and its split count) for the coming steps, from the
+        host's lengths. The schedule in use keeps a 10 % advantage so that a batch near a boundary
+        does not flip (a graph runner holds one graph per schedule)."""
         plan = self.decode_plan
         counts = self.executor.req_tokens_manager.req_token_count
-        plan.choose_schedule([counts[r] for r in self.request_ids], margin=1.0 if plan.per_sequence else 1.2)
+        plan.choose_schedule([counts[r] for r in self.request_ids], hysteresis=1.1)
 
     @property
     def max_actual_seq_len(self) -> int:
@@ -322,7 +322,7 @@ class DecodeGraphRunner:
         device = getattr(atten_info, "device_decode", None)
         plan = getattr(atten_info, "decode_plan", None)
         # a graph holds the kernels of the decode schedule it was captured with
-        per_sequence = bool(plan is not None and plan.per_sequence)
+        per_sequence = int(plan.schedule) if plan is not None else 0   # 0 balanced, else splits per sequence
         if device is not None:
             return key + (id(device), per_sequence)   # the graph is tied to that batch's tensors
         # Host-metadata steps replay through a static plan built at capture: the graph holds that
@@ -356,7 +356,7 @@ class DecodeGraphRunner:
                                               plan.num_kv_heads, plan.num_pages, plan.chunks, plan.page_size,
                                               plan.shared_pages, token_bytes=plan.token_bytes,
                                               kv_dtype=getattr(plan, "kv_dtype", None))
-            info.decode_plan.per_sequence = bool(plan.per_sequence)
+            info.decode_plan.set_schedule(plan.schedule)
         return info
 
     def capture(self, input_ids: torch.Tensor, position_ids: torch.Tensor, atten_info) -> bool:

@@ -57,13 +57,14 @@ def flash_decoding(q, k_cache, v_cache, qk_scale, b_req_tokens_table, b_seq_len,
     b = q.shape[0]
     cols = ((int(max_actual_seq_len) + PAGE_SIZE - 1) // PAGE_SIZE) * PAGE_SIZE
     table = _block_table_of(b_req_tokens_table[:b, :cols])
-    # The host knows the batch size and the longest sequence: for steps small enough (every
-    # sequence taken to be that long) one wavefront per sequence and kv head is the faster schedule.
+    # The host knows the batch size and the longest sequence: with every sequence taken to be that
+    # long, small steps go one or several wavefronts per sequence and kv head, the rest balanced.
     hkv, d = k_cache.shape[1], k_cache.shape[2]
     max_pages = cols // PAGE_SIZE
-    if ops.per_sequence_decode_is_faster(b, hkv, max_pages, b * max_pages, 2 * hkv * d * q.element_size(),
-                                         heads_per_kv_head=q.shape[1] // hkv):
-        return ops.paged_decode(q, pool, table, b_seq_len, float(qk_scale), num_splits=1, schedule="splits")
+    splits = ops.decode_schedule(b, hkv, max_pages, b * max_pages, 2 * hkv * d * q.element_size(),
+                                 heads_per_kv_head=q.shape[1] // hkv)
+    if splits:
+        return ops.paged_decode(q, pool, table, b_seq_len, float(qk_scale), num_splits=splits, schedule="splits")
     return ops.paged_decode(q, pool, table, b_seq_len, float(qk_scale))
 
 

@@ -287,11 +287,56 @@ def per_sequence_decode_is_faster(batch: int, num_kv_heads: int, max_pages: int,
     if batch <= 0 or total_pages <= 0:
         return False
     nbytes = float(total_pages) * page_size * token_bytes
-    per_sequence = max(5.0 + 0.57 * max_pages, 3.0 + nbytes / 5.0e6, 3.0 + 5.5e-3 * batch * num_kv_heads)
+    chain_pages = (max_pages * page_size + PAGE_SIZE - 1) // PAGE_SIZE     # the kernels step by 16 tokens
+    per_sequence = max(5.0 + 0.57 * chain_pages, 3.0 + nbytes / 5.0e6, 3.0 + 5.5e-3 * batch * num_kv_heads)
     balanced = 13.0 + nbytes / 5.6e6 + 0.03 * batch
     if heads_per_kv_head > 8:
         balanced *= 1.1
     return per_sequence * margin < balanced
+
+
+SPLIT_COUNTS = (4, 8, 16)
+
+
+def decode_schedule(batch: int, num_kv_heads: int, max_pages: int, total_pages: int, token_bytes: int,
+                    page_size: int = PAGE_SIZE, heads_per_kv_head: int = 8, current: Optional[int] = None,
+                    hysteresis: float = 1.0) -> int:
+    """Which decode schedule a step should take, from what the host knows about it: 0 = balanced,
+    1 = one wavefront per (sequence, kv head) in one launch, 4 / 8 / 16 = that many splits per
+    sequence and the merge launch.
+
+    The first two are estimated as in ``per_sequence_decode_is_faster``. Several splits per sequence
+    are for small batches, where the balanced schedule's fixed cost (plan look-ups, a merge over
+    every chunk of the device) is most of its time: 6.8 us for the two launches, the longest
+    sequence's pages per split at 0.63 us a page (a wavefront's dependent chain) against the bytes
+    at 6.1 MB/us, whichever is larger, and 1.5 ns per wavefront launched; splits are considered while
+    the launch has at most 2048 wavefronts. Where the bytes dominate, uneven sequences make uneven
+    splits which the balanced cut does not have, so the estimate grows by up to a quarter with the
+    bytes' share. Constants are fits to 290 measured shapes on an MI355X (1 to 128 sequences of 64
+    to 16384 tokens: equal, ragged, one long among short; 64/8 and 16/8 heads; every schedule
+    replayed from a graph): choosing by this rule is 1.7 % slower on average than always choosing
+    the fastest schedule (26 % at worst), the two-way rule 9 % (73 %). ``current``: the schedule in
+    use; the others must be estimated ``hysteresis`` times faster to replace it."""
+    if batch <= 0 or total_pages <= 0:
+        return 0
+    nbytes = float(total_pages) * page_size * token_bytes
+    chain_pages = (max_pages * page_size + PAGE_SIZE - 1) // PAGE_SIZE     # the kernels step by 16 tokens
+    estimates = {
+        0: (13.0 + nbytes / 5.6e6 + 0.03 * batch) * (1.1 if heads_per_kv_head > 8 else 1.0),
+        1: 1.1 * max(5.0 + 0.57 * chain_pages, 3.0 + nbytes / 5.0e6, 3.0 + 5.5e-3 * batch * num_kv_heads),
+    }
+    slices = (heads_per_kv_head + 15) // 16                                # wavefronts per kv head
+    for n in SPLIT_COUNTS:
+        wavefronts = batch * n * num_kv_heads * slices
+        if wavefronts > 2048:
+            continue
+        chain = 0.63 * ((chain_pages + n - 1) // n)
+        stream = nbytes / 6.1e6
+        both = (chain ** 3.2 + stream ** 3.2) ** (1.0 / 3.2)
+        estimates[n] = (6.8 + both + 1.5e-3 * wavefronts) * (1.0 + 0.25 * stream / (chain + stream))
+    if current in estimates:
+        estimates[current] /= hysteresis
+    return min(estimates, key=estimates.get)
 
 
 class DecodePlan:
@@ -300,8 +345,9 @@ class DecodePlan:
     Balanced schedule (default): the cut of the batch's pages into equal chunks (one launch), the
     device plan buffer (chunk entries) and the partial-result workspace. Launches that share a
     plan share its workspace and must run one after the other (same stream).
-    Per-sequence schedule (``per_sequence`` True, see ``choose_schedule``): nothing to build;
-    ``decode_step`` then runs one wavefront per (sequence, kv head), the append fused in.
+    Per-sequence schedule (``per_sequence`` True, see ``choose_schedule``): no cut to build;
+    ``decode_step`` then runs ``splits`` wavefronts per (sequence, kv head), the append fused in,
+    and with more than one split the merge launch over ``split_workspace``.
     """
 
     def __init__(self, block_table: torch.Tensor, seq_lens: torch.Tensor, num_q_heads: int,
@@ -312,13 +358,15 @@ class DecodePlan:
         """``shared_pages``: leading block-table entries that are the same physical pages in every
         row (a shared cached prefix); they are then attended once for the whole batch.
         ``host_seq_lens``: the lengths as the host knows them; with them the plan picks the
-        per-sequence schedule where ``per_sequence_decode_is_faster`` says so. ``token_bytes``:
+        per-sequence schedule (and its split count) where ``decode_schedule`` says so. ``token_bytes``:
         K + V bytes of one token in the pool (default: fp16). ``kv_dtype``: the pool's element type
         (default fp16); with a shared prefix it decides how the default chunk count is chosen."""
         lib = _lib.load()
         self.shared_pages = int(shared_pages)
         self.kv_dtype = kv_dtype
         self.per_sequence = False
+        self.splits = 1
+        self.split_workspace: Optional[torch.Tensor] = None
         self.token_bytes = int(token_bytes) if token_bytes is not None else 2 * int(num_kv_heads) * HEAD_DIM * 2
         _need(0 <= self.shared_pages <= block_table.shape[1], "shared_pages out of range")
         _need(block_table.dim() == 2, "block_table must be [B, max_blocks]")
@@ -350,16 +398,36 @@ class DecodePlan:
             self.choose_schedule(host_seq_lens)
         self.refresh()
 
-    def choose_schedule(self, host_seq_lens: Sequence[int], margin: float = 1.1) -> bool:
-        """Sets ``per_sequence`` from the lengths as the host knows them (no device read). A plan
-        with a shared prefix stays balanced. Returns the choice."""
+    def set_schedule(self, splits: int) -> None:
+        """0: balanced; otherwise the per-sequence schedule with that many splits per sequence
+        (the partial-result buffer of several splits is allocated here, not at the launch)."""
+        self.per_sequence = splits > 0
+        self.splits = max(1, int(splits))
+        if self.splits > 1:
+            need = int(_lib.load().litekv_paged_decode_workspace_bytes(self.batch, self.num_q_heads, HEAD_DIM,
+                                                                       self.splits)) // 4
+            if self.split_workspace is None or self.split_workspace.numel() < need:
+                self.split_workspace = torch.empty(need, dtype=torch.float32, device=self.block_table.device)
+
+    @property
+    def schedule(self) -> int:
+        """0 on the balanced schedule, else the splits per sequence."""
+        return self.splits if self.per_sequence else 0
+
+    def choose_schedule(self, host_seq_lens: Sequence[int], hysteresis: float = 1.0) -> bool:
+        """Sets the schedule from the lengths as the host knows them (no device read): see
+        ``decode_schedule``; the schedule in use keeps a ``hysteresis`` advantage. A plan with a
+        shared prefix stays balanced. Returns ``per_sequence``."""
         if self.shared_pages > 0:
-            self.per_sequence = False
+            self.set_schedule(0)
             return False
         pages = [(int(n) + self.page_size - 1) // self.page_size for n in host_seq_lens if n > 0]
-        self.per_sequence = bool(pages) and per_sequence_decode_is_faster(
-            self.batch, self.num_kv_heads, max(pages), sum(pages), self.token_bytes, self.page_size, margin,
-            self.num_q_heads // self.num_kv_heads)
+        if not pages:
+            self.set_schedule(0)
+            return False
+        self.set_schedule(decode_schedule(self.batch, self.num_kv_heads, max(pages), sum(pages), self.token_bytes,
+                                          self.page_size, self.num_q_heads // self.num_kv_heads,
+                                          current=self.schedule, hysteresis=hysteresis))
         return self.per_sequence
 
     def refresh(self, block_table: Optional[torch.Tensor] = None, seq_lens: Optional[torch.Tensor] = None) -> None:
@@ -430,10 +498,12 @@ def decode_step(q: torch.Tensor, kv_pool: torch.Tensor, plan: DecodePlan,
     """One layer of a decode step under ``plan``. Balanced schedule: optional append of k_new / v_new
     ([B, Hkv, D]) at logical position seq_lens[b] - 1 fused into the attention of q [B, Hq, D] over
     the planned pages, then the merge of the sequences that span several chunks. Per-sequence
-    schedule (``plan.per_sequence``): the same in one launch of one wavefront per (sequence, kv
-    head), no merge. An fp8 pool (uint8 / float8_e4m3fn) comes with its per-head ``kv_scales``."""
+    schedule (``plan.per_sequence``): the same by ``plan.splits`` wavefronts per (sequence, kv
+    head); one launch and no merge with one split. An fp8 pool (uint8 / float8_e4m3fn) comes with
+    its per-head ``kv_scales``."""
     if plan.per_sequence:
-        return paged_decode(q, kv_pool, plan.block_table, plan.seq_lens, softmax_scale, num_splits=1, out=out,
+        return paged_decode(q, kv_pool, plan.block_table, plan.seq_lens, softmax_scale, num_splits=plan.splits,
+                            out=out, workspace=plan.split_workspace if plan.splits > 1 else None,
                             page_size=plan.page_size, schedule="splits", kv_scales=kv_scales,
                             k_new=k_new, v_new=v_new)
     _dev_half("q", q)

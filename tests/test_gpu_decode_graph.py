@@ -173,7 +173,7 @@ def test_refused_row_appends_nothing_and_attends_nothing():
     case = workloads.make_decode_case("refused", 31, [30, 15, 47], HQ, HKV, device=DEV)
     capacity = torch.tensor([32, 15, 48], dtype=torch.int32, device=DEV)     # row 1: 15 cached, no room
     ids = torch.arange(3, dtype=torch.int32, device=DEV)
-    for per_sequence in (False, True):
+    for per_sequence in (0, 1, 4):                       # balanced, one wavefront, four splits per sequence
         pool = case.kv_pool.clone()
         seq = case.context_lens.to(DEV).to(torch.int32).clone()
         slot = torch.zeros(3, dtype=torch.int32, device=DEV)
@@ -183,7 +183,7 @@ def test_refused_row_appends_nothing_and_attends_nothing():
         torch.cuda.synchronize()
         assert seq.tolist() == [31, -1, 48] and int(flag.item()) == 1 and int(slot[1]) == -1
         plan = ops.DecodePlan(rows, seq, HQ, HKV, case.num_pages, chunks=5)
-        plan.per_sequence = per_sequence
+        plan.set_schedule(per_sequence)
         out = ops.decode_step(case.q, pool, plan, case.k_new, case.v_new, SCALE)
         torch.cuda.synchronize()
         want_pool = case.kv_pool.clone()                 # index assignment of the two live rows only
@@ -204,8 +204,13 @@ def test_refused_row_appends_nothing_and_attends_nothing():
         assert seq.tolist() == [32, -1, -1] and slot.tolist()[1:] == [-1, -1]
 
 
-def test_replayed_steps_equal_eager_steps_bit_for_bit():
-    print("graph replay (device metadata) vs eager host metadata", flush=True)
+@pytest.mark.parametrize("pinned", [0, 1, 8], ids=["balanced", "one_wavefront", "eight_splits"])
+def test_replayed_steps_equal_eager_steps_bit_for_bit(pinned, monkeypatch):
+    """Both executors are held on one decode schedule (the host rule would let the device batch keep
+    a schedule a little longer than a plan built afresh every step, and two schedules differ in the
+    order of their sums)."""
+    print(f"graph replay (device metadata) vs eager host metadata, schedule {pinned}", flush=True)
+    monkeypatch.setattr(ops, "decode_schedule", lambda *args, **kwargs: pinned)
     host, dev = _executor(), _executor()
     model_h, model_d = TinyModel(), TinyModel()
     lens = [1, 17, 48, 100, 31]

@@ -84,33 +84,75 @@ def test_fp8_pools_take_it_too():
     assert_attention_close(out_b, ref, "fp8 balanced")
 
 
-def test_graph_replay_follows_a_change_of_schedule():
-    """A small batch starts on the per-sequence schedule and outgrows it: the device batch moves
-    to the balanced one, the runner captures a second graph, and every step still matches an
-    executor that builds its metadata on the host."""
+def test_graph_replay_follows_a_change_of_schedule(monkeypatch):
+    """A small batch starts with one wavefront per sequence, moves to several splits per sequence
+    and then to the balanced schedule as it grows: the device batch follows, the runner captures
+    one graph per schedule, and every step still matches an executor that builds its metadata on
+    the host. (The thresholds are set by the test: the measured rule keeps four sequences off the
+    balanced schedule up to thousands of tokens.)"""
     from tests.test_gpu_decode_graph import TinyModel, _executor, _host_step, _next_tokens, _prefill
 
-    print("graph replay across a change of decode schedule", flush=True)
+    print("graph replay across changes of decode schedule", flush=True)
+
+    def by_longest(batch, num_kv_heads, max_pages, total_pages, token_bytes, page_size=16, heads_per_kv_head=8,
+                   current=None, hysteresis=1.0):
+        return 1 if max_pages <= 8 else 8 if max_pages <= 12 else 0
+
+    monkeypatch.setattr(ops, "decode_schedule", by_longest)
     host, graphed = _executor(num_pages=400, max_seq_len=512), _executor(num_pages=400, max_seq_len=512)
     model_h, model_g = TinyModel(), TinyModel()
     lens = [100, 20, 90, 5]
     ids_h, ids_g = _prefill(host, lens, 4), _prefill(graphed, lens, 4)
     graphed.attach_model(model_g, "qwen3")
     batch = graphed.activate_device_decode_batch(ids_g, reserve_tokens=32)
-    assert batch.decode_plan.per_sequence
+    assert batch.decode_plan.schedule == 1
     tok_h = tok_g = torch.tensor([[7], [8], [9], [10]], device=DEV)
-    seen = set()
+    seen = []
     for step in range(160):
         out_h = _host_step(host, model_h, ids_h, tok_h)
         graphed.extend_paged_requests(ids_g)
         out_g = graphed.forward(tok_g)
         torch.cuda.synchronize()
-        seen.add(batch.decode_plan.per_sequence)
+        if batch.decode_plan.schedule not in seen:
+            seen.append(batch.decode_plan.schedule)
         assert float((out_h - out_g).abs().max()) <= 3 * 2e-3, f"step {step}"     # three layers summed
         tok_h = tok_g = _next_tokens(out_h)
-    assert seen == {True, False} and not batch.decode_plan.per_sequence
-    assert graphed.graph_runner.capture_count == 2
+    assert seen == [1, 8, 0] and not batch.decode_plan.per_sequence
+    assert graphed.graph_runner.capture_count == 3
     batch.check()
+
+
+def test_small_batches_take_several_splits_per_sequence_with_the_same_result():
+    """Where the host rule picks several splits per sequence (a few sequences of some hundred
+    tokens), the step appends and attends like the balanced one: pool bit for bit, attention within
+    the tolerance of the oracle; a plan keeps its partial-result buffer between steps."""
+    for hq, hkv, lens in ((64, 8, [300, 1000, 37, 512]), (16, 8, [420, 16, 0, 777, 2100]), (32, 4, [900])):
+        print(f"several splits per sequence: heads {hq}/{hkv} lens {lens}", flush=True)
+        case = workloads.make_decode_case("sched", 36, lens, hq, hkv, device=DEV)
+        routed, balanced = _plans(case, hq, hkv, lens, token_bytes=2 * hkv * 128 * 2)
+        assert routed.per_sequence and routed.splits in ops.SPLIT_COUNTS and routed.schedule == routed.splits
+        assert routed.split_workspace is not None and balanced.schedule == 0
+        pool_a, pool_b = case.kv_pool.clone(), case.kv_pool.clone()
+        out_a = ops.decode_step(case.q, pool_a, routed, case.k_new, case.v_new, case.softmax_scale)
+        out_b = ops.decode_step(case.q, pool_b, balanced, case.k_new, case.v_new, case.softmax_scale)
+        torch.cuda.synchronize()
+        assert torch.equal(pool_a.view(torch.int16), pool_b.view(torch.int16))
+        ref = c_oracle.paged_decode(to_np16(case.q), to_np16(pool_a), case.block_table.cpu().numpy(),
+                                    case.seq_lens.cpu().numpy(), case.softmax_scale)
+        assert_attention_close(out_a, ref, "several splits")
+        assert_attention_close(out_b, ref, "balanced")
+        held = routed.split_workspace.data_ptr()
+        again = ops.decode_step(case.q, pool_a, routed, None, None, case.softmax_scale)
+        assert torch.equal(again, out_a) and routed.split_workspace.data_ptr() == held
+        # moving the plan to another split count (or back to balanced) needs no new plan
+        routed.set_schedule(4)
+        four = ops.decode_step(case.q, pool_a, routed, None, None, case.softmax_scale)
+        routed.set_schedule(0)
+        routed.refresh()
+        cut = ops.decode_step(case.q, pool_a, routed, None, None, case.softmax_scale)
+        torch.cuda.synchronize()
+        assert_attention_close(four, ref, "four splits")
+        assert_attention_close(cut, ref, "back to balanced")
 
 
 @pytest.mark.parametrize("splits", [1, 2, 5, 16])
@@ -166,10 +208,11 @@ def test_fused_append_argument_checks():
                          k_new=case.k_new[:1], v_new=case.v_new[:1])
 
 
-@pytest.mark.parametrize("lens", [[30, 100, 64, 7], [40, 2500, 900, 16]], ids=["short", "long"])
-def test_drop_in_flash_decoding_on_either_schedule(lens):
+@pytest.mark.parametrize("lens,expected", [([30, 100, 64, 7], 8), ([40, 2500, 900, 16], 16), ([40, 9000, 900, 16], 0)],
+                         ids=["short", "long", "longer"])
+def test_drop_in_flash_decoding_on_either_schedule(lens, expected):
     """The reference-signature wrapper picks the schedule from the batch size and the longest
-    sequence it is told; both choices give the oracle's attention."""
+    sequence it is told; each choice gives the oracle's attention."""
     from llama_lite_npu_amd import kernels as compat
 
     hq, hkv = 16, 8
@@ -180,9 +223,9 @@ def test_drop_in_flash_decoding_on_either_schedule(lens):
     # the reference's per-token table: slot of every logical position
     token_table = (case.block_table.long()[:, :, None] * 16 + torch.arange(16, device=DEV)).reshape(len(lens), -1)
     max_len = max(lens) + 1
-    picks_per_sequence = ops.per_sequence_decode_is_faster(len(lens), hkv, (max_len + 15) // 16,
-                                                           len(lens) * ((max_len + 15) // 16), 2 * hkv * 128 * 2)
-    assert picks_per_sequence == (max(lens) < 200)
+    picked = ops.decode_schedule(len(lens), hkv, (max_len + 15) // 16, len(lens) * ((max_len + 15) // 16),
+                                 2 * hkv * 128 * 2, heads_per_kv_head=hq // hkv)
+    assert picked == expected
     out = compat.flash_decoding(case.q, pool[:, :hkv], pool[:, hkv:], case.softmax_scale,
                                 token_table.to(torch.int32), case.seq_lens.long(), max_len)
     torch.cuda.synchronize()
