@@ -267,35 +267,49 @@ def prefix_chunks(batch: int, num_q_heads: int, num_kv_heads: int, shared_pages:
                                                              1 if fp16_pool else 0))
 
 
-def per_sequence_decode_is_faster(batch: int, num_kv_heads: int, max_pages: int, total_pages: int,
-                                  token_bytes: int, page_size: int = PAGE_SIZE, margin: float = 1.1,
-                                  heads_per_kv_head: int = 8) -> bool:
-    """Which of the two decode schedules a step should take, from what the host knows about it.
-
-    One wavefront per (sequence, kv head) (``num_splits=1`` of the splits schedule with the append
-    fused in: one launch, no merge) costs a dependent chain of page steps as long as the longest
-    sequence, the bytes at the rate such unbalanced streams reach, or the placement of its
-    wavefronts, whichever is largest. The balanced schedule (fused step + merge) costs two launches
-    whose fixed part is larger, the bytes at a higher rate, and a little per sequence. Constants
-    (us, bytes per us) are fits to 248 measured shapes on an MI355X (8 to 2048 sequences, 32 to 4096
-    tokens, uniform and ragged, 64/8 and 32/4 heads, each schedule replayed from a graph): choosing
-    by this rule is within 0.4 % of always choosing the faster schedule on average (worst case 14 %),
-    always balanced is 29 % slower on average. ``margin``: how much faster the per-sequence estimate
-    must be to be chosen. With more than 8 query heads per kv head the balanced schedule works on
-    two column tiles and merges twice the rows (measured 10 to 30 % slower, the other schedule
-    unchanged): its estimate grows by a tenth."""
-    if batch <= 0 or total_pages <= 0:
-        return False
-    nbytes = float(total_pages) * page_size * token_bytes
-    chain_pages = (max_pages * page_size + PAGE_SIZE - 1) // PAGE_SIZE     # the kernels step by 16 tokens
-    per_sequence = max(5.0 + 0.57 * chain_pages, 3.0 + nbytes / 5.0e6, 3.0 + 5.5e-3 * batch * num_kv_heads)
-    balanced = 13.0 + nbytes / 5.6e6 + 0.03 * batch
-    if heads_per_kv_head > 8:
-        balanced *= 1.1
-    return per_sequence * margin < balanced
-
-
 SPLIT_COUNTS = (4, 8, 16)
+
+
+def decode_schedule_estimates(batch: int, num_kv_heads: int, max_pages: int, total_pages: int, token_bytes: int,
+                              page_size: int = PAGE_SIZE, heads_per_kv_head: int = 8) -> dict:
+    """Estimated microseconds per layer of every decode schedule a step could take, keyed as
+    ``decode_schedule`` returns them. Fits to 554 measured shapes on an MI355X (1 to 2048 sequences
+    of 32 to 16384 tokens: equal, ragged, one long among short; 64/8 and 16/8 heads; every
+    schedule replayed from a graph; ``tune_decode_schedule`` re-measures the table):
+
+    * 1, one wavefront per (sequence, kv head), one launch: 4.2 us + the largest (a 2.3-norm) of the
+      longest sequence's dependent chain of 16-token steps at 0.6 us each, the placement of the
+      launch's wavefronts at 2.7 ns each, and the bytes at 5.9 MB/us (unbalanced streams).
+    * 4 / 8 / 16 splits per sequence + the merge launch, for launches of at most 2048 wavefronts:
+      6.8 us for the two launches, the chain of a split against the bytes at 6.1 MB/us (a 3.1-norm),
+      1.3 ns per wavefront; where the bytes dominate, uneven sequences make uneven splits, which
+      the balanced cut does not have: up to 15 % more with the bytes' share.
+    * 0, balanced (fused step + merge): 7.8 us, 0.15 us per piece the merge folds for the longest
+      sequence (up to 42), 3.3 ns + 0.26 ns per query head for every sequence, and the bytes at
+      6.7 MB/us against the chain inside one of the 256 chunks; a tenth more with over 8 query
+      heads per kv head (two column tiles, twice the rows to merge)."""
+    steps = max(1, page_size // PAGE_SIZE)                 # the kernels step by 16 tokens
+    chain = max_pages * steps
+    total = total_pages * steps
+    nbytes = float(total_pages) * page_size * token_bytes
+    num_q_heads = num_kv_heads * heads_per_kv_head
+    slices = (heads_per_kv_head + 15) // 16                # wavefronts per kv head
+    norm = lambda p, *xs: sum(x ** p for x in xs) ** (1.0 / p)
+    pieces = chain / max(1.0, total / 256.0)
+    estimates = {
+        0: (7.8 + 0.149 * min(pieces, 42.0) + (3.3e-3 + 2.6e-4 * num_q_heads) * batch
+            + norm(2.0, nbytes / 6.67e6, 0.605 * ((total + 255) // 256))) * (1.1 if heads_per_kv_head > 8 else 1.0),
+        1: 4.2 + norm(2.3, 0.605 * chain, 2.7e-3 * batch * num_kv_heads * slices, nbytes / 5.86e6),
+    }
+    for n in SPLIT_COUNTS:
+        wavefronts = batch * n * num_kv_heads * slices
+        if wavefronts > 2048:
+            continue
+        split_chain = 0.634 * ((chain + n - 1) // n)
+        stream = nbytes / 6.06e6
+        estimates[n] = ((6.76 + norm(3.1, split_chain, stream) + 1.3e-3 * wavefronts)
+                        * (1.0 + 0.15 * stream / (split_chain + stream)))
+    return estimates
 
 
 def decode_schedule(batch: int, num_kv_heads: int, max_pages: int, total_pages: int, token_bytes: int,
@@ -303,37 +317,14 @@ def decode_schedule(batch: int, num_kv_heads: int, max_pages: int, total_pages: 
                     hysteresis: float = 1.0) -> int:
     """Which decode schedule a step should take, from what the host knows about it: 0 = balanced,
     1 = one wavefront per (sequence, kv head) in one launch, 4 / 8 / 16 = that many splits per
-    sequence and the merge launch.
-
-    The first two are estimated as in ``per_sequence_decode_is_faster``. Several splits per sequence
-    are for small batches, where the balanced schedule's fixed cost (plan look-ups, a merge over
-    every chunk of the device) is most of its time: 6.8 us for the two launches, the longest
-    sequence's pages per split at 0.63 us a page (a wavefront's dependent chain) against the bytes
-    at 6.1 MB/us, whichever is larger, and 1.5 ns per wavefront launched; splits are considered while
-    the launch has at most 2048 wavefronts. Where the bytes dominate, uneven sequences make uneven
-    splits which the balanced cut does not have, so the estimate grows by up to a quarter with the
-    bytes' share. Constants are fits to 290 measured shapes on an MI355X (1 to 128 sequences of 64
-    to 16384 tokens: equal, ragged, one long among short; 64/8 and 16/8 heads; every schedule
-    replayed from a graph): choosing by this rule is 1.7 % slower on average than always choosing
-    the fastest schedule (26 % at worst), the two-way rule 9 % (73 %). ``current``: the schedule in
-    use; the others must be estimated ``hysteresis`` times faster to replace it."""
-    if batch <= 0 or total_pages <= 0:
+    sequence and the merge launch: the smallest of ``decode_schedule_estimates``. Choosing by this
+    rule is 1.1 % slower on average than always choosing the fastest schedule on the measured
+    shapes (29 % at worst); always balanced is 19 % slower on average. ``current``: the schedule
+    in use; another must be estimated ``hysteresis`` times faster to replace it."""
+    if batch <= 0 or total_pages <= 0 or max_pages <= 0:
         return 0
-    nbytes = float(total_pages) * page_size * token_bytes
-    chain_pages = (max_pages * page_size + PAGE_SIZE - 1) // PAGE_SIZE     # the kernels step by 16 tokens
-    estimates = {
-        0: (13.0 + nbytes / 5.6e6 + 0.03 * batch) * (1.1 if heads_per_kv_head > 8 else 1.0),
-        1: 1.1 * max(5.0 + 0.57 * chain_pages, 3.0 + nbytes / 5.0e6, 3.0 + 5.5e-3 * batch * num_kv_heads),
-    }
-    slices = (heads_per_kv_head + 15) // 16                                # wavefronts per kv head
-    for n in SPLIT_COUNTS:
-        wavefronts = batch * n * num_kv_heads * slices
-        if wavefronts > 2048:
-            continue
-        chain = 0.63 * ((chain_pages + n - 1) // n)
-        stream = nbytes / 6.1e6
-        both = (chain ** 3.2 + stream ** 3.2) ** (1.0 / 3.2)
-        estimates[n] = (6.8 + both + 1.5e-3 * wavefronts) * (1.0 + 0.25 * stream / (chain + stream))
+    estimates = decode_schedule_estimates(batch, num_kv_heads, max_pages, total_pages, token_bytes, page_size,
+                                          heads_per_kv_head)
     if current in estimates:
         estimates[current] /= hysteresis
     return min(estimates, key=estimates.get)

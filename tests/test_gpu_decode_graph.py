@@ -264,8 +264,11 @@ def test_replayed_steps_equal_eager_steps_bit_for_bit(pinned, monkeypatch):
     assert _pools_equal(host, dev)
 
 
-def test_host_metadata_steps_replay_through_static_copies():
+def test_host_metadata_steps_replay_through_static_copies(monkeypatch):
     print("graph replay (host metadata, static copies) vs eager", flush=True)
+    # one decode schedule for the whole run: a change of schedule is a graph of its own, which
+    # test_graph_replay_follows_a_change_of_schedule covers
+    monkeypatch.setattr(ops, "decode_schedule", lambda *args, **kwargs: 1)
     host, graphed = _executor(), _executor()
     model_h, model_g = TinyModel(), TinyModel()
     lens = [30, 5, 64]
@@ -312,11 +315,12 @@ def _shared_prefix_batch(ex, model):
     return tuple(batch_ids)
 
 
-def test_graph_of_a_shared_prefix_batch_is_not_replayed_for_a_batch_sharing_nothing():
+def test_graph_of_a_shared_prefix_batch_is_not_replayed_for_a_batch_sharing_nothing(monkeypatch):
     """Host-metadata steps replay through a static plan made at capture. A batch that shares a
     cached prefix and a batch of the same size that shares nothing need different plans: each
     must get its own graph, every replay equal to the eager step bit for bit."""
     print("graph replay: shared-prefix batch, then a same-size batch without one", flush=True)
+    monkeypatch.setattr(ops, "decode_schedule", lambda *args, **kwargs: 1)   # the private batch on one schedule
     host, graphed = _executor(num_pages=200, max_requests=8), _executor(num_pages=200, max_requests=8)
     model_h, model_g = TinyModel(), TinyModel()
     shared_h, shared_g = _shared_prefix_batch(host, model_h), _shared_prefix_batch(graphed, model_g)

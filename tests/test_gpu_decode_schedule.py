@@ -49,7 +49,7 @@ def test_short_batches_take_the_per_sequence_schedule_with_the_same_result(hq, h
 
 def test_long_sequences_and_shared_prefixes_stay_balanced():
     print("per-sequence schedule: cases that must not take it", flush=True)
-    lens = [37, 128, 511, 3000]
+    lens = [37, 128, 511, 12000]
     case = workloads.make_decode_case("sched", 32, lens, 16, 8, device=DEV)
     routed, _ = _plans(case, 16, 8, lens)
     assert not routed.per_sequence
