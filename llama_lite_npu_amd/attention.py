@@ -6,8 +6,9 @@ arguments, driven by the same ``AttentionInfo``. Differences:
 
 * no ``torch.cat([xk, xv])``: K and V rows go to the pool straight from their own tensors;
 * decode follows the step's ``DecodePlan``: one fused launch (append + attention) and a merge
-  on the balanced schedule, or an append and one wavefront per (sequence, kv head) where the
-  plan found the step small enough for that to be faster;
+  on the balanced schedule, or the append fused into one wavefront (no merge) or several splits
+  (+ merge) per (sequence, kv head) where the plan found the step small enough for that to be
+  faster;
 * prefill reads K/V through the block table (context 0 for a fresh prompt, history for later
   chunks), so one kernel serves both branches of the reference;
 * ``qkv_epilogue`` folds the step before the append (QK RMSNorm, rotary embedding,
