@@ -752,7 +752,7 @@ def measure(name: str, args, device: str, cpu_budget_s: float, schedule=None, kv
             schedule = "per_sequence" if splits > 0 else "balanced"
         res = run_decode(case, layers, steps, warmup, device, case.name, schedule, shared,
                          graph=not args.no_graph, kv_dtype=kv_dtype, splits=splits)
-    traffic, stamp = measured_traffic(name, schedule, kv_dtype)
+    traffic, stamp = measured_traffic(name, None if name == "c3" else schedule, kv_dtype)
     res["roofline"]["traffic_source"] = stamp
     if traffic is not None and (name != "c4" or not args.no_shared_prefix):
         if name == "c3":
