@@ -277,9 +277,11 @@ def decode_schedule_estimates(batch: int, num_kv_heads: int, max_pages: int, tot
     of 32 to 16384 tokens: equal, ragged, one long among short; 64/8 and 16/8 heads; every
     schedule replayed from a graph; ``tune_decode_schedule`` re-measures the table):
 
-    * 1, one wavefront per (sequence, kv head), one launch: 4.2 us + the largest (a 2.3-norm) of the
-      longest sequence's dependent chain of 16-token steps at 0.6 us each, the placement of the
-      launch's wavefronts at 2.7 ns each, and the bytes at 5.9 MB/us (unbalanced streams).
+    * 1, one wavefront per (sequence, kv head), one launch: 4.3 us + the largest (a 3.6-norm) of the
+      longest sequence's dependent chain of 16-token steps at 0.58 us each -- up to half as much
+      again when the launch has 2048 wavefronts or more, whose loads share the compute units'
+      memory paths with the chain's --, the placement of the launch's wavefronts at 2.9 ns each,
+      and the bytes at 5.7 MB/us (unbalanced streams).
     * 4 / 8 / 16 splits per sequence + the merge launch, for launches of at most 2048 wavefronts:
       6.8 us for the two launches, the chain of a split against the bytes at 6.1 MB/us (a 3.1-norm),
       1.3 ns per wavefront; where the bytes dominate, uneven sequences make uneven splits, which
@@ -295,11 +297,12 @@ def decode_schedule_estimates(batch: int, num_kv_heads: int, max_pages: int, tot
     num_q_heads = num_kv_heads * heads_per_kv_head
     slices = (heads_per_kv_head + 15) // 16                # wavefronts per kv head
     norm = lambda p, *xs: sum(x ** p for x in xs) ** (1.0 / p)
+    lone = batch * num_kv_heads * slices                   # wavefronts of a launch with one per sequence
     pieces = chain / max(1.0, total / 256.0)
     estimates = {
         0: (7.8 + 0.149 * min(pieces, 42.0) + (3.3e-3 + 2.6e-4 * num_q_heads) * batch
             + norm(2.0, nbytes / 6.67e6, 0.605 * ((total + 255) // 256))) * (1.1 if heads_per_kv_head > 8 else 1.0),
-        1: 4.2 + norm(2.3, 0.605 * chain, 2.7e-3 * batch * num_kv_heads * slices, nbytes / 5.86e6),
+        1: 4.27 + norm(3.6, 0.584 * chain * (1.0 + 0.49 * min(1.0, lone / 2048.0)), 2.9e-3 * lone, nbytes / 5.70e6),
     }
     for n in SPLIT_COUNTS:
         wavefronts = batch * n * num_kv_heads * slices
@@ -319,7 +322,8 @@ def decode_schedule(batch: int, num_kv_heads: int, max_pages: int, total_pages: 
     1 = one wavefront per (sequence, kv head) in one launch, 4 / 8 / 16 = that many splits per
     sequence and the merge launch: the smallest of ``decode_schedule_estimates``. Choosing by this
     rule is 1.1 % slower on average than always choosing the fastest schedule on the measured
-    shapes (29 % at worst); always balanced is 19 % slower on average. ``current``: the schedule
+    shapes (29 % at worst; 1.4 to 1.7 % and 29 to 34 % on three head layouts the constants were not
+    fitted on); always balanced is 19 % slower on average. ``current``: the schedule
     in use; another must be estimated ``hysteresis`` times faster to replace it."""
     if batch <= 0 or total_pages <= 0 or max_pages <= 0:
         return 0
