@@ -611,6 +611,47 @@ def run_prefill(case, steps: int, warmup: int, device: str, label: str) -> dict:
     }
 
 
+def time_chunk_prefill(device: str, rows: int = 128, history: int = 32768, hq: int = 64, hkv: int = 8) -> dict:
+    """One request's prefill chunk (the reference's chunked prefill) of `rows` tokens over `history`
+    cached tokens: too few query rows to fill the device, so the library also cuts the launch along
+    the keys (ops.paged_prefill, key_slices chosen by the library) -- timed beside the same launch
+    with the cut switched off. Median of 20 launches each, torch events around each launch."""
+    import torch
+    from llama_lite_npu_amd import _lib, ops
+
+    g = torch.Generator(device=device).manual_seed(77)
+    pages = (history + rows + 15) // 16
+    pool = torch.empty((pages * 16, 2 * hkv, 128), dtype=torch.float16, device=device).normal_(generator=g)
+    q = torch.empty((rows, hq, 128), dtype=torch.float16, device=device).normal_(generator=g)
+    table = torch.randperm(pages, generator=g, device=device).to(torch.int32).reshape(1, pages)
+    cu = torch.tensor([0, rows], dtype=torch.int32, device=device)
+    ctx = torch.tensor([history], dtype=torch.int32, device=device)
+    out = torch.empty_like(q)
+    slices = int(_lib.load().litekv_paged_prefill_key_slices(1, hq, hkv, 128, rows, history + rows))
+    ws = torch.empty(max(4, ops.paged_prefill_workspace_floats(rows, hq, 128, max(slices, 1))), dtype=torch.float32,
+                     device=device)
+
+    def timed(key_slices):
+        run = lambda: ops.paged_prefill(q, pool, table, cu, ctx, rows, None, out=out, key_slices=key_slices,
+                                        workspace=ws if key_slices > 1 else None)
+        for _ in range(3):
+            run()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(20)]
+        for a, b in evs:
+            a.record()
+            run()
+            b.record()
+        torch.cuda.synchronize()
+        return _median([a.elapsed_time(b) for a, b in evs]) * 1e3
+
+    flops = 4.0 * hq * 128 * rows * (history + (rows + 1) / 2.0)
+    plain, cut = timed(1), timed(slices)
+    return {"chunk_prefill": {"rows": rows, "history_tokens": history, "key_slices": slices,
+                              "us_uncut": plain, "us": cut, "tflops": flops / (cut * 1e-6) / 1e12,
+                              "tflops_uncut": flops / (plain * 1e-6) / 1e12}}
+
+
 def cpu_baseline_decode(case, budget_s: float = 10.0, max_sequences=None, kv_dtype: str = "f16") -> dict:
     """The reference's torch CPU path (append + gathered fp32 attention) for ONE layer of `case`,
     on the host cores: 1 warm-up, then repetitions for about `budget_s` seconds, min taken.
@@ -797,6 +838,7 @@ def measure(name: str, args, device: str, cpu_budget_s: float, schedule=None, kv
         row["pct_of_mfma_peak"] = 100.0 * res["roofline"]["frac"]
         row["detail"].update(time_qk_epilogue(int(case.seq_lens.sum()), case.num_q_heads, case.num_kv_heads,
                                               case.slot_mapping, case.kv_pool))
+        row["detail"].update(time_chunk_prefill(device))
         if not args.no_cpu_baseline:
             row["cpu_baseline"] = cpu_baseline_prefill(case, cpu_budget_s)
     del case
