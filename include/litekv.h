@@ -548,11 +548,12 @@ int litekv_paged_prefill(const void *q, int64_t q_token_stride,
  * they differ from litekv_paged_prefill's within fp32 rounding of the merge).
  * head_dim 64 or 128, 2 <= key_slices <= 8.
  *
- *   litekv_paged_prefill_key_slices  the count that brings the launch's
- *       workgroups to the device's resident slots with at least 32 key tiles
- *       (2048 keys) per slice when the longest row sees max_kv_len keys;
- *       1: do not split
- *       (call litekv_paged_prefill)
+ *   litekv_paged_prefill_key_slices  the count with the smallest estimated
+ *       time when the longest row sees max_kv_len keys (history + chunk):
+ *       key tiles per workgroup at the rate its share of a compute unit
+ *       gives, against a merge launch and a partial row per query row, head
+ *       and slice; 1: do not split (call litekv_paged_prefill) -- launches
+ *       that fill the device, short histories, fresh prompts
  *   num_tokens    T, the query rows of the launch (= cu_q_lens[batch])
  *   workspace     litekv_paged_prefill_split_workspace_bytes(T, Hq, D,
  *                 key_slices) bytes, 16-byte aligned; launches that share it

@@ -83,17 +83,22 @@ static size_t prefill_split_workspace_bytes(int64_t num_tokens, int32_t num_q_he
   return (size_t)key_slices * (size_t)num_tokens * (size_t)num_q_heads * (kHD + 1) * sizeof(float);
 }
 
-// Key slices that fill the device for a paged prefill whose row blocks alone would not: as many as
-// bring its workgroups to the device's resident slots, at most kMaxPrefillKeySlices, each with at
-// least 32 key tiles (2048 keys) if the longest row sees `max_kv_len` keys: a slice costs a partial
-// row (fp32) written and read back per query row and head, and the launch a merge. 1 means: do
-// not split. (64 query / 8 kv heads, one request's chunk over 32k cached tokens, plain against
-// sliced: 128 rows 527 -> 176 us, 256 rows 533 -> 298 us, 512 rows 609 -> 551 us; 512 rows over
-// 2048 tokens in two slices 77 -> 90 us, which the 32 tiles rule out.)
+// Key slices for a paged prefill whose row blocks alone would not fill the device, if the longest
+// row sees `max_kv_len` keys: the count (at most kMaxPrefillKeySlices) with the smallest estimated
+// time, 1 (do not split) unless that is at least 5 % less than unsplit. The estimate, in
+// microseconds, head dim 128 (fits to one request's chunk of 64 to 512 rows over 0 to 32k cached
+// tokens, 64 query / 8 kv heads): a workgroup walks max_kv_len / 64 / n key tiles at 1.0 us each
+// while it has its compute unit to itself and at 1.7 us once the launch has more workgroups than
+// compute units (two share one), times the rounds the launch needs on the device's resident
+// slots; a cut costs the merge launch, 6 us, and a partial row (fp32) written and read back per
+// query row, head and slice at 6 MB/us. (One chunk over 32k tokens, plain against sliced:
+// 128 rows 527 -> 176 us, 256 rows 533 -> 298 us, 512 rows 609 -> 551 us; 128 rows over 2048 tokens
+// 40 -> 30 us in four slices; 512 rows over 2048 tokens in two slices 49 -> 60 us and 128 rows of a
+// fresh prompt in eight 14 -> 29 us, which the estimate rules out.)
 static int32_t prefill_key_slices(int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
                                   int32_t max_q_len, int64_t max_kv_len) {
   if (batch <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0 ||
-      max_q_len <= 0 || num_q_heads / num_kv_heads > kMaxGroup) {
+      max_q_len <= 0 || max_kv_len <= 0 || num_q_heads / num_kv_heads > kMaxGroup) {
     return 1;
   }
   const PrefillShape s = prefill_shape(num_q_heads / num_kv_heads, max_q_len, kColTiles * kTiledWaves);
@@ -110,13 +115,28 @@ static int32_t prefill_key_slices(int32_t batch, int32_t num_q_heads, int32_t nu
     cached_device = dev;
     cached_cus = cus;
   }
-  const int64_t slots = (int64_t)cached_cus * (kHD == 64 ? 3 : 2);
+  const int64_t cus = cached_cus;
+  const int64_t slots = cus * (kHD == 64 ? 3 : 2);
   if (2 * wgs > slots) return 1;
-  int64_t n = slots / wgs;
-  n = n < kMaxPrefillKeySlices ? n : kMaxPrefillKeySlices;
-  const int64_t tiles = max_kv_len / kKvTile;
-  while (n > 1 && tiles / n < 32) --n;
-  return (int32_t)n;
+  const double tile_us = kHD == 64 ? 0.6 : 1.0;
+  const double tiles = (double)((max_kv_len + kKvTile - 1) / kKvTile);
+  const double partial_us = (double)batch * max_q_len * num_q_heads * (kHD + 1) * 2.0 * sizeof(float) / 6.0e6;
+  auto estimate = [&](int64_t n) {
+    const int64_t resident = wgs * n;
+    const double per_tile = resident <= cus ? tile_us : 1.7 * tile_us * (double)((resident + slots - 1) / slots);
+    return tiles / (double)n * per_tile + (n > 1 ? 6.0 + partial_us * (double)n : 0.0);
+  };
+  const double unsplit = estimate(1);
+  int64_t best = 1;
+  double best_us = 0.95 * unsplit;
+  for (int64_t n = 2; n <= kMaxPrefillKeySlices; ++n) {
+    const double t = estimate(n);
+    if (t < best_us) {
+      best = n;
+      best_us = t;
+    }
+  }
+  return (int32_t)best;
 }
 
 // Causal chunk attention over paged KV; `kv_scales` selects the fp8 pool.

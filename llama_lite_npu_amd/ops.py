@@ -698,8 +698,8 @@ def paged_prefill(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Ten
     A launch with too few query rows to fill the device (one request's chunk over a long history)
     is cut along the keys as well: ``key_slices`` workgroups per row block and a merge launch
     (head_dim 64 / 128, any pool format). None lets the library choose from the launch shape and
-    ``max_kv_len`` (the most keys a row sees: history + chunk; default: what the block table can
-    name); 1 switches it off. ``workspace`` (float32, see ``paged_prefill_workspace_floats``) is
+    ``max_kv_len`` (the most keys a row sees: history + chunk, as the host knows it; without it
+    the launch is not cut); 1 switches it off. ``workspace`` (float32, see ``paged_prefill_workspace_floats``) is
     allocated when not given."""
     _dev_half("q", q)
     fp8 = is_quantised_pool(kv_pool)
@@ -725,10 +725,10 @@ def paged_prefill(q: torch.Tensor, kv_pool: torch.Tensor, block_table: torch.Ten
         out = torch.empty((t, hq, d), dtype=torch.float16, device=q.device)
     lib = _lib.load()
     if key_slices is None:
-        if max_kv_len is None:
-            max_kv_len = block_table.shape[1] * page_size
-        # a workgroup takes 128 (row, head) columns: beyond 512 of them the device is full as it is
-        few_rows = 0 < t * hq <= 128 * 512
+        # a workgroup takes 128 (row, head) columns: beyond 512 of them the device is full as it is;
+        # and without the lengths on the host there is nothing to choose by (what the block table
+        # could name says little: a fresh prompt cut into eight slices takes twice as long)
+        few_rows = 0 < t * hq <= 128 * 512 and max_kv_len is not None
         key_slices = int(lib.litekv_paged_prefill_key_slices(b, hq, hkv, d, int(max_q_len), int(max_kv_len))) if few_rows else 1
     key_slices = int(key_slices)
     if key_slices > 1:

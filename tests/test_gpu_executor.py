@@ -111,10 +111,10 @@ def test_chunked_prefill_matches_one_shot_prefill():
 
 
 def test_lone_chunk_over_a_long_history_is_cut_along_its_keys():
-    """One request prefilled 128 rows at a time: from 4224 cached tokens on, the chunk's launch has
-    too few row blocks for the device and the attention layer's prefill call cuts it along its
-    keys (the executor's host-side lengths say how far the rows see). Every chunk against the
-    oracle on the whole prompt."""
+    """One request prefilled 128 rows at a time: a chunk's launch has too few row blocks for the
+    device, and once the history is long enough for a cut to pay the attention layer's prefill call
+    cuts it along its keys (the executor's host-side lengths say how far the rows see). Every chunk
+    against the oracle on the whole prompt."""
     print("executor: chunked prefill over a long history", flush=True)
     attn = Attention(HQ, HKV, D)
     n, chunk = 4608, 128
@@ -132,7 +132,7 @@ def test_lone_chunk_over_a_long_history_is_cut_along_its_keys():
         outs.append(attn.context_forward(q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous(), info, 0,
                                          SCALE * LOG2E))
     torch.cuda.synchronize()
-    assert sliced >= 3                      # the last chunks see 4224 keys and more: two slices of 2048 at least
+    assert sliced >= 3                      # the last chunks see 4224 keys and more
     ref = c_oracle.varlen_prefill(to_np16(q), to_np16(k), to_np16(v), np.array([0], dtype=np.int32),
                                   np.array([n], dtype=np.int32), SCALE)
     assert_attention_close(torch.cat(outs), ref, "chunks over a growing history")

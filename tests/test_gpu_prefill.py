@@ -320,24 +320,33 @@ def test_key_slices_are_chosen_for_launches_that_leave_the_device_idle():
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     rule = lambda *a: int(lib.litekv_paged_prefill_key_slices(*a))
     # 512 rows x 64/8 heads = 32 row blocks x 8 kv heads = 256 workgroups on 2 per compute unit
-    assert rule(1, 64, 8, 128, 512, 32768 + 512) == (2 * cus) // 256
-    assert rule(1, 64, 8, 128, 128, 32768) == min(8, (2 * cus) // 64)
+    assert rule(1, 64, 8, 128, 128, 32768) >= 4
+    if cus == 256:
+        assert rule(1, 64, 8, 128, 512, 32768 + 512) == 2         # measured 609 -> 551 us
+        assert rule(1, 64, 8, 128, 128, 32768) == 8               # 64 workgroups: eight slices fill the slots
+        assert rule(1, 64, 8, 128, 128, 2048 + 128) == 4           # measured 40 -> 30 us
+        assert rule(1, 64, 8, 128, 64, 8192 + 64) == 8             # measured 130 -> 36 us
     assert rule(4, 64, 8, 128, 512, 32768) == 1                    # four such chunks fill it
     assert rule(1, 64, 8, 128, 512, 700) == 1                      # too few keys to share out
-    assert rule(1, 64, 8, 128, 128, 64 * 32 * 3) == 3              # 32 key tiles per slice at least
-    assert rule(1, 64, 8, 128, 512, 2048 + 512) == 1               # two slices of 20 tiles would not pay
+    assert rule(1, 64, 8, 128, 512, 2048 + 512) == 1               # two slices would not pay (49 -> 60 us)
+    assert rule(1, 64, 8, 128, 512, 4096 + 512) == 1               # nor here (82 -> 88 us)
+    for rows in (64, 128, 256, 512):                               # a fresh prompt is never cut (14 -> 29 us in eight)
+        assert rule(1, 64, 8, 128, rows, rows) == 1 and rule(1, 64, 8, 128, rows, 256 + rows) == 1
     assert rule(1, 64, 8, 256, 128, 32768) == 1 and rule(1, 64, 8, 32, 128, 32768) == 1
     assert rule(1, 32, 8, 64, 256, 16384) >= 2                     # head dim 64 has its own build
-    # chosen by default from what the block table can name
+    # chosen by default from the longest row's keys as the caller knows them; not at all without them
     case = workloads.make_prefill_case("ksr", 7400, [256], 64, 8, context_lens=[6000], device=DEV)
     _append(case)
-    auto = ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, case.context_lens,
-                             case.max_q_len, case.softmax_scale)
-    forced = ops.paged_prefill(case.q, case.kv_pool, case.block_table, case.cu_q_lens, case.context_lens,
-                               case.max_q_len, case.softmax_scale,
-                               key_slices=rule(1, 64, 8, 128, 256, case.block_table.shape[1] * 16))
+    args = (case.q, case.kv_pool, case.block_table, case.cu_q_lens, case.context_lens, case.max_q_len,
+            case.softmax_scale)
+    picked = rule(1, 64, 8, 128, 256, 6256)
+    assert picked > 1
+    auto = ops.paged_prefill(*args, max_kv_len=6256)
+    forced = ops.paged_prefill(*args, key_slices=picked)
+    blind = ops.paged_prefill(*args)
+    plain = ops.paged_prefill(*args, key_slices=1)
     torch.cuda.synchronize()
-    assert torch.equal(auto, forced)
+    assert torch.equal(auto, forced) and torch.equal(blind, plain)
     assert_attention_close(auto, _oracle_paged(case), "key slices by default")
 
 
