@@ -838,7 +838,8 @@ def measure(name: str, args, device: str, cpu_budget_s: float, schedule=None, kv
         row["pct_of_mfma_peak"] = 100.0 * res["roofline"]["frac"]
         row["detail"].update(time_qk_epilogue(int(case.seq_lens.sum()), case.num_q_heads, case.num_kv_heads,
                                               case.slot_mapping, case.kv_pool))
-        row["detail"].update(time_chunk_prefill(device))
+        if not args.no_chunk_prefill:
+            row["detail"].update(time_chunk_prefill(device))
         if not args.no_cpu_baseline:
             row["cpu_baseline"] = cpu_baseline_prefill(case, cpu_budget_s)
     del case
@@ -870,6 +871,9 @@ def main() -> int:
     ap.add_argument("--kv-dtype", default="f16", choices=["f16", "fp8", "int8"],
                     help="storage of the KV pools (fp8: E4M3 codes, int8: signed codes, both with per-head "
                          "scales; decode configs only)")
+    ap.add_argument("--no-chunk-prefill", action="store_true",
+                    help="c3: skip the chunk-over-a-long-history launches timed beside the workload (they run the "
+                         "same kernel at another shape, which a per-kernel profile of the run would mix in)")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the leg that replays the decode step as one HIP graph")
     ap.add_argument("--out-dir", default="bench_out",
