@@ -322,7 +322,7 @@ def decode_schedule(batch: int, num_kv_heads: int, max_pages: int, total_pages: 
     1 = one wavefront per (sequence, kv head) in one launch, 4 / 8 / 16 = that many splits per
     sequence and the merge launch: the smallest of ``decode_schedule_estimates``. Choosing by this
     rule is 1.1 % slower on average than always choosing the fastest schedule on the measured
-    shapes (29 % at worst; 1.4 to 1.7 % and 29 to 34 % on three head layouts the constants were not
+    shapes (30 % at worst; 1.3 to 1.7 % and 27 to 32 % on three head layouts the constants were not
     fitted on); always balanced is 19 % slower on average. ``current``: the schedule
     in use; another must be estimated ``hysteresis`` times faster to replace it."""
     if batch <= 0 or total_pages <= 0 or max_pages <= 0:
