@@ -997,6 +997,98 @@ __device__ __forceinline__ void merge_row_wide(const float *__restrict__ lse, in
   if (live_col) *(half2_t *)(out_row + mcol) = half2_t{(half_t)(o0 * inv), (half_t)(o1 * inv)};
 }
 
+// The same merge with the row's elements shared out among kMergeDimSlices workgroups of 32
+// elements each, for steps of a few long sequences: their rows are few (one per query head and
+// sequence) and one workgroup per row reads its 256 pieces through a single compute unit's memory
+// path (a 16k-token sequence alone: 6.7 us of a 22 us layer, on 64 of 256 compute units). Sixteen
+// lanes read the slice's 128 bytes of a piece, so the 256 threads take 16 pieces per load and each
+// thread every sixteenth piece, all its loads in flight at once for up to 256 pieces; the sixteen
+// partial sums are added in index order by the first sixteen lanes.
+constexpr int kMergeSliceDims = 32;
+constexpr int kMergeDimSlices = kHD / kMergeSliceDims;
+constexpr int kMergeRedFloats = 8 + 16 * kMergeSliceDims + 16 > 8 + kMergeWaves * kHD + kMergeWaves
+                                    ? 8 + 16 * kMergeSliceDims + 16
+                                    : 8 + kMergeWaves * kHD + kMergeWaves;
+
+__device__ __forceinline__ void merge_row_sliced(const float *__restrict__ lse, int64_t lse_stride,
+                                                 const float *__restrict__ po, int64_t po_stride,
+                                                 int n_parts, half_t *out_row, int tid, int slice,
+                                                 float *red) {
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int l16 = tid & 15;
+  const int r = tid >> 4;  // 0..15: which of 16 pieces per sweep
+  const int col = slice * kMergeSliceDims + 2 * l16;
+  float den = 0.f, num0 = 0.f, num1 = 0.f;
+  auto block_max = [&](float mx) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, xor_lane(mx, off));
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  };
+  // the thread's pieces base, base + 16, ...: their log-sum-exps and its two elements of their rows
+  auto request = [&](int base, float (&l)[16], float2 (&row)[16]) {
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int s = base + 16 * u;
+      const bool live = s < n_parts;
+      const int at = live ? s : base;
+      l[u] = live ? lse[(int64_t)at * lse_stride] : -INFINITY;
+      row[u] = *(const float2 *)(po + (int64_t)at * po_stride + col);
+    }
+  };
+  auto add = [&](const float (&l)[16], const float2 (&row)[16], float mx) {
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const float w = fast_exp2((l[u] - mx) * kLog2e);  // 0 for a piece past the end
+      den += w;
+      num0 += w * row[u].x;
+      num1 += w * row[u].y;
+    }
+  };
+  if (n_parts <= 256) {
+    // one sweep: rows and log-sum-exps are requested together, the maximum comes from the
+    // log-sum-exps the threads hold (every piece is held by sixteen of them): one round trip
+    float l[16];
+    float2 row[16];
+    request(r < n_parts ? r : 0, l, row);
+    float mine = -INFINITY;
+    if (r < n_parts) {
+#pragma unroll
+      for (int u = 0; u < 16; ++u) mine = fmaxf(mine, l[u]);
+    }
+    const float mx = block_max(mine);
+    if (r < n_parts) add(l, row, mx);
+  } else {
+    float mine = -INFINITY;
+    for (int s = tid; s < n_parts; s += kMergeWaves * kWave) mine = fmaxf(mine, lse[(int64_t)s * lse_stride]);
+    const float mx = block_max(mine);
+    for (int base = r; base < n_parts; base += 256) {
+      float l[16];
+      float2 row[16];
+      request(base, l, row);
+      add(l, row, mx);
+    }
+  }
+  float *sums = red + 8;  // [16][kMergeSliceDims], then the sixteen denominators
+  sums[r * kMergeSliceDims + 2 * l16] = num0;
+  sums[r * kMergeSliceDims + 2 * l16 + 1] = num1;
+  if (l16 == 0) sums[16 * kMergeSliceDims + r] = den;
+  __syncthreads();
+  if (tid >= 16) return;
+  float d = 0.f, o0 = 0.f, o1 = 0.f;
+#pragma unroll
+  for (int r2 = 0; r2 < 16; ++r2) {
+    o0 += sums[r2 * kMergeSliceDims + 2 * l16];
+    o1 += sums[r2 * kMergeSliceDims + 2 * l16 + 1];
+    d += sums[16 * kMergeSliceDims + r2];
+  }
+  const float inv = 1.0f / d;
+  typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+  *(half2_t *)(out_row + col) = half2_t{(half_t)(o0 * inv), (half_t)(o1 * inv)};
+}
+
 // Balanced-schedule merge, one workgroup per (query head, sequence) -- or, without a shared
 // prefix and with more sequences than chunk boundaries, per (query head, boundary): only a
 // sequence that crosses a boundary has pieces to merge -- : combines the sequence's
@@ -1009,7 +1101,7 @@ __global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merg
     const float *__restrict__ part_lse, const float *__restrict__ pre_o,
     const float *__restrict__ pre_lse, int32_t pre_splits, int32_t batch, int32_t num_q_heads,
     int32_t by_boundary, int32_t bt_stride, int32_t chunks, int32_t heads_per_wg) {
-  __shared__ float red[8 + kMergeWaves * kHD + kMergeWaves];
+  __shared__ float red[kMergeRedFloats];
   // heads_per_wg 1: the workgroup has one row (query head); 4: each wavefront has its own
   const int hq = blockIdx.x * heads_per_wg + (heads_per_wg > 1 ? (int)(threadIdx.x >> 6) : 0);
   int b = blockIdx.y;
@@ -1033,6 +1125,16 @@ __global__ __launch_bounds__(kMergeWaves *kWave) void paged_decode_balanced_merg
   const int64_t pre0 = (int64_t)b * num_q_heads + hq;
   const int64_t pre_step = (int64_t)batch * num_q_heads;
   half_t *out_row = out + ((int64_t)b * num_q_heads + hq) * kHD;
+  if (gridDim.z > 1) {
+    // the launch shares a long row's elements out among the workgroups z (heads_per_wg is 1);
+    // any other row is the first one's alone
+    if (pre_splits == 0 && n_parts > 16) {
+      merge_row_sliced(part_lse + cell0, num_q_heads, part_o + cell0 * kHD, (int64_t)num_q_heads * kHD,
+                       n_parts, out_row, threadIdx.x, (int)blockIdx.z, red);
+      return;
+    }
+    if (blockIdx.z != 0) return;
+  }
   if (pre_splits == 0 && n_parts > 16 && blockDim.x == kMergeWaves * kWave) {  // uniform in the workgroup
     // a long row takes the whole workgroup; with a row per wavefront the rows take turns
     for (int r = 0; r < heads_per_wg; ++r) {
@@ -1805,8 +1907,15 @@ static int launch_balanced(const char *what, const void *q, int64_t q_batch_stri
                            (int64_t)merge_rows * num_q_heads >= 8192)
                               ? kMergeWaves
                               : 1;
+  // Few rows that may be long (a handful of long sequences): a row's elements go to
+  // kMergeDimSlices workgroups, so that its pieces are read through as many compute units
+  // (see merge_row_sliced); with more rows than that the workgroups already cover the device.
+  const int dim_slices = (merge_waves == kMergeWaves && merge_heads == 1 &&
+                          (int64_t)merge_rows * num_q_heads * kMergeDimSlices <= 4 * (int64_t)device_cus())
+                             ? kMergeDimSlices
+                             : 1;
   hipLaunchKernelGGL(paged_decode_balanced_merge_kernel,
-                     dim3((unsigned)(num_q_heads / merge_heads), (unsigned)merge_rows),
+                     dim3((unsigned)(num_q_heads / merge_heads), (unsigned)merge_rows, (unsigned)dim_slices),
                      dim3(merge_waves * kWave), 0,
                      static_cast<hipStream_t>(stream), static_cast<const int32_t *>(plan), seq_lens,
                      static_cast<half_t *>(out), part_o, part_lse, pre_o, pre_lse, pre_splits,

@@ -286,9 +286,10 @@ def decode_schedule_estimates(batch: int, num_kv_heads: int, max_pages: int, tot
       6.8 us for the two launches, the chain of a split against the bytes at 6.1 MB/us (a 3.1-norm),
       1.3 ns per wavefront; where the bytes dominate, uneven sequences make uneven splits, which
       the balanced cut does not have: up to 15 % more with the bytes' share.
-    * 0, balanced (fused step + merge): 7.8 us, 0.15 us per piece the merge folds for the longest
-      sequence (up to 42), 3.3 ns + 0.26 ns per query head for every sequence, and the bytes at
-      6.7 MB/us against the chain inside one of the 256 chunks; a tenth more with over 8 query
+    * 0, balanced (fused step + merge): 7.6 us, 0.17 us per piece the merge folds for the longest
+      sequence (up to 36; 0.06 us where a step of few rows shares a long row out among several
+      workgroups), 3.4 ns + 0.26 ns per query head for every sequence, and the bytes at
+      6.8 MB/us against the chain inside one of the 256 chunks; a tenth more with over 8 query
       heads per kv head (two column tiles, twice the rows to merge)."""
     steps = max(1, page_size // PAGE_SIZE)                 # the kernels step by 16 tokens
     chain = max_pages * steps
@@ -299,9 +300,11 @@ def decode_schedule_estimates(batch: int, num_kv_heads: int, max_pages: int, tot
     norm = lambda p, *xs: sum(x ** p for x in xs) ** (1.0 / p)
     lone = batch * num_kv_heads * slices                   # wavefronts of a launch with one per sequence
     pieces = chain / max(1.0, total / 256.0)
+    # rows of more than 16 pieces are merged by several workgroups each while the step has few rows
+    per_piece = 0.057 if pieces > 16 and batch * num_q_heads <= 256 else 0.170
     estimates = {
-        0: (7.8 + 0.149 * min(pieces, 42.0) + (3.3e-3 + 2.6e-4 * num_q_heads) * batch
-            + norm(2.0, nbytes / 6.67e6, 0.605 * ((total + 255) // 256))) * (1.1 if heads_per_kv_head > 8 else 1.0),
+        0: (7.6 + per_piece * min(pieces, 36.0) + (3.4e-3 + 2.6e-4 * num_q_heads) * batch
+            + norm(2.0, nbytes / 6.81e6, 0.82 * ((total + 255) // 256))) * (1.1 if heads_per_kv_head > 8 else 1.0),
         1: 4.27 + norm(3.6, 0.584 * chain * (1.0 + 0.49 * min(1.0, lone / 2048.0)), 2.9e-3 * lone, nbytes / 5.70e6),
     }
     for n in SPLIT_COUNTS:

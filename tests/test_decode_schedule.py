@@ -23,10 +23,14 @@ def test_many_short_sequences_take_one_wavefront_each():
 
 
 def test_small_batches_take_several_splits_per_sequence():
-    # measured: 1 to 8 sequences of 256 to 2048 tokens run 1.3 to 1.5 times faster in 8 or 16 splits
+    # measured: 1 to 8 sequences of 256 to 1024 tokens run 1.2 to 1.5 times faster in 8 or 16 splits
     for batch in (1, 2, 4, 8):
-        for tokens in (256, 1024, 2048):
+        for tokens in (256, 1024):
             assert uniform(batch, tokens) in (8, 16), (batch, tokens)
+    assert uniform(8, 2048) in (8, 16)
+    # from a few thousand tokens on, a step of few rows merges its long rows over several workgroups
+    # and the balanced cut is the faster one again
+    assert uniform(1, 4096) == 0 and uniform(2, 8192) == 0 and uniform(4, 8192) == 0
     c1 = [38, 129, 512, 1001]
     assert decode_schedule(4, 8, max(map(pages, c1)), sum(map(pages, c1)), TOK, heads_per_kv_head=2) in (8, 16)
 

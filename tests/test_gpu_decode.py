@@ -657,3 +657,26 @@ def test_prefix_chunk_count_leaves_room_for_the_prefix_role():
                           torch.full((64,), 2100, dtype=torch.int32, device=DEV), 64, 8, 4096,
                           shared_pages=128, kv_dtype=torch.float16)
     assert plan.chunks == c4
+
+
+@pytest.mark.parametrize("head_dim", [128, 64])
+@pytest.mark.parametrize("hq,hkv", [(64, 8), (16, 2)])
+def test_few_long_sequences_merge_their_many_pieces(hq, hkv, head_dim):
+    """One to three long sequences on the balanced schedule: each spans far more than 16 chunks,
+    and with so few rows the merge shares every row's elements out among several workgroups (more
+    than 256 pieces: several sweeps). A short and an empty sequence ride along (fewer pieces: the
+    ordinary paths of the same launch). Against the oracle, and twice bit for bit; nine such
+    sequences take the one-workgroup-per-row merge of long rows."""
+    for lens, chunks in (([9000], None), ([5000, 70, 0, 4100], None), ([9000, 3000, 33], 700), ([2600] * 9, None)):
+        print(f"long rows {hq}/{hkv} d{head_dim} lens {lens} chunks {chunks}", flush=True)
+        case = workloads.make_decode_case("long", 1300 + hq + head_dim, lens, hq, hkv, device=DEV, head_dim=head_dim)
+        ops.kv_append(case.k_new, case.v_new, case.slot_mapping, case.kv_pool)
+        for i, n in enumerate(lens):
+            if n == 0:
+                case.seq_lens[i] = 0
+        ref = _oracle(case)
+        kw = dict(schedule="balanced") if chunks is None else dict(schedule="balanced", chunks=chunks)
+        out = _run(case, **kw)
+        again = _run(case, **kw)
+        assert torch.equal(out, again)
+        assert_attention_close(out, ref, f"long rows {lens}")
